@@ -1,0 +1,260 @@
+/*
+ * sdk_mapped_ops.h - C ABI of the MI355X (gfx950) mapped-operation backend.
+ *
+ * One shared library, libsdk_mapped_ops.so, built from hand-written HIP
+ * kernels.  Every entry point takes plain device pointers, sizes and a HIP
+ * stream; no torch (or any other framework) type crosses this boundary.
+ *
+ * The entry points are what the reference package's per-family pybind11
+ * extension modules (package `_spherical_distortion_ext`, reference setup.py:62-199)
+ * bind for the device side of this path: each comment cites the reference
+ * interface the function replaces (paths relative to the reference tree).
+ *
+ * Conventions
+ *   - All tensors are dense, row-major ("contiguous NCHW"); device memory.
+ *   - sample_map holds (x, y) pairs in pixel units, x = column, y = row, with
+ *     the data's floating type.  Unweighted layout [..., 2] is selected by
+ *     num_interp_pts == 0; weighted layout [..., P, 2] with interp_weights
+ *     [..., P] by num_interp_pts == P >= 1 (interp_weights must be non-NULL).
+ *   - interp: 0 nearest (round half away from zero, no wrap), 1 bilinear
+ *     (out-of-range taps read as zero / are dropped), 2 bispherical (bilinear
+ *     whose columns wrap modulo the width; rows are still bounds-checked).
+ *     Any other value behaves as nearest, like the reference's switch default
+ *     (ext_modules/include/core/resample.h:48-50, :72-76).
+ *   - dtype: SDK_F32 or SDK_F64 for data, map and weights alike.
+ *   - Outputs are fully written by the call (scatter targets are zero-filled
+ *     first, on the same stream); inputs are never modified.
+ *   - All work is enqueued on `stream` (a hipStream_t, NULL = default stream)
+ *     and the call returns without synchronising.
+ *   - Return value: SDK_OK (0) or a negative sdk_status; sdk_last_error()
+ *     gives the message of the calling thread's most recent failure.  The
+ *     reference prints and calls std::exit(-1) on a device error
+ *     (ext_modules/include/cuda_helper.h:5-10); this library returns instead.
+ *   - A plane (H*W, or OH*OW) must have fewer than 2^31 elements.
+ */
+#ifndef SDK_MAPPED_OPS_H_
+#define SDK_MAPPED_OPS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sdk_status {
+  SDK_OK = 0,
+  SDK_ERR_INVALID_ARGUMENT = -1, /* NULL pointer, bad size, unknown dtype */
+  SDK_ERR_UNSUPPORTED = -2,      /* valid request this build cannot serve */
+  SDK_ERR_WORKSPACE = -3,        /* workspace missing or too small */
+  SDK_ERR_DEVICE = -4            /* HIP runtime reported an error */
+} sdk_status;
+
+typedef enum sdk_dtype { SDK_F32 = 0, SDK_F64 = 1 } sdk_dtype;
+
+/* ext_modules/include/enums.h:12-16 (exported by include/layers/enum_export.h:10-18) */
+typedef enum sdk_interp { SDK_NEAREST = 0, SDK_BILINEAR = 1, SDK_BISPHERICAL = 2 } sdk_interp;
+
+/* Arithmetic used by the dense contraction inside the convolution entry points.
+ * SDK_COMPUTE_NATIVE: the tensors' own type (fp32 MFMA for SDK_F32).
+ * SDK_COMPUTE_BF16:   operands rounded to bf16, fp32 accumulation (SDK_F32 only). */
+typedef enum sdk_compute { SDK_COMPUTE_NATIVE = 0, SDK_COMPUTE_BF16 = 1 } sdk_compute;
+
+typedef void* sdk_stream_t; /* hipStream_t */
+
+const char* sdk_last_error(void);
+int sdk_version(void);
+
+/* ------------------------------------------------------------------------- *
+ * Resampling.
+ * ------------------------------------------------------------------------- */
+
+/* Gather: out[b,c,my,mx] = interp(image[b,c], sample_map[my,mx]).
+ * image [B,C,H,W]; sample_map [MH,MW,(P,)2]; out [B,C,MH,MW].
+ * Replaces `_resample.resample_from_map` / `_weighted_resample.weighted_resample_from_map`
+ * (ext_modules/include/layers/resample_layer.h:62-80,
+ *  ext_modules/include/layers/weighted_resample_layer.h:76-101;
+ *  device side ext_modules/src/cuda/resample_layer.cu, include/cuda/resample.cuh:50-81, :127-164). */
+int sdk_resample_from_map(const void* image, const void* sample_map, const void* interp_weights,
+                          void* out, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t map_height, int64_t map_width,
+                          int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                          sdk_stream_t stream);
+
+/* Scatter: out (zero-filled) accumulates input[b,c,my,mx] at sample_map[my,mx].
+ * input [B,C,MH,MW]; out [B,C,H,W].  If weight_sum is non-NULL it receives, as
+ * one [H,W] plane, the same scatter applied to an all-ones input plane (the
+ * per-pixel sum of splat weights; batch- and channel-invariant).
+ * Replaces `_resample.resample_to_map` / `_weighted_resample.weighted_resample_to_map`
+ * (ext_modules/include/layers/resample_layer.h:40-60,
+ *  ext_modules/include/layers/weighted_resample_layer.h:49-74;
+ *  device side include/cuda/resample.cuh:14-47, :87-124). */
+int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, void* weight_sum, int64_t batch, int64_t channels,
+                        int64_t map_height, int64_t map_width, int64_t height, int64_t width,
+                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                        sdk_stream_t stream);
+
+/* data[p, i] /= (weight_sum[i] + eps) for p < planes, i < plane_size, in place.
+ * The reference does this in Python for its weighted splat
+ * (layers/functional/sphere_ops.py:74-80, eps 1e-12). */
+int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, int64_t planes,
+                                int64_t plane_size, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Mapped im2col / col2im (batched).
+ * col[b, c*K + k, pix] with pix = y_out*OW + x_out, out_pixels = OH*OW.
+ * sample_map [OH,OW,K,(P,)2].
+ * Replace the device launchers MappedIm2Col2D / MappedCol2Im2D (+Weighted)
+ * (ext_modules/include/cuda/mapped_im2col.cuh:28-49, :67-94, :113-136, :158-184),
+ * which the reference calls once per batch element.
+ * ------------------------------------------------------------------------- */
+int sdk_mapped_im2col(const void* image, const void* sample_map, const void* interp_weights,
+                      void* columns, int64_t batch, int64_t channels, int64_t height,
+                      int64_t width, int64_t out_pixels, int64_t kernel_size,
+                      int32_t num_interp_pts, int32_t interp, int32_t dtype, sdk_stream_t stream);
+
+/* image [B,C,H,W] is zero-filled by the call, then accumulated into. */
+int sdk_mapped_col2im(const void* columns, const void* sample_map, const void* interp_weights,
+                      void* image, int64_t batch, int64_t channels, int64_t height,
+                      int64_t width, int64_t out_pixels, int64_t kernel_size,
+                      int32_t num_interp_pts, int32_t interp, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Mapped max pooling.
+ * ------------------------------------------------------------------------- */
+
+/* out[b,c,oy,ox] = max_k interp(input[b,c], sample_map[oy,ox,k]) with strict `>`
+ * (first maximum wins, NaN never wins) starting from -FLT_MAX;
+ * indices[b,c,oy,ox] (int64) = flat element offset, inside sample_map, of the
+ * winning sample's x coordinate (of its first interpolation point when
+ * weighted), or -1 when no sample exceeded the start value.
+ * Replaces `_mapped_max_pooling.mapped_max_pool` /
+ * `_weighted_mapped_max_pooling.weighted_mapped_max_pool`
+ * (ext_modules/include/layers/mapped_max_pooling_layer.h:42-62,
+ *  weighted_mapped_max_pooling_layer.h:42-66; body
+ *  ext_modules/include/common/mapped_max_pool.h:13-57, :81-133, device branch). */
+int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, int64_t* indices, int64_t batch, int64_t channels,
+                        int64_t height, int64_t width, int64_t out_height, int64_t out_width,
+                        int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                        int32_t dtype, sdk_stream_t stream);
+
+/* grad_input [B,C,H,W] (zero-filled by the call) receives grad_output[b,c,oy,ox]
+ * splatted at the sample the stored index names, with the same interpolation.
+ * Negative or out-of-range indices contribute nothing.
+ * Replaces `_mapped_max_pooling.mapped_max_unpool` /
+ * `_weighted_mapped_max_pooling.weighted_mapped_max_unpool`
+ * (ext_modules/include/layers/mapped_max_pooling_layer.h:64-88,
+ *  weighted_mapped_max_pooling_layer.h:68-99; body common/mapped_max_pool.h:60-78, :136-171). */
+int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,
+                          const void* interp_weights, void* grad_input, int64_t batch,
+                          int64_t channels, int64_t height, int64_t width, int64_t out_height,
+                          int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
+                          int32_t interp, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Mapped convolution.  weight [Cout, Cin, K]; bias [Cout];
+ * input [B,Cin,H,W]; sample_map [OH,OW,K,(P,)2]; output [B,Cout,OH,OW].
+ *
+ * Some shape/dtype combinations run as separate im2col/col2im + GEMM kernels
+ * and need device scratch: ask sdk_mapped_conv_workspace_bytes() (same
+ * arguments for the forward, backward and transposed entry points of one
+ * layer call) and pass at least that many bytes (256-byte aligned).  A
+ * result of 0 means the fused kernels serve the request and workspace may be
+ * NULL.
+ * ------------------------------------------------------------------------- */
+size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
+                                       int64_t gather_pixels, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute);
+
+/* output[b] = weight[Cout, Cin*K] x im2col(input[b]) + bias.
+ * Replaces `_mapped_convolution.mapped_conv_forward` /
+ * `_weighted_mapped_convolution.weighted_mapped_conv_forward`
+ * (ext_modules/include/layers/mapped_convolution_layer.h:62-87,
+ *  weighted_mapped_convolution_layer.h:69-101; device side
+ *  ext_modules/src/cuda/mapped_convolution_layer.cu:16-74). */
+int sdk_mapped_conv_forward(const void* input, const void* sample_map, const void* interp_weights,
+                            const void* weight, const void* bias, void* output, void* workspace,
+                            size_t workspace_bytes, int64_t batch, int64_t in_channels,
+                            int64_t height, int64_t width, int64_t out_channels,
+                            int64_t out_height, int64_t out_width, int64_t kernel_size,
+                            int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                            int32_t compute, sdk_stream_t stream);
+
+/* grad_input[b] = col2im(weight^T x grad_output[b]).
+ * Replaces cuda::MappedConvBackwardInput, first half of `mapped_conv_backward`
+ * (ext_modules/include/layers/mapped_convolution_layer.h:89-134;
+ *  ext_modules/src/cuda/mapped_convolution_layer.cu:76-133). */
+int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_map,
+                                   const void* interp_weights, const void* weight,
+                                   void* grad_input, void* workspace, size_t workspace_bytes,
+                                   int64_t batch, int64_t in_channels, int64_t height,
+                                   int64_t width, int64_t out_channels, int64_t out_height,
+                                   int64_t out_width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   int32_t compute, sdk_stream_t stream);
+
+/* grad_weight[Cout, Cin*K] = sum_b grad_output[b] x im2col(input[b])^T.
+ * Replaces cuda::MappedConvBackwardWeight
+ * (ext_modules/src/cuda/mapped_convolution_layer.cu:135-194). */
+int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                    const void* interp_weights, const void* input,
+                                    void* grad_weight, void* workspace, size_t workspace_bytes,
+                                    int64_t batch, int64_t in_channels, int64_t height,
+                                    int64_t width, int64_t out_channels, int64_t out_height,
+                                    int64_t out_width, int64_t kernel_size,
+                                    int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                    int32_t compute, sdk_stream_t stream);
+
+/* grad_bias[c] = sum over batch and pixels of grad_output[b,c,:]
+ * (`grad_output.sum({0, 2, 3})`, ext_modules/include/layers/mapped_convolution_layer.h:130). */
+int sdk_bias_grad(const void* grad_output, void* grad_bias, int64_t batch, int64_t channels,
+                  int64_t pixels, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Mapped transposed convolution.  weight [Cin, Cout, K]; bias [Cout];
+ * input [B,Cin,IH,IW]; sample_map [IH,IW,K,(P,)2] pointing into the
+ * [OH,OW] output; output [B,Cout,OH,OW].
+ * Replace `_mapped_transposed_convolution.mapped_transposed_conv_forward/_backward`
+ * and the weighted twins
+ * (ext_modules/include/layers/mapped_transposed_convolution_layer.h:62-93, :95-140;
+ *  device side ext_modules/src/cuda/mapped_transposed_convolution_layer.cu:53-223).
+ * ------------------------------------------------------------------------- */
+int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map,
+                                       const void* interp_weights, const void* weight,
+                                       const void* bias, void* output, void* workspace,
+                                       size_t workspace_bytes, int64_t batch,
+                                       int64_t in_channels, int64_t in_height, int64_t in_width,
+                                       int64_t out_channels, int64_t out_height,
+                                       int64_t out_width, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute, sdk_stream_t stream);
+
+int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const void* sample_map,
+                                              const void* interp_weights, const void* weight,
+                                              void* grad_input, void* workspace,
+                                              size_t workspace_bytes, int64_t batch,
+                                              int64_t in_channels, int64_t in_height,
+                                              int64_t in_width, int64_t out_channels,
+                                              int64_t out_height, int64_t out_width,
+                                              int64_t kernel_size, int32_t num_interp_pts,
+                                              int32_t interp, int32_t dtype, int32_t compute,
+                                              sdk_stream_t stream);
+
+int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                               const void* interp_weights, const void* input,
+                                               void* grad_weight, void* workspace,
+                                               size_t workspace_bytes, int64_t batch,
+                                               int64_t in_channels, int64_t in_height,
+                                               int64_t in_width, int64_t out_channels,
+                                               int64_t out_height, int64_t out_width,
+                                               int64_t kernel_size, int32_t num_interp_pts,
+                                               int32_t interp, int32_t dtype, int32_t compute,
+                                               sdk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SDK_MAPPED_OPS_H_ */

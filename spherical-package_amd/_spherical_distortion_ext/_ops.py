@@ -1,0 +1,354 @@
+"""PyTorch-ROCm custom operators over the C ABI.
+
+Every operator here checks its tensors the way the reference's pybind entry
+points do (contiguous, all on the GPU: ext_modules/include/cuda_helper.h:12-18),
+allocates the outputs with torch, fetches the current HIP stream and makes one
+call into libsdk_mapped_ops.so.  The operators are registered in the
+``sdk_mapped_ops`` namespace of torch.library for the CUDA (= HIP on ROCm)
+dispatch key only: calling them with CPU tensors raises, there is no CPU path.
+"""
+import ctypes
+
+import torch
+
+from . import _capi
+
+_NS = "sdk_mapped_ops"
+_DTYPES = {torch.float32: _capi.SDK_F32, torch.float64: _capi.SDK_F64}
+
+# Arithmetic of the dense contraction inside the convolution operators:
+# "native" (the tensors' type) or "bf16" (bf16 operands, fp32 accumulate).
+_compute_mode = _capi.SDK_COMPUTE_NATIVE
+
+
+def set_conv_compute(mode):
+    """Selects the GEMM arithmetic of the mapped (transposed) convolutions."""
+    global _compute_mode
+    modes = {"native": _capi.SDK_COMPUTE_NATIVE, "fp32": _capi.SDK_COMPUTE_NATIVE,
+             "bf16": _capi.SDK_COMPUTE_BF16}
+    if mode not in modes:
+        raise ValueError("compute mode must be one of %s" % sorted(modes))
+    _compute_mode = modes[mode]
+
+
+def get_conv_compute():
+    return "bf16" if _compute_mode == _capi.SDK_COMPUTE_BF16 else "native"
+
+
+# --------------------------------------------------------------------------- checks
+def _check(ref, **tensors):
+    """ref: the tensor that decides device and dtype (first argument of the op)."""
+    if not ref.is_cuda:
+        raise RuntimeError("this backend runs on the GPU only: tensors must be CUDA/HIP tensors")
+    if ref.dtype not in _DTYPES:
+        raise RuntimeError("unsupported dtype %s (float32 and float64 only)" % ref.dtype)
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if not t.is_contiguous():
+            raise RuntimeError("%s must be contiguous" % name)
+        if not t.is_cuda or t.device != ref.device:
+            raise RuntimeError("%s must be a CUDA tensor on %s" % (name, ref.device))
+        if t.dtype != ref.dtype and name != "idx_mask":
+            raise RuntimeError("%s must have dtype %s (got %s)" % (name, ref.dtype, t.dtype))
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(ref):
+    return ctypes.c_void_p(torch.cuda.current_stream(ref.device).cuda_stream)
+
+
+def _npts(sample_map, interp_weights, map_rank_unweighted):
+    """0 for the unweighted map layout, P for the weighted one."""
+    if interp_weights is None:
+        if sample_map.dim() != map_rank_unweighted or sample_map.shape[-1] != 2:
+            raise RuntimeError("sample_map must have %d dimensions ending in 2, got %s"
+                               % (map_rank_unweighted, tuple(sample_map.shape)))
+        return 0
+    if sample_map.dim() != map_rank_unweighted + 1 or sample_map.shape[-1] != 2:
+        raise RuntimeError("weighted sample_map must have %d dimensions ending in 2, got %s"
+                           % (map_rank_unweighted + 1, tuple(sample_map.shape)))
+    if tuple(interp_weights.shape) != tuple(sample_map.shape[:-1]):
+        raise RuntimeError("interp_weights shape %s does not match sample_map %s"
+                           % (tuple(interp_weights.shape), tuple(sample_map.shape)))
+    return int(interp_weights.shape[-1])
+
+
+def _workspace(ref, batch, cin, cout, pixels, K, P, interp):
+    n = _capi.load().sdk_mapped_conv_workspace_bytes(
+        batch, cin, cout, pixels, K, P, interp, _DTYPES[ref.dtype], _compute_mode)
+    if n == 0:
+        return None, 0
+    return torch.empty(n, dtype=torch.uint8, device=ref.device), n
+
+
+# --------------------------------------------------------------------------- resample
+def resample_from_map(x, sample_map, interp_weights, interp):
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 3)
+    B, C, H, W = x.shape
+    MH, MW = sample_map.shape[:2]
+    out = torch.empty((B, C, MH, MW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_resample_from_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(out), B, C, H, W, MH, MW, P, int(interp), _DTYPES[x.dtype], _stream(x))
+    return out
+
+
+def resample_to_map(x, sample_map, interp_weights, out_h, out_w, interp):
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 3)
+    B, C, MH, MW = x.shape
+    if tuple(sample_map.shape[:2]) != (MH, MW):
+        raise RuntimeError("sample_map grid %s must match the input's %s"
+                           % (tuple(sample_map.shape[:2]), (MH, MW)))
+    out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(out), ctypes.c_void_p(0), B, C, MH, MW, int(out_h), int(out_w), P,
+                   int(interp), _DTYPES[x.dtype], _stream(x))
+    return out
+
+
+def resample_to_map_normalized(x, sample_map, interp_weights, out_h, out_w, interp, eps):
+    """resample_to_map(x) / (resample_to_map(ones) + eps) with one weight-sum plane."""
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 3)
+    B, C, MH, MW = x.shape
+    if tuple(sample_map.shape[:2]) != (MH, MW):
+        raise RuntimeError("sample_map grid must match the input's")
+    out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
+    wsum = torch.empty((int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(out), _ptr(wsum), B, C, MH, MW, int(out_h), int(out_w), P, int(interp),
+                   _DTYPES[x.dtype], _stream(x))
+        _capi.call("sdk_normalize_by_weight_sum", _ptr(out), _ptr(wsum), float(eps), B * C,
+                   int(out_h) * int(out_w), _DTYPES[x.dtype], _stream(x))
+    return out, wsum
+
+
+# --------------------------------------------------------------------------- im2col / col2im
+def mapped_im2col(x, sample_map, interp_weights, interp):
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, H, W = x.shape
+    OH, OW, K = sample_map.shape[:3]
+    col = torch.empty((B, C * K, OH * OW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_mapped_im2col", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(col), B, C, H, W, OH * OW, K, P, int(interp), _DTYPES[x.dtype],
+                   _stream(x))
+    return col
+
+
+def mapped_col2im(col, sample_map, interp_weights, height, width, interp):
+    _check(col, col=col, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 4)
+    OH, OW, K = sample_map.shape[:3]
+    B, CK, M = col.shape
+    if M != OH * OW or CK % K:
+        raise RuntimeError("columns %s do not match sample_map %s"
+                           % (tuple(col.shape), tuple(sample_map.shape)))
+    C = CK // K
+    im = torch.empty((B, C, int(height), int(width)), dtype=col.dtype, device=col.device)
+    with torch.cuda.device(col.device):
+        _capi.call("sdk_mapped_col2im", _ptr(col), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(im), B, C, int(height), int(width), M, K, P, int(interp),
+                   _DTYPES[col.dtype], _stream(col))
+    return im
+
+
+# --------------------------------------------------------------------------- pooling
+def mapped_max_pool(x, sample_map, interp_weights, kernel_size, interp):
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, H, W = x.shape
+    OH, OW, K = sample_map.shape[:3]
+    if K != int(kernel_size):
+        raise RuntimeError("kernel_size %d does not match sample_map %s"
+                           % (int(kernel_size), tuple(sample_map.shape)))
+    out = torch.empty((B, C, OH, OW), dtype=x.dtype, device=x.device)
+    idx = torch.empty((B, C, OH, OW), dtype=torch.int64, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_mapped_max_pool", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(out), _ptr(idx), B, C, H, W, OH, OW, K, P, int(interp),
+                   _DTYPES[x.dtype], _stream(x))
+    return out, idx
+
+
+def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, in_w,
+                      kernel_size, interp):
+    _check(grad_output, grad_output=grad_output, idx_mask=idx_mask, sample_map=sample_map,
+           interp_weights=interp_weights)
+    if idx_mask.dtype != torch.int64 or idx_mask.shape != grad_output.shape:
+        raise RuntimeError("idx_mask must be an int64 tensor shaped like grad_output")
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, OH, OW = grad_output.shape
+    if tuple(sample_map.shape[:3]) != (OH, OW, int(kernel_size)):
+        raise RuntimeError("sample_map %s does not match grad_output %s / kernel_size %d"
+                           % (tuple(sample_map.shape), tuple(grad_output.shape), int(kernel_size)))
+    gin = torch.empty((B, C, int(in_h), int(in_w)), dtype=grad_output.dtype,
+                      device=grad_output.device)
+    with torch.cuda.device(grad_output.device):
+        _capi.call("sdk_mapped_max_unpool", _ptr(grad_output), _ptr(idx_mask), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(gin), B, C, int(in_h), int(in_w), OH, OW,
+                   int(kernel_size), P, int(interp), _DTYPES[grad_output.dtype],
+                   _stream(grad_output))
+    return gin
+
+
+# --------------------------------------------------------------------------- convolution
+def _conv_dims(x_shape, weight, sample_map, kernel_size, transposed):
+    K = int(kernel_size)
+    if sample_map.shape[2] != K or weight.shape[2] != K:
+        raise RuntimeError("kernel_size %d does not match sample_map %s / weight %s"
+                           % (K, tuple(sample_map.shape), tuple(weight.shape)))
+    B, Cin = int(x_shape[0]), int(x_shape[1])
+    if weight.shape[0 if transposed else 1] != Cin:
+        raise RuntimeError("weight %s does not match %d input channels"
+                           % (tuple(weight.shape), Cin))
+    Cout = int(weight.shape[1 if transposed else 0])
+    return B, Cin, Cout, K
+
+
+def mapped_conv_forward(x, sample_map, interp_weights, weight, bias, kernel_size, interp):
+    _check(x, input=x, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+           bias=bias)
+    P = _npts(sample_map, interp_weights, 4)
+    B, Cin, Cout, K = _conv_dims(x.shape, weight, sample_map, kernel_size, False)
+    H, W = x.shape[2:]
+    OH, OW = sample_map.shape[:2]
+    out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        ws, nws = _workspace(x, B, Cin, Cout, OH * OW, K, P, int(interp))
+        _capi.call("sdk_mapped_conv_forward", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B, Cin, H, W, Cout, OH,
+                   OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode, _stream(x))
+    return out
+
+
+def mapped_conv_backward(grad_output, sample_map, interp_weights, x, weight, bias, kernel_size,
+                         interp):
+    # The reference checks input, sample_map, weight and bias here, not grad_output
+    # (include/layers/mapped_convolution_layer.h:93-96); the kernels need it dense too.
+    grad_output = grad_output.contiguous()
+    _check(grad_output, grad_output=grad_output, input=x, sample_map=sample_map,
+           interp_weights=interp_weights, weight=weight, bias=bias)
+    P = _npts(sample_map, interp_weights, 4)
+    B, Cin, Cout, K = _conv_dims(x.shape, weight, sample_map, kernel_size, False)
+    H, W = x.shape[2:]
+    OH, OW = sample_map.shape[:2]
+    gi = torch.empty_like(x)
+    gw = torch.empty_like(weight)
+    gb = torch.empty((Cout,), dtype=x.dtype, device=x.device)
+    dt = _DTYPES[x.dtype]
+    with torch.cuda.device(x.device):
+        ws, nws = _workspace(x, B, Cin, Cout, OH * OW, K, P, int(interp))
+        s = _stream(x)
+        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
+        _capi.call("sdk_mapped_conv_backward_input", _ptr(grad_output), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(weight), _ptr(gi), _ptr(ws), nws, *dims)
+        _capi.call("sdk_mapped_conv_backward_weight", _ptr(grad_output), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(x), _ptr(gw), _ptr(ws), nws, *dims)
+        _capi.call("sdk_bias_grad", _ptr(grad_output), _ptr(gb), B, Cout, OH * OW, dt, s)
+    return gi, gw, gb
+
+
+def mapped_transposed_conv_forward(x, sample_map, interp_weights, weight, bias, out_h, out_w,
+                                   kernel_size, interp):
+    _check(x, input=x, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+           bias=bias)
+    P = _npts(sample_map, interp_weights, 4)
+    B, Cin, Cout, K = _conv_dims(x.shape, weight, sample_map, kernel_size, True)
+    IH, IW = x.shape[2:]
+    if tuple(sample_map.shape[:2]) != (IH, IW):
+        raise RuntimeError("sample_map grid %s must match the input's %s"
+                           % (tuple(sample_map.shape[:2]), (IH, IW)))
+    OH, OW = int(out_h), int(out_w)
+    out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        ws, nws = _workspace(x, B, Cin, Cout, IH * IW, K, P, int(interp))
+        _capi.call("sdk_mapped_transposed_conv_forward", _ptr(x), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B,
+                   Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype],
+                   _compute_mode, _stream(x))
+    return out
+
+
+def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, weight, bias,
+                                    kernel_size, interp):
+    grad_output = grad_output.contiguous()
+    _check(grad_output, grad_output=grad_output, input=x, sample_map=sample_map,
+           interp_weights=interp_weights, weight=weight, bias=bias)
+    P = _npts(sample_map, interp_weights, 4)
+    B, Cin, Cout, K = _conv_dims(x.shape, weight, sample_map, kernel_size, True)
+    IH, IW = x.shape[2:]
+    OH, OW = grad_output.shape[2:]
+    gi = torch.empty_like(x)
+    gw = torch.empty_like(weight)
+    gb = torch.empty((Cout,), dtype=x.dtype, device=x.device)
+    dt = _DTYPES[x.dtype]
+    with torch.cuda.device(x.device):
+        ws, nws = _workspace(x, B, Cin, Cout, IH * IW, K, P, int(interp))
+        s = _stream(x)
+        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
+        _capi.call("sdk_mapped_transposed_conv_backward_input", _ptr(grad_output),
+                   _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(gi), _ptr(ws), nws,
+                   *dims)
+        _capi.call("sdk_mapped_transposed_conv_backward_weight", _ptr(grad_output),
+                   _ptr(sample_map), _ptr(interp_weights), _ptr(x), _ptr(gw), _ptr(ws), nws,
+                   *dims)
+        _capi.call("sdk_bias_grad", _ptr(grad_output), _ptr(gb), B, Cout, OH * OW, dt, s)
+    return gi, gw, gb
+
+
+# --------------------------------------------------------------------------- registration
+_SCHEMAS = (
+    ("resample_from_map",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int interp) -> Tensor",
+     resample_from_map),
+    ("resample_to_map",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int out_h, int out_w, int interp)"
+     " -> Tensor", resample_to_map),
+    ("resample_to_map_normalized",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int out_h, int out_w, int interp,"
+     " float eps) -> (Tensor, Tensor)", resample_to_map_normalized),
+    ("mapped_im2col",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int interp) -> Tensor",
+     mapped_im2col),
+    ("mapped_col2im",
+     "(Tensor col, Tensor sample_map, Tensor? interp_weights, int height, int width, int interp)"
+     " -> Tensor", mapped_col2im),
+    ("mapped_max_pool",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int kernel_size, int interp)"
+     " -> (Tensor, Tensor)", mapped_max_pool),
+    ("mapped_max_unpool",
+     "(Tensor grad_output, Tensor idx_mask, Tensor sample_map, Tensor? interp_weights, int in_h,"
+     " int in_w, int kernel_size, int interp) -> Tensor", mapped_max_unpool),
+    ("mapped_conv_forward",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, Tensor weight, Tensor bias,"
+     " int kernel_size, int interp) -> Tensor", mapped_conv_forward),
+    ("mapped_conv_backward",
+     "(Tensor grad_output, Tensor sample_map, Tensor? interp_weights, Tensor x, Tensor weight,"
+     " Tensor bias, int kernel_size, int interp) -> (Tensor, Tensor, Tensor)",
+     mapped_conv_backward),
+    ("mapped_transposed_conv_forward",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, Tensor weight, Tensor bias,"
+     " int out_h, int out_w, int kernel_size, int interp) -> Tensor",
+     mapped_transposed_conv_forward),
+    ("mapped_transposed_conv_backward",
+     "(Tensor grad_output, Tensor sample_map, Tensor? interp_weights, Tensor x, Tensor weight,"
+     " Tensor bias, int kernel_size, int interp) -> (Tensor, Tensor, Tensor)",
+     mapped_transposed_conv_backward),
+)
+
+_library = torch.library.Library(_NS, "DEF")
+for _name, _schema, _fn in _SCHEMAS:
+    _library.define(_name + _schema)
+    _library.impl(_name, _fn, "CUDA")
+
+ops = getattr(torch.ops, _NS)

@@ -1,0 +1,238 @@
+// C entry points of mapped convolution and mapped transposed convolution.
+// Each call is reduced to one of three contractions over a ConvGeom (see
+// conv_internal.hpp) and routed to the fused MFMA kernels when they cover the
+// request, otherwise to the generic im2col/col2im + GEMM path.
+#include <hip/hip_runtime.h>
+
+#include "conv_fused.hpp"
+#include "conv_internal.hpp"
+#include "sdk_host.hpp"
+
+using namespace sdk;
+
+namespace {
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+size_t generic_workspace_bytes(int64_t gather_channels, int64_t K, int64_t M, int dtype) {
+  return align256((size_t)gather_channels * K * M * (dtype == SDK_F64 ? 8 : 4));
+}
+
+int check_common(const char* what, int64_t B, int64_t Cg, int64_t H, int64_t W, int64_t Cp,
+                 int64_t M, int64_t K, int32_t P, const void* wts, int32_t dtype,
+                 int32_t compute) {
+  SDK_REQUIRE(B >= 0 && Cg >= 1 && Cp >= 1 && K >= 1, "%s: bad size", what);
+  SDK_REQUIRE(H >= 1 && W >= 1 && H * W < ((int64_t)1 << 31), "%s: bad plane size", what);
+  SDK_REQUIRE(M >= 1 && M < ((int64_t)1 << 31), "%s: bad pixel count", what);
+  SDK_REQUIRE(Cg * K < ((int64_t)1 << 24) && Cp < ((int64_t)1 << 24), "%s: too many channels",
+              what);
+  SDK_REQUIRE(P >= 0 && (P == 0 || wts), "%s: weighted map needs interp_weights", what);
+  SDK_REQUIRE(dtype == SDK_F32 || dtype == SDK_F64, "%s: unknown dtype %d", what, dtype);
+  SDK_REQUIRE(compute == SDK_COMPUTE_NATIVE || compute == SDK_COMPUTE_BF16,
+              "%s: unknown compute mode %d", what, compute);
+  if (compute == SDK_COMPUTE_BF16 && dtype != SDK_F32)
+    return fail(SDK_ERR_UNSUPPORTED, "%s: bf16 compute needs float32 tensors", what);
+  return SDK_OK;
+}
+
+int check_workspace(const char* what, const ConvGeom& g, int dtype, void* ws, size_t ws_bytes) {
+  const size_t need = generic_workspace_bytes(g.Cg, g.K, g.M, dtype);
+  if (!ws || ws_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", what, need,
+                ws ? ws_bytes : (size_t)0);
+  return SDK_OK;
+}
+
+enum Op { GATHER_GEMM, GEMM_SCATTER, GATHER_WGRAD };
+
+// a: pixel-side tensor for GEMM_SCATTER / GATHER_WGRAD inputs, image otherwise (see call sites).
+int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, const void* in0,
+        const void* map, const void* wts, const void* in1, const void* bias, void* out, void* ws,
+        size_t ws_bytes, hipStream_t stream) {
+  if (g.B == 0 && op != GATHER_WGRAD) return SDK_OK;
+  if (dtype == SDK_F32 && fused_supported(g)) {
+    const float* m = (const float*)map;
+    const float* w = (const float*)wts;
+    switch (op) {
+      case GATHER_GEMM:
+        return fused_gather_gemm(g, compute, (const float*)in0, m, w, (const float*)in1,
+                                 (const float*)bias, (float*)out, stream);
+      case GEMM_SCATTER:
+        return fused_gemm_scatter(g, compute, (const float*)in0, m, w, (const float*)in1,
+                                  (const float*)bias, (float*)out, stream);
+      case GATHER_WGRAD:
+        return fused_gather_wgrad(g, compute, (const float*)in0, m, w, (const float*)in1,
+                                  (float*)out, stream);
+    }
+  }
+  if (compute == SDK_COMPUTE_BF16)
+    return fail(SDK_ERR_UNSUPPORTED, "%s: bf16 compute is not available for this shape", what);
+  int rc = check_workspace(what, g, dtype, ws, ws_bytes);
+  if (rc) return rc;
+  SDK_DISPATCH_DTYPE(dtype, {
+    switch (op) {
+      case GATHER_GEMM:
+        return generic_gather_gemm<T>(g, (const T*)in0, (const T*)map, (const T*)wts,
+                                      (const T*)in1, (const T*)bias, (T*)out, (T*)ws, stream);
+      case GEMM_SCATTER:
+        return generic_gemm_scatter<T>(g, (const T*)in0, (const T*)map, (const T*)wts,
+                                       (const T*)in1, (const T*)bias, (T*)out, (T*)ws, stream);
+      case GATHER_WGRAD:
+        return generic_gather_wgrad<T>(g, (const T*)in0, (const T*)map, (const T*)wts,
+                                       (const T*)in1, (T*)out, (T*)ws, stream);
+    }
+  });
+  return SDK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
+                                       int64_t gather_pixels, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute) {
+  (void)compute;
+  // Upper bound over the conv (gather side = in_channels) and transposed conv
+  // (gather side = out_channels) roles, so one query serves a whole layer call.
+  ConvGeom a{batch, (int)in_channels, 1, 1, (int)out_channels, (int)gather_pixels,
+             (int)kernel_size, num_interp_pts, interp};
+  ConvGeom b{batch, (int)out_channels, 1, 1, (int)in_channels, (int)gather_pixels,
+             (int)kernel_size, num_interp_pts, interp};
+  if (dtype == SDK_F32 && fused_supported(a) && fused_supported(b)) return 0;
+  return generic_workspace_bytes(std::max(in_channels, out_channels), kernel_size, gather_pixels,
+                                 dtype);
+}
+
+int sdk_mapped_conv_forward(const void* input, const void* sample_map, const void* interp_weights,
+                            const void* weight, const void* bias, void* output, void* workspace,
+                            size_t workspace_bytes, int64_t batch, int64_t in_channels,
+                            int64_t height, int64_t width, int64_t out_channels,
+                            int64_t out_height, int64_t out_width, int64_t kernel_size,
+                            int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                            int32_t compute, sdk_stream_t stream) {
+  const char* what = "mapped_conv_forward";
+  SDK_REQUIRE(input && sample_map && weight && bias && output, "%s: NULL pointer", what);
+  SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
+  const int64_t M = out_height * out_width;
+  int rc = check_common(what, batch, in_channels, height, width, out_channels, M, kernel_size,
+                        num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GATHER_GEMM, g, dtype, compute, input, sample_map, interp_weights, weight, bias,
+             output, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_map,
+                                   const void* interp_weights, const void* weight,
+                                   void* grad_input, void* workspace, size_t workspace_bytes,
+                                   int64_t batch, int64_t in_channels, int64_t height,
+                                   int64_t width, int64_t out_channels, int64_t out_height,
+                                   int64_t out_width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   int32_t compute, sdk_stream_t stream) {
+  const char* what = "mapped_conv_backward_input";
+  SDK_REQUIRE(grad_output && sample_map && weight && grad_input, "%s: NULL pointer", what);
+  SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
+  const int64_t M = out_height * out_width;
+  int rc = check_common(what, batch, in_channels, height, width, out_channels, M, kernel_size,
+                        num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights,
+             weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                    const void* interp_weights, const void* input,
+                                    void* grad_weight, void* workspace, size_t workspace_bytes,
+                                    int64_t batch, int64_t in_channels, int64_t height,
+                                    int64_t width, int64_t out_channels, int64_t out_height,
+                                    int64_t out_width, int64_t kernel_size,
+                                    int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                    int32_t compute, sdk_stream_t stream) {
+  const char* what = "mapped_conv_backward_weight";
+  SDK_REQUIRE(grad_output && sample_map && input && grad_weight, "%s: NULL pointer", what);
+  SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
+  const int64_t M = out_height * out_width;
+  int rc = check_common(what, batch, in_channels, height, width, out_channels, M, kernel_size,
+                        num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
+             nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map,
+                                       const void* interp_weights, const void* weight,
+                                       const void* bias, void* output, void* workspace,
+                                       size_t workspace_bytes, int64_t batch,
+                                       int64_t in_channels, int64_t in_height, int64_t in_width,
+                                       int64_t out_channels, int64_t out_height,
+                                       int64_t out_width, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute, sdk_stream_t stream) {
+  const char* what = "mapped_transposed_conv_forward";
+  SDK_REQUIRE(input && sample_map && weight && bias && output, "%s: NULL pointer", what);
+  SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
+  const int64_t M = in_height * in_width;
+  int rc = check_common(what, batch, out_channels, out_height, out_width, in_channels, M,
+                        kernel_size, num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GEMM_SCATTER, g, dtype, compute, input, sample_map, interp_weights, weight,
+             bias, output, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const void* sample_map,
+                                              const void* interp_weights, const void* weight,
+                                              void* grad_input, void* workspace,
+                                              size_t workspace_bytes, int64_t batch,
+                                              int64_t in_channels, int64_t in_height,
+                                              int64_t in_width, int64_t out_channels,
+                                              int64_t out_height, int64_t out_width,
+                                              int64_t kernel_size, int32_t num_interp_pts,
+                                              int32_t interp, int32_t dtype, int32_t compute,
+                                              sdk_stream_t stream) {
+  const char* what = "mapped_transposed_conv_backward_input";
+  SDK_REQUIRE(grad_output && sample_map && weight && grad_input, "%s: NULL pointer", what);
+  SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
+  const int64_t M = in_height * in_width;
+  int rc = check_common(what, batch, out_channels, out_height, out_width, in_channels, M,
+                        kernel_size, num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GATHER_GEMM, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
+             nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                               const void* interp_weights, const void* input,
+                                               void* grad_weight, void* workspace,
+                                               size_t workspace_bytes, int64_t batch,
+                                               int64_t in_channels, int64_t in_height,
+                                               int64_t in_width, int64_t out_channels,
+                                               int64_t out_height, int64_t out_width,
+                                               int64_t kernel_size, int32_t num_interp_pts,
+                                               int32_t interp, int32_t dtype, int32_t compute,
+                                               sdk_stream_t stream) {
+  const char* what = "mapped_transposed_conv_backward_weight";
+  SDK_REQUIRE(grad_output && sample_map && input && grad_weight, "%s: NULL pointer", what);
+  SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
+  const int64_t M = in_height * in_width;
+  int rc = check_common(what, batch, out_channels, out_height, out_width, in_channels, M,
+                        kernel_size, num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp};
+  return run(what, GATHER_WGRAD, g, dtype, compute, input, sample_map, interp_weights,
+             grad_output, nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

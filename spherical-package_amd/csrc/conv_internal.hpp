@@ -1,0 +1,50 @@
+// Internal interfaces between the convolution drivers and the kernels they
+// chain.  Not part of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace sdk {
+
+int zero_fill(void* ptr, size_t bytes, hipStream_t stream);
+
+// Batched mapped im2col / col2im over `planes` image planes (see
+// mapped_gather_scatter.hip).  col2im accumulates onto what `im` holds.
+template <typename T>
+int launch_mapped_im2col(const T* im, const T* map, const T* wts, T* col, int64_t planes, int H,
+                         int W, int M, int K, int P, int interp, hipStream_t stream);
+template <typename T>
+int launch_mapped_col2im(const T* col, const T* map, const T* wts, T* im, int64_t planes, int H,
+                         int W, int M, int K, int P, int interp, hipStream_t stream);
+
+// Geometry of one convolution-shaped call, shared by the generic and the fused
+// drivers.  "gather side" is the image the sample map points into, "pixel side"
+// the grid the map is defined on:
+//   mapped conv:            gather side = input  [Cg = Cin,  H x W],  pixel side = output (Cp = Cout, M = OH*OW)
+//   mapped transposed conv: gather side = output [Cg = Cout, OH x OW], pixel side = input (Cp = Cin,  M = IH*IW)
+// The weight matrix is always [Cp, Cg*K] row-major.
+struct ConvGeom {
+  int64_t B;
+  int Cg, H, W;  // gather-side channels and plane size
+  int Cp, M;     // pixel-side channels and pixel count
+  int K, P, interp;
+};
+
+// The three contractions, for the tensors' own floating type, as separate
+// im2col/col2im + GEMM launches with `workspace` holding one batch element's
+// columns [Cg*K, M].
+//   gather_gemm:  pix[b] = Wm x im2col(img[b]) (+ bias per row)       (conv forward, transposed backward-input)
+//   gemm_scatter: img[b] (+)= col2im(Wm^T x pix[b]), img pre-filled    (conv backward-input, transposed forward)
+//   gather_wgrad: gW = sum_b pix[b] x im2col(img[b])^T                 (both backward-weight)
+template <typename T>
+int generic_gather_gemm(const ConvGeom& g, const T* img, const T* map, const T* wts, const T* Wm,
+                        const T* bias, T* pix, T* workspace, hipStream_t stream);
+template <typename T>
+int generic_gemm_scatter(const ConvGeom& g, const T* pix, const T* map, const T* wts, const T* Wm,
+                         const T* bias, T* img, T* workspace, hipStream_t stream);
+template <typename T>
+int generic_gather_wgrad(const ConvGeom& g, const T* pix, const T* map, const T* wts, const T* img,
+                         T* gW, T* workspace, hipStream_t stream);
+
+}  // namespace sdk

@@ -1,0 +1,498 @@
+// Memory-bound mapped gather / scatter kernels for gfx950 and their C entry
+// points: resample_from_map / resample_to_map, mapped im2col / col2im, mapped
+// max pool / unpool.
+//
+// Common shape of every kernel: one thread owns one map pixel (lanes of a
+// wavefront own consecutive pixels, so sample-map reads, value reads and value
+// writes are contiguous across the wave) and applies the pixel's taps to a
+// chunk of PC image planes held in registers, so the tap arithmetic and the
+// map traffic are amortised over PC planes and PC independent loads are in
+// flight per lane.  grid.x walks pixels, grid.y walks plane chunks.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+
+#include "sdk_host.hpp"
+#include "sdk_taps.hpp"
+
+namespace sdk {
+
+constexpr int kBlock = 256;  // 4 wavefronts
+constexpr int kPC = 8;       // planes per thread
+
+// ---------------------------------------------------------------------------
+// Fill kernels (scatter targets start from zero; hipMemsetAsync is avoided so
+// that callers may capture these entry points into a HIP graph).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fill_kernel(T* __restrict__ p, size_t n, T v) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+// 16-byte stores for the bulk of a zero fill.
+__global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) p[i] = z;
+}
+
+int zero_fill(void* ptr, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return SDK_OK;
+  // ptr comes from a framework allocator (>= 256-byte aligned) and all element
+  // sizes divide 16, so only a tail of < 16 bytes needs the scalar kernel.
+  const size_t n16 = ((uintptr_t)ptr % 16 == 0) ? bytes / 16 : 0;
+  if (n16) {
+    const int blocks = (int)std::min<size_t>(ceil_div((int64_t)n16, kBlock), 256 * 16);
+    launch(zero16_kernel, dim3(blocks), dim3(kBlock), stream, (uint4*)ptr, n16);
+  }
+  const size_t done = n16 * 16;
+  if (done < bytes) {
+    const size_t rest = bytes - done;
+    const int blocks = (int)std::min<size_t>(ceil_div((int64_t)rest, kBlock), 256 * 16);
+    launch(fill_kernel<unsigned char>, dim3(blocks), dim3(kBlock), stream,
+                       (unsigned char*)ptr + done, rest, (unsigned char)0);
+  }
+  SDK_LAUNCH_CHECK("zero_fill");
+  return SDK_OK;
+}
+
+// ---------------------------------------------------------------------------
+// resample_from_map (gather).  Body: ext_modules/include/common/resample.h:34-52,
+// :85-107.  planes = B*C; image plane stride HW; out plane stride MP.
+// ---------------------------------------------------------------------------
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
+    const T* __restrict__ image, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ out, int planes, int H, int W, int MP, int P) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= MP) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  T acc[kPC];
+  gather_sample<T, INTERP, WEIGHTED, kPC>(image + (size_t)plane0 * HW, HW, np,
+                                          map + (size_t)pix * q * 2,
+                                          WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W, acc);
+#pragma unroll
+  for (int j = 0; j < kPC; ++j)
+    if (j < np) out[(size_t)(plane0 + j) * MP + pix] = acc[j];
+}
+
+// ---------------------------------------------------------------------------
+// resample_to_map (scatter).  Body: common/resample.h:11-31, :55-82.
+// ONES: the input is an implicit all-ones plane (weight-sum pass).
+// ---------------------------------------------------------------------------
+template <typename T, int INTERP, bool WEIGHTED, bool ONES>
+__global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
+    const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ out, int planes, int H, int W, int MP, int P) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= MP) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  T val[kPC];
+#pragma unroll
+  for (int j = 0; j < kPC; ++j)
+    val[j] = ONES ? T(1) : (j < np ? in[(size_t)(plane0 + j) * MP + pix] : T(0));
+  scatter_sample<T, INTERP, WEIGHTED, kPC>(out + (size_t)plane0 * HW, HW, np,
+                                           map + (size_t)pix * q * 2,
+                                           WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W, val);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void normalize_kernel(T* __restrict__ data,
+                                                           const T* __restrict__ wsum, T eps,
+                                                           size_t plane_size, size_t total) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride)
+    data[i] = data[i] / (wsum[i % plane_size] + eps);
+}
+
+// ---------------------------------------------------------------------------
+// mapped im2col / col2im, batched.  Bodies: common/mapped_im2col.h:11-41, :44-77,
+// :80-116, :119-158.  grid.y walks chunks of the B*C image planes; a plane's K
+// column rows are (plane*K + k).
+// ---------------------------------------------------------------------------
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_im2col_kernel(
+    const T* __restrict__ im, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ col, int planes, int H, int W, int M, int K, int P) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= M) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  for (int k = 0; k < K; ++k) {
+    const size_t s = ((size_t)pix * K + k) * q;
+    T acc[kPC];
+    gather_sample<T, INTERP, WEIGHTED, kPC>(im + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                            WEIGHTED ? wts + s : nullptr, P, H, W, acc);
+#pragma unroll
+    for (int j = 0; j < kPC; ++j)
+      if (j < np) col[((size_t)(plane0 + j) * K + k) * M + pix] = acc[j];
+  }
+}
+
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_col2im_kernel(
+    const T* __restrict__ col, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ im, int planes, int H, int W, int M, int K, int P) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= M) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  for (int k = 0; k < K; ++k) {
+    const size_t s = ((size_t)pix * K + k) * q;
+    T val[kPC];
+#pragma unroll
+    for (int j = 0; j < kPC; ++j)
+      val[j] = j < np ? col[((size_t)(plane0 + j) * K + k) * M + pix] : T(0);
+    scatter_sample<T, INTERP, WEIGHTED, kPC>(im + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                             WEIGHTED ? wts + s : nullptr, P, H, W, val);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// mapped max pool.  Body: common/mapped_max_pool.h:13-57, :81-133 (device
+// branch: running maximum starts at -FLT_MAX for every T, index at -1).
+// ---------------------------------------------------------------------------
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
+    const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ out, int64_t* __restrict__ idx, int planes, int H, int W, int M, int K,
+    int P) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= M) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  T best[kPC];
+  int best_k[kPC];
+#pragma unroll
+  for (int j = 0; j < kPC; ++j) {
+    best[j] = T(-FLT_MAX);
+    best_k[j] = -1;
+  }
+  for (int k = 0; k < K; ++k) {
+    const size_t s = ((size_t)pix * K + k) * q;
+    T v[kPC];
+    gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                            WEIGHTED ? wts + s : nullptr, P, H, W, v);
+#pragma unroll
+    for (int j = 0; j < kPC; ++j)
+      if (v[j] > best[j]) {  // strict: first maximum wins, NaN never wins
+        best[j] = v[j];
+        best_k[j] = k;
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < kPC; ++j)
+    if (j < np) {
+      const size_t o = (size_t)(plane0 + j) * M + pix;
+      out[o] = best[j];
+      idx[o] = best_k[j] < 0 ? (int64_t)-1
+                             : (int64_t)(((size_t)pix * K + best_k[j]) * q * 2);
+    }
+}
+
+// Unpool: body common/mapped_max_pool.h:60-78, :136-171.  One thread per pooled
+// element; the stored index names the winning sample inside the map (and,
+// halved, inside the weights).  Indices outside [0, map_elems) contribute nothing.
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_max_unpool_kernel(
+    const T* __restrict__ gout, const int64_t* __restrict__ idx, const T* __restrict__ map,
+    const T* __restrict__ wts, T* __restrict__ gin, size_t total, int H, int W, int M, int P,
+    int64_t map_elems) {
+  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= total) return;
+  const size_t plane = i / (size_t)M;
+  const int64_t s = idx[i];
+  const int q = WEIGHTED ? P : 1;
+  if (s < 0 || s + 2 * q > map_elems) return;
+  const T val[1] = {gout[i]};
+  scatter_sample<T, INTERP, WEIGHTED, 1>(gin + plane * (size_t)H * W, 0, 1, map + s,
+                                         WEIGHTED ? wts + s / 2 : nullptr, P, H, W, val);
+}
+
+// ---------------------------------------------------------------------------
+// Host-side launch helpers.
+// ---------------------------------------------------------------------------
+static int check_plane(int64_t h, int64_t w, const char* what) {
+  if (h <= 0 || w <= 0 || h * w >= ((int64_t)1 << 31))
+    return fail(SDK_ERR_INVALID_ARGUMENT, "%s: plane %lld x %lld must have 1 .. 2^31-1 elements",
+                what, (long long)h, (long long)w);
+  return SDK_OK;
+}
+
+static int check_grid_y(int64_t planes, const char* what) {
+  if (ceil_div(planes, kPC) > 65535)
+    return fail(SDK_ERR_UNSUPPORTED, "%s: batch*channels = %lld exceeds %d", what,
+                (long long)planes, 65535 * kPC);
+  return SDK_OK;
+}
+
+template <typename T>
+static int launch_resample_from_map(const T* image, const T* map, const T* wts, T* out,
+                                    int64_t planes, int H, int W, int MP, int P, int interp,
+                                    hipStream_t stream) {
+  const dim3 grid((unsigned)ceil_div(MP, kBlock), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((resample_from_map_kernel<T, INTERP, WEIGHTED>), grid,
+                                          dim3(kBlock), stream, image, map, wts, out,
+                                          (int)planes, H, W, MP, P)));
+  SDK_LAUNCH_CHECK("resample_from_map");
+  return SDK_OK;
+}
+
+template <typename T>
+static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
+                                  int64_t planes, int H, int W, int MP, int P, int interp,
+                                  hipStream_t stream) {
+  int rc = zero_fill(out, sizeof(T) * (size_t)planes * H * W, stream);
+  if (rc != SDK_OK) return rc;
+  const dim3 grid((unsigned)ceil_div(MP, kBlock), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, false>),
+                                          grid, dim3(kBlock), stream, in, map, wts, out,
+                                          (int)planes, H, W, MP, P)));
+  SDK_LAUNCH_CHECK("resample_to_map");
+  if (wsum) {
+    rc = zero_fill(wsum, sizeof(T) * (size_t)H * W, stream);
+    if (rc != SDK_OK) return rc;
+    const dim3 g1((unsigned)ceil_div(MP, kBlock), 1);
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, true>),
+                                            g1, dim3(kBlock), stream, (const T*)nullptr, map,
+                                            wts, wsum, 1, H, W, MP, P)));
+    SDK_LAUNCH_CHECK("resample_to_map(weight_sum)");
+  }
+  return SDK_OK;
+}
+
+// Shared with the convolution drivers (declared in conv_internal.hpp).
+template <typename T>
+int launch_mapped_im2col(const T* im, const T* map, const T* wts, T* col, int64_t planes, int H,
+                         int W, int M, int K, int P, int interp, hipStream_t stream) {
+  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((mapped_im2col_kernel<T, INTERP, WEIGHTED>), grid,
+                                          dim3(kBlock), stream, im, map, wts, col, (int)planes,
+                                          H, W, M, K, P)));
+  SDK_LAUNCH_CHECK("mapped_im2col");
+  return SDK_OK;
+}
+
+// `im` must already hold the values to accumulate onto (zeros, or a bias fill).
+template <typename T>
+int launch_mapped_col2im(const T* col, const T* map, const T* wts, T* im, int64_t planes, int H,
+                         int W, int M, int K, int P, int interp, hipStream_t stream) {
+  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((mapped_col2im_kernel<T, INTERP, WEIGHTED>), grid,
+                                          dim3(kBlock), stream, col, map, wts, im, (int)planes,
+                                          H, W, M, K, P)));
+  SDK_LAUNCH_CHECK("mapped_col2im");
+  return SDK_OK;
+}
+
+template int launch_mapped_im2col<float>(const float*, const float*, const float*, float*, int64_t,
+                                         int, int, int, int, int, int, hipStream_t);
+template int launch_mapped_im2col<double>(const double*, const double*, const double*, double*,
+                                          int64_t, int, int, int, int, int, int, hipStream_t);
+template int launch_mapped_col2im<float>(const float*, const float*, const float*, float*, int64_t,
+                                         int, int, int, int, int, int, hipStream_t);
+template int launch_mapped_col2im<double>(const double*, const double*, const double*, double*,
+                                          int64_t, int, int, int, int, int, int, hipStream_t);
+
+}  // namespace sdk
+
+using namespace sdk;
+
+// ---------------------------------------------------------------------------
+// C entry points.
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int sdk_resample_from_map(const void* image, const void* sample_map, const void* interp_weights,
+                          void* out, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t map_height, int64_t map_width,
+                          int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                          sdk_stream_t stream) {
+  SDK_REQUIRE(image && sample_map && out, "resample_from_map: NULL pointer");
+  SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
+              "resample_from_map: weighted map needs interp_weights");
+  SDK_REQUIRE(batch >= 0 && channels >= 0, "resample_from_map: negative size");
+  int rc = check_plane(height, width, "resample_from_map(image)");
+  if (rc) return rc;
+  rc = check_plane(map_height, map_width, "resample_from_map(map)");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  rc = check_grid_y(planes, "resample_from_map");
+  if (rc) return rc;
+  SDK_DISPATCH_DTYPE(dtype, return launch_resample_from_map<T>(
+                                (const T*)image, (const T*)sample_map, (const T*)interp_weights,
+                                (T*)out, planes, (int)height, (int)width,
+                                (int)(map_height * map_width), num_interp_pts, interp,
+                                (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, void* weight_sum, int64_t batch, int64_t channels,
+                        int64_t map_height, int64_t map_width, int64_t height, int64_t width,
+                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                        sdk_stream_t stream) {
+  SDK_REQUIRE(input && sample_map && out, "resample_to_map: NULL pointer");
+  SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
+              "resample_to_map: weighted map needs interp_weights");
+  SDK_REQUIRE(batch >= 0 && channels >= 0, "resample_to_map: negative size");
+  int rc = check_plane(height, width, "resample_to_map(out)");
+  if (rc) return rc;
+  rc = check_plane(map_height, map_width, "resample_to_map(map)");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  rc = check_grid_y(planes, "resample_to_map");
+  if (rc) return rc;
+  if (planes == 0 && !weight_sum) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_resample_to_map<T>(
+                                (const T*)input, (const T*)sample_map, (const T*)interp_weights,
+                                (T*)out, (T*)weight_sum, planes, (int)height, (int)width,
+                                (int)(map_height * map_width), num_interp_pts, interp,
+                                (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, int64_t planes,
+                                int64_t plane_size, int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(data && weight_sum, "normalize_by_weight_sum: NULL pointer");
+  SDK_REQUIRE(planes >= 0 && plane_size >= 0, "normalize_by_weight_sum: negative size");
+  const size_t total = (size_t)planes * plane_size;
+  if (total == 0) return SDK_OK;
+  const int blocks = (int)std::min<int64_t>(ceil_div((int64_t)total, kBlock), 256 * 16);
+  SDK_DISPATCH_DTYPE(dtype, (launch(normalize_kernel<T>, dim3(blocks), dim3(kBlock),
+                                                (hipStream_t)stream, (T*)data,
+                                                (const T*)weight_sum, (T)eps, (size_t)plane_size,
+                                                total)));
+  SDK_LAUNCH_CHECK("normalize_by_weight_sum");
+  return SDK_OK;
+}
+
+static int check_mapped(const void* a, const void* map, const void* wts, const void* b,
+                        int64_t batch, int64_t channels, int64_t height, int64_t width,
+                        int64_t out_pixels, int64_t K, int32_t P, const char* what) {
+  SDK_REQUIRE(a && map && b, "%s: NULL pointer", what);
+  SDK_REQUIRE(P >= 0 && (P == 0 || wts), "%s: weighted map needs interp_weights", what);
+  SDK_REQUIRE(batch >= 0 && channels >= 0 && K >= 1, "%s: bad size", what);
+  SDK_REQUIRE(out_pixels > 0 && out_pixels < ((int64_t)1 << 31), "%s: bad output pixel count",
+              what);
+  int rc = check_plane(height, width, what);
+  if (rc) return rc;
+  return check_grid_y(batch * channels, what);
+}
+
+int sdk_mapped_im2col(const void* image, const void* sample_map, const void* interp_weights,
+                      void* columns, int64_t batch, int64_t channels, int64_t height,
+                      int64_t width, int64_t out_pixels, int64_t kernel_size,
+                      int32_t num_interp_pts, int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  int rc = check_mapped(image, sample_map, interp_weights, columns, batch, channels, height, width,
+                        out_pixels, kernel_size, num_interp_pts, "mapped_im2col");
+  if (rc) return rc;
+  if (batch * channels == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_mapped_im2col<T>(
+                                (const T*)image, (const T*)sample_map, (const T*)interp_weights,
+                                (T*)columns, batch * channels, (int)height, (int)width,
+                                (int)out_pixels, (int)kernel_size, num_interp_pts, interp,
+                                (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_mapped_col2im(const void* columns, const void* sample_map, const void* interp_weights,
+                      void* image, int64_t batch, int64_t channels, int64_t height,
+                      int64_t width, int64_t out_pixels, int64_t kernel_size,
+                      int32_t num_interp_pts, int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  int rc = check_mapped(columns, sample_map, interp_weights, image, batch, channels, height, width,
+                        out_pixels, kernel_size, num_interp_pts, "mapped_col2im");
+  if (rc) return rc;
+  if (batch * channels == 0) return SDK_OK;
+  const size_t esz = dtype == SDK_F64 ? 8 : 4;
+  rc = zero_fill(image, esz * (size_t)(batch * channels) * height * width, (hipStream_t)stream);
+  if (rc) return rc;
+  SDK_DISPATCH_DTYPE(dtype, return launch_mapped_col2im<T>(
+                                (const T*)columns, (const T*)sample_map,
+                                (const T*)interp_weights, (T*)image, batch * channels, (int)height,
+                                (int)width, (int)out_pixels, (int)kernel_size, num_interp_pts,
+                                interp, (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, int64_t* indices, int64_t batch, int64_t channels,
+                        int64_t height, int64_t width, int64_t out_height, int64_t out_width,
+                        int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                        int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(indices, "mapped_max_pool: NULL indices");
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_pool: bad output size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(input, sample_map, interp_weights, out, batch, channels, height, width, M,
+                        kernel_size, num_interp_pts, "mapped_max_pool");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_DTYPE(
+      dtype,
+      SDK_DISPATCH_INTERP(interp, num_interp_pts,
+                          (launch((mapped_max_pool_kernel<T, INTERP, WEIGHTED>), grid,
+                                              dim3(kBlock), (hipStream_t)stream,
+                                              (const T*)input, (const T*)sample_map,
+                                              (const T*)interp_weights, (T*)out, indices,
+                                              (int)planes, (int)height, (int)width, (int)M,
+                                              (int)kernel_size, num_interp_pts))));
+  SDK_LAUNCH_CHECK("mapped_max_pool");
+  return SDK_OK;
+}
+
+int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,
+                          const void* interp_weights, void* grad_input, int64_t batch,
+                          int64_t channels, int64_t height, int64_t width, int64_t out_height,
+                          int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
+                          int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(indices, "mapped_max_unpool: NULL indices");
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_unpool: bad pooled size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(grad_output, sample_map, interp_weights, grad_input, batch, channels,
+                        height, width, M, kernel_size, num_interp_pts, "mapped_max_unpool");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  const size_t esz = dtype == SDK_F64 ? 8 : 4;
+  rc = zero_fill(grad_input, esz * (size_t)planes * height * width, (hipStream_t)stream);
+  if (rc) return rc;
+  const size_t total = (size_t)planes * M;
+  const int64_t map_elems = M * kernel_size * pts(num_interp_pts) * 2;
+  SDK_REQUIRE(ceil_div((int64_t)total, kBlock) < ((int64_t)1 << 31),
+              "mapped_max_unpool: too many elements");
+  const dim3 grid((unsigned)ceil_div((int64_t)total, kBlock));
+  SDK_DISPATCH_DTYPE(
+      dtype,
+      SDK_DISPATCH_INTERP(interp, num_interp_pts,
+                          (launch((mapped_max_unpool_kernel<T, INTERP, WEIGHTED>),
+                                              grid, dim3(kBlock), (hipStream_t)stream,
+                                              (const T*)grad_output, indices,
+                                              (const T*)sample_map, (const T*)interp_weights,
+                                              (T*)grad_input, total, (int)height, (int)width,
+                                              (int)M, num_interp_pts, map_elems))));
+  SDK_LAUNCH_CHECK("mapped_max_unpool");
+  return SDK_OK;
+}
+
+}  // extern "C"

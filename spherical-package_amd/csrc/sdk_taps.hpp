@@ -1,0 +1,172 @@
+// Device-side interpolation primitives: a sample coordinate is turned once into
+// up to four (offset, weight) taps, which are then applied to any number of
+// image planes.  Semantics follow the reference's point functions
+// (ext_modules/include/core/interpolation.h:97-247, blend order :17-33, splat
+// :36-61); translation units including this header must be compiled with
+// -ffp-contract=off so products and sums round exactly as on the reference CPU.
+//
+// One deliberate difference: a tap whose weight is exactly zero is neither read
+// nor written.  For finite data the result is identical (the reference adds
+// 0*value); only a non-finite value under a zero weight, which the reference
+// would turn into NaN, is ignored here.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace sdk {
+
+template <typename T>
+__device__ __forceinline__ void atomic_add_noret(T* addr, T v) {
+  // Relaxed, device-scope; with -munsafe-fp-atomics this is one
+  // global_atomic_add_f32 / _f64 without return value.
+  (void)__hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ int to_int_clamped(float v) {
+  return (int)fminf(fmaxf(v, -2.0e9f), 2.0e9f);
+}
+__device__ __forceinline__ int to_int_clamped(double v) {
+  return (int)fmin(fmax(v, -2.0e9), 2.0e9);
+}
+__device__ __forceinline__ float floor_t(float v) { return floorf(v); }
+__device__ __forceinline__ double floor_t(double v) { return floor(v); }
+// Round half away from zero, the rule of llround() used by the reference
+// (core/interpolation.h:102-103).
+__device__ __forceinline__ float round_t(float v) { return roundf(v); }
+__device__ __forceinline__ double round_t(double v) { return round(v); }
+
+// ((v % n) + n) % n for n > 0 (core/util.h:59-62), with the common in-range case first.
+__device__ __forceinline__ int wrap_index(int v, int n) {
+  if ((unsigned)v < (unsigned)n) return v;
+  int r = v % n;
+  return r < 0 ? r + n : r;
+}
+
+// INTERP: 0 nearest, 1 bilinear, 2 bispherical.
+template <typename T, int INTERP>
+struct PointTaps {
+  static constexpr int N = (INTERP == 0) ? 1 : 4;
+  int off[N];  // element offset inside one H x W plane, or -1 (inactive tap)
+  T w[N];
+
+  __device__ __forceinline__ void set(T x, T y, int H, int W) {
+    if constexpr (INTERP == 0) {
+      const int xi = to_int_clamped(round_t(x));
+      const int yi = to_int_clamped(round_t(y));
+      const bool ok = (unsigned)xi < (unsigned)W && (unsigned)yi < (unsigned)H;
+      off[0] = ok ? yi * W + xi : -1;
+      w[0] = T(1);
+    } else {
+      const T fx = floor_t(x), fy = floor_t(y);
+      const int x1 = to_int_clamped(fx), y1 = to_int_clamped(fy);
+      // Weights against the unwrapped integer neighbours x1, x1+1, y1, y1+1.
+      const T A = (fy + T(1)) - y, B = (fx + T(1)) - x, C = x - fx, D = y - fy;
+      const bool y1ok = (unsigned)y1 < (unsigned)H;
+      const bool y2ok = y1 >= -1 && y1 < H - 1;
+      int c1, c2;
+      bool x1ok, x2ok;
+      if constexpr (INTERP == 2) {
+        c1 = wrap_index(x1, W);
+        c2 = (c1 + 1 == W) ? 0 : c1 + 1;
+        x1ok = x2ok = true;
+      } else {
+        c1 = x1;
+        c2 = x1 + 1;
+        x1ok = (unsigned)x1 < (unsigned)W;
+        x2ok = x1 >= -1 && x1 < W - 1;
+      }
+      w[0] = A * B;
+      w[1] = A * C;
+      w[2] = D * B;
+      w[3] = D * C;
+      const int r1 = y1 * W, r2 = r1 + W;
+      off[0] = (x1ok && y1ok && w[0] != T(0)) ? r1 + c1 : -1;
+      off[1] = (x2ok && y1ok && w[1] != T(0)) ? r1 + c2 : -1;
+      off[2] = (x1ok && y2ok && w[2] != T(0)) ? r2 + c1 : -1;
+      off[3] = (x2ok && y2ok && w[3] != T(0)) ? r2 + c2 : -1;
+    }
+  }
+
+  // Branch-free guarded read: inactive taps read element 0 and discard it.
+  static __device__ __forceinline__ T read(const T* __restrict__ plane, int o) {
+    const T d = plane[o < 0 ? 0 : o];
+    return o < 0 ? T(0) : d;
+  }
+
+  __device__ __forceinline__ T gather(const T* __restrict__ plane) const {
+    if constexpr (INTERP == 0) {
+      return read(plane, off[0]);
+    } else {
+      const T t0 = w[0] * read(plane, off[0]);
+      const T t1 = w[1] * read(plane, off[1]);
+      const T t2 = w[2] * read(plane, off[2]);
+      const T t3 = w[3] * read(plane, off[3]);
+      return t0 + t1 + t2 + t3;
+    }
+  }
+
+  __device__ __forceinline__ void scatter(T* __restrict__ plane, T v) const {
+    if constexpr (INTERP == 0) {
+      if (off[0] >= 0) atomic_add_noret(plane + off[0], v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (off[i] >= 0) atomic_add_noret(plane + off[i], w[i] * v);
+    }
+  }
+};
+
+// Applies one map sample (1 point, or P weighted points accumulated in
+// ascending order: core/resample.h:144-161) to PC planes that are `stride`
+// elements apart.  Planes j >= np are not touched (acc[j] = 0).
+template <typename T, int INTERP, bool WEIGHTED, int PC>
+__device__ __forceinline__ void gather_sample(const T* __restrict__ base, size_t stride, int np,
+                                              const T* __restrict__ coords,
+                                              const T* __restrict__ wts, int P, int H, int W,
+                                              T (&acc)[PC]) {
+  PointTaps<T, INTERP> t;
+  if constexpr (!WEIGHTED) {
+    t.set(coords[0], coords[1], H, W);
+#pragma unroll
+    for (int j = 0; j < PC; ++j) {
+      const T v = t.gather(base + (size_t)(j < np ? j : 0) * stride);
+      acc[j] = j < np ? v : T(0);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < PC; ++j) acc[j] = T(0);
+    for (int p = 0; p < P; ++p) {
+      t.set(coords[2 * p], coords[2 * p + 1], H, W);
+      const T wt = wts[p];
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        const T v = t.gather(base + (size_t)(j < np ? j : 0) * stride);
+        if (j < np) acc[j] += wt * v;
+      }
+    }
+  }
+}
+
+// Adjoint of gather_sample (core/resample.h:127-141): splats val[j] into plane j.
+template <typename T, int INTERP, bool WEIGHTED, int PC>
+__device__ __forceinline__ void scatter_sample(T* __restrict__ base, size_t stride, int np,
+                                               const T* __restrict__ coords,
+                                               const T* __restrict__ wts, int P, int H, int W,
+                                               const T (&val)[PC]) {
+  PointTaps<T, INTERP> t;
+  if constexpr (!WEIGHTED) {
+    t.set(coords[0], coords[1], H, W);
+#pragma unroll
+    for (int j = 0; j < PC; ++j)
+      if (j < np) t.scatter(base + (size_t)j * stride, val[j]);
+  } else {
+    for (int p = 0; p < P; ++p) {
+      t.set(coords[2 * p], coords[2 * p + 1], H, W);
+      const T wt = wts[p];
+#pragma unroll
+      for (int j = 0; j < PC; ++j)
+        if (j < np) t.scatter(base + (size_t)j * stride, wt * val[j]);
+    }
+  }
+}
+
+}  // namespace sdk

@@ -1,0 +1,212 @@
+"""Autograd functions and functional entry points of the mapped operations.
+
+Counterpart of the reference's layers/functional/{mapped_convolution,
+mapped_pooling,resample}.py: same call signatures, same choice between the
+weighted and unweighted extension modules, same gradient tuple arity.
+"""
+import torch
+
+import _spherical_distortion_ext._mapped_convolution as _mapped_conv
+import _spherical_distortion_ext._mapped_max_pooling as _mapped_max_pool
+import _spherical_distortion_ext._mapped_transposed_convolution as _mapped_transposed_conv
+import _spherical_distortion_ext._resample as _resample
+import _spherical_distortion_ext._weighted_mapped_convolution as _weighted_mapped_conv
+import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mapped_max_pool
+import _spherical_distortion_ext._weighted_mapped_transposed_convolution as _weighted_mapped_transposed_conv
+import _spherical_distortion_ext._weighted_resample as _weighted_resample
+
+from ..layer_utils import InterpolationType, check_args, check_input_map_shape
+
+
+class MappedConvolutionFunction(torch.autograd.Function):
+    """layers/functional/mapped_convolution.py:14-61."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias, sample_map, kernel_size, interp, interp_weights=None):
+        ctx.save_for_backward(input, weight, bias, sample_map, interp_weights)
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = InterpolationType(interp)
+        if interp_weights is None:
+            return _mapped_conv.mapped_conv_forward(input, sample_map, weight, bias,
+                                                    ctx.kernel_size, ctx.interp)
+        return _weighted_mapped_conv.weighted_mapped_conv_forward(
+            input, sample_map, interp_weights, weight, bias, ctx.kernel_size, ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight, bias, sample_map, interp_weights = ctx.saved_tensors
+        if interp_weights is None:
+            grads = _mapped_conv.mapped_conv_backward(grad_output, sample_map, input, weight, bias,
+                                                      ctx.kernel_size, ctx.interp)
+        else:
+            grads = _weighted_mapped_conv.weighted_mapped_conv_backward(
+                grad_output, sample_map, interp_weights, input, weight, bias, ctx.kernel_size,
+                ctx.interp)
+        grad_input, grad_weight, grad_bias = grads
+        return grad_input, grad_weight, grad_bias, None, None, None, None
+
+
+class MappedTransposedConvolutionFunction(torch.autograd.Function):
+    """layers/functional/mapped_convolution.py:64-113."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias, sample_map, output_height, output_width, kernel_size,
+                interp, interp_weights=None):
+        ctx.save_for_backward(input, sample_map, weight, bias, interp_weights)
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = InterpolationType(interp)
+        if interp_weights is None:
+            return _mapped_transposed_conv.mapped_transposed_conv_forward(
+                input, sample_map, weight, bias, output_height, output_width, ctx.kernel_size,
+                ctx.interp)
+        return _weighted_mapped_transposed_conv.weighted_mapped_transposed_conv_forward(
+            input, sample_map, interp_weights, weight, bias, output_height, output_width,
+            ctx.kernel_size, ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, sample_map, weight, bias, interp_weights = ctx.saved_tensors
+        if interp_weights is None:
+            grads = _mapped_transposed_conv.mapped_transposed_conv_backward(
+                grad_output, sample_map, input, weight, bias, ctx.kernel_size, ctx.interp)
+        else:
+            grads = _weighted_mapped_transposed_conv.weighted_mapped_transposed_conv_backward(
+                grad_output, sample_map, interp_weights, input, weight, bias, ctx.kernel_size,
+                ctx.interp)
+        grad_input, grad_weight, grad_bias = grads
+        return grad_input, grad_weight, grad_bias, None, None, None, None, None, None
+
+
+class MappedMaxPoolFunction(torch.autograd.Function):
+    """layers/functional/mapped_pooling.py:106-153: returns (pooled, idx_mask);
+    idx_mask is not differentiable."""
+
+    @staticmethod
+    def forward(ctx, input, sample_map, kernel_size, interp, interp_weights=None):
+        interp = InterpolationType(interp)
+        if interp_weights is None:
+            pooled, idx_mask = _mapped_max_pool.mapped_max_pool(input, sample_map, kernel_size,
+                                                                interp)
+        else:
+            pooled, idx_mask = _weighted_mapped_max_pool.weighted_mapped_max_pool(
+                input, sample_map, interp_weights, kernel_size, interp)
+        ctx.mark_non_differentiable(idx_mask)
+        ctx.save_for_backward(idx_mask, sample_map, interp_weights)
+        ctx.in_hw = (int(input.shape[2]), int(input.shape[3]))
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = interp
+        return pooled, idx_mask
+
+    @staticmethod
+    def backward(ctx, grad_output, idx_mask_grad=None):
+        idx_mask, sample_map, interp_weights = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if interp_weights is None:
+            grad_input = _mapped_max_pool.mapped_max_unpool(
+                grad_output, idx_mask, sample_map, ctx.in_hw[0], ctx.in_hw[1], ctx.kernel_size,
+                ctx.interp)
+        else:
+            grad_input = _weighted_mapped_max_pool.weighted_mapped_max_unpool(
+                grad_output, idx_mask, sample_map, interp_weights, ctx.in_hw[0], ctx.in_hw[1],
+                ctx.kernel_size, ctx.interp)
+        return grad_input, None, None, None, None
+
+
+class ResampleFunction(torch.autograd.Function):
+    """Forward scatter, backward gather (layers/functional/resample.py:11-48)."""
+
+    @staticmethod
+    def forward(ctx, input, sample_map, output_shape, interp, interp_weights=None):
+        ctx.save_for_backward(sample_map, interp_weights)
+        ctx.interp = InterpolationType(interp)
+        if interp_weights is None:
+            return _resample.resample_to_map(input, sample_map, output_shape[0], output_shape[1],
+                                             ctx.interp)
+        return _weighted_resample.weighted_resample_to_map(
+            input, sample_map, interp_weights, output_shape[0], output_shape[1], ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        sample_map, interp_weights = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if interp_weights is None:
+            grad = _resample.resample_from_map(grad_output, sample_map, ctx.interp)
+        else:
+            grad = _weighted_resample.weighted_resample_from_map(grad_output, sample_map,
+                                                                 interp_weights, ctx.interp)
+        return grad, None, None, None, None
+
+
+class UnresampleFunction(torch.autograd.Function):
+    """Forward gather, backward scatter (layers/functional/resample.py:51-83)."""
+
+    @staticmethod
+    def forward(ctx, input, sample_map, interp, interp_weights=None):
+        ctx.save_for_backward(sample_map, interp_weights)
+        ctx.interp = InterpolationType(interp)
+        ctx.in_hw = (int(input.shape[2]), int(input.shape[3]))
+        if interp_weights is None:
+            return _resample.resample_from_map(input, sample_map, ctx.interp)
+        return _weighted_resample.weighted_resample_from_map(input, sample_map, interp_weights,
+                                                             ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        sample_map, interp_weights = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if interp_weights is None:
+            grad = _resample.resample_to_map(grad_output, sample_map, ctx.in_hw[0], ctx.in_hw[1],
+                                             ctx.interp)
+        else:
+            grad = _weighted_resample.weighted_resample_to_map(
+                grad_output, sample_map, interp_weights, ctx.in_hw[0], ctx.in_hw[1], ctx.interp)
+        return grad, None, None, None
+
+
+# ----------------------------------------------------------------------------- entry points
+def mapped_convolution(input, weight, bias, sample_map, kernel_size, interp,
+                       interp_weights=None):
+    """layers/functional/mapped_convolution.py:121-131."""
+    check_args(input, sample_map, interp_weights, weight.shape[1], weight.shape[2])
+    return MappedConvolutionFunction.apply(input, weight, bias, sample_map, kernel_size, interp,
+                                           interp_weights)
+
+
+def mapped_transposed_convolution(input, weight, bias, sample_map, output_height, output_width,
+                                  kernel_size, interp, interp_weights=None):
+    """layers/functional/mapped_convolution.py:134-148."""
+    check_args(input, sample_map, interp_weights, weight.shape[0], weight.shape[2])
+    check_input_map_shape(input, sample_map)
+    return MappedTransposedConvolutionFunction.apply(input, weight, bias, sample_map,
+                                                     output_height, output_width, kernel_size,
+                                                     interp, interp_weights)
+
+
+def mapped_max_pool(input, sample_map, kernel_size, interp, interp_weights=None):
+    """-> (pooled, idx_mask); layers/functional/mapped_pooling.py:225-232."""
+    check_args(input, sample_map, interp_weights, None, kernel_size)
+    return MappedMaxPoolFunction.apply(input, sample_map, kernel_size, interp, interp_weights)
+
+
+def _with_batch_dim(input):
+    assert input.dim() in [3, 4], \
+        'Input must have 3 or 4 dimensions (input.dim() == {})'.format(input.dim())
+    return (input.unsqueeze(0), True) if input.dim() == 3 else (input, False)
+
+
+def resample(input, sample_map, output_shape, interp, interp_weights=None):
+    """Scatter `input` through the map; a 3-D input is treated as one batch element
+    (layers/functional/resample.py:113-134)."""
+    batched, added = _with_batch_dim(input)
+    check_args(batched, sample_map, interp_weights, None, None)
+    check_input_map_shape(batched, sample_map)
+    out = ResampleFunction.apply(batched, sample_map, output_shape, interp, interp_weights)
+    return out.squeeze(0) if added else out
+
+
+def unresample(input, sample_map, interp, interp_weights=None):
+    """Gather from `input` at the map (layers/functional/resample.py:137-157)."""
+    batched, added = _with_batch_dim(input)
+    check_args(batched, sample_map, interp_weights, None, None)
+    out = UnresampleFunction.apply(batched, sample_map, interp, interp_weights)
+    return out.squeeze(0) if added else out

@@ -1,0 +1,248 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on identical seeded inputs,
+and against the fixtures the reference's compiled CPU code produced.
+
+Tolerances (norm-relative, max|a-b| / max|b|):
+  nearest gather and pooling indices      bit-exact
+  float32 forward                         1e-5
+  float32 backward (atomic reorder)       1e-4
+  float64                                 1e-12
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN_DIR, relerr
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FWD_TOL = {np.float32: 1e-5, np.float64: 1e-12}
+BWD_TOL = {np.float32: 1e-4, np.float64: 1e-12}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from _spherical_distortion_ext import _ops
+    return _ops
+
+
+def _t(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _n(t):
+    return t.detach().cpu().numpy()
+
+
+def _coords(rng, shape, h, w, dtype, margin=2.0):
+    xy = rng.uniform(-margin, [w - 1 + margin, h - 1 + margin], size=tuple(shape) + (2,))
+    sel = rng.uniform(size=shape) < 0.25
+    xy[sel] = np.round(xy[sel])
+    sel = rng.uniform(size=shape) < 0.1
+    xy[sel] = np.floor(xy[sel]) + 0.5
+    return np.ascontiguousarray(xy.astype(dtype))
+
+
+CASES = [(i, wgt, dt) for i in (0, 1, 2) for wgt in (False, True)
+         for dt in (np.float32, np.float64)]
+
+
+def _ids(c):
+    return "interp%d-%s-%s" % (c[0], "weighted" if c[1] else "plain", np.dtype(c[2]).name)
+
+
+@pytest.mark.parametrize("case", CASES, ids=_ids)
+def test_resample_both_directions(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(100 + interp)
+    B, C, H, W, MH, MW, P = 3, 5, 37, 53, 29, 41, 3   # ragged: nothing divides a tile size
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    m = _coords(rng, (MH, MW, P) if weighted else (MH, MW), H, W, dt)
+    iw = rng.uniform(0.1, 1, (MH, MW, P)).astype(dt) if weighted else None
+    got = _n(ops.resample_from_map(_t(x), _t(m), _t(iw), interp))
+    want = oracle.resample_from_map(x, m, interp, iw)
+    if interp == 0 and not weighted:
+        assert np.array_equal(got, want)          # nearest resampling: bit-exact
+    assert np.array_equal(got, want) or relerr(got, want) <= FWD_TOL[dt]
+    y = rng.standard_normal((B, C, MH, MW)).astype(dt)
+    got = _n(ops.resample_to_map(_t(y), _t(m), _t(iw), H, W, interp))
+    want = oracle.resample_to_map(y, m, H, W, interp, iw)
+    assert relerr(got, want) <= BWD_TOL[dt]
+    # normalised variant == scatter(y) / (scatter(ones) + eps)
+    gotn, wsum = ops.resample_to_map_normalized(_t(y), _t(m), _t(iw), H, W, interp, 1e-12)
+    ones = oracle.resample_to_map(np.ones((1, 1, MH, MW), dt), m, H, W, interp, iw)[0, 0]
+    assert relerr(_n(wsum), ones) <= BWD_TOL[dt]
+    assert relerr(_n(gotn), want / (ones + dt(1e-12))) <= 10 * BWD_TOL[dt]
+
+
+@pytest.mark.parametrize("case", CASES, ids=_ids)
+def test_im2col_col2im(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(200 + interp)
+    B, C, H, W, OH, OW, K, P = 2, 11, 19, 23, 13, 17, 5, 2
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if weighted else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if weighted else None
+    got = _n(ops.mapped_im2col(_t(x), _t(m), _t(iw), interp))
+    want = np.stack([oracle.mapped_im2col(x[b], m, interp, iw) for b in range(B)])
+    assert np.array_equal(got, want) or relerr(got, want) <= FWD_TOL[dt]
+    if interp == 0 and not weighted:
+        assert np.array_equal(got, want)
+    col = rng.standard_normal((B, C * K, OH * OW)).astype(dt)
+    got = _n(ops.mapped_col2im(_t(col), _t(m), _t(iw), H, W, interp))
+    want = np.stack([oracle.mapped_col2im(col[b], m, H, W, interp, iw) for b in range(B)])
+    assert relerr(got, want) <= BWD_TOL[dt]
+
+
+@pytest.mark.parametrize("case", CASES, ids=_ids)
+def test_max_pool_and_unpool(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(300 + interp)
+    B, C, H, W, OH, OW, K, P = 2, 9, 21, 27, 10, 13, 9, 2
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if weighted else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if weighted else None
+    val, idx = ops.mapped_max_pool(_t(x), _t(m), _t(iw), K, interp)
+    wval, widx = oracle.mapped_max_pool(x, m, K, interp, iw)          # device-branch init
+    assert np.array_equal(_n(idx), widx)                              # indices: bit-exact
+    assert np.array_equal(_n(val), wval)
+    # against the reference host branch: identical wherever it found a winner
+    hval, hidx = oracle.mapped_max_pool(x, m, K, interp, iw, host_init_quirk=True)
+    ok = hidx >= 0
+    assert np.array_equal(_n(idx)[ok], hidx[ok]) and np.array_equal(_n(val)[ok], hval[ok])
+    g = rng.standard_normal((B, C, OH, OW)).astype(dt)
+    got = _n(ops.mapped_max_unpool(_t(g), idx, _t(m), _t(iw), H, W, K, interp))
+    want = oracle.mapped_max_unpool(g, widx, m, H, W, K, interp, iw)
+    assert relerr(got, want) <= BWD_TOL[dt]
+
+
+def test_pool_ties_nan_and_no_winner(ops, oracle):
+    """First maximum wins; NaN never wins; a window below -FLT_MAX has index -1."""
+    x = np.zeros((1, 1, 2, 4), np.float32)
+    x[0, 0, 0] = [5, 5, np.nan, 1]
+    x[0, 0, 1] = [-np.inf, -np.inf, -np.inf, -np.inf]
+    m = np.array([[[[0, 0], [1, 0], [2, 0]], [[2, 0], [3, 0], [0, 0]],
+                   [[0, 1], [1, 1], [2, 1]], [[9, 9], [9, 9], [9, 9]]]], np.float32)
+    val, idx = ops.mapped_max_pool(_t(x), _t(m), None, 3, 0)
+    wval, widx = oracle.mapped_max_pool(x, m, 3, 0)
+    assert np.array_equal(_n(idx), widx) and np.array_equal(_n(val), wval)
+    assert _n(idx).reshape(-1).tolist() == [0, 6 + 4, -1, 18]
+    g = np.ones((1, 1, 1, 4), np.float32)
+    got = _n(ops.mapped_max_unpool(_t(g), idx, _t(m), None, 2, 4, 3, 0))
+    assert got.reshape(-1).tolist() == [2, 0, 0, 0, 0, 0, 0, 0]  # -1 and out-of-image drop out
+
+
+CONV_CASES = [(i, wgt, dt) for i in (0, 1, 2) for wgt in (False, True)
+              for dt in (np.float32, np.float64)]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=_ids)
+def test_mapped_convolution(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(400 + interp)
+    B, Cin, Cout, H, W, OH, OW, K, P = 2, 7, 5, 17, 19, 11, 13, 4, 3
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if weighted else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if weighted else None
+    wt = rng.standard_normal((Cout, Cin, K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), K, interp))
+    assert relerr(got, oracle.mapped_conv_forward(x, m, wt, b, K, interp, iw)) <= FWD_TOL[dt]
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= BWD_TOL[dt]
+    assert relerr(_n(gw), ww) <= BWD_TOL[dt]
+    assert relerr(_n(gb), wb) <= BWD_TOL[dt]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=_ids)
+def test_mapped_transposed_convolution(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(500 + interp)
+    B, Cin, Cout, IH, IW, OH, OW, K, P = 2, 6, 4, 9, 11, 15, 18, 3, 2
+    x = rng.standard_normal((B, Cin, IH, IW)).astype(dt)
+    m = _coords(rng, (IH, IW, K, P) if weighted else (IH, IW, K), OH, OW, dt)
+    iw = rng.uniform(0.1, 1, (IH, IW, K, P)).astype(dt) if weighted else None
+    wt = rng.standard_normal((Cin, Cout, K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), OH, OW, K,
+                                                interp))
+    want = oracle.mapped_transposed_conv_forward(x, m, wt, b, OH, OW, K, interp, iw)
+    assert relerr(got, want) <= BWD_TOL[dt]      # the forward is the scatter here
+    gi, gw, gb = ops.mapped_transposed_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b),
+                                                     K, interp)
+    wi, ww, wb = oracle.mapped_transposed_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= BWD_TOL[dt]
+    assert relerr(_n(gw), ww) <= BWD_TOL[dt]
+    assert relerr(_n(gb), wb) <= BWD_TOL[dt]
+
+
+# ------------------------------------------------------------------------------------------
+# Against the compiled reference's fixtures directly (no oracle in between).
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("d", ["f64", "f32"])
+@pytest.mark.parametrize("interp", [0, 1, 2])
+def test_against_reference_fixtures(ops, d, interp):
+    fx = np.load(os.path.join(GOLDEN_DIR, "ref_fixtures.npz"))
+    dt = np.float64 if d == "f64" else np.float32
+    ftol, btol = (1e-12, 1e-12) if d == "f64" else (1e-5, 1e-4)
+    g = lambda n: _t(fx["%s/in/%s" % (d, n)])  # noqa: E731
+    pre = "%s/i%d/" % (d, interp)
+    H, W, K = 6, 7, 3
+    assert np.array_equal(_n(ops.resample_from_map(g("x"), g("r_u"), None, interp)),
+                          fx[pre + "from"])
+    got = _n(ops.resample_from_map(g("x"), g("r_w"), g("riw"), interp))
+    assert np.array_equal(got, fx[pre + "wfrom"]) or relerr(got, fx[pre + "wfrom"]) <= ftol
+    assert relerr(_n(ops.resample_to_map(g("rin"), g("r_u"), None, H, W, interp)),
+                  fx[pre + "to"]) <= btol
+    assert relerr(_n(ops.resample_to_map(g("rin"), g("r_w"), g("riw"), H, W, interp)),
+                  fx[pre + "wto"]) <= btol
+    for wtag, m, iw in (("", g("m_u"), None), ("w", g("m_w"), g("iw"))):
+        out = ops.mapped_conv_forward(g("x"), m, iw, g("weight"), g("bias"), K, interp)
+        assert relerr(_n(out), fx[pre + wtag + "conv_fwd"]) <= ftol
+        gi, gw, gb = ops.mapped_conv_backward(g("gout"), m, iw, g("x"), g("weight"), g("bias"),
+                                              K, interp)
+        assert relerr(_n(gi), fx[pre + wtag + "conv_gi"]) <= btol
+        assert relerr(_n(gw), fx[pre + wtag + "conv_gw"]) <= btol
+        assert relerr(_n(gb), fx[pre + wtag + "conv_gb"]) <= btol
+        oh, ow = fx["%s/in/tgout" % d].shape[2:]
+        out = ops.mapped_transposed_conv_forward(g("tx"), m, iw, g("tweight"), g("bias"), oh, ow,
+                                                 K, interp)
+        assert relerr(_n(out), fx[pre + wtag + "tconv_fwd"]) <= btol
+        gi, gw, gb = ops.mapped_transposed_conv_backward(g("tgout"), m, iw, g("tx"), g("tweight"),
+                                                         g("bias"), K, interp)
+        assert relerr(_n(gi), fx[pre + wtag + "tconv_gi"]) <= btol
+        assert relerr(_n(gw), fx[pre + wtag + "tconv_gw"]) <= btol
+        assert relerr(_n(gb), fx[pre + wtag + "tconv_gb"]) <= btol
+        # pooling: the GPU follows the reference's device branch; it equals the host-branch
+        # fixture wherever that found a winner (index >= 0)
+        val, idx = ops.mapped_max_pool(g("x"), m, iw, K, interp)
+        ok = fx[pre + wtag + "pool_idx"] >= 0
+        assert np.array_equal(_n(idx)[ok], fx[pre + wtag + "pool_idx"][ok])
+        assert np.array_equal(_n(val)[ok], fx[pre + wtag + "pool_val"][ok])
+    for wtag, m, iw in (("", g("m_ui"), None), ("w", g("m_wi"), g("iw"))):
+        val, idx = ops.mapped_max_pool(g("xpos"), m, iw, K, interp)
+        assert np.array_equal(_n(idx), fx[pre + wtag + "pospool_idx"])
+        assert np.array_equal(_n(val), fx[pre + wtag + "pospool_val"])
+        got = _n(ops.mapped_max_unpool(g("gpool"), idx, m, iw, H, W, K, interp))
+        assert relerr(got, fx[pre + wtag + "unpool"]) <= btol
+    assert dt is not None
+
+
+def test_errors_are_raised_not_fatal(ops):
+    x = torch.zeros(1, 2, 4, 5, device=DEV)
+    m = torch.zeros(3, 3, 2, device=DEV)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.resample_from_map(x.transpose(2, 3), m, None, 1)
+    with pytest.raises(RuntimeError, match="dtype"):
+        ops.resample_from_map(x, m.double(), None, 1)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ops.resample_from_map(x, m.cpu(), None, 1)
+    with pytest.raises(RuntimeError, match="unsupported dtype"):
+        ops.resample_from_map(x.half(), m.half(), None, 1)
+    # unknown interpolation values fall back to nearest like the reference's switch default
+    a = ops.resample_from_map(x + 1, m, None, 7)
+    assert torch.equal(a, ops.resample_from_map(x + 1, m, None, 0))

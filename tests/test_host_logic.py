@@ -1,0 +1,130 @@
+"""CPU-only checks of the host side: the C-ABI library exports what the header declares,
+the Python layers mirror the reference's interface, and nothing runs without the GPU."""
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import PKG, ROOT
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sdk_mapped_ops.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sdk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib_path = os.path.join(PKG, "libsdk_mapped_ops.so")
+    assert os.path.exists(lib_path), "build first: python -c 'import __graft_entry__ as g; g.build()'"
+    lib = ctypes.CDLL(lib_path)
+    names = _declared_symbols()
+    assert len(names) >= 17
+    for n in names:
+        assert hasattr(lib, n), "missing export " + n
+
+
+def test_ctypes_table_matches_header():
+    from _spherical_distortion_ext import _capi
+    declared = set(_declared_symbols())
+    bound = set(_capi.SIGNATURES) | set(_capi.OTHER_SYMBOLS)
+    assert declared == bound
+    assert _capi.load().sdk_version() >= 100
+
+
+def test_enum_values_and_tensor_round_trip():
+    from spherical_distortion.nn import InterpolationType as IT
+    assert (int(IT.NEAREST), int(IT.BILINEAR), int(IT.BISPHERICAL)) == (0, 1, 2)
+    assert IT(torch.tensor(2)) is IT.BISPHERICAL
+    assert IT(torch.tensor(int(IT.NEAREST))) is IT.NEAREST
+
+
+def test_module_parameters_follow_the_reference_layout():
+    from spherical_distortion.nn import (MappedConvolution, MappedMaxPool,
+                                         MappedTransposedConvolution)
+    conv = MappedConvolution(6, 4, kernel_size=9)
+    assert conv.weight.shape == (4, 6, 9) and conv.bias.shape == (4,)
+    bound = 1 / math.sqrt(6 * 9)
+    assert conv.weight.abs().max() <= bound and conv.bias.abs().max() <= bound
+    assert conv.weight.std() > 0.3 * bound
+    assert int(conv.interp) == 1
+    nb = MappedConvolution(6, 4, kernel_size=9, bias=False)
+    assert isinstance(nb.bias, torch.nn.Parameter) and (nb.bias == 0).all()
+    t = MappedTransposedConvolution(6, 4, kernel_size=7)
+    assert t.weight.shape == (6, 4, 7) and t.bias.shape == (4,)
+    assert t.weight.abs().max() <= 1 / math.sqrt(6 * 7)
+    assert set(dict(conv.state_dict())) == {"weight", "bias"}
+    assert MappedMaxPool(4).return_indices is False
+
+
+def test_check_args_assertions():
+    from spherical_distortion import functional as F
+    from spherical_distortion.layer_utils import check_args
+    x = torch.zeros(1, 2, 4, 5)
+    with pytest.raises(AssertionError, match="4 dimensions"):
+        check_args(x[0], torch.zeros(4, 5, 3, 2), None, 2, 3)
+    with pytest.raises(AssertionError, match="Sample map must have 4"):
+        check_args(x, torch.zeros(4, 5, 2), None, 2, 3)
+    with pytest.raises(AssertionError, match="Sample map must have 5"):
+        check_args(x, torch.zeros(4, 5, 3, 2), torch.zeros(4, 5, 3, 2), 2, 3)
+    with pytest.raises(AssertionError, match="size 2"):
+        check_args(x, torch.zeros(4, 5, 3, 3), None, 2, 3)
+    with pytest.raises(AssertionError, match="same dtype"):
+        check_args(x, torch.zeros(4, 5, 3, 2).double(), None, 2, 3)
+    with pytest.raises(AssertionError, match="input channels"):
+        check_args(x, torch.zeros(4, 5, 3, 2), None, 3, 3)
+    with pytest.raises(AssertionError, match="Kernel size"):
+        check_args(x, torch.zeros(4, 5, 3, 2), None, 2, 4)
+    with pytest.raises(AssertionError, match="interpolation points"):
+        check_args(x, torch.zeros(4, 5, 3, 2, 2), torch.zeros(4, 5, 3, 3), 2, 3)
+    check_args(x, torch.zeros(4, 5, 3, 2, 2), torch.zeros(4, 5, 3, 2), 2, 3)
+    check_args(x, torch.zeros(7, 7, 2), None, None, None)  # resample: rank-3 map
+    with pytest.raises(AssertionError, match="must match sample map"):
+        F.mapped_transposed_convolution(x, torch.zeros(2, 3, 3), torch.zeros(3),
+                                        torch.zeros(4, 6, 3, 2), 8, 8, 3, 1)
+    with pytest.raises(AssertionError, match="3 or 4 dimensions"):
+        F.unresample(torch.zeros(4, 5), torch.zeros(2, 2, 2), 1)
+
+
+def test_cpu_tensors_are_refused_loudly():
+    """There is no CPU path: the operators exist for the GPU dispatch key only."""
+    from spherical_distortion.nn import MappedConvolution, MappedMaxPool, Unresample
+    x = torch.zeros(1, 2, 4, 5)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        MappedConvolution(2, 3, 4)(x, torch.zeros(4, 5, 4, 2))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        MappedMaxPool(4)(x, torch.zeros(4, 5, 4, 2))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        Unresample()(x, torch.zeros(3, 3, 2))
+
+
+def test_product_code_never_touches_the_oracle():
+    bad = []
+    for base, _, files in os.walk(PKG):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")) or f == "Makefile":
+                text = open(os.path.join(base, f)).read()
+                if re.search(r"\boracle\b|_ref\b|sdk_oracle", text):
+                    bad.append(os.path.join(base, f))
+    assert not bad, bad
+
+
+def test_workload_generators_shapes():
+    import numpy as np
+    import workloads as wl
+    m = wl.gnomonic_kernel_map(16, 32, stride=2, dilation=2)
+    assert m.shape == (8, 16, 9, 2) and np.isfinite(m).all()
+    assert np.array_equal(m[3, 5, 4], [10.0, 6.0])  # centre sample is the pixel itself
+    m4, w4 = wl.four_nearest_weighted(wl.gnomonic_kernel_map(16, 32, dtype=np.float64), 16, 32)
+    assert m4.shape == (16, 32, 9, 4, 2) and np.allclose(w4.sum(-1), 1, atol=1e-6)
+    assert (m4 == np.round(m4)).all() and m4[..., 0].max() <= 31 and m4[..., 1].max() <= 15
+    v, f = wl.icosphere(3)
+    assert v.shape == (642, 3) and f.shape == (1280, 3)
+    ring = wl.vertex_ring_map(3)
+    assert ring.shape == (1, 642, 7, 2) and (ring[..., 1] == 0).all()
+    nb = ring[0, :, 1:, 0].astype(int)
+    assert all(v_ in nb[n] for v_ in range(40) for n in nb[v_])  # neighbourhood is symmetric
+    assert wl.tangent_patch_map(64, 128, 1, 8).shape == (80, 64, 2)
