@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the mapped-operation backend on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME]] [--no-cpu]
+
+One "step" is one forward + backward pass of the large weighted mapped
+convolution (configuration 4: x 8x128x256x512 -> 128 channels, K = 9, P = 4
+bispherical interpolation points, float32), with every tensor already resident
+in HBM.  The headline value is images per second over K timed steps.  The same
+JSON line also carries, under "kernels", the achieved rate of every other hot
+kernel (tangent-image gather / scatter, mapped max pool / unpool, icosphere
+convolution and transposed convolution) against its roofline, the roofline
+object of the dominant kernel and a CPU baseline measured in the same run.
+
+Algorithmic bytes / flops per launch (what "achieved" divides by the measured
+duration) are the minimal tensor traffic of each operator:
+    gather   : image + map + output
+    scatter  : input + map + output (+ one weight-sum plane when normalising)
+    pool     : input + map + values + int64 indices;  unpool: grad_out + indices + map + grad_in
+    conv     : 2 * Cout * Cin * K * OH*OW * B flops per contraction
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "spherical-package_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_FP32_TFLOPS = 157.3     # dense matrix fp32
+MFMA_BF16_TFLOPS = 2500.0    # dense bf16
+
+
+def _nbytes(*arrays):
+    return float(sum(a.numel() * a.element_size() for a in arrays if a is not None))
+
+
+class Timer:
+    """HIP-event timing on torch's current stream (the stream every kernel of this
+    library is launched on)."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def run(self, fn, steps, warmup):
+        t = self.torch
+        for _ in range(warmup):
+            fn()
+        t.cuda.synchronize()
+        evs = [(t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True))
+               for _ in range(steps)]
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        t.cuda.synchronize()
+        ms = [a.elapsed_time(b) for a, b in evs]
+        return float(np.mean(ms)), float(np.min(ms))
+
+
+def _roof(bound, work, ms, traffic=None, peak=None):
+    if bound == "hbm":
+        peak = HBM_PEAK_GBS
+        achieved = work / (ms * 1e-3) / 1e9
+        unit = "GB/s"
+    else:
+        achieved = work / (ms * 1e-3) / 1e12
+        unit = "TFLOP/s"
+    return {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": traffic}
+
+
+def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
+    import workloads
+    cfg = workloads.config4(batch=batch)
+    dev = "cuda:0"
+    x, m, iw, w, b, g = (torch.from_numpy(cfg[k]).to(dev) for k in
+                         ("x", "sample_map", "interp_weights", "weight", "bias", "grad_output"))
+    K, interp = cfg["kernel_size"], cfg["interp"]
+    B, Cin, H, W = x.shape
+    Cout = w.shape[0]
+    flops = 2.0 * Cout * Cin * K * H * W * B
+    ops.set_conv_compute(compute)
+    try:
+        def step():
+            ops.mapped_conv_forward(x, m, iw, w, b, K, interp)
+            ops.mapped_conv_backward(g, m, iw, x, w, b, K, interp)
+        ms, ms_min = timer.run(step, steps, warmup)
+        ms_f, _ = timer.run(lambda: ops.mapped_conv_forward(x, m, iw, w, b, K, interp),
+                            max(2, steps // 2), 1)
+    finally:
+        ops.set_conv_compute("native")
+    peak = MFMA_FP32_TFLOPS if compute == "native" else MFMA_BF16_TFLOPS
+    return {"ms_per_step": ms, "ms_min": ms_min, "images_per_s": B / (ms * 1e-3),
+            "forward_ms": ms_f, "flops_per_step": 3 * flops,
+            "roofline_step": _roof("mfma", 3 * flops, ms, peak=peak),
+            "roofline_forward": _roof("mfma", flops, ms_f, peak=peak),
+            "tensors": (cfg, None)}
+
+
+def bench_resample2(torch, ops, timer, steps, warmup):
+    import workloads
+    cfg = workloads.config2()
+    dev = "cuda:0"
+    x = torch.from_numpy(cfg["x"]).to(dev)
+    m = torch.from_numpy(cfg["sample_map"]).to(dev)
+    H, W = cfg["out_shape"]
+    patches = ops.resample_from_map(x, m, None, 1)
+    ms_g, _ = timer.run(lambda: ops.resample_from_map(x, m, None, 1), steps, warmup)
+    ms_s, _ = timer.run(lambda: ops.resample_to_map_normalized(patches, m, None, H, W, 1, 1e-12),
+                        steps, warmup)
+    gather_bytes = _nbytes(x, m, patches)
+    scatter_bytes = _nbytes(patches, m, x) + H * W * 4.0
+    return {"gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g)),
+            "scatter_normalise": dict(ms=ms_s, **_roof("hbm", scatter_bytes, ms_s))}
+
+
+def bench_pool3(torch, ops, timer, steps, warmup):
+    import workloads
+    cfg = workloads.config3()
+    dev = "cuda:0"
+    x = torch.from_numpy(cfg["x"]).to(dev)
+    m = torch.from_numpy(cfg["sample_map"]).to(dev)
+    g = torch.from_numpy(cfg["grad_output"]).to(dev)
+    K = cfg["kernel_size"]
+    H, W = x.shape[2:]
+    val, idx = ops.mapped_max_pool(x, m, None, K, 0)
+    ms_f, _ = timer.run(lambda: ops.mapped_max_pool(x, m, None, K, 0), steps, warmup)
+    ms_b, _ = timer.run(lambda: ops.mapped_max_unpool(g, idx, m, None, H, W, K, 0), steps, warmup)
+    fwd_bytes = _nbytes(x, m, val, idx)
+    bwd_bytes = _nbytes(g, idx, m, x)
+    return {"pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f)),
+            "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b)),
+            "no_winner_outputs": int((idx < 0).sum().item())}
+
+
+def bench_ico5(torch, ops, timer, steps, warmup):
+    import workloads
+    cfg = workloads.config5()
+    dev = "cuda:0"
+    t = {k: torch.from_numpy(v).to(dev) for k, v in cfg.items() if isinstance(v, np.ndarray)}
+    K = cfg["kernel_size"]
+    B, C, _, V = t["x"].shape
+    flops = 2.0 * C * C * K * V * B
+
+    def conv_step():
+        ops.mapped_conv_forward(t["x"], t["sample_map"], None, t["weight"], t["bias"], K, 0)
+        ops.mapped_conv_backward(t["grad_output"], t["sample_map"], None, t["x"], t["weight"],
+                                 t["bias"], K, 0)
+    ms_c, _ = timer.run(conv_step, steps, warmup)
+    oh, ow = cfg["out_hw"]
+    Vc = t["x_coarse"].shape[3]
+    ms_t, _ = timer.run(lambda: ops.mapped_transposed_conv_forward(
+        t["x_coarse"], t["up_map"], None, t["up_weight"], t["up_bias"], oh, ow, K, 0), steps,
+        warmup)
+    tflops = 2.0 * C * C * K * Vc * B
+    return {"icosphere_conv_fwd_bwd": dict(ms=ms_c, images_per_s=B / (ms_c * 1e-3),
+                                           **_roof("mfma", 3 * flops, ms_c,
+                                                   peak=MFMA_FP32_TFLOPS)),
+            "transposed_conv_forward": dict(ms=ms_t, **_roof("mfma", tflops, ms_t,
+                                                             peak=MFMA_FP32_TFLOPS))}
+
+
+def cpu_baseline(budget_s=25.0):
+    """Times the CPU checker on a bounded sample of configuration 4 (batch 1, a
+    band of output rows when needed) and scales to images per second."""
+    import torch
+    import workloads
+    from oracle import oracle as orc
+    try:
+        from oracle import ref
+        R = ref.load() if ref.available() else None
+    except Exception:
+        R = None
+    H, W = 256, 512
+    cfg = workloads.config4(batch=1)
+    rows = 64 if R is None else H             # band of output rows (a bounded sample)
+    m = np.ascontiguousarray(cfg["sample_map"][:rows])
+    iw = np.ascontiguousarray(cfg["interp_weights"][:rows])
+    g = np.ascontiguousarray(cfg["grad_output"][:, :, :rows])
+    K = 9
+    t0 = time.time()
+    if R is not None:
+        tt = [torch.from_numpy(a) for a in (cfg["x"], m, iw, cfg["weight"], cfg["bias"], g)]
+        it = R.InterpolationType(2)
+        R._weighted_mapped_convolution.weighted_mapped_conv_forward(
+            tt[0], tt[1], tt[2], tt[3], tt[4], K, it)
+        R._weighted_mapped_convolution.weighted_mapped_conv_backward(
+            tt[5], tt[1], tt[2], tt[0], tt[3], tt[4], K, it)
+        kind, cores = "reference", torch.get_num_threads()
+    else:
+        orc.mapped_conv_forward(cfg["x"], m, cfg["weight"], cfg["bias"], K, 2, iw)
+        orc.mapped_conv_backward(g, m, cfg["x"], cfg["weight"], cfg["bias"], K, 2, iw)
+        kind, cores = "port", orc.num_threads()
+    dt = time.time() - t0
+    frac = rows / float(H)                    # share of one image's output pixels
+    return {"value": round(frac / dt, 4), "unit": "images/s", "cores": int(cores), "kind": kind,
+            "sample": "configuration 4, batch 1, output rows 0..%d of %d (%.1f s of CPU work), "
+                      "fwd+bwd, scaled by the pixel share" % (rows - 1, H, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--only", default="", help="comma list of: conv4,conv4_bf16,resample2,pool3,ico5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); "
+                 "multi-GPU sharding is described in DESIGN.md, not built")
+
+    import torch
+    from _spherical_distortion_ext import _ops as ops
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    timer = Timer(torch)
+    only = [s for s in args.only.split(",") if s]
+    want = lambda n: not only or n in only  # noqa: E731
+
+    kernels = {}
+    head = None
+    if want("conv4"):
+        head = bench_conv4(torch, ops, timer, args.steps, args.warmup)
+        head.pop("tensors")
+        kernels["conv4_fp32"] = {k: head[k] for k in ("ms_per_step", "forward_ms", "images_per_s",
+                                                     "roofline_step", "roofline_forward")}
+        torch.cuda.empty_cache()
+    if want("conv4_bf16"):
+        try:
+            r = bench_conv4(torch, ops, timer, args.steps, args.warmup, compute="bf16")
+            r.pop("tensors")
+            kernels["conv4_bf16"] = {k: r[k] for k in ("ms_per_step", "forward_ms", "images_per_s",
+                                                      "roofline_step", "roofline_forward")}
+        except RuntimeError as e:
+            kernels["conv4_bf16"] = {"error": str(e)[:200]}
+        torch.cuda.empty_cache()
+    if want("resample2"):
+        kernels.update(bench_resample2(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
+    if want("pool3"):
+        kernels.update(bench_pool3(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
+        torch.cuda.empty_cache()
+    if want("ico5"):
+        kernels.update(bench_ico5(torch, ops, timer, args.steps, args.warmup))
+        torch.cuda.empty_cache()
+
+    line = {"metric": "mapped_conv_fwd_bwd_images_per_sec", "unit": "images/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "configuration 4: weighted (P=4) bispherical mapped convolution "
+                                   "fwd+bwd, x 8x128x256x512 -> 128 channels, K=9, float32",
+                       "global_batch": 8}}
+    if head is not None:
+        line.update(value=round(head["images_per_s"], 3), ms_per_step=round(head["ms_per_step"], 4),
+                    roofline=head["roofline_step"])
+    else:
+        line.update(value=None, ms_per_step=None, roofline=None)
+    line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    line["kernels"] = kernels
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -55,10 +55,16 @@ typedef enum sdk_dtype { SDK_F32 = 0, SDK_F64 = 1 } sdk_dtype;
 /* ext_modules/include/enums.h:12-16 (exported by include/layers/enum_export.h:10-18) */
 typedef enum sdk_interp { SDK_NEAREST = 0, SDK_BILINEAR = 1, SDK_BISPHERICAL = 2 } sdk_interp;
 
-/* Arithmetic used by the dense contraction inside the convolution entry points.
- * SDK_COMPUTE_NATIVE: the tensors' own type (fp32 MFMA for SDK_F32).
- * SDK_COMPUTE_BF16:   operands rounded to bf16, fp32 accumulation (SDK_F32 only). */
-typedef enum sdk_compute { SDK_COMPUTE_NATIVE = 0, SDK_COMPUTE_BF16 = 1 } sdk_compute;
+/* Arithmetic / kernel choice of the dense contraction inside the convolution entry points.
+ * SDK_COMPUTE_NATIVE:  the tensors' own type; float32 runs the fused gather + fp32-MFMA kernels.
+ * SDK_COMPUTE_BF16:    operands rounded to bf16, fp32 accumulation (SDK_F32 only).
+ * SDK_COMPUTE_UNFUSED: separate im2col/col2im and plain-FMA GEMM kernels through a column
+ *                      workspace (always used for SDK_F64; kept selectable as a cross-check). */
+typedef enum sdk_compute {
+  SDK_COMPUTE_NATIVE = 0,
+  SDK_COMPUTE_BF16 = 1,
+  SDK_COMPUTE_UNFUSED = 2
+} sdk_compute;
 
 typedef void* sdk_stream_t; /* hipStream_t */
 
@@ -157,12 +163,12 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
  * Mapped convolution.  weight [Cout, Cin, K]; bias [Cout];
  * input [B,Cin,H,W]; sample_map [OH,OW,K,(P,)2]; output [B,Cout,OH,OW].
  *
- * Some shape/dtype combinations run as separate im2col/col2im + GEMM kernels
- * and need device scratch: ask sdk_mapped_conv_workspace_bytes() (same
- * arguments for the forward, backward and transposed entry points of one
- * layer call) and pass at least that many bytes (256-byte aligned).  A
- * result of 0 means the fused kernels serve the request and workspace may be
- * NULL.
+ * Every convolution entry point needs device scratch (re-laid-out weights for
+ * the fused kernels, one batch element's column matrix for the unfused path):
+ * ask sdk_mapped_conv_workspace_bytes() (same arguments for the forward,
+ * backward and transposed entry points of one layer call; gather_pixels is the
+ * number of sample-map pixels OH*OW, resp. IH*IW for the transposed layer) and
+ * pass at least that many bytes, 256-byte aligned.
  * ------------------------------------------------------------------------- */
 size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
                                        int64_t gather_pixels, int64_t kernel_size,

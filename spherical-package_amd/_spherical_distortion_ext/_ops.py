@@ -16,8 +16,9 @@ from . import _capi
 _NS = "sdk_mapped_ops"
 _DTYPES = {torch.float32: _capi.SDK_F32, torch.float64: _capi.SDK_F64}
 
-# Arithmetic of the dense contraction inside the convolution operators:
-# "native" (the tensors' type) or "bf16" (bf16 operands, fp32 accumulate).
+# Arithmetic of the dense contraction inside the convolution operators: "native"
+# (the tensors' type), "bf16" (bf16 operands, fp32 accumulate) or "unfused"
+# (separate im2col/col2im + GEMM kernels, the cross-check path).
 _compute_mode = _capi.SDK_COMPUTE_NATIVE
 
 
@@ -25,14 +26,15 @@ def set_conv_compute(mode):
     """Selects the GEMM arithmetic of the mapped (transposed) convolutions."""
     global _compute_mode
     modes = {"native": _capi.SDK_COMPUTE_NATIVE, "fp32": _capi.SDK_COMPUTE_NATIVE,
-             "bf16": _capi.SDK_COMPUTE_BF16}
+             "bf16": _capi.SDK_COMPUTE_BF16, "unfused": _capi.SDK_COMPUTE_UNFUSED}
     if mode not in modes:
         raise ValueError("compute mode must be one of %s" % sorted(modes))
     _compute_mode = modes[mode]
 
 
 def get_conv_compute():
-    return "bf16" if _compute_mode == _capi.SDK_COMPUTE_BF16 else "native"
+    return {_capi.SDK_COMPUTE_BF16: "bf16", _capi.SDK_COMPUTE_UNFUSED: "unfused"}.get(
+        _compute_mode, "native")
 
 
 # --------------------------------------------------------------------------- checks

@@ -28,15 +28,15 @@ int check_common(const char* what, int64_t B, int64_t Cg, int64_t H, int64_t W, 
               what);
   SDK_REQUIRE(P >= 0 && (P == 0 || wts), "%s: weighted map needs interp_weights", what);
   SDK_REQUIRE(dtype == SDK_F32 || dtype == SDK_F64, "%s: unknown dtype %d", what, dtype);
-  SDK_REQUIRE(compute == SDK_COMPUTE_NATIVE || compute == SDK_COMPUTE_BF16,
+  SDK_REQUIRE(compute == SDK_COMPUTE_NATIVE || compute == SDK_COMPUTE_BF16 ||
+                  compute == SDK_COMPUTE_UNFUSED,
               "%s: unknown compute mode %d", what, compute);
   if (compute == SDK_COMPUTE_BF16 && dtype != SDK_F32)
     return fail(SDK_ERR_UNSUPPORTED, "%s: bf16 compute needs float32 tensors", what);
   return SDK_OK;
 }
 
-int check_workspace(const char* what, const ConvGeom& g, int dtype, void* ws, size_t ws_bytes) {
-  const size_t need = generic_workspace_bytes(g.Cg, g.K, g.M, dtype);
+int check_workspace(const char* what, size_t need, void* ws, size_t ws_bytes) {
   if (!ws || ws_bytes < need)
     return fail(SDK_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", what, need,
                 ws ? ws_bytes : (size_t)0);
@@ -50,16 +50,20 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
         const void* map, const void* wts, const void* in1, const void* bias, void* out, void* ws,
         size_t ws_bytes, hipStream_t stream) {
   if (g.B == 0 && op != GATHER_WGRAD) return SDK_OK;
-  if (dtype == SDK_F32 && fused_supported(g)) {
+  if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(g)) {
+    if (op != GATHER_WGRAD) {
+      int rc = check_workspace(what, fused_workspace_bytes(g), ws, ws_bytes);
+      if (rc) return rc;
+    }
     const float* m = (const float*)map;
     const float* w = (const float*)wts;
     switch (op) {
       case GATHER_GEMM:
         return fused_gather_gemm(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                 (const float*)bias, (float*)out, stream);
+                                 (const float*)bias, (float*)out, (float*)ws, stream);
       case GEMM_SCATTER:
         return fused_gemm_scatter(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                  (const float*)bias, (float*)out, stream);
+                                  (const float*)bias, (float*)out, (float*)ws, stream);
       case GATHER_WGRAD:
         return fused_gather_wgrad(g, compute, (const float*)in0, m, w, (const float*)in1,
                                   (float*)out, stream);
@@ -67,7 +71,7 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
   }
   if (compute == SDK_COMPUTE_BF16)
     return fail(SDK_ERR_UNSUPPORTED, "%s: bf16 compute is not available for this shape", what);
-  int rc = check_workspace(what, g, dtype, ws, ws_bytes);
+  int rc = check_workspace(what, generic_workspace_bytes(g.Cg, g.K, g.M, dtype), ws, ws_bytes);
   if (rc) return rc;
   SDK_DISPATCH_DTYPE(dtype, {
     switch (op) {
@@ -93,14 +97,15 @@ size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64
                                        int64_t gather_pixels, int64_t kernel_size,
                                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
                                        int32_t compute) {
-  (void)compute;
   // Upper bound over the conv (gather side = in_channels) and transposed conv
   // (gather side = out_channels) roles, so one query serves a whole layer call.
   ConvGeom a{batch, (int)in_channels, 1, 1, (int)out_channels, (int)gather_pixels,
              (int)kernel_size, num_interp_pts, interp};
   ConvGeom b{batch, (int)out_channels, 1, 1, (int)in_channels, (int)gather_pixels,
              (int)kernel_size, num_interp_pts, interp};
-  if (dtype == SDK_F32 && fused_supported(a) && fused_supported(b)) return 0;
+  if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(a) &&
+      fused_supported(b))
+    return align256(std::max(fused_workspace_bytes(a), fused_workspace_bytes(b)));
   return generic_workspace_bytes(std::max(in_channels, out_channels), kernel_size, gather_pixels,
                                  dtype);
 }

@@ -1,19 +1,538 @@
+// Fused mapped-convolution kernels for gfx950 (float32 tensors).
+//
+// The im2col column matrix never exists in HBM.  Three kernels cover the six
+// contractions of mapped / mapped-transposed convolution (see ConvGeom):
+//
+//   gather_gemm   pix[b][n,m]  = sum_{c,k} Wm[n,(c,k)] * gather(img[b,c], tap(m,k)) + bias[n]
+//   gemm_scatter  img[b,c]    += scatter_{tap(m,k)}( sum_n Wm[n,(c,k)] * pix[b][n,m] )
+//   gather_wgrad  gW[n,(c,k)]  = sum_{b,m} pix[b][n,m] * gather(img[b,c], tap(m,k))
+//
+// Common structure: a 256-thread workgroup (4 wavefronts) owns a tile of
+// pixels.  For one kernel sample k at a time it turns the tile's sample-map
+// entries into a compact per-pixel tap list in LDS (offset + coefficient; the
+// interpolation weight and the per-point weight are folded into one
+// coefficient, zero-weight taps are dropped), which is then reused for every
+// channel.  Column values are produced straight into an LDS operand tile (or
+// consumed straight from MFMA accumulators) and contracted with
+// v_mfma_f32_32x32x2_f32; each wavefront owns a 64 x 64 block of the 128 x 128
+// (or 64 x 256) workgroup tile as 2 x 2 MFMA accumulators.
+//
+// MFMA 32x32x2 f32 register layout used below (wave64, lane l):
+//   A operand: A[i = l % 32][k = l / 32]        B operand: B[k = l / 32][j = l % 32]
+//   D, 16 registers v: D[i = 8*(v/4) + 4*(l/32) + v%4][j = l % 32]
 #include "conv_fused.hpp"
 
+#include <hip/hip_runtime.h>
+
 #include "sdk_host.hpp"
+#include "sdk_taps.hpp"
 
 namespace sdk {
-bool fused_supported(const ConvGeom&) { return false; }
-int fused_gather_gemm(const ConvGeom&, int, const float*, const float*, const float*, const float*,
-                      const float*, float*, hipStream_t) {
-  return fail(SDK_ERR_UNSUPPORTED, "fused path not built");
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kKC = 32;         // reduction rows staged per step
+constexpr int kMaxSlots = 64;   // tap slots per pixel and kernel sample (points * taps)
+
+__host__ __device__ constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// Row of D held in accumulator register v of lane l (see layout above).
+__device__ __forceinline__ int mfma_row(int v, int lane) {
+  return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
 }
-int fused_gemm_scatter(const ConvGeom&, int, const float*, const float*, const float*,
-                       const float*, const float*, float*, hipStream_t) {
-  return fail(SDK_ERR_UNSUPPORTED, "fused path not built");
+
+// XCD-aware tile order: hardware workgroup ids go round-robin over the 8 XCDs
+// (each with its own L2); give every XCD a contiguous band of tiles so that
+// neighbouring pixel tiles, which share input rows, meet in one L2.
+__device__ __forceinline__ int xcd_band_tile(int bid, int ntiles) {
+  constexpr int X = 8;
+  const int per = ntiles / X;           // full bands
+  if (bid >= per * X) return bid;       // remainder keeps its natural order
+  return (bid % X) * per + bid / X;
 }
-int fused_gather_wgrad(const ConvGeom&, int, const float*, const float*, const float*,
-                       const float*, float*, hipStream_t) {
-  return fail(SDK_ERR_UNSUPPORTED, "fused path not built");
+
+// ---------------------------------------------------------------------------
+// Tap table of one kernel sample k for TP consecutive pixels starting at pix0.
+// Layout tap_off[slot][TP], tap_co[slot][TP] (slot-major, so lanes that own
+// consecutive pixels hit consecutive LDS banks).  Every pixel's active taps are
+// packed to the front; slots up to the tile-wide maximum *smax are padded with
+// coefficient 0.  Must be called by all threads of the workgroup.
+// ---------------------------------------------------------------------------
+template <int INTERP, bool WEIGHTED, int TP>
+__device__ __forceinline__ void build_taps(const float* __restrict__ map,
+                                           const float* __restrict__ wts, int pix0, int M, int K,
+                                           int k, int P, int H, int W, int* __restrict__ tap_off,
+                                           float* __restrict__ tap_co, int* __restrict__ smax) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *smax = 0;
+  __syncthreads();
+  int cnt = 0;
+  if (tid < TP) {
+    const int pix = pix0 + tid;
+    if (pix < M) {
+      const int q = WEIGHTED ? P : 1;
+      const size_t s = ((size_t)pix * K + k) * q;
+      PointTaps<float, INTERP> t;
+      for (int p = 0; p < q; ++p) {
+        t.set(map[(s + p) * 2], map[(s + p) * 2 + 1], H, W);
+        const float wt = WEIGHTED ? wts[s + p] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < PointTaps<float, INTERP>::N; ++i) {
+          const float co = WEIGHTED ? wt * t.w[i] : t.w[i];
+          if (t.off[i] >= 0 && co != 0.0f) {
+            tap_off[cnt * TP + tid] = t.off[i];
+            tap_co[cnt * TP + tid] = co;
+            ++cnt;
+          }
+        }
+      }
+    }
+    atomicMax(smax, cnt);
+  }
+  __syncthreads();
+  if (tid < TP) {
+    const int top = *smax;
+    for (int sidx = cnt; sidx < top; ++sidx) {
+      tap_off[sidx * TP + tid] = 0;
+      tap_co[sidx * TP + tid] = 0.0f;
+    }
+  }
+  __syncthreads();
 }
+
+// One reduction chunk of kKC rows: D(64 x 64 per wave) += A^T-tile x B-tile.
+// As[r][lda] holds the A operand r-major (row index i contiguous), Bs[r][ldb]
+// the B operand r-major (column index j contiguous).
+__device__ __forceinline__ void mfma_chunk(const float* __restrict__ As, int lda, int a_base,
+                                           const float* __restrict__ Bs, int ldb, int b_base,
+                                           int rows, floatx16 (&acc)[2][2]) {
+  const int lane = threadIdx.x & 63;
+  const int lk = lane >> 5, lj = lane & 31;
+#pragma unroll 4
+  for (int r = 0; r < rows; r += 2) {
+    const float a0 = As[(r + lk) * lda + a_base + lj];
+    const float a1 = As[(r + lk) * lda + a_base + 32 + lj];
+    const float b0 = Bs[(r + lk) * ldb + b_base + lj];
+    const float b1 = Bs[(r + lk) * ldb + b_base + 32 + lj];
+    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ void zero_acc(floatx16 (&acc)[2][2]) {
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+}
+
+// ---------------------------------------------------------------------------
+// Weight re-layout (once per call, a few hundred KB): from Wm[Cp][Cg*K] to
+//   Wg[k][c][n]  (n contiguous, padded to CgP x CpP)   for gather_gemm
+//   Ws[k][n][c]  (c contiguous, padded to CpP x CgP)   for gemm_scatter
+// Padding is zero so the hot loops need no channel guards on the weight side.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
+    const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int CpP, int CgP,
+    int n_fastest) {
+  const size_t total = (size_t)K * CpP * CgP;
+  for (size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x; e < total;
+       e += (size_t)gridDim.x * kThreads) {
+    int n, c, k;
+    if (n_fastest) {
+      n = (int)(e % CpP);
+      c = (int)((e / CpP) % CgP);
+      k = (int)(e / ((size_t)CpP * CgP));
+    } else {
+      c = (int)(e % CgP);
+      n = (int)((e / CgP) % CpP);
+      k = (int)(e / ((size_t)CpP * CgP));
+    }
+    out[e] = (n < Cp && c < Cg) ? Wm[(size_t)n * Cg * K + (size_t)c * K + k] : 0.0f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gather_gemm.  Workgroup tile: TN pixel-side channels x TM pixels, TN*TM = 16384.
+// grid.x = pixel tiles * n tiles, grid.y = batch.
+// LDS: Bs[kKC][TM] column tile, As[kKC][TN] weight tile, tap table.
+// ---------------------------------------------------------------------------
+template <int INTERP, bool WEIGHTED, int TN, int TM>
+__global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
+    const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
+    const float* __restrict__ Wg, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
+    int H, int W, int Cp, int M, int K, int P, int CgP, int CpP, int slots, int m_tiles) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* Bs = reinterpret_cast<float*>(smem);             // [kKC][TM]
+  float* As = Bs + kKC * TM;                               // [kKC][TN]
+  int* tap_off = reinterpret_cast<int*>(As + kKC * TN);    // [slots][TM]
+  float* tap_co = reinterpret_cast<float*>(tap_off + slots * TM);
+  int* smax = reinterpret_cast<int*>(tap_co + slots * TM);
+
+  constexpr int WAVES_N = TN / 64;           // waves along n
+  constexpr int SPLIT = kThreads / TM;       // threads sharing one pixel in the gather
+  constexpr int RPT = kKC / SPLIT;           // column rows per thread and chunk
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n_tiles = CpP / TN;
+  const int tile = xcd_band_tile(blockIdx.x, m_tiles * n_tiles);
+  const int m0 = (tile / n_tiles) * TM, n0 = (tile % n_tiles) * TN;
+  const int a_base = (wave % WAVES_N) * 64, b_base = (wave / WAVES_N) * 64;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
+  const int gm = tid % TM, gpart = tid / TM;
+
+  floatx16 acc[2][2];
+  zero_acc(acc);
+
+  for (int k = 0; k < K; ++k) {
+    build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    const int ns = *smax;
+    for (int c0 = 0; c0 < CgP; c0 += kKC) {
+      // ---- gather kKC column rows (channels c0.., sample k) for TM pixels
+      float col[RPT];
+#pragma unroll
+      for (int j = 0; j < RPT; ++j) col[j] = 0.0f;
+      const int cfirst = c0 + gpart * RPT;
+      for (int s = 0; s < ns; ++s) {
+        const int off = tap_off[s * TM + gm];
+        const float co = tap_co[s * TM + gm];
+#pragma unroll
+        for (int j = 0; j < RPT; ++j) {
+          const int c = min(cfirst + j, Cg - 1);   // padded rows meet zero weights
+          const float d = img_b[(size_t)c * HW + off];
+          col[j] += co * (co != 0.0f ? d : 0.0f);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < RPT; ++j) Bs[(gpart * RPT + j) * TM + gm] = col[j];
+      // ---- weight tile As[r][n] = Wg[k][c0 + r][n0 + n]
+      const float4* src = reinterpret_cast<const float4*>(Wg + ((size_t)k * CgP + c0) * CpP + n0);
+      for (int e = tid; e < kKC * TN / 4; e += kThreads) {
+        const int r = e / (TN / 4), n4 = e % (TN / 4);
+        reinterpret_cast<float4*>(As)[e] = src[(size_t)r * (CpP / 4) + n4];
+      }
+      __syncthreads();
+      mfma_chunk(As, TN, a_base, Bs, TM, b_base, kKC, acc);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: + bias, store (lanes along pixels: 128-byte rows)
+  float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int m = m0 + b_base + 32 * b + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + a_base + 32 * a + mfma_row(v, lane);
+        if (n < Cp && m < M) pix_b[(size_t)n * M + m] = acc[a][b][v] + (bias ? bias[n] : 0.0f);
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// gemm_scatter.  Workgroup tile: TC gather-side channels x TM pixels.  For every
+// kernel sample k and channel tile: D[c][m] = sum_n Ws[k][n][c] * pix[b][n][m],
+// then each accumulator is splatted through the pixel's taps with hardware
+// float atomics (lanes own consecutive pixels, so a wave's atomics fall on
+// neighbouring addresses).  img must be pre-filled (zeros or bias).
+// grid.x = pixel tiles, grid.y = batch.
+// ---------------------------------------------------------------------------
+template <int INTERP, bool WEIGHTED, int TC, int TM>
+__global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
+    const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
+    const float* __restrict__ Wsc, float* __restrict__ img, int Cg, int H, int W, int Cp, int M,
+    int K, int P, int CgP, int CpP, int slots, int m_tiles) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* Bs = reinterpret_cast<float*>(smem);             // [kKC][TM]  pix chunk
+  float* As = Bs + kKC * TM;                               // [kKC][TC]  weight chunk
+  int* tap_off = reinterpret_cast<int*>(As + kKC * TC);
+  float* tap_co = reinterpret_cast<float*>(tap_off + slots * TM);
+  int* smax = reinterpret_cast<int*>(tap_co + slots * TM);
+
+  constexpr int WAVES_C = TC / 64;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tile = xcd_band_tile(blockIdx.x, m_tiles);
+  const int m0 = tile * TM;
+  const int a_base = (wave % WAVES_C) * 64, b_base = (wave / WAVES_C) * 64;
+  const size_t HW = (size_t)H * W;
+  const float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
+  float* img_b = img + (size_t)blockIdx.y * Cg * HW;
+  const bool vec_ok = (M % 4 == 0);
+
+  for (int k = 0; k < K; ++k) {
+    build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    const int ns = *smax;
+    for (int c0 = 0; c0 < CgP; c0 += TC) {
+      floatx16 acc[2][2];
+      zero_acc(acc);
+      for (int nn0 = 0; nn0 < CpP; nn0 += kKC) {
+        // pix chunk Bs[r][m] = pix[b][nn0 + r][m0 + m]
+        if (vec_ok) {
+          for (int e = tid; e < kKC * TM / 4; e += kThreads) {
+            const int r = e / (TM / 4), m4 = (e % (TM / 4)) * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (nn0 + r < Cp && m0 + m4 < M)
+              v = *reinterpret_cast<const float4*>(pix_b + (size_t)(nn0 + r) * M + m0 + m4);
+            reinterpret_cast<float4*>(Bs)[e] = v;
+          }
+        } else {
+          for (int e = tid; e < kKC * TM; e += kThreads) {
+            const int r = e / TM, m = e % TM;
+            Bs[e] = (nn0 + r < Cp && m0 + m < M) ? pix_b[(size_t)(nn0 + r) * M + m0 + m] : 0.0f;
+          }
+        }
+        // weight chunk As[r][c] = Ws[k][nn0 + r][c0 + c]
+        const float4* src =
+            reinterpret_cast<const float4*>(Wsc + ((size_t)k * CpP + nn0) * CgP + c0);
+        for (int e = tid; e < kKC * TC / 4; e += kThreads) {
+          const int r = e / (TC / 4), c4 = e % (TC / 4);
+          reinterpret_cast<float4*>(As)[e] = src[(size_t)r * (CgP / 4) + c4];
+        }
+        __syncthreads();
+        mfma_chunk(As, TC, a_base, Bs, TM, b_base, kKC, acc);
+        __syncthreads();
+      }
+      // ---- scatter the 64 x 64 block of this wave
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int ml = b_base + 32 * b + (lane & 31);
+        for (int s = 0; s < ns; ++s) {
+          const int off = tap_off[s * TM + ml];
+          const float co = tap_co[s * TM + ml];
+          if (co != 0.0f) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) {
+                const int c = c0 + a_base + 32 * a + mfma_row(v, lane);
+                if (c < Cg) atomic_add_noret(img_b + (size_t)c * HW + off, co * acc[a][b][v]);
+              }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gather_wgrad.  Workgroup: one kernel sample k, one TC x TN tile of gW, one
+// batch element and one range of pixels; D[n][c] = sum_m pix[b][n][m] * col[(c,k)][m]
+// accumulated over the range in chunks of KM pixels, then added atomically to gW.
+// grid.x = K * c tiles * n tiles, grid.y = pixel ranges, grid.z = batch.
+// LDS: As[KM][TN+1] (pix, transposed), Bs[KM][TC+1] (columns, transposed), taps.
+// ---------------------------------------------------------------------------
+template <int INTERP, bool WEIGHTED, int KM>
+__global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
+    const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
+    const float* __restrict__ img, float* __restrict__ gW, int Cg, int H, int W, int Cp, int M,
+    int K, int P, int slots, int c_tiles, int n_tiles, int chunks_per_range) {
+  constexpr int TN = 128, TC = 128, LDA = TN + 1, LDB = TC + 1;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* As = reinterpret_cast<float*>(smem);              // [KM][LDA]
+  float* Bs = As + KM * LDA;                               // [KM][LDB]
+  int* tap_off = reinterpret_cast<int*>(Bs + KM * LDB);    // [slots][KM]
+  float* tap_co = reinterpret_cast<float*>(tap_off + slots * KM);
+  int* smax = reinterpret_cast<int*>(tap_co + slots * KM);
+
+  constexpr int GROUPS = kThreads / KM;   // channel groups in the gather
+  constexpr int CPT = TC / GROUPS;        // channels per thread
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int k = blockIdx.x / (c_tiles * n_tiles);
+  const int c0 = ((blockIdx.x / n_tiles) % c_tiles) * TC;
+  const int n0 = (blockIdx.x % n_tiles) * TN;
+  const int a_base = (wave & 1) * 64, b_base = (wave >> 1) * 64;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + (size_t)blockIdx.z * Cg * HW;
+  const float* pix_b = pix + (size_t)blockIdx.z * Cp * M;
+  const int gm = tid % KM, grp = tid / KM;
+
+  floatx16 acc[2][2];
+  zero_acc(acc);
+
+  const int chunk_beg = blockIdx.y * chunks_per_range;
+  const int chunk_end = min(chunk_beg + chunks_per_range, (M + KM - 1) / KM);
+  for (int ch = chunk_beg; ch < chunk_end; ++ch) {
+    const int m0 = ch * KM;
+    build_taps<INTERP, WEIGHTED, KM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    const int ns = *smax;
+    // ---- gather columns for KM pixels x TC channels -> Bs[m][c]
+    float col[CPT];
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) col[j] = 0.0f;
+    const int cfirst = c0 + grp * CPT;
+    for (int s = 0; s < ns; ++s) {
+      const int off = tap_off[s * KM + gm];
+      const float co = tap_co[s * KM + gm];
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) {
+        const int c = min(cfirst + j, Cg - 1);
+        const float d = img_b[(size_t)c * HW + off];
+        col[j] += co * (co != 0.0f ? d : 0.0f);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < CPT; ++j)
+      Bs[gm * LDB + grp * CPT + j] = (cfirst + j < Cg) ? col[j] : 0.0f;
+    // ---- pix tile As[m][n] = pix[b][n0 + n][m0 + m]
+    {
+      constexpr int NPT = TN / GROUPS;
+      const bool mok = m0 + gm < M;
+#pragma unroll
+      for (int j = 0; j < NPT; ++j) {
+        const int n = grp * NPT + j;
+        As[gm * LDA + n] = (mok && n0 + n < Cp) ? pix_b[(size_t)(n0 + n) * M + m0 + gm] : 0.0f;
+      }
+    }
+    __syncthreads();
+    mfma_chunk(As, LDA, a_base, Bs, LDB, b_base, KM, acc);
+    // the next build_taps() starts with a barrier, which also protects As / Bs
+  }
+
+  // ---- epilogue: gW[n][c*K + k] += D[n][c]
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int c = c0 + b_base + 32 * b + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + a_base + 32 * a + mfma_row(v, lane);
+        if (n < Cp && c < Cg)
+          atomic_add_noret(gW + (size_t)n * Cg * K + (size_t)c * K + k, acc[a][b][v]);
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side.
+// ---------------------------------------------------------------------------
+static int slots_for(const ConvGeom& g) {
+  const int nt = (g.interp == 1 || g.interp == 2) ? 4 : 1;
+  return pts(g.P) * nt;
+}
+
+bool fused_supported(const ConvGeom& g) {
+  if (slots_for(g) > kMaxSlots) return false;
+  if (g.B > 65535) return false;
+  return true;
+}
+
+size_t fused_workspace_bytes(const ConvGeom& g) {
+  const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
+  return (size_t)g.K * CpP * CgP * sizeof(float);
+}
+
+static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
+                    bool n_fastest, hipStream_t stream) {
+  const size_t total = (size_t)g.K * CpP * CgP;
+  const int blocks = (int)std::min<size_t>((total + kThreads - 1) / kThreads, 2048);
+  launch(relayout_weight_kernel, dim3(blocks), dim3(kThreads), stream, Wm, out, g.Cp, g.Cg, g.K,
+         CpP, CgP, n_fastest ? 1 : 0);
+  SDK_LAUNCH_CHECK("relayout_weight");
+  return SDK_OK;
+}
+
+template <typename Kern, typename... Args>
+static int launch_smem(const char* what, Kern kern, dim3 grid, size_t smem, hipStream_t stream,
+                       Args... args) {
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess)
+      return fail(SDK_ERR_DEVICE, "%s: cannot reserve %zu bytes of LDS: %s", what, smem,
+                  hipGetErrorString(e));
+  }
+  kern<<<grid, dim3(kThreads), smem, stream>>>(args...);
+  SDK_LAUNCH_CHECK(what);
+  return SDK_OK;
+}
+
+int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
+                      const float* wts, const float* Wm, const float* bias, float* pix,
+                      float* workspace, hipStream_t stream) {
+  if (compute != SDK_COMPUTE_NATIVE)
+    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  const int slots = slots_for(g);
+  const bool narrow = g.Cp <= 64;
+  const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
+  const int CpP = round_up(g.Cp, TN), CgP = round_up(g.Cg, kKC);
+  int rc = relayout(g, Wm, workspace, CpP, CgP, true, stream);
+  if (rc) return rc;
+  const int m_tiles = (int)ceil_div(g.M, TM), n_tiles = CpP / TN;
+  const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
+  const size_t smem = sizeof(float) * (kKC * TM + kKC * TN) + (size_t)slots * TM * 8 + 16;
+#define GG(TNv, TMv)                                                                          \
+  SDK_DISPATCH_INTERP(g.interp, g.P,                                                          \
+                      (rc = launch_smem("gather_gemm",                                        \
+                                        gather_gemm_kernel<INTERP, WEIGHTED, TNv, TMv>, grid, \
+                                        smem, stream, img, map, wts, (const float*)workspace, \
+                                        bias, pix, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP,  \
+                                        CpP, slots, m_tiles)))
+  if (narrow) GG(64, 256); else GG(128, 128);
+#undef GG
+  return rc;
+}
+
+int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const float* map,
+                       const float* wts, const float* Wm, const float* bias, float* img,
+                       float* workspace, hipStream_t stream) {
+  if (compute != SDK_COMPUTE_NATIVE)
+    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+  if (rc) return rc;
+  const int slots = slots_for(g);
+  const bool narrow = g.Cg <= 64;
+  const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;
+  const int CgP = round_up(g.Cg, TC), CpP = round_up(g.Cp, kKC);
+  rc = relayout(g, Wm, workspace, CpP, CgP, false, stream);
+  if (rc) return rc;
+  const int m_tiles = (int)ceil_div(g.M, TM);
+  const dim3 grid((unsigned)m_tiles, (unsigned)g.B);
+  const size_t smem = sizeof(float) * (kKC * TM + kKC * TC) + (size_t)slots * TM * 8 + 16;
+#define GS(TCv, TMv)                                                                           \
+  SDK_DISPATCH_INTERP(g.interp, g.P,                                                           \
+                      (rc = launch_smem("gemm_scatter",                                        \
+                                        gemm_scatter_kernel<INTERP, WEIGHTED, TCv, TMv>, grid, \
+                                        smem, stream, pix, map, wts, (const float*)workspace,  \
+                                        img, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP, CpP,    \
+                                        slots, m_tiles)))
+  if (narrow) GS(64, 256); else GS(128, 128);
+#undef GS
+  return rc;
+}
+
+int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
+                       const float* wts, const float* img, float* gW, hipStream_t stream) {
+  if (compute != SDK_COMPUTE_NATIVE)
+    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
+  if (rc) return rc;
+  if (g.B == 0) return SDK_OK;
+  constexpr int KM = 64;
+  const int slots = slots_for(g);
+  const int c_tiles = (int)ceil_div(g.Cg, 128), n_tiles = (int)ceil_div(g.Cp, 128);
+  const int chunks = (int)ceil_div(g.M, KM);
+  // enough pixel ranges for ~8 workgroups per CU overall, at least 8 chunks each
+  const int64_t base = (int64_t)g.K * c_tiles * n_tiles * g.B;
+  int ranges = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, base), ceil_div(chunks, 8)));
+  ranges = std::min(ranges, 65535);
+  const int cpr = (int)ceil_div(chunks, ranges);
+  ranges = (int)ceil_div(chunks, cpr);
+  const dim3 grid((unsigned)(g.K * c_tiles * n_tiles), (unsigned)ranges, (unsigned)g.B);
+  const size_t smem = sizeof(float) * (size_t)KM * (129 + 129) + (size_t)slots * KM * 8 + 16;
+  SDK_DISPATCH_INTERP(g.interp, g.P,
+                      (rc = launch_smem("gather_wgrad", gather_wgrad_kernel<INTERP, WEIGHTED, KM>,
+                                        grid, smem, stream, pix, map, wts, img, gW, g.Cg, g.H,
+                                        g.W, g.Cp, g.M, g.K, g.P, slots, c_tiles, n_tiles, cpr)));
+  return rc;
+}
+
 }  // namespace sdk

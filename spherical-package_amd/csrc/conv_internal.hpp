@@ -18,6 +18,10 @@ template <typename T>
 int launch_mapped_col2im(const T* col, const T* map, const T* wts, T* im, int64_t planes, int H,
                          int W, int M, int K, int P, int interp, hipStream_t stream);
 
+// dst[(b*C + c)*n + i] = bias ? bias[c] : 0 for `planes` = B*C planes of n elements.
+template <typename T>
+int plane_fill(T* dst, const T* bias, int64_t planes, int C, size_t n, hipStream_t stream);
+
 // Geometry of one convolution-shaped call, shared by the generic and the fused
 // drivers.  "gather side" is the image the sample map points into, "pixel side"
 // the grid the map is defined on:

@@ -180,6 +180,67 @@ def test_mapped_transposed_convolution(ops, oracle, case):
     assert relerr(_n(gb), wb) <= BWD_TOL[dt]
 
 
+@pytest.fixture
+def unfused(ops):
+    ops.set_conv_compute("unfused")
+    yield
+    ops.set_conv_compute("native")
+
+
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[2] is np.float32], ids=_ids)
+def test_unfused_float32_path(ops, oracle, unfused, case):
+    """float32 normally runs the fused MFMA kernels; the separate im2col/col2im + GEMM
+    kernels (the float64 route) must give the same answers in float32."""
+    test_mapped_convolution(ops, oracle, case)
+    test_mapped_transposed_convolution(ops, oracle, case)
+
+
+# shapes that straddle the fused kernels' tiles: (Cin, Cout, H, W, OH, OW, K, P, interp)
+TILE_CASES = [
+    (40, 72, 20, 24, 19, 23, 5, 0, 1),     # wide tiles, ragged pixels, 2 reduction chunks
+    (130, 130, 9, 12, 9, 12, 3, 2, 2),     # two channel tiles on both sides, weighted
+    (33, 64, 16, 40, 8, 40, 9, 0, 0),      # narrow tiles (<= 64 channels), nearest
+    (64, 33, 10, 30, 10, 29, 7, 4, 1),     # 16 tap slots per sample
+    (3, 16, 64, 128, 64, 128, 9, 0, 1),    # configuration 1's shape
+]
+
+
+@pytest.mark.parametrize("tc", TILE_CASES, ids=lambda t: "x".join(map(str, t)))
+def test_fused_conv_tile_edges(ops, oracle, tc):
+    Cin, Cout, H, W, OH, OW, K, P, interp = tc
+    dt = np.float32
+    rng = np.random.default_rng(sum(tc))
+    B = 3
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if P else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if P else None
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), K, interp))
+    assert relerr(got, oracle.mapped_conv_forward(x, m, wt, b, K, interp, iw)) <= 1e-5
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    assert relerr(_n(gb), wb) <= 1e-4
+    # transposed layer over the same map: input lives on the OH x OW grid, output on H x W
+    xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+    bt = rng.standard_normal(Cin).astype(dt)
+    gt = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), _t(iw), _t(wtt), _t(bt), H, W, K,
+                                                interp))
+    assert relerr(got, oracle.mapped_transposed_conv_forward(xt, m, wtt, bt, H, W, K, interp,
+                                                             iw)) <= 1e-4
+    gi, gw, gb = ops.mapped_transposed_conv_backward(_t(gt), _t(m), _t(iw), _t(xt), _t(wtt),
+                                                     _t(bt), K, interp)
+    wi, ww, wb = oracle.mapped_transposed_conv_backward(gt, m, xt, wtt, bt, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    assert relerr(_n(gb), wb) <= 1e-4
+
+
 # ------------------------------------------------------------------------------------------
 # Against the compiled reference's fixtures directly (no oracle in between).
 # ------------------------------------------------------------------------------------------
