@@ -198,14 +198,24 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
 #pragma unroll
       for (int j = 0; j < RPT; ++j) col[j] = 0.0f;
       const int cfirst = c0 + gpart * RPT;
-      for (int s = 0; s < ns; ++s) {
-        const int off = tap_off[s * TM + gm];
-        const float co = tap_co[s * TM + gm];
+      for (int s0 = 0; s0 < ns; s0 += 4) {
+        int off[4];
+        float co[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const bool on = s0 + u < ns;
+          off[u] = on ? tap_off[(s0 + u) * TM + gm] : 0;
+          co[u] = on ? tap_co[(s0 + u) * TM + gm] : 0.0f;
+        }
 #pragma unroll
         for (int j = 0; j < RPT; ++j) {
           const int c = min(cfirst + j, Cg - 1);   // padded rows meet zero weights
-          const float d = img_b[(size_t)c * HW + off];
-          col[j] += co * (co != 0.0f ? d : 0.0f);
+          const float* plane = img_b + (size_t)c * HW;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const float d = plane[off[u]];
+            col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
+          }
         }
       }
 #pragma unroll
@@ -368,14 +378,24 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
 #pragma unroll
     for (int j = 0; j < CPT; ++j) col[j] = 0.0f;
     const int cfirst = c0 + grp * CPT;
-    for (int s = 0; s < ns; ++s) {
-      const int off = tap_off[s * KM + gm];
-      const float co = tap_co[s * KM + gm];
+    for (int s0 = 0; s0 < ns; s0 += 4) {
+      int off[4];
+      float co[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool on = s0 + u < ns;
+        off[u] = on ? tap_off[(s0 + u) * KM + gm] : 0;
+        co[u] = on ? tap_co[(s0 + u) * KM + gm] : 0.0f;
+      }
 #pragma unroll
       for (int j = 0; j < CPT; ++j) {
         const int c = min(cfirst + j, Cg - 1);
-        const float d = img_b[(size_t)c * HW + off];
-        col[j] += co * (co != 0.0f ? d : 0.0f);
+        const float* plane = img_b + (size_t)c * HW;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float d = plane[off[u]];
+          col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
+        }
       }
     }
 #pragma unroll
