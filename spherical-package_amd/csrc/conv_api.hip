@@ -100,9 +100,9 @@ size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64
   // Upper bound over the conv (gather side = in_channels) and transposed conv
   // (gather side = out_channels) roles, so one query serves a whole layer call.
   ConvGeom a{batch, (int)in_channels, 1, 1, (int)out_channels, (int)gather_pixels,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, 1};
   ConvGeom b{batch, (int)out_channels, 1, 1, (int)in_channels, (int)gather_pixels,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, 1};
   if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(a) &&
       fused_supported(b))
     return align256(std::max(fused_workspace_bytes(a), fused_workspace_bytes(b)));
@@ -125,7 +125,7 @@ int sdk_mapped_conv_forward(const void* input, const void* sample_map, const voi
                         num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GATHER_GEMM, g, dtype, compute, input, sample_map, interp_weights, weight, bias,
              output, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -146,7 +146,7 @@ int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_m
                         num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights,
              weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -167,7 +167,7 @@ int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_
                         num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
              nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -189,7 +189,7 @@ int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map
                         kernel_size, num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GEMM_SCATTER, g, dtype, compute, input, sample_map, interp_weights, weight,
              bias, output, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -212,7 +212,7 @@ int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const voi
                         kernel_size, num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GATHER_GEMM, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
              nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -235,7 +235,7 @@ int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const vo
                         kernel_size, num_interp_pts, interp_weights, dtype, compute);
   if (rc) return rc;
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
-             (int)kernel_size, num_interp_pts, interp};
+             (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GATHER_WGRAD, g, dtype, compute, input, sample_map, interp_weights,
              grad_output, nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
 }

@@ -24,6 +24,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
 
@@ -197,7 +199,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
       float col[RPT];
 #pragma unroll
       for (int j = 0; j < RPT; ++j) col[j] = 0.0f;
-      const int cfirst = c0 + gpart * RPT;
+      // gpart is the same for all lanes of a wave when TM >= 64: keep the channel
+      // base in scalar registers so each load needs only a 32-bit lane offset
+      const int cfirst = c0 + (TM >= 64 ? __builtin_amdgcn_readfirstlane(gpart) : gpart) * RPT;
       for (int s0 = 0; s0 < ns; s0 += 4) {
         int off[4];
         float co[4];
@@ -207,13 +211,16 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
           off[u] = on ? tap_off[(s0 + u) * TM + gm] : 0;
           co[u] = on ? tap_co[(s0 + u) * TM + gm] : 0.0f;
         }
+        // one scalar base for the chunk; every load adds a 32-bit lane offset
+        const char* base = reinterpret_cast<const char*>(img_b + (size_t)min(cfirst, Cg - 1) * HW);
+        const unsigned plane_bytes = (unsigned)HW * 4u;
 #pragma unroll
         for (int j = 0; j < RPT; ++j) {
-          const int c = min(cfirst + j, Cg - 1);   // padded rows meet zero weights
-          const float* plane = img_b + (size_t)c * HW;
+          // padded rows re-read the last channel and meet zero weights
+          const unsigned cj = (unsigned)(min(cfirst + j, Cg - 1) - min(cfirst, Cg - 1)) * plane_bytes;
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
-            const float d = plane[off[u]];
+            const float d = *reinterpret_cast<const float*>(base + ((unsigned)off[u] * 4u + cj));
             col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
           }
         }
@@ -377,7 +384,7 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
     float col[CPT];
 #pragma unroll
     for (int j = 0; j < CPT; ++j) col[j] = 0.0f;
-    const int cfirst = c0 + grp * CPT;
+    const int cfirst = c0 + (KM >= 64 ? __builtin_amdgcn_readfirstlane(grp) : grp) * CPT;
     for (int s0 = 0; s0 < ns; s0 += 4) {
       int off[4];
       float co[4];
@@ -387,13 +394,14 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
         off[u] = on ? tap_off[(s0 + u) * KM + gm] : 0;
         co[u] = on ? tap_co[(s0 + u) * KM + gm] : 0.0f;
       }
+      const char* base = reinterpret_cast<const char*>(img_b + (size_t)min(cfirst, Cg - 1) * HW);
+      const unsigned plane_bytes = (unsigned)HW * 4u;
 #pragma unroll
       for (int j = 0; j < CPT; ++j) {
-        const int c = min(cfirst + j, Cg - 1);
-        const float* plane = img_b + (size_t)c * HW;
+        const unsigned cj = (unsigned)(min(cfirst + j, Cg - 1) - min(cfirst, Cg - 1)) * plane_bytes;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const float d = plane[off[u]];
+          const float d = *reinterpret_cast<const float*>(base + ((unsigned)off[u] * 4u + cj));
           col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
         }
       }
@@ -441,13 +449,14 @@ static int slots_for(const ConvGeom& g) {
 
 bool fused_supported(const ConvGeom& g) {
   if (slots_for(g) > kMaxSlots) return false;
+  if ((int64_t)g.H * g.W > ((int64_t)1 << 24)) return false;  // 32-bit byte offsets over 32 planes
   if (g.B > 65535) return false;
   return true;
 }
 
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
-  return (size_t)g.K * CpP * CgP * sizeof(float);
+  return std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
 }
 
 static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
@@ -480,6 +489,8 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                       float* workspace, hipStream_t stream) {
   if (compute != SDK_COMPUTE_NATIVE)
     return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  if (staged_supported(g) && getenv("SDK_STAGED"))
+    return staged_gather_gemm(g, img, map, wts, Wm, bias, pix, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -508,6 +519,8 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
+  if (scatter_staged_supported(g) && !getenv("SDK_NO_STAGED_SCATTER"))
+    return staged_gemm_scatter(g, pix, map, wts, Wm, img, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;

@@ -21,4 +21,16 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* img, float* gW, hipStream_t stream);
 
+// LDS-staged kernels (conv_staged.hip): the tile's image window lives in LDS.
+bool staged_supported(const ConvGeom& g);
+size_t staged_workspace_bytes(const ConvGeom& g);
+int staged_gather_gemm(const ConvGeom& g, const float* img, const float* map, const float* wts,
+                       const float* Wm, const float* bias, float* pix, float* workspace,
+                       hipStream_t stream);
+
+// img must be pre-filled (zeros or bias); needs Cp <= 128 (scatter_staged_supported).
+bool scatter_staged_supported(const ConvGeom& g);
+int staged_gemm_scatter(const ConvGeom& g, const float* pix, const float* map, const float* wts,
+                        const float* Wm, float* img, float* workspace, hipStream_t stream);
+
 }  // namespace sdk

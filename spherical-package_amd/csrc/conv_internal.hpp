@@ -33,6 +33,7 @@ struct ConvGeom {
   int Cg, H, W;  // gather-side channels and plane size
   int Cp, M;     // pixel-side channels and pixel count
   int K, P, interp;
+  int OW;        // width of the pixel grid (M = OH * OW)
 };
 
 // The three contractions, for the tensors' own floating type, as separate
