@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
   constexpr int NT = Taps2D<INTERP>::N;
 
   const Region rg = find_region<INTERP, WEIGHTED>(map, wts, pt, ty0, tx0, oy, ox, pix_ok, K, P, H,
-                                                  W, bb);
+                                                  W, bb, nullptr);
   build_region_lut(rg, H, W, src);
 
   floatx16 acc[NB];
@@ -231,6 +231,10 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
     const float* __restrict__ Ws, float* __restrict__ img, int Cg, int H, int W, int Cp, int K,
     int P, int chunks, PixelTiling pt) {
   __shared__ float region[kCC * (kRegionCap + 1)];
+  __shared__ int tc_e[4 * kTapRows * 32];
+  __shared__ float tc_co[4 * kTapRows * 32];
+  __shared__ int tc_rs[4 * (kTapKMax + 1)];
+  __shared__ int tc_ns[4 * kTapKMax];
   __shared__ int src[kRegionCap];
   __shared__ int bb[4];
 
@@ -249,8 +253,10 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
   constexpr int NT = Taps2D<INTERP>::N;
 
   const Region rg = find_region<INTERP, WEIGHTED>(map, wts, pt, ty0, tx0, oy, ox, pix_ok, K, P, H,
-                                                  W, bb);
+                                                  W, bb, tc_ns);
   build_region_lut(rg, H, W, src);
+  const TapCache tc = build_tap_cache<INTERP, WEIGHTED>(map, wts, pt, oy, ox, pix_ok, K, P, H, W,
+                                                        rg, tc_ns, tc_e, tc_co, tc_rs);
 
   // pixel-side operand, resident in registers: step s holds channel 2*s + half
   float bfrag[NS];
@@ -279,33 +285,39 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc, 0, 0, 0);
       }
       // splat: accumulator register v of this lane is channel c0 + row(v), pixel m
-      if (pix_ok) {
+      auto splat = [&](int e, float co) {
+        if (co != 0.0f) {
+          if (e >= 0) {
+            float* dst = region + (4 * half) * rg.RSp + e;
+            int offs[16];
+            float vals[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              offs[v] = (8 * (v >> 2) + (v & 3)) * rg.RSp;
+              vals[v] = co * acc[v];
+            }
+            lds_add_f32_batch<16>(dst, offs, vals);
+          } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int c = c0 + st_mfma_row(v, lane);
+              if (c < Cg) atomic_add_noret(img_b + (size_t)c * HW + (-e - 1), co * acc[v]);
+            }
+          }
+        }
+      };
+      if (k < tc.kc) {
+        const int r1 = tc.rs[k + 1];
+        for (int r = tc.rs[k]; r < r1; ++r) splat(tc.e[r * 32 + (lane & 31)], tc.co[r * 32 + (lane & 31)]);
+      } else if (pix_ok) {
         const size_t sbase = ((size_t)m * K + k) * q;
         Taps2D<INTERP> t;
         for (int p = 0; p < q; ++p) {
           t.set(map[(sbase + p) * 2], map[(sbase + p) * 2 + 1], H, W,
                 WEIGHTED ? wts[sbase + p] : 1.0f);
 #pragma unroll
-          for (int i = 0; i < NT; ++i) {
-            const float co = t.w[i];
-            if (__any(co != 0.0f)) {
-              const int e = rg.encode(t.y[i], t.x[i], W);
-              if (co != 0.0f) {
-                if (e >= 0) {
-                  float* dst = region + (4 * half) * rg.RSp + e;
-#pragma unroll
-                  for (int v = 0; v < 16; ++v)
-                    lds_add_f32(dst + (8 * (v >> 2) + (v & 3)) * rg.RSp, co * acc[v]);
-                } else {
-#pragma unroll
-                  for (int v = 0; v < 16; ++v) {
-                    const int c = c0 + st_mfma_row(v, lane);
-                    if (c < Cg) atomic_add_noret(img_b + (size_t)c * HW + (-e - 1), co * acc[v]);
-                  }
-                }
-              }
-            }
-          }
+          for (int i = 0; i < NT; ++i)
+            if (__any(t.w[i] != 0.0f)) splat(rg.encode(t.y[i], t.x[i], W), t.w[i]);
         }
       }
     }

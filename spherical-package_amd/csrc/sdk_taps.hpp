@@ -35,6 +35,31 @@ __device__ __forceinline__ void lds_add_f32(float* addr, float v) {
   }
 }
 
+// N independent float adds into LDS: all loads, then all compare-and-swaps, are
+// issued back to back so their latencies overlap; an add whose swap lost a race
+// is redone with the single-word loop.
+template <int N>
+__device__ __forceinline__ void lds_add_f32_batch(float* base, const int (&offs)[N],
+                                                  const float (&vals)[N]) {
+  int old[N], got[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+    old[i] = __hip_atomic_load(reinterpret_cast<int*>(base + offs[i]), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+    got[i] = atomicCAS(reinterpret_cast<int*>(base + offs[i]), old[i],
+                       __float_as_int(__int_as_float(old[i]) + vals[i]));
+  bool lost = false;
+#pragma unroll
+  for (int i = 0; i < N; ++i) lost |= got[i] != old[i];
+  if (lost) {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if (got[i] != old[i]) lds_add_f32(base + offs[i], vals[i]);
+  }
+}
+
 __device__ __forceinline__ int to_int_clamped(float v) {
   return (int)fminf(fmaxf(v, -2.0e9f), 2.0e9f);
 }
