@@ -343,14 +343,15 @@ __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
 // gather_wgrad.  Workgroup: one kernel sample k, one TC x TN tile of gW, one
 // batch element and one range of pixels; D[n][c] = sum_m pix[b][n][m] * col[(c,k)][m]
 // accumulated over the range in chunks of KM pixels, then added atomically to gW.
-// grid.x = K * c tiles * n tiles, grid.y = pixel ranges, grid.z = batch.
+// grid.x = 8 * ceil(ranges * batch / 8) * K * c tiles * n tiles; ids past the last range exit.
 // LDS: As[KM][TN+1] (pix, transposed), Bs[KM][TC+1] (columns, transposed), taps.
 // ---------------------------------------------------------------------------
 template <int INTERP, bool WEIGHTED, int KM>
 __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ img, float* __restrict__ gW, int Cg, int H, int W, int Cp, int M,
-    int K, int P, int slots, int c_tiles, int n_tiles, int chunks_per_range) {
+    int K, int P, int slots, int c_tiles, int n_tiles, int chunks_per_range, int ranges,
+    int batches) {
   constexpr int TN = 128, TC = 128, LDA = TN + 1, LDB = TC + 1;
   extern __shared__ __align__(16) unsigned char smem[];
   float* As = reinterpret_cast<float*>(smem);              // [KM][LDA]
@@ -362,19 +363,27 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
   constexpr int GROUPS = kThreads / KM;   // channel groups in the gather
   constexpr int CPT = TC / GROUPS;        // channels per thread
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int k = blockIdx.x / (c_tiles * n_tiles);
-  const int c0 = ((blockIdx.x / n_tiles) % c_tiles) * TC;
-  const int n0 = (blockIdx.x % n_tiles) * TN;
+  // 1-D grid.  Workgroup ids go round-robin over the 8 XCDs; all K * c_tiles * n_tiles
+  // output tiles of one pixel range read the same pixels of img and pix, so they are
+  // given consecutive slots of one XCD and meet in its L2.
+  const int kinds = K * c_tiles * n_tiles;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int kind = slot % kinds, range_id = (slot / kinds) * 8 + xcd;
+  if (range_id >= ranges * batches) return;
+  const int range = range_id % ranges, batch = range_id / ranges;
+  const int k = kind / (c_tiles * n_tiles);
+  const int c0 = ((kind / n_tiles) % c_tiles) * TC;
+  const int n0 = (kind % n_tiles) * TN;
   const int a_base = (wave & 1) * 64, b_base = (wave >> 1) * 64;
   const size_t HW = (size_t)H * W;
-  const float* img_b = img + (size_t)blockIdx.z * Cg * HW;
-  const float* pix_b = pix + (size_t)blockIdx.z * Cp * M;
+  const float* img_b = img + (size_t)batch * Cg * HW;
+  const float* pix_b = pix + (size_t)batch * Cp * M;
   const int gm = tid % KM, grp = tid / KM;
 
   floatx16 acc[2][2];
   zero_acc(acc);
 
-  const int chunk_beg = blockIdx.y * chunks_per_range;
+  const int chunk_beg = range * chunks_per_range;
   const int chunk_end = min(chunk_beg + chunks_per_range, (M + KM - 1) / KM);
   for (int ch = chunk_beg; ch < chunk_end; ++ch) {
     const int m0 = ch * KM;
@@ -559,12 +568,15 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   ranges = std::min(ranges, 65535);
   const int cpr = (int)ceil_div(chunks, ranges);
   ranges = (int)ceil_div(chunks, cpr);
-  const dim3 grid((unsigned)(g.K * c_tiles * n_tiles), (unsigned)ranges, (unsigned)g.B);
+  const int64_t slots_total = ceil_div((int64_t)ranges * g.B, 8) * 8 * g.K * c_tiles * n_tiles;
+  if (slots_total >= ((int64_t)1 << 31))
+    return fail(SDK_ERR_UNSUPPORTED, "gather_wgrad: grid too large");
+  const dim3 grid((unsigned)slots_total, 1, 1);
   const size_t smem = sizeof(float) * (size_t)KM * (129 + 129) + (size_t)slots * KM * 8 + 16;
   SDK_DISPATCH_INTERP(g.interp, g.P,
                       (rc = launch_smem("gather_wgrad", gather_wgrad_kernel<INTERP, WEIGHTED, KM>,
                                         grid, smem, stream, pix, map, wts, img, gW, g.Cg, g.H,
-                                        g.W, g.Cp, g.M, g.K, g.P, slots, c_tiles, n_tiles, cpr)));
+                                        g.W, g.Cp, g.M, g.K, g.P, slots, c_tiles, n_tiles, cpr, ranges, (int)g.B)));
   return rc;
 }
 
