@@ -76,6 +76,33 @@ def _roof(bound, work, ms, traffic=None, peak=None):
             "frac": round(achieved / peak, 4), "traffic": traffic}
 
 
+def _conv_entry_points(torch, ops, x, m, iw, w, b, g, K, interp, compute):
+    """The three contractions of one mapped-convolution layer call as separate C-ABI
+    launches (what the autograd function issues), for per-kernel timing."""
+    from _spherical_distortion_ext import _capi
+    B, Cin, H, W = x.shape
+    Cout = w.shape[0]
+    OH, OW = m.shape[:2]
+    P = 0 if iw is None else int(iw.shape[-1])
+    mode = {"native": _capi.SDK_COMPUTE_NATIVE, "bf16": _capi.SDK_COMPUTE_BF16}[compute]
+    nws = _capi.load().sdk_mapped_conv_workspace_bytes(B, Cin, Cout, OH * OW, K, P, interp, 0, mode)
+    ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=x.device)
+    out = torch.empty(B, Cout, OH, OW, device=x.device)
+    gi, gw = torch.empty_like(x), torch.empty_like(w)
+    gb = torch.empty(Cout, device=x.device)
+    p, s = ops._ptr, ops._stream(x)
+    dims = (B, Cin, H, W, Cout, OH, OW, K, P, interp, 0, mode, s)
+    return {
+        "forward": lambda: _capi.call("sdk_mapped_conv_forward", p(x), p(m), p(iw), p(w), p(b),
+                                      p(out), p(ws), nws, *dims),
+        "backward_input": lambda: _capi.call("sdk_mapped_conv_backward_input", p(g), p(m), p(iw),
+                                             p(w), p(gi), p(ws), nws, *dims),
+        "backward_weight": lambda: _capi.call("sdk_mapped_conv_backward_weight", p(g), p(m),
+                                              p(iw), p(x), p(gw), p(ws), nws, *dims),
+        "bias_grad": lambda: _capi.call("sdk_bias_grad", p(g), p(gb), B, Cout, OH * OW, 0, s),
+    }, (ws, out, gi, gw, gb)
+
+
 def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
     import workloads
     cfg = workloads.config4(batch=batch)
@@ -86,22 +113,25 @@ def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
     B, Cin, H, W = x.shape
     Cout = w.shape[0]
     flops = 2.0 * Cout * Cin * K * H * W * B
+    peak = MFMA_FP32_TFLOPS if compute == "native" else MFMA_BF16_TFLOPS
     ops.set_conv_compute(compute)
     try:
         def step():
             ops.mapped_conv_forward(x, m, iw, w, b, K, interp)
             ops.mapped_conv_backward(g, m, iw, x, w, b, K, interp)
         ms, ms_min = timer.run(step, steps, warmup)
-        ms_f, _ = timer.run(lambda: ops.mapped_conv_forward(x, m, iw, w, b, K, interp),
-                            max(2, steps // 2), 1)
     finally:
         ops.set_conv_compute("native")
-    peak = MFMA_FP32_TFLOPS if compute == "native" else MFMA_BF16_TFLOPS
+    calls, keep = _conv_entry_points(torch, ops, x, m, iw, w, b, g, K, interp, compute)
+    parts = {}
+    for name, fn in calls.items():
+        t, _ = timer.run(fn, max(3, steps // 2), 1)
+        parts[name] = dict(ms=t, **(_roof("mfma", flops, t, peak=peak) if name != "bias_grad"
+                                    else _roof("hbm", _nbytes(g), t)))
+    del keep
+    dominant = max(("forward", "backward_input", "backward_weight"), key=lambda n: parts[n]["ms"])
     return {"ms_per_step": ms, "ms_min": ms_min, "images_per_s": B / (ms * 1e-3),
-            "forward_ms": ms_f, "flops_per_step": 3 * flops,
-            "roofline_step": _roof("mfma", 3 * flops, ms, peak=peak),
-            "roofline_forward": _roof("mfma", flops, ms_f, peak=peak),
-            "tensors": (cfg, None)}
+            "flops_per_contraction": flops, "parts": parts, "dominant": dominant}
 
 
 def bench_resample2(torch, ops, timer, steps, warmup):
@@ -167,9 +197,20 @@ def bench_ico5(torch, ops, timer, steps, warmup):
                                                              peak=MFMA_FP32_TFLOPS))}
 
 
-def cpu_baseline(budget_s=25.0):
-    """Times the CPU checker on a bounded sample of configuration 4 (batch 1, a
-    band of output rows when needed) and scales to images per second."""
+def _measured_traffic(kernel):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
+    a copy kernel of known size); kept with the profile summaries, None when not measured."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(kernel)
+
+
+def cpu_baseline(budget_s=12.0):
+    """Times the CPU checker on a bounded sample of configuration 4 and reports images per
+    second: whole batch-1 images (forward + backward) repeated for about `budget_s` seconds
+    with the compiled reference, or one band of output rows, scaled, with the slower port."""
     import torch
     import workloads
     from oracle import oracle as orc
@@ -178,29 +219,38 @@ def cpu_baseline(budget_s=25.0):
         R = ref.load() if ref.available() else None
     except Exception:
         R = None
-    H, W = 256, 512
+    H = 256
     cfg = workloads.config4(batch=1)
-    rows = 64 if R is None else H             # band of output rows (a bounded sample)
+    K = 9
+    if R is not None:
+        tt = [torch.from_numpy(cfg[k]) for k in ("x", "sample_map", "interp_weights", "weight",
+                                                 "bias", "grad_output")]
+        it = R.InterpolationType(2)
+        mod = R._weighted_mapped_convolution
+
+        def one():
+            mod.weighted_mapped_conv_forward(tt[0], tt[1], tt[2], tt[3], tt[4], K, it)
+            mod.weighted_mapped_conv_backward(tt[5], tt[1], tt[2], tt[0], tt[3], tt[4], K, it)
+        one()  # warm-up
+        reps, t0 = 0, time.time()
+        while reps < 1 or (time.time() - t0 < budget_s and reps < 16):
+            one()
+            reps += 1
+        dt = time.time() - t0
+        return {"value": round(reps / dt, 4), "unit": "images/s",
+                "cores": int(torch.get_num_threads()), "kind": "reference",
+                "sample": "configuration 4 at batch 1 (one 128x256x512 image, fwd+bwd), %d "
+                          "repetitions in %.1f s after one warm-up" % (reps, dt)}
+    rows = 64
     m = np.ascontiguousarray(cfg["sample_map"][:rows])
     iw = np.ascontiguousarray(cfg["interp_weights"][:rows])
     g = np.ascontiguousarray(cfg["grad_output"][:, :, :rows])
-    K = 9
     t0 = time.time()
-    if R is not None:
-        tt = [torch.from_numpy(a) for a in (cfg["x"], m, iw, cfg["weight"], cfg["bias"], g)]
-        it = R.InterpolationType(2)
-        R._weighted_mapped_convolution.weighted_mapped_conv_forward(
-            tt[0], tt[1], tt[2], tt[3], tt[4], K, it)
-        R._weighted_mapped_convolution.weighted_mapped_conv_backward(
-            tt[5], tt[1], tt[2], tt[0], tt[3], tt[4], K, it)
-        kind, cores = "reference", torch.get_num_threads()
-    else:
-        orc.mapped_conv_forward(cfg["x"], m, cfg["weight"], cfg["bias"], K, 2, iw)
-        orc.mapped_conv_backward(g, m, cfg["x"], cfg["weight"], cfg["bias"], K, 2, iw)
-        kind, cores = "port", orc.num_threads()
+    orc.mapped_conv_forward(cfg["x"], m, cfg["weight"], cfg["bias"], K, 2, iw)
+    orc.mapped_conv_backward(g, m, cfg["x"], cfg["weight"], cfg["bias"], K, 2, iw)
     dt = time.time() - t0
-    frac = rows / float(H)                    # share of one image's output pixels
-    return {"value": round(frac / dt, 4), "unit": "images/s", "cores": int(cores), "kind": kind,
+    return {"value": round(rows / float(H) / dt, 4), "unit": "images/s",
+            "cores": int(orc.num_threads()), "kind": "port",
             "sample": "configuration 4, batch 1, output rows 0..%d of %d (%.1f s of CPU work), "
                       "fwd+bwd, scaled by the pixel share" % (rows - 1, H, dt)}
 
@@ -229,16 +279,14 @@ def main():
     head = None
     if want("conv4"):
         head = bench_conv4(torch, ops, timer, args.steps, args.warmup)
-        head.pop("tensors")
-        kernels["conv4_fp32"] = {k: head[k] for k in ("ms_per_step", "forward_ms", "images_per_s",
-                                                     "roofline_step", "roofline_forward")}
+        kernels["conv4_fp32"] = dict(ms_per_step=head["ms_per_step"],
+                                     images_per_s=head["images_per_s"], **head["parts"])
         torch.cuda.empty_cache()
     if want("conv4_bf16"):
         try:
             r = bench_conv4(torch, ops, timer, args.steps, args.warmup, compute="bf16")
-            r.pop("tensors")
-            kernels["conv4_bf16"] = {k: r[k] for k in ("ms_per_step", "forward_ms", "images_per_s",
-                                                      "roofline_step", "roofline_forward")}
+            kernels["conv4_bf16"] = dict(ms_per_step=r["ms_per_step"],
+                                         images_per_s=r["images_per_s"], **r["parts"])
         except RuntimeError as e:
             kernels["conv4_bf16"] = {"error": str(e)[:200]}
         torch.cuda.empty_cache()
@@ -258,8 +306,12 @@ def main():
                                    "fwd+bwd, x 8x128x256x512 -> 128 channels, K=9, float32",
                        "global_batch": 8}}
     if head is not None:
+        dom = head["parts"][head["dominant"]]
+        roof = {k: dom[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+        roof["kernel"] = "mapped_conv_" + head["dominant"]
+        roof["traffic"] = _measured_traffic(roof["kernel"])
         line.update(value=round(head["images_per_s"], 3), ms_per_step=round(head["ms_per_step"], 4),
-                    roofline=head["roofline_step"])
+                    roofline=roof)
     else:
         line.update(value=None, ms_per_step=None, roofline=None)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()

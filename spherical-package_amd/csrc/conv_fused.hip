@@ -24,8 +24,6 @@
 
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
-
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
 
@@ -498,8 +496,6 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                       float* workspace, hipStream_t stream) {
   if (compute != SDK_COMPUTE_NATIVE)
     return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
-  if (staged_supported(g) && getenv("SDK_STAGED"))
-    return staged_gather_gemm(g, img, map, wts, Wm, bias, pix, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -528,7 +524,7 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
-  if (scatter_staged_supported(g) && !getenv("SDK_NO_STAGED_SCATTER"))
+  if (scatter_staged_supported(g))
     return staged_gemm_scatter(g, pix, map, wts, Wm, img, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;

@@ -82,6 +82,10 @@ __global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
     const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
     int H, int W, int Cp, int K, int P, int CgP, int n_tiles, PixelTiling pt) {
   __shared__ float region[kCC * (kRegionCap + 1)];
+  __shared__ int tc_e[4 * kTapRows * 32];
+  __shared__ float tc_co[4 * kTapRows * 32];
+  __shared__ int tc_rs[4 * (kTapKMax + 1)];
+  __shared__ int tc_ns[4 * kTapKMax];
   __shared__ int src[kRegionCap];
   __shared__ int bb[4];
 
@@ -101,8 +105,10 @@ __global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
   constexpr int NT = Taps2D<INTERP>::N;
 
   const Region rg = find_region<INTERP, WEIGHTED>(map, wts, pt, ty0, tx0, oy, ox, pix_ok, K, P, H,
-                                                  W, bb, nullptr);
+                                                  W, bb, tc_ns);
   build_region_lut(rg, H, W, src);
+  const TapCache tc = build_tap_cache<INTERP, WEIGHTED>(map, wts, pt, oy, ox, pix_ok, K, P, H, W,
+                                                        rg, tc_ns, tc_e, tc_co, tc_rs);
 
   floatx16 acc[NB];
 #pragma unroll
@@ -111,50 +117,53 @@ __global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
 
   for (int c0 = 0; c0 < CgP; c0 += kCC) {
-    __syncthreads();  // LUT ready / previous chunk's readers are done
+    __syncthreads();  // previous chunk's readers are done
     load_region(img_b, HW, Cg, c0, rg, src, region);
     __syncthreads();
     // this lane's column rows inside the chunk: 2*step + half
     const float* reg_half = region + half * rg.RSp;
-    const float* img_half = img_b + (size_t)min(c0 + half, Cg - 1) * HW;
     for (int k = 0; k < K; ++k) {
       float col[kCC / 2];
 #pragma unroll
       for (int s = 0; s < kCC / 2; ++s) col[s] = 0.0f;
-      if (pix_ok) {
-        const size_t sbase = ((size_t)m * K + k) * q;
+      // adds one tap (encoded index e, coefficient co) of this lane's pixel to its column rows
+      auto gather = [&](int e, float co) {
+        if (__all(e >= 0 || co == 0.0f)) {
+          const int ee = e >= 0 ? e : 0;
+#pragma unroll
+          for (int s = 0; s < kCC / 2; ++s) col[s] += co * reg_half[2 * s * rg.RSp + ee];
+        } else {
+          // some lane's tap lies outside the staged window
+#pragma unroll
+          for (int s = 0; s < kCC / 2; ++s) {
+            float d;
+            if (e >= 0) {
+              d = reg_half[2 * s * rg.RSp + e];
+            } else {
+              const int c = c0 + 2 * s + half;
+              d = (co != 0.0f && c < Cg) ? img_b[(size_t)c * HW + (-e - 1)] : 0.0f;
+            }
+            col[s] += co * d;
+          }
+        }
+      };
+      if (k < tc.kc) {
+        const int r1 = tc.rs[k + 1];
+        for (int r = tc.rs[k]; r < r1; ++r)
+          gather(tc.e[r * 32 + (lane & 31)], tc.co[r * 32 + (lane & 31)]);
+      } else {
+        const size_t sbase = ((size_t)(pix_ok ? m : 0) * K + k) * q;
         Taps2D<INTERP> t;
         for (int p = 0; p < q; ++p) {
           t.set(map[(sbase + p) * 2], map[(sbase + p) * 2 + 1], H, W,
                 WEIGHTED ? wts[sbase + p] : 1.0f);
 #pragma unroll
           for (int i = 0; i < NT; ++i) {
-            const float co = t.w[i];
-            if (__any(co != 0.0f)) {
-              const int e = rg.encode(t.y[i], t.x[i], W);
-              if (__all(e >= 0 || co == 0.0f)) {
-                const int ee = e >= 0 ? e : 0;
-#pragma unroll
-                for (int s = 0; s < kCC / 2; ++s) col[s] += co * reg_half[2 * s * rg.RSp + ee];
-              } else {
-                // some lane's tap lies outside the staged window
-#pragma unroll
-                for (int s = 0; s < kCC / 2; ++s) {
-                  float d;
-                  if (e >= 0) {
-                    d = reg_half[2 * s * rg.RSp + e];
-                  } else {
-                    const int c = c0 + 2 * s + half;
-                    d = (co != 0.0f && c < Cg) ? img_b[(size_t)c * HW + (-e - 1)] : 0.0f;
-                  }
-                  col[s] += co * d;
-                }
-              }
-            }
+            const float co = pix_ok ? t.w[i] : 0.0f;
+            if (__any(co != 0.0f)) gather(rg.encode(t.y[i], t.x[i], W), co);
           }
         }
       }
-      (void)img_half;
       // weights: one 16-byte fragment per lane and step, rows c0 + 2*step + half
       const float* wrow = Wp + (((size_t)k * CgP + c0 + half) * n_tiles + nt) * TN + (lane & 31) * NB;
 #pragma unroll
