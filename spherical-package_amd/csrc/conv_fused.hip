@@ -25,11 +25,10 @@
 #include <hip/hip_runtime.h>
 
 #include "sdk_host.hpp"
+#include "sdk_mfma.hpp"
 #include "sdk_taps.hpp"
 
 namespace sdk {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
 constexpr int kKC = 32;         // reduction rows staged per step
@@ -122,6 +121,43 @@ __device__ __forceinline__ void mfma_chunk(const float* __restrict__ As, int lda
   }
 }
 
+// Same contraction with operands rounded to bf16 (fp32 accumulate): the LDS tiles stay
+// fp32 and are converted while the fragments are read; rows must be a multiple of 16.
+__device__ __forceinline__ void mfma_chunk_bf16(const float* __restrict__ As, int lda, int a_base,
+                                                const float* __restrict__ Bs, int ldb, int b_base,
+                                                int rows, floatx16 (&acc)[2][2]) {
+  const int lane = threadIdx.x & 63;
+  const int lk = lane >> 5, lj = lane & 31;
+  for (int r = 0; r < rows; r += 16) {
+    Bf16Frag a[2], b[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      float fa[8], fb[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        fa[j] = As[(r + 8 * lk + j) * lda + a_base + 32 * blk + lj];
+        fb[j] = Bs[(r + 8 * lk + j) * ldb + b_base + 32 * blk + lj];
+      }
+      a[blk] = pack_bf16x8(fa);
+      b[blk] = pack_bf16x8(fb);
+    }
+    acc[0][0] = mfma_bf16(a[0], b[0], acc[0][0]);
+    acc[0][1] = mfma_bf16(a[0], b[1], acc[0][1]);
+    acc[1][0] = mfma_bf16(a[1], b[0], acc[1][0]);
+    acc[1][1] = mfma_bf16(a[1], b[1], acc[1][1]);
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ void mfma_chunk_any(const float* __restrict__ As, int lda, int a_base,
+                                               const float* __restrict__ Bs, int ldb, int b_base,
+                                               int rows, floatx16 (&acc)[2][2]) {
+  if constexpr (BF16)
+    mfma_chunk_bf16(As, lda, a_base, Bs, ldb, b_base, rows, acc);
+  else
+    mfma_chunk(As, lda, a_base, Bs, ldb, b_base, rows, acc);
+}
+
 __device__ __forceinline__ void zero_acc(floatx16 (&acc)[2][2]) {
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -162,7 +198,7 @@ __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
 // grid.x = pixel tiles * n tiles, grid.y = batch.
 // LDS: Bs[kKC][TM] column tile, As[kKC][TN] weight tile, tap table.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int TN, int TM>
+template <int INTERP, bool WEIGHTED, int TN, int TM, bool BF16>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wg, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
@@ -232,7 +268,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
         reinterpret_cast<float4*>(As)[e] = src[(size_t)r * (CpP / 4) + n4];
       }
       __syncthreads();
-      mfma_chunk(As, TN, a_base, Bs, TM, b_base, kKC, acc);
+      mfma_chunk_any<BF16>(As, TN, a_base, Bs, TM, b_base, kKC, acc);
       __syncthreads();
     }
   }
@@ -260,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
 // neighbouring addresses).  img must be pre-filled (zeros or bias).
 // grid.x = pixel tiles, grid.y = batch.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int TC, int TM>
+template <int INTERP, bool WEIGHTED, int TC, int TM, bool BF16>
 __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
     const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wsc, float* __restrict__ img, int Cg, int H, int W, int Cp, int M,
@@ -312,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
           reinterpret_cast<float4*>(As)[e] = src[(size_t)r * (CgP / 4) + c4];
         }
         __syncthreads();
-        mfma_chunk(As, TC, a_base, Bs, TM, b_base, kKC, acc);
+        mfma_chunk_any<BF16>(As, TC, a_base, Bs, TM, b_base, kKC, acc);
         __syncthreads();
       }
       // ---- scatter the 64 x 64 block of this wave
@@ -344,7 +380,7 @@ __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
 // grid.x = 8 * ceil(ranges * batch / 8) * K * c tiles * n tiles; ids past the last range exit.
 // LDS: As[KM][TN+1] (pix, transposed), Bs[KM][TC+1] (columns, transposed), taps.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int KM>
+template <int INTERP, bool WEIGHTED, int KM, bool BF16>
 __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ img, float* __restrict__ gW, int Cg, int H, int W, int Cp, int M,
@@ -427,7 +463,7 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
       }
     }
     __syncthreads();
-    mfma_chunk(As, LDA, a_base, Bs, LDB, b_base, KM, acc);
+    mfma_chunk_any<BF16>(As, LDA, a_base, Bs, LDB, b_base, KM, acc);
     // the next build_taps() starts with a barrier, which also protects As / Bs
   }
 
@@ -494,8 +530,7 @@ static int launch_smem(const char* what, Kern kern, dim3 grid, size_t smem, hipS
 int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
                       const float* wts, const float* Wm, const float* bias, float* pix,
                       float* workspace, hipStream_t stream) {
-  if (compute != SDK_COMPUTE_NATIVE)
-    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  const bool bf16 = compute == SDK_COMPUTE_BF16;
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -505,14 +540,15 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
   const int m_tiles = (int)ceil_div(g.M, TM), n_tiles = CpP / TN;
   const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
   const size_t smem = sizeof(float) * (kKC * TM + kKC * TN) + (size_t)slots * TM * 8 + 16;
-#define GG(TNv, TMv)                                                                          \
+#define GG(TNv, TMv, BFv)                                                                          \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                          \
                       (rc = launch_smem("gather_gemm",                                        \
-                                        gather_gemm_kernel<INTERP, WEIGHTED, TNv, TMv>, grid, \
+                                        gather_gemm_kernel<INTERP, WEIGHTED, TNv, TMv, BFv>, grid, \
                                         smem, stream, img, map, wts, (const float*)workspace, \
                                         bias, pix, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP,  \
                                         CpP, slots, m_tiles)))
-  if (narrow) GG(64, 256); else GG(128, 128);
+  if (bf16) { if (narrow) GG(64, 256, true); else GG(128, 128, true); }
+  else { if (narrow) GG(64, 256, false); else GG(128, 128, false); }
 #undef GG
   return rc;
 }
@@ -520,12 +556,11 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
 int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* Wm, const float* bias, float* img,
                        float* workspace, hipStream_t stream) {
-  if (compute != SDK_COMPUTE_NATIVE)
-    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
   if (scatter_staged_supported(g))
-    return staged_gemm_scatter(g, pix, map, wts, Wm, img, workspace, stream);
+    return staged_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -535,22 +570,22 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
   const int m_tiles = (int)ceil_div(g.M, TM);
   const dim3 grid((unsigned)m_tiles, (unsigned)g.B);
   const size_t smem = sizeof(float) * (kKC * TM + kKC * TC) + (size_t)slots * TM * 8 + 16;
-#define GS(TCv, TMv)                                                                           \
+#define GS(TCv, TMv, BFv)                                                                           \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                           \
                       (rc = launch_smem("gemm_scatter",                                        \
-                                        gemm_scatter_kernel<INTERP, WEIGHTED, TCv, TMv>, grid, \
+                                        gemm_scatter_kernel<INTERP, WEIGHTED, TCv, TMv, BFv>, grid, \
                                         smem, stream, pix, map, wts, (const float*)workspace,  \
                                         img, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP, CpP,    \
                                         slots, m_tiles)))
-  if (narrow) GS(64, 256); else GS(128, 128);
+  if (bf16) { if (narrow) GS(64, 256, true); else GS(128, 128, true); }
+  else { if (narrow) GS(64, 256, false); else GS(128, 128, false); }
 #undef GS
   return rc;
 }
 
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* img, float* gW, hipStream_t stream) {
-  if (compute != SDK_COMPUTE_NATIVE)
-    return fail(SDK_ERR_UNSUPPORTED, "bf16 compute is not built for the fused kernels yet");
+  const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
@@ -569,10 +604,15 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
     return fail(SDK_ERR_UNSUPPORTED, "gather_wgrad: grid too large");
   const dim3 grid((unsigned)slots_total, 1, 1);
   const size_t smem = sizeof(float) * (size_t)KM * (129 + 129) + (size_t)slots * KM * 8 + 16;
-  SDK_DISPATCH_INTERP(g.interp, g.P,
-                      (rc = launch_smem("gather_wgrad", gather_wgrad_kernel<INTERP, WEIGHTED, KM>,
-                                        grid, smem, stream, pix, map, wts, img, gW, g.Cg, g.H,
-                                        g.W, g.Cp, g.M, g.K, g.P, slots, c_tiles, n_tiles, cpr, ranges, (int)g.B)));
+#define GW(BFv)                                                                                 \
+  SDK_DISPATCH_INTERP(g.interp, g.P,                                                            \
+                      (rc = launch_smem("gather_wgrad",                                         \
+                                        gather_wgrad_kernel<INTERP, WEIGHTED, KM, BFv>, grid,   \
+                                        smem, stream, pix, map, wts, img, gW, g.Cg, g.H, g.W,   \
+                                        g.Cp, g.M, g.K, g.P, slots, c_tiles, n_tiles, cpr,      \
+                                        ranges, (int)g.B)))
+  if (bf16) GW(true); else GW(false);
+#undef GW
   return rc;
 }
 

@@ -30,7 +30,7 @@ int staged_gather_gemm(const ConvGeom& g, const float* img, const float* map, co
 
 // img must be pre-filled (zeros or bias); needs Cp <= 128 (scatter_staged_supported).
 bool scatter_staged_supported(const ConvGeom& g);
-int staged_gemm_scatter(const ConvGeom& g, const float* pix, const float* map, const float* wts,
+int staged_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map, const float* wts,
                         const float* Wm, float* img, float* workspace, hipStream_t stream);
 
 }  // namespace sdk

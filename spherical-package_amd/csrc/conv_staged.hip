@@ -20,10 +20,10 @@
 #include "conv_fused.hpp"
 #include "conv_staged.hpp"
 #include "sdk_host.hpp"
+#include "sdk_mfma.hpp"
 
 namespace sdk {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kStThreads = 256;
 
@@ -214,27 +214,41 @@ __global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
 // Weight copy Ws[k][chunk][g][half][c % 32][j]: value for n = 2*(4g + j) + half,
 // so a lane fetches the A fragments of four consecutive MFMA steps as 16 bytes.
 // ---------------------------------------------------------------------------
+// With bf16 != 0 the order is Ws[k][chunk][t][half][c % 32][j], n = 16*t + 8*half + j: the
+// eight values a lane packs into one bf16 A fragment are 32 contiguous bytes.
 __global__ __launch_bounds__(kStThreads) void permute_weight_scatter_kernel(
     const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int chunks,
-    int NS) {
+    int NS, int bf16) {
   const size_t per_k = (size_t)chunks * NS * 64;
   const size_t total = (size_t)K * per_k;
   for (size_t e = (size_t)blockIdx.x * kStThreads + threadIdx.x; e < total;
        e += (size_t)gridDim.x * kStThreads) {
-    const int j = (int)(e & 3);
-    const int cl = (int)((e >> 2) & 31);
-    const int half = (int)((e >> 7) & 1);
-    const size_t rest = e >> 8;               // (k * chunks + chunk) * (NS/4) + g
-    const int g = (int)(rest % (NS / 4));
-    const int chunk = (int)((rest / (NS / 4)) % chunks);
-    const int k = (int)(rest / ((size_t)(NS / 4) * chunks));
-    const int n = 2 * (4 * g + j) + half;
+    int j, cl, half, g, chunk, k, n;
+    if (bf16) {
+      j = (int)(e & 7);
+      cl = (int)((e >> 3) & 31);
+      half = (int)((e >> 8) & 1);
+      const size_t rest = e >> 9;             // (k * chunks + chunk) * (NS/8) + t
+      g = (int)(rest % (NS / 8));
+      chunk = (int)((rest / (NS / 8)) % chunks);
+      k = (int)(rest / ((size_t)(NS / 8) * chunks));
+      n = 16 * g + 8 * half + j;
+    } else {
+      j = (int)(e & 3);
+      cl = (int)((e >> 2) & 31);
+      half = (int)((e >> 7) & 1);
+      const size_t rest = e >> 8;             // (k * chunks + chunk) * (NS/4) + g
+      g = (int)(rest % (NS / 4));
+      chunk = (int)((rest / (NS / 4)) % chunks);
+      k = (int)(rest / ((size_t)(NS / 4) * chunks));
+      n = 2 * (4 * g + j) + half;
+    }
     const int c = chunk * kCC + cl;
     out[e] = (n < Cp && c < Cg) ? Wm[(size_t)n * Cg * K + (size_t)c * K + k] : 0.0f;
   }
 }
 
-template <int INTERP, bool WEIGHTED, int NS>
+template <int INTERP, bool WEIGHTED, int NS, bool BF16>
 __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
     const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Ws, float* __restrict__ img, int Cg, int H, int W, int Cp, int K,
@@ -267,12 +281,27 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
   const TapCache tc = build_tap_cache<INTERP, WEIGHTED>(map, wts, pt, oy, ox, pix_ok, K, P, H, W,
                                                         rg, tc_ns, tc_e, tc_co, tc_rs);
 
-  // pixel-side operand, resident in registers: step s holds channel 2*s + half
-  float bfrag[NS];
+  // pixel-side operand, resident in registers.  fp32: step s holds channel 2*s + half;
+  // bf16: fragment t holds channels 16*t + 8*half + 0..7, two per register.
+  float bfrag[BF16 ? 1 : NS];
+  Bf16Frag bfrag16[BF16 ? NS / 8 : 1];
+  if constexpr (BF16) {
 #pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    const int n = 2 * s + half;
-    bfrag[s] = (pix_ok && n < Cp) ? pix_b[(size_t)n * M + m] : 0.0f;
+    for (int t = 0; t < NS / 8; ++t) {
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int n = 16 * t + 8 * half + j;
+        f[j] = (pix_ok && n < Cp) ? pix_b[(size_t)n * M + m] : 0.0f;
+      }
+      bfrag16[t] = pack_bf16x8(f);
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int n = 2 * s + half;
+      bfrag[s] = (pix_ok && n < Cp) ? pix_b[(size_t)n * M + m] : 0.0f;
+    }
   }
   for (int e = tid; e < kCC * rg.RSp; e += kStThreads) region[e] = 0.0f;
   __syncthreads();
@@ -285,13 +314,27 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
       for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
       const float4* wp = reinterpret_cast<const float4*>(
                              Ws + ((size_t)k * chunks + chunk) * NS * 64) + half * 32 + (lane & 31);
+      if constexpr (BF16) {
+        // per fragment t: 64 lanes x 8 floats = 128 float4; this lane's pair starts at
+        // (half * 32 + lane % 32) * 2
+        const float4* wb = reinterpret_cast<const float4*>(
+                               Ws + ((size_t)k * chunks + chunk) * NS * 64) +
+                           (half * 32 + (lane & 31)) * 2;
 #pragma unroll
-      for (int g = 0; g < NS / 4; ++g) {
-        const float4 a = wp[g * 64];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bfrag[4 * g + 0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bfrag[4 * g + 1], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bfrag[4 * g + 2], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc, 0, 0, 0);
+        for (int t = 0; t < NS / 8; ++t) {
+          const float4 lo = wb[t * 128], hi = wb[t * 128 + 1];
+          const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+          acc = mfma_bf16(pack_bf16x8(f), bfrag16[t], acc);
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < NS / 4; ++g) {
+          const float4 a = wp[g * 64];
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bfrag[4 * g + 0], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bfrag[4 * g + 1], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bfrag[4 * g + 2], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc, 0, 0, 0);
+        }
       }
       // splat: accumulator register v of this lane is channel c0 + row(v), pixel m
       auto splat = [&](int e, float co) {
@@ -402,8 +445,9 @@ int staged_gather_gemm(const ConvGeom& g, const float* img, const float* map, co
   return SDK_OK;
 }
 
-int staged_gemm_scatter(const ConvGeom& g, const float* pix, const float* map, const float* wts,
-                        const float* Wm, float* img, float* workspace, hipStream_t stream) {
+int staged_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
+                        const float* wts, const float* Wm, float* img, float* workspace,
+                        hipStream_t stream) {
   const PixelTiling pt = make_tiling(g);
   const int NS = g.Cp > 64 ? 64 : (g.Cp > 32 ? 32 : 16);   // MFMA steps: 2 channels each
   const int chunks = (int)ceil_div(g.Cg, kCC);
@@ -411,16 +455,17 @@ int staged_gemm_scatter(const ConvGeom& g, const float* pix, const float* map, c
     const size_t total = (size_t)g.K * chunks * NS * 64;
     const int blocks = (int)std::min<size_t>((total + kStThreads - 1) / kStThreads, 2048);
     launch(permute_weight_scatter_kernel, dim3(blocks), dim3(kStThreads), stream, Wm, workspace,
-           g.Cp, g.Cg, g.K, chunks, NS);
+           g.Cp, g.Cg, g.K, chunks, NS, bf16 ? 1 : 0);
     SDK_LAUNCH_CHECK("permute_weight_scatter");
   }
   const dim3 grid((unsigned)(pt.tiles_x * pt.tiles_y), (unsigned)g.B);
-#define SS(NSv)                                                                                  \
+#define SS(NSv, BFv)                                                                                  \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                             \
-                      (launch(staged_gemm_scatter_kernel<INTERP, WEIGHTED, NSv>, grid,           \
+                      (launch(staged_gemm_scatter_kernel<INTERP, WEIGHTED, NSv, BFv>, grid,      \
                               dim3(kStThreads), stream, pix, map, wts, (const float*)workspace,  \
                               img, g.Cg, g.H, g.W, g.Cp, g.K, g.P, chunks, pt)))
-  if (NS == 64) SS(64); else if (NS == 32) SS(32); else SS(16);
+  if (bf16) { if (NS == 64) SS(64, true); else if (NS == 32) SS(32, true); else SS(16, true); }
+  else { if (NS == 64) SS(64, false); else if (NS == 32) SS(32, false); else SS(16, false); }
 #undef SS
   SDK_LAUNCH_CHECK("staged_gemm_scatter");
   return SDK_OK;

@@ -241,6 +241,44 @@ def test_fused_conv_tile_edges(ops, oracle, tc):
     assert relerr(_n(gb), wb) <= 1e-4
 
 
+@pytest.fixture
+def bf16_compute(ops):
+    ops.set_conv_compute("bf16")
+    yield
+    ops.set_conv_compute("native")
+
+
+@pytest.mark.parametrize("tc", TILE_CASES[:4], ids=lambda t: "x".join(map(str, t)))
+def test_bf16_compute_within_1e_2(ops, oracle, bf16_compute, tc):
+    """bf16 operands with fp32 accumulation in the MFMA contraction: every output within
+    1e-2 (norm-relative) of the float32 CPU result."""
+    Cin, Cout, H, W, OH, OW, K, P, interp = tc
+    dt = np.float32
+    rng = np.random.default_rng(7 + sum(tc))
+    B = 2
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if P else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if P else None
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), K, interp))
+    want = oracle.mapped_conv_forward(x, m, wt, b, K, interp, iw)
+    assert 1e-6 < relerr(got, want) <= 1e-2      # really bf16, and inside the tolerance
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-2
+    assert relerr(_n(gw), ww) <= 1e-2
+    assert relerr(_n(gb), wb) <= 1e-4
+    xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+    bt = rng.standard_normal(Cin).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), _t(iw), _t(wtt), _t(bt), H, W, K,
+                                                interp))
+    assert relerr(got, oracle.mapped_transposed_conv_forward(xt, m, wtt, bt, H, W, K, interp,
+                                                             iw)) <= 1e-2
+
+
 # ------------------------------------------------------------------------------------------
 # Against the compiled reference's fixtures directly (no oracle in between).
 # ------------------------------------------------------------------------------------------
