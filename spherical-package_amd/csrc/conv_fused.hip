@@ -21,6 +21,7 @@
 //   A operand: A[i = l % 32][k = l / 32]        B operand: B[k = l / 32][j = l % 32]
 //   D, 16 registers v: D[i = 8*(v/4) + 4*(l/32) + v%4][j = l % 32]
 #include "conv_fused.hpp"
+#include "conv_plan.hpp"
 
 #include <hip/hip_runtime.h>
 
@@ -499,7 +500,9 @@ bool fused_supported(const ConvGeom& g) {
 
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
-  return std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
+  size_t need = std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
+  if (plan_supported(g)) need = std::max(need, plan_bytes(g));
+  return need;
 }
 
 static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
@@ -584,11 +587,18 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
 }
 
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
-                       const float* wts, const float* img, float* gW, hipStream_t stream) {
+                       const float* wts, const float* img, float* gW, float* workspace,
+                       hipStream_t stream) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
+  if (planned_wgrad_supported(g)) {
+    Plan plan;
+    rc = build_plan(g, map, wts, workspace, stream, &plan);
+    if (rc) return rc;
+    return planned_wgrad(g, bf16, plan, pix, img, gW, stream);
+  }
   constexpr int KM = 64;
   const int slots = slots_for(g);
   const int c_tiles = (int)ceil_div(g.Cg, 128), n_tiles = (int)ceil_div(g.Cp, 128);

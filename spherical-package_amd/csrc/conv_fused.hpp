@@ -19,7 +19,8 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                        const float* wts, const float* Wm, const float* bias, float* img,
                        float* workspace, hipStream_t stream);
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
-                       const float* wts, const float* img, float* gW, hipStream_t stream);
+                       const float* wts, const float* img, float* gW, float* workspace,
+                       hipStream_t stream);
 
 // LDS-staged kernels (conv_staged.hip): the tile's image window lives in LDS.
 bool staged_supported(const ConvGeom& g);

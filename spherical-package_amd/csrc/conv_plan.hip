@@ -1,0 +1,508 @@
+// Tap plan construction and the plan-driven weight-gradient kernel (gfx950,
+// float32 tensors).  Layout of a plan: conv_plan.hpp.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "conv_plan.hpp"
+#include "sdk_host.hpp"
+#include "sdk_mfma.hpp"
+
+namespace sdk {
+
+constexpr int kPlThreads = 256;
+
+// ---------------------------------------------------------------------------
+// Plan construction: one workgroup per tile.  Thread = (pixel of the tile,
+// parity of the kernel sample).  Pass 1 finds the bounding box of all active
+// taps and the per-sample row counts, pass 2 writes the encoded rows.
+// ---------------------------------------------------------------------------
+template <int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kPlThreads) void plan_kernel(
+    const float* __restrict__ map, const float* __restrict__ wts, PixelTiling pt, int K, int P,
+    int H, int W, int S, int* __restrict__ hdr, int* __restrict__ ns_out,
+    int2* __restrict__ taps) {
+  __shared__ int bb[4];
+  __shared__ int ns_l[kPlanKMax];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int tile = blockIdx.x;
+  const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
+  const int p = tid & 127, kpar = tid >> 7;
+  const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
+  const bool pix_ok = oy < pt.OH && ox < pt.OW;
+  const int q = WEIGHTED ? P : 1;
+  constexpr int NT = Taps2D<INTERP>::N;
+
+  // anchor: centre-ish sample of the tile's first pixel (same value in every thread)
+  const size_t s0 = (((size_t)ty0 * pt.OW + tx0) * K + K / 2) * q;
+  const int ax = wrap_index(to_int_clamped(round_t(map[s0 * 2])), W);
+  const int ay = min(max(to_int_clamped(round_t(map[s0 * 2 + 1])), 0), H - 1);
+
+  for (int k = tid; k < K; k += kPlThreads) ns_l[k] = 0;
+  if (tid == 0) {
+    bb[0] = INT_MAX;
+    bb[1] = INT_MIN;
+    bb[2] = INT_MAX;
+    bb[3] = INT_MIN;
+  }
+  __syncthreads();
+
+  const size_t base = ((size_t)oy * pt.OW + ox) * K;
+  Taps2D<INTERP> t;
+  int dy0 = INT_MAX, dy1 = INT_MIN, dx0 = INT_MAX, dx1 = INT_MIN;
+  for (int k = kpar; k < K; k += 2) {
+    int cnt = 0;
+    if (pix_ok) {
+      for (int pp = 0; pp < q; ++pp) {
+        const size_t s = (base + k) * q + pp;
+        t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+          if (t.w[i] != 0.0f) {
+            const int dy = t.y[i] - ay;
+            int dx = t.x[i] - ax;
+            dx += (dx > W / 2) ? -W : ((dx < -(W / 2)) ? W : 0);
+            dy0 = min(dy0, dy);
+            dy1 = max(dy1, dy);
+            dx0 = min(dx0, dx);
+            dx1 = max(dx1, dx);
+            ++cnt;
+          }
+        }
+      }
+    }
+    cnt = wave_max(cnt);
+    if (lane == 0) atomicMax(&ns_l[k], cnt);
+  }
+  dy0 = wave_min(dy0);
+  dy1 = wave_max(dy1);
+  dx0 = wave_min(dx0);
+  dx1 = wave_max(dx1);
+  if (lane == 0) {
+    atomicMin(&bb[0], dy0);
+    atomicMax(&bb[1], dy1);
+    atomicMin(&bb[2], dx0);
+    atomicMax(&bb[3], dx1);
+  }
+  __syncthreads();
+  const Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, pt.TY(), pt.TX(), W);
+  if (tid == 0) {
+    hdr[tile * 8 + 0] = rg.ry0;
+    hdr[tile * 8 + 1] = rg.rx0;
+    hdr[tile * 8 + 2] = rg.RH;
+    hdr[tile * 8 + 3] = rg.RW;
+  }
+  for (int k = tid; k < K; k += kPlThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
+
+  for (int k = kpar; k < K; k += 2) {
+    const int n = ns_l[k];
+    int2* row = taps + ((size_t)tile * K + k) * S * 128 + p;
+    int cnt = 0;
+    if (pix_ok) {
+      for (int pp = 0; pp < q; ++pp) {
+        const size_t s = (base + k) * q + pp;
+        t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+          if (t.w[i] != 0.0f) {
+            row[(size_t)cnt * 128] = make_int2(rg.encode(t.y[i], t.x[i], W), __float_as_int(t.w[i]));
+            ++cnt;
+          }
+        }
+      }
+    }
+    for (; cnt < n; ++cnt) row[(size_t)cnt * 128] = make_int2(0, 0);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// planned_wgrad:  gW[n][c][k] += sum_{b, m} pix[b][n][m] * col[b][(c, k)][m]
+//
+// Workgroup (256 threads, 4 waves): one chunk of 32 image channels c, one tile
+// of 128 pixel-side channels n (wave w owns rows 32w .. 32w+31), one block of
+// KB kernel samples, one batch element and a run of consecutive pixel tiles.
+// One 32 x 32 accumulator per kernel sample stays in registers over the whole
+// run and is added to gW once at the end.
+//
+// Per pixel tile the 32 channels of the tile's image window are staged in LDS
+// with coalesced loads.  The tile is processed in two halves of 64 pixels.  Per
+// half all global reads are issued together: each lane's A fragments (pix values
+// of its row n for the 64 pixels) and the half's plan rows, which go to LDS.
+// Then, per kernel sample, every lane gathers the column values of one pixel and
+// 8 channels from the LDS window (plan row -> ds_read + fma), the 32 x 64 column
+// tile is exchanged through LDS and each wave multiplies it with its A
+// fragments.  No global read sits between two samples.
+//
+// Contraction order inside a half (m = pixel 0..63 of the half), fp32
+// v_mfma_f32_32x32x2_f32: step 4g+i of lane half h contracts m = 8g + 4h + i, so
+// a lane reads its A values and its column values as 16-byte vectors.  bf16
+// v_mfma_f32_32x32x16_bf16: instruction t contracts m = 16t + 8h + 0..7.
+// ---------------------------------------------------------------------------
+constexpr int kColLd = 68;            // column tile row stride (floats): 16-byte rows, 4-bank skew
+constexpr int kRegionLd = kRegionCap + 16;  // largest window stride, see region_stride()
+constexpr int kRowCap = 36;           // plan rows of one half held in LDS at a time
+
+// Window stride: a multiple of 32 plus 16, so the two channel groups a half-wave
+// reads in one ds_read (channels 4j and 4j+1) fall on disjoint bank halves.
+__device__ __forceinline__ int region_stride(int RS) { return ((RS + 31) & ~31) + 16; }
+
+template <int KB, bool BF16>
+__global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
+    const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
+    const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW, int Cg,
+    int H, int W, int Cp, int K, int S, PixelTiling pt, int tiles,
+    int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
+  __shared__ __align__(16) float region[kCC * kRegionLd];
+  __shared__ __align__(16) float colT[2][kCC * kColLd];
+  __shared__ __align__(16) int2 prow[kRowCap * 64];
+  __shared__ int src[kRegionCap];
+  __shared__ int ns_l[KB];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // 1-D grid; workgroup ids go round-robin over the 8 XCDs.  All workgroups of one
+  // tile run (every batch element, channel chunk and sample block) read the same
+  // plan rows, and those of one batch element the same pix tiles; they are given
+  // consecutive slots of one XCD, so they meet in its L2.
+  const int kinds = c_chunks * n_tiles * kblocks * batches;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int kind = slot % kinds, group = (slot / kinds) * 8 + xcd;
+  if (group >= groups) return;
+  const int kb = kind % kblocks, nt = (kind / kblocks) % n_tiles;
+  const int cc = (kind / (kblocks * n_tiles)) % c_chunks;
+  const int batch = kind / (kblocks * n_tiles * c_chunks);
+  const int k0 = kb * KB, kcount = min(KB, K - k0);
+  const int c0 = cc * kCC, n0 = nt * 128;
+  const int M = pt.OH * pt.OW;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + ((size_t)batch * Cg) * HW;
+  const float* pix_b = pix + ((size_t)batch * Cp) * M;
+
+  // roles: gather (pixel px16 of the wave's 16, channel group cg), MFMA (row/column nl, half h)
+  const int px16 = lane & 15, cg = lane >> 4;
+  const int m_local = wave * 16 + px16;
+  const int nl = lane & 31, h = lane >> 5;
+  const int n_row = n0 + 32 * wave + nl;
+  const bool n_ok = n_row < Cp;
+  const float* pix_row = pix_b + (size_t)(n_ok ? n_row : 0) * M;
+
+  floatx16 acc[KB];
+#pragma unroll
+  for (int i = 0; i < KB; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
+
+  // Tiles are dealt round-robin to the tile runs: costly tiles (taps outside the window,
+  // e.g. polar rows of a spherical map) are spread over all workgroups.
+  int buf = 0;
+  for (int tile = group; tile < tiles; tile += groups) {
+    const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
+    // pixel index (inside the image of the pixel side) of tile-local pixel p, or -1
+    auto pixel_index = [&](int p) -> int {
+      const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
+      return (oy < pt.OH && ox < pt.OW) ? oy * pt.OW + ox : -1;
+    };
+    Region rg;
+    rg.ry0 = hdr[tile * 8 + 0];
+    rg.rx0 = hdr[tile * 8 + 1];
+    rg.RH = hdr[tile * 8 + 2];
+    rg.RW = hdr[tile * 8 + 3];
+    rg.RS = rg.RH * rg.RW;
+    rg.RSp = region_stride(rg.RS);
+    // plan rows of this tile and sample block: uniform base, 32-bit lane offsets
+    const char* tile_taps = reinterpret_cast<const char*>(taps + ((size_t)tile * K + k0) * S * 128);
+
+    __syncthreads();  // every wave is done with the previous tile's window, rows and column tiles
+    if (tid < kcount) ns_l[tid] = ns[(size_t)tile * K + k0 + tid];
+    build_region_lut(rg, H, W, src);
+    __syncthreads();
+    {
+      // wave w stages channels 8w .. 8w+7; a lane owns window elements lane, lane+64, ...
+      // (at most 5 of them) and has all its loads in flight before the first LDS write
+      constexpr int PER_WAVE = kCC / 4, ITER = (kRegionCap + 63) / 64;
+      const char* cbase = reinterpret_cast<const char*>(
+          img_b + (size_t)min(c0 + wave * PER_WAVE, Cg - 1) * HW);
+      const unsigned plane = (unsigned)HW * 4u;
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j) {
+        const bool c_ok = c0 + wave * PER_WAVE + j < Cg;
+        float v[ITER];
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+          const int e = lane + 64 * it;
+          const int o = e < rg.RS ? src[e] : -1;
+          const bool ok = o >= 0 && c_ok;
+          const float d = *reinterpret_cast<const float*>(
+              cbase + (ok ? (unsigned)j * plane + (unsigned)o * 4u : 0u));
+          v[it] = ok ? d : 0.0f;
+        }
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+          const int e = lane + 64 * it;
+          if (e < rg.RS) region[(wave * PER_WAVE + j) * rg.RSp + e] = v[it];
+        }
+      }
+    }
+    // (the window becomes visible with the barrier that follows the first row staging)
+
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+      // ---- A fragments of this lane's row n for the 64 pixels of the half
+      float afrag[BF16 ? 1 : 32];
+      Bf16Frag afrag16[BF16 ? 4 : 1];
+      {
+        constexpr int GROUPS = BF16 ? 4 : 8;   // groups of 8 consecutive pixels per lane half ...
+        constexpr int RUN = BF16 ? 8 : 4;      // ... of which this lane holds RUN
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+          const int p0 = half * 64 + (BF16 ? 16 * g + 8 * h : 8 * g + 4 * h);
+          float f[RUN];
+          if (vec4) {
+            const int m0 = pixel_index(p0);
+#pragma unroll
+            for (int u = 0; u < RUN / 4; ++u) {
+              float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+              if (n_ok && m0 >= 0) x = *reinterpret_cast<const float4*>(pix_row + m0 + 4 * u);
+              f[4 * u + 0] = x.x;
+              f[4 * u + 1] = x.y;
+              f[4 * u + 2] = x.z;
+              f[4 * u + 3] = x.w;
+            }
+          } else {
+#pragma unroll
+            for (int u = 0; u < RUN; ++u) {
+              const int mi = pixel_index(p0 + u);
+              f[u] = (n_ok && mi >= 0) ? pix_row[mi] : 0.0f;
+            }
+          }
+          if constexpr (BF16) {
+            afrag16[g] = pack_bf16x8(reinterpret_cast<const float(&)[8]>(f));
+          } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) afrag[4 * g + u] = f[u];
+          }
+        }
+      }
+
+      // Samples are taken in runs whose plan rows fit the LDS row buffer.
+      int kk_beg = 0;
+      while (kk_beg < kcount) {
+        int kk_end = kk_beg, rows = 0;
+        while (kk_end < kcount && rows + ns_l[kk_end] <= kRowCap) rows += ns_l[kk_end++];
+        // (ns <= S <= kRowCap is a launch condition, so every run holds at least one sample)
+        // ---- stage the rows of samples kk_beg .. kk_end-1 for the 64 pixels of the half
+        {
+          int kk = kk_beg, r0 = 0;   // row r of the run belongs to sample kk, its row r - r0
+          for (int i = tid; i < rows * 64; i += kPlThreads) {
+            const int r = i >> 6, p = i & 63;
+            while (r - r0 >= ns_l[kk]) r0 += ns_l[kk++];
+            const char* row = tile_taps + (size_t)(kk * S + (r - r0)) * (128 * sizeof(int2));
+            prow[i] = *reinterpret_cast<const int2*>(row + (unsigned)(half * 64 + p) * (unsigned)sizeof(int2));
+          }
+        }
+        __syncthreads();
+
+        int row0 = 0;
+#pragma unroll 1
+        for (int kk = kk_beg; kk < kk_end; ++kk) {
+          const int nrows = ns_l[kk];
+          // ---- gather: column values of pixel m_local, channels 4j + cg
+          float col[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) col[j] = 0.0f;
+          // adds one row (window index or image offset e, coefficient co) to col[]
+          auto tap_any = [&](int e, float co) {
+            // some lane's tap lies outside the window: that lane reads the image directly
+            // (uniform base, 32-bit byte offsets; 32 planes of < 2^24 elements fit)
+            const bool out = e < 0 && co != 0.0f;
+            const float* rp = region + cg * rg.RSp + (e >= 0 ? e : 0);
+            const char* gbase = reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
+            const unsigned plane = (unsigned)HW * 4u;
+            const unsigned o0 = out ? (unsigned)cg * plane + (unsigned)(-e - 1) * 4u : 0u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const bool g_ok = out && c0 + 4 * j + cg < Cg;
+              const float dg =
+                  *reinterpret_cast<const float*>(gbase + (g_ok ? o0 + 4u * j * plane : 0u));
+              const float dl = rp[4 * j * rg.RSp];
+              col[j] += co * (e >= 0 ? dl : (g_ok ? dg : 0.0f));
+            }
+          };
+          for (int r = 0; r < nrows; r += 2) {
+            // two rows per step so that their LDS reads overlap
+            const int2 ec0 = prow[(row0 + r) * 64 + m_local];
+            const int2 ec1 = (r + 1 < nrows) ? prow[(row0 + r + 1) * 64 + m_local] : make_int2(0, 0);
+            const float co0 = __int_as_float(ec0.y), co1 = __int_as_float(ec1.y);
+            if (__all((ec0.x >= 0 || co0 == 0.0f) && (ec1.x >= 0 || co1 == 0.0f))) {
+              const float* rp0 = region + cg * rg.RSp + (ec0.x >= 0 ? ec0.x : 0);
+              const float* rp1 = region + cg * rg.RSp + (ec1.x >= 0 ? ec1.x : 0);
+              float d0[8], d1[8];
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                d0[j] = rp0[4 * j * rg.RSp];
+                d1[j] = rp1[4 * j * rg.RSp];
+              }
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                col[j] += co0 * d0[j];
+                col[j] += co1 * d1[j];
+              }
+            } else {
+              tap_any(ec0.x, co0);
+              tap_any(ec1.x, co1);
+            }
+          }
+          row0 += nrows;
+          float* ct = colT[buf];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ct[(4 * j + cg) * kColLd + m_local] = col[j];
+          __syncthreads();
+
+          // ---- D[n][c] += A[n][m] * col[c][m]; one copy of this block per accumulator
+          const float* bt = ct + nl * kColLd;
+          auto mma = [&](floatx16& d) {
+            if constexpr (BF16) {
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const float4 lo = *reinterpret_cast<const float4*>(bt + 16 * t + 8 * h);
+                const float4 hi = *reinterpret_cast<const float4*>(bt + 16 * t + 8 * h + 4);
+                const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
+              }
+            } else {
+              float4 b = *reinterpret_cast<const float4*>(bt + 4 * h);
+#pragma unroll
+              for (int g = 0; g < 8; ++g) {
+                float4 bn = b;
+                if (g < 7) bn = *reinterpret_cast<const float4*>(bt + 8 * (g + 1) + 4 * h);
+                d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 0], b.x, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 1], b.y, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 2], b.z, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 3], b.w, d, 0, 0, 0);
+                b = bn;
+              }
+            }
+          };
+#pragma unroll
+          for (int u = 0; u < KB; ++u)
+            if (u == kk) mma(acc[u]);
+          buf ^= 1;
+        }
+        kk_beg = kk_end;
+      }
+    }
+  }
+
+  // ---- gW[n][c*K + k] += D[n][c]; accumulator register v: row 8*(v/4) + 4*h + v%4, column nl
+  const int c = c0 + nl;
+  if (c < Cg) {
+#pragma unroll
+    for (int kk = 0; kk < KB; ++kk) {
+      if (kk < kcount) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int n = n0 + 32 * wave + 8 * (v >> 2) + 4 * h + (v & 3);
+          if (n < Cp)
+            atomic_add_noret(gW + (size_t)n * Cg * K + (size_t)c * K + k0 + kk, acc[kk][v]);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side.
+// ---------------------------------------------------------------------------
+PixelTiling plan_tiling(int OH, int OW) {
+  PixelTiling pt;
+  pt.OH = OH;
+  pt.OW = OW;
+  pt.tx_shift = (OH >= 8) ? 4 : (OH >= 4 ? 5 : (OH >= 2 ? 6 : 7));
+  // narrow grids: no wider than the grid needs
+  while (pt.tx_shift > 0 && (1 << (pt.tx_shift - 1)) >= OW) --pt.tx_shift;
+  pt.tiles_x = (int)ceil_div(OW, pt.TX());
+  pt.tiles_y = (int)ceil_div(OH, pt.TY());
+  return pt;
+}
+
+static int plan_slots(const ConvGeom& g) {
+  return pts(g.P) * ((g.interp == 1 || g.interp == 2) ? 4 : 1);
+}
+
+bool plan_supported(const ConvGeom& g) {
+  if (g.OW < 1 || g.M % g.OW != 0 || g.K > kPlanKMax) return false;
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  const int64_t tiles = (int64_t)pt.tiles_x * pt.tiles_y;
+  return tiles * g.K * plan_slots(g) * 128 < ((int64_t)1 << 40) && tiles * 8 < ((int64_t)1 << 31);
+}
+
+static size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
+
+size_t plan_bytes(const ConvGeom& g) {
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
+  return align16(tiles * 8 * sizeof(int)) + align16(tiles * g.K * sizeof(int)) +
+         tiles * g.K * plan_slots(g) * 128 * sizeof(int2);
+}
+
+int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+               hipStream_t stream, Plan* plan) {
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
+  const int S = plan_slots(g);
+  char* base = static_cast<char*>(workspace);
+  int* hdr = reinterpret_cast<int*>(base);
+  int* ns = reinterpret_cast<int*>(base + align16(tiles * 8 * sizeof(int)));
+  int2* taps = reinterpret_cast<int2*>(base + align16(tiles * 8 * sizeof(int)) +
+                                       align16(tiles * g.K * sizeof(int)));
+  SDK_DISPATCH_INTERP(g.interp, g.P,
+                      (launch(plan_kernel<INTERP, WEIGHTED>, dim3((unsigned)tiles),
+                              dim3(kPlThreads), stream, map, wts, pt, g.K, g.P, g.H, g.W, S, hdr,
+                              ns, taps)));
+  SDK_LAUNCH_CHECK("plan");
+  plan->pt = pt;
+  plan->tiles = (int)tiles;
+  plan->S = S;
+  plan->hdr = hdr;
+  plan->ns = ns;
+  plan->taps = taps;
+  return SDK_OK;
+}
+
+bool planned_wgrad_supported(const ConvGeom& g) {
+  return plan_supported(g) && plan_slots(g) <= kRowCap && g.B <= 65535;
+}
+
+int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* pix,
+                  const float* img, float* gW, hipStream_t stream) {
+  const int kblocks = (int)ceil_div(g.K, 9);
+  const int per = (int)ceil_div(g.K, kblocks);
+  const int KB = per <= 1 ? 1 : (per <= 4 ? 4 : (per <= 7 ? 7 : 9));
+  const int kb_count = (int)ceil_div(g.K, KB);
+  const int c_chunks = (int)ceil_div(g.Cg, kCC), n_tiles = (int)ceil_div(g.Cp, 128);
+  const int64_t kinds = (int64_t)c_chunks * n_tiles * kb_count * g.B;
+  // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall
+  int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, kinds), 8) * 8);
+  int groups = (int)std::min<int64_t>(plan.tiles, want);
+  const int tpg = (int)ceil_div(plan.tiles, groups);
+  groups = (int)ceil_div(plan.tiles, tpg);
+  const int64_t slots = ceil_div(groups, 8) * 8 * kinds;
+  if (slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "planned_wgrad: grid too large");
+  const int TX = plan.pt.TX();
+  const int vec4 = (g.OW % 4 == 0 && TX >= (bf16 ? 8 : 4) &&
+                    reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
+  const dim3 grid((unsigned)slots);
+#define PW(KBv, BFv)                                                                            \
+  launch(planned_wgrad_kernel<KBv, BFv>, grid, dim3(kPlThreads), stream, pix, img, plan.hdr,    \
+         plan.ns, plan.taps, gW, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, plan.tiles,        \
+         groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4)
+  if (bf16) {
+    if (KB == 1) PW(1, true); else if (KB == 4) PW(4, true); else if (KB == 7) PW(7, true); else PW(9, true);
+  } else {
+    if (KB == 1) PW(1, false); else if (KB == 4) PW(4, false); else if (KB == 7) PW(7, false); else PW(9, false);
+  }
+#undef PW
+  SDK_LAUNCH_CHECK("planned_wgrad");
+  return SDK_OK;
+}
+
+}  // namespace sdk

@@ -1,0 +1,47 @@
+// Tap plan: the sample map of one convolution call, resolved once per call into
+// per-tile lists of (window index, coefficient) pairs that every batch element
+// and channel chunk reuses.
+//
+// The pixel grid is cut into 2-D tiles of 128 pixels (PixelTiling).  For tile t:
+//   hdr[8*t + 0..3]  window of the image the tile's taps fall into: first row,
+//                    first column, rows, columns (columns wrap modulo W)
+//   ns[t*K + k]      rows of kernel sample k: the largest number of active taps
+//                    any pixel of the tile has for that sample
+//   taps[((t*K + k)*S + r)*128 + p]   row r < ns of pixel p (tile-local index):
+//                    .x >= 0: element index inside the window (row * columns + column)
+//                    .x <  0: -(flat offset inside the image plane) - 1 (outside the window)
+//                    .y: float bits of the coefficient (interpolation weight times
+//                    point weight); pixels with fewer taps are padded with 0.
+// S = points per sample * taps per point bounds the rows of one sample.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "conv_internal.hpp"
+#include "conv_staged.hpp"
+
+namespace sdk {
+
+constexpr int kPlanKMax = 256;  // kernel samples a plan can hold
+
+struct Plan {
+  PixelTiling pt;
+  int tiles, S;
+  const int* hdr;
+  const int* ns;
+  const int2* taps;
+};
+
+PixelTiling plan_tiling(int OH, int OW);
+bool plan_supported(const ConvGeom& g);
+size_t plan_bytes(const ConvGeom& g);
+
+// Builds the plan of (g, map, wts) in `workspace` (plan_bytes(g) bytes, 16-byte aligned).
+int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+               hipStream_t stream, Plan* plan);
+
+// gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
+bool planned_wgrad_supported(const ConvGeom& g);
+int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* pix,
+                  const float* img, float* gW, hipStream_t stream);
+
+}  // namespace sdk

@@ -107,6 +107,41 @@ struct PixelTiling {
   __host__ __device__ int TY() const { return 128 >> tx_shift; }
 };
 
+// Turns the bounding box [dy0, dy1] x [dx0, dx1] of a tile's taps (relative to the
+// anchor (ay, ax), columns unwrapped) into the staged window: the whole box when it
+// fits the capacity, otherwise a window around the tile; what falls outside is
+// served from global memory.
+__device__ __forceinline__ Region choose_region(int dy0, int dy1, int dx0, int dx1, int ay, int ax,
+                                                int TY, int TX, int W) {
+  Region r;
+  if (dy0 > dy1) {  // no active tap at all
+    r.ry0 = ay;
+    r.rx0 = ax;
+    r.RH = 1;
+    r.RW = 1;
+  } else {
+    int RH = dy1 - dy0 + 1, RW = min(dx1 - dx0 + 1, W);
+    int ry0 = ay + dy0, rx0 = ax + dx0;
+    if (RH * RW > kRegionCap) {
+      const int RHc = min(RH, 16);
+      const int RWc = min(RW, kRegionCap / RHc);
+      const int cy = (RH <= 2 * RHc) ? ay + (dy0 + dy1) / 2 : ay + TY / 2;
+      const int cx = (RW <= 2 * RWc) ? ax + (dx0 + dx1) / 2 : ax + TX / 2;
+      ry0 = cy - RHc / 2;
+      rx0 = cx - RWc / 2;
+      RH = RHc;
+      RW = RWc;
+    }
+    r.ry0 = ry0;
+    r.rx0 = wrap_index(rx0, W);
+    r.RH = RH;
+    r.RW = RW;
+  }
+  r.RS = r.RH * r.RW;
+  r.RSp = r.RS | 1;
+  return r;
+}
+
 // Determines the region of this workgroup's tile: bounding box, relative to an
 // anchor near the tile, of every active tap of every sample (pass over all K
 // samples and points), clipped to the region capacity.  `bb` is 4 ints of LDS.
@@ -180,34 +215,7 @@ __device__ __forceinline__ Region find_region(const float* __restrict__ map,
   dy1 = bb[1];
   dx0 = bb[2];
   dx1 = bb[3];
-  Region r;
-  if (dy0 > dy1) {  // no active tap at all
-    r.ry0 = ay;
-    r.rx0 = ax;
-    r.RH = 1;
-    r.RW = 1;
-  } else {
-    int RH = dy1 - dy0 + 1, RW = min(dx1 - dx0 + 1, W);
-    int ry0 = ay + dy0, rx0 = ax + dx0;
-    if (RH * RW > kRegionCap) {
-      // keep a window around the tile; what falls outside is served from global memory
-      const int RHc = min(RH, 16);
-      const int RWc = min(RW, kRegionCap / RHc);
-      const int cy = (RH <= 2 * RHc) ? ay + (dy0 + dy1) / 2 : ay + pt.TY() / 2;
-      const int cx = (RW <= 2 * RWc) ? ax + (dx0 + dx1) / 2 : ax + pt.TX() / 2;
-      ry0 = cy - RHc / 2;
-      rx0 = cx - RWc / 2;
-      RH = RHc;
-      RW = RWc;
-    }
-    r.ry0 = ry0;
-    r.rx0 = wrap_index(rx0, W);
-    r.RH = RH;
-    r.RW = RW;
-  }
-  r.RS = r.RH * r.RW;
-  r.RSp = r.RS | 1;
-  return r;
+  return choose_region(dy0, dy1, dx0, dx1, ay, ax, pt.TY(), pt.TX(), W);
 }
 
 // Per-wave cache of encoded taps: for kernel sample k < kc, rows rs[k] .. rs[k+1]-1
