@@ -501,7 +501,7 @@ bool fused_supported(const ConvGeom& g) {
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
   size_t need = std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
-  if (plan_supported(g)) need = std::max(need, plan_bytes(g));
+  if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
   return need;
 }
 
@@ -562,8 +562,8 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
-  if (scatter_staged_supported(g))
-    return staged_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, stream);
+  if (planned_scatter_supported(g))
+    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, stream);
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;

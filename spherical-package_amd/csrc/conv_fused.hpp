@@ -22,16 +22,13 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
                        const float* wts, const float* img, float* gW, float* workspace,
                        hipStream_t stream);
 
-// LDS-staged kernels (conv_staged.hip): the tile's image window lives in LDS.
-bool staged_supported(const ConvGeom& g);
+// Bytes of the permuted weight copy the plan-driven scatter kernel reads.
 size_t staged_workspace_bytes(const ConvGeom& g);
-int staged_gather_gemm(const ConvGeom& g, const float* img, const float* map, const float* wts,
-                       const float* Wm, const float* bias, float* pix, float* workspace,
-                       hipStream_t stream);
 
-// img must be pre-filled (zeros or bias); needs Cp <= 128 (scatter_staged_supported).
-bool scatter_staged_supported(const ConvGeom& g);
-int staged_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map, const float* wts,
-                        const float* Wm, float* img, float* workspace, hipStream_t stream);
+// Plan-driven variant (conv_plan.hpp); workspace = permuted weights + plan.
+bool planned_scatter_supported(const ConvGeom& g);
+int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
+                         const float* wts, const float* Wm, float* img, float* workspace,
+                         hipStream_t stream);
 
 }  // namespace sdk

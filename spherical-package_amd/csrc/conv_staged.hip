@@ -1,16 +1,8 @@
-// LDS-staged fused convolution kernels for gfx950 (float32 tensors, fp32 MFMA).
+// Plan-driven MFMA -> scatter kernel for gfx950 (float32 tensors):
 //
-// gather_gemm:  pix[b][n, m] = sum_{c,k} Wm[n,(c,k)] * gather(img[b,c], tap(m,k)) + bias[n]
+//   img[b,c] += scatter_{tap(m,k)}( sum_n Wm[n,(c,k)] * pix[b][n,m] )
 //
-// A 256-thread workgroup owns a 2-D tile of 128 map pixels and NB*32 output
-// channels.  Each of its 4 wavefronts owns 32 of the pixels and all NB*32
-// channels (NB MFMA accumulators of 32 x 32).  Per chunk of kCC image channels
-// the tile's image window is staged in LDS (conv_staged.hpp); then, for every
-// kernel sample k, each lane turns its pixel's sample points into taps, gathers
-// the column values of its pixel from LDS straight into the MFMA B-operand
-// registers (lane l: pixel l%32, channel parity l/32) and multiplies with weight
-// fragments loaded as one 16-byte read per lane from a pre-permuted weight
-// copy.  No column tile and no barrier inside the k loop.
+// used for conv backward-input and transposed-conv forward.
 //
 // MFMA 32x32x2 f32 register layout (wave64, lane l):
 //   A operand: A[i = l % 32][k = l / 32]        B operand: B[k = l / 32][j = l % 32]
@@ -19,6 +11,7 @@
 
 #include "conv_fused.hpp"
 #include "conv_staged.hpp"
+#include "conv_plan.hpp"
 #include "sdk_host.hpp"
 #include "sdk_mfma.hpp"
 
@@ -38,183 +31,9 @@ __device__ __forceinline__ int st_xcd_band(int bid, int n) {
   return (bid % X) * per + bid / X;
 }
 
-// Weight copy for gather_gemm: Wp[k][c][nt][(n % 32) * NB + (n / 32) % NB] for
-// n-tiles of NB*32 channels, zero padded to CgP x (n_tiles * NB * 32).
-__global__ __launch_bounds__(kStThreads) void permute_weight_gather_kernel(
-    const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int CgP,
-    int n_tiles, int NB) {
-  const int TN = NB * 32;
-  const size_t total = (size_t)K * CgP * n_tiles * TN;
-  for (size_t e = (size_t)blockIdx.x * kStThreads + threadIdx.x; e < total;
-       e += (size_t)gridDim.x * kStThreads) {
-    const int inner = (int)(e % TN);
-    const int nt = (int)((e / TN) % n_tiles);
-    const int c = (int)((e / ((size_t)TN * n_tiles)) % CgP);
-    const int k = (int)(e / ((size_t)TN * n_tiles * CgP));
-    const int n = nt * TN + (inner % NB) * 32 + inner / NB;
-    out[e] = (n < Cp && c < Cg) ? Wm[(size_t)n * Cg * K + (size_t)c * K + k] : 0.0f;
-  }
-}
-
-// Stages channels [c0, c0 + kCC) of the tile's window: region[cl * RSp + e].
-__device__ __forceinline__ void load_region(const float* __restrict__ img_b, size_t HW, int Cg,
-                                            int c0, const Region& rg,
-                                            const int* __restrict__ src,
-                                            float* __restrict__ region) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  constexpr int PER_WAVE = kCC / 4;
-  for (int e = lane; e < rg.RS; e += 64) {
-    const int o = src[e];
-    float v[PER_WAVE];
-#pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) {
-      const int c = c0 + wave * PER_WAVE + j;
-      v[j] = (o >= 0 && c < Cg) ? img_b[(size_t)c * HW + o] : 0.0f;
-    }
-#pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) region[(wave * PER_WAVE + j) * rg.RSp + e] = v[j];
-  }
-}
-
-template <int INTERP, bool WEIGHTED, int NB>
-__global__ __launch_bounds__(kStThreads) void staged_gather_gemm_kernel(
-    const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
-    const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
-    int H, int W, int Cp, int K, int P, int CgP, int n_tiles, PixelTiling pt) {
-  __shared__ float region[kCC * (kRegionCap + 1)];
-  __shared__ int tc_e[4 * kTapRows * 32];
-  __shared__ float tc_co[4 * kTapRows * 32];
-  __shared__ int tc_rs[4 * (kTapKMax + 1)];
-  __shared__ int tc_ns[4 * kTapKMax];
-  __shared__ int src[kRegionCap];
-  __shared__ int bb[4];
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
-  const int tile = st_xcd_band(blockIdx.x, pt.tiles_x * pt.tiles_y * n_tiles);
-  const int nt = tile % n_tiles, ptile = tile / n_tiles;
-  const int ty0 = (ptile / pt.tiles_x) * pt.TY(), tx0 = (ptile % pt.tiles_x) << pt.tx_shift;
-  const int p_local = wave * 32 + (lane & 31);
-  const int oy = ty0 + (p_local >> pt.tx_shift), ox = tx0 + (p_local & (pt.TX() - 1));
-  const bool pix_ok = oy < pt.OH && ox < pt.OW;
-  const int m = oy * pt.OW + ox;
-  const int M = pt.OH * pt.OW;
-  const size_t HW = (size_t)H * W;
-  const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
-  const int q = WEIGHTED ? P : 1;
-  constexpr int TN = NB * 32;
-  constexpr int NT = Taps2D<INTERP>::N;
-
-  const Region rg = find_region<INTERP, WEIGHTED>(map, wts, pt, ty0, tx0, oy, ox, pix_ok, K, P, H,
-                                                  W, bb, tc_ns);
-  build_region_lut(rg, H, W, src);
-  const TapCache tc = build_tap_cache<INTERP, WEIGHTED>(map, wts, pt, oy, ox, pix_ok, K, P, H, W,
-                                                        rg, tc_ns, tc_e, tc_co, tc_rs);
-
-  floatx16 acc[NB];
-#pragma unroll
-  for (int i = 0; i < NB; ++i)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
-
-  for (int c0 = 0; c0 < CgP; c0 += kCC) {
-    __syncthreads();  // previous chunk's readers are done
-    load_region(img_b, HW, Cg, c0, rg, src, region);
-    __syncthreads();
-    // this lane's column rows inside the chunk: 2*step + half
-    const float* reg_half = region + half * rg.RSp;
-    for (int k = 0; k < K; ++k) {
-      float col[kCC / 2];
-#pragma unroll
-      for (int s = 0; s < kCC / 2; ++s) col[s] = 0.0f;
-      // adds one tap (encoded index e, coefficient co) of this lane's pixel to its column rows
-      auto gather = [&](int e, float co) {
-        if (__all(e >= 0 || co == 0.0f)) {
-          const int ee = e >= 0 ? e : 0;
-#pragma unroll
-          for (int s = 0; s < kCC / 2; ++s) col[s] += co * reg_half[2 * s * rg.RSp + ee];
-        } else {
-          // some lane's tap lies outside the staged window
-#pragma unroll
-          for (int s = 0; s < kCC / 2; ++s) {
-            float d;
-            if (e >= 0) {
-              d = reg_half[2 * s * rg.RSp + e];
-            } else {
-              const int c = c0 + 2 * s + half;
-              d = (co != 0.0f && c < Cg) ? img_b[(size_t)c * HW + (-e - 1)] : 0.0f;
-            }
-            col[s] += co * d;
-          }
-        }
-      };
-      if (k < tc.kc) {
-        const int r1 = tc.rs[k + 1];
-        for (int r = tc.rs[k]; r < r1; ++r)
-          gather(tc.e[r * 32 + (lane & 31)], tc.co[r * 32 + (lane & 31)]);
-      } else {
-        const size_t sbase = ((size_t)(pix_ok ? m : 0) * K + k) * q;
-        Taps2D<INTERP> t;
-        for (int p = 0; p < q; ++p) {
-          t.set(map[(sbase + p) * 2], map[(sbase + p) * 2 + 1], H, W,
-                WEIGHTED ? wts[sbase + p] : 1.0f);
-#pragma unroll
-          for (int i = 0; i < NT; ++i) {
-            const float co = pix_ok ? t.w[i] : 0.0f;
-            if (__any(co != 0.0f)) gather(rg.encode(t.y[i], t.x[i], W), co);
-          }
-        }
-      }
-      // weights: one 16-byte fragment per lane and step, rows c0 + 2*step + half
-      const float* wrow = Wp + (((size_t)k * CgP + c0 + half) * n_tiles + nt) * TN + (lane & 31) * NB;
-#pragma unroll
-      for (int s = 0; s < kCC / 2; ++s) {
-        float a[NB];
-        const float* wp = wrow + (size_t)(2 * s) * n_tiles * TN;
-        if constexpr (NB == 4) {
-          const float4 f = *reinterpret_cast<const float4*>(wp);
-          a[0] = f.x; a[1] = f.y; a[2] = f.z; a[3] = f.w;
-        } else if constexpr (NB == 2) {
-          const float2 f = *reinterpret_cast<const float2*>(wp);
-          a[0] = f.x; a[1] = f.y;
-        } else {
-          a[0] = *wp;
-        }
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], col[s], acc[i], 0, 0, 0);
-      }
-    }
-  }
-
-  // epilogue: + bias, store; lanes own consecutive pixels of the tile
-  if (pix_ok) {
-    float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int n = nt * TN + 32 * i + st_mfma_row(v, lane);
-        if (n < Cp) pix_b[(size_t)n * M + m] = acc[i][v] + (bias ? bias[n] : 0.0f);
-      }
-  }
-}
-
-// ---------------------------------------------------------------------------
-// gemm_scatter:  img[b,c] += scatter_{tap(m,k)}( sum_n Wm[n,(c,k)] * pix[b][n,m] )
-//
-// Same tile / wave / lane ownership as gather_gemm.  The pixel-side operand of
-// a lane's 32 pixels (all Cp <= 2*NS channels) stays in registers as MFMA B
-// fragments for the whole kernel.  For every chunk of kCC image channels and
-// every kernel sample k one 32 x 32 accumulator per wave receives
-// D[c][m] = sum_n W[n,(c,k)] pix[n,m]; each lane then splats its accumulator
-// rows through its pixel's taps into the LDS window (lds_add_f32; global
-// atomics only for taps outside the window).  After the K samples the window
-// is flushed to the image with one atomic per element and cleared.
-//
-// Weight copy Ws[k][chunk][g][half][c % 32][j]: value for n = 2*(4g + j) + half,
-// so a lane fetches the A fragments of four consecutive MFMA steps as 16 bytes.
-// ---------------------------------------------------------------------------
-// With bf16 != 0 the order is Ws[k][chunk][t][half][c % 32][j], n = 16*t + 8*half + j: the
+// Weight copy for the scatter kernel.  fp32: Ws[k][chunk][g][half][c % 32][j] holds the
+// value for n = 2*(4g + j) + half, so a lane fetches the A fragments of four consecutive
+// MFMA steps as 16 bytes.  bf16: Ws[k][chunk][t][half][c % 32][j], n = 16*t + 8*half + j: the
 // eight values a lane packs into one bf16 A fragment are 32 contiguous bytes.
 __global__ __launch_bounds__(kStThreads) void permute_weight_scatter_kernel(
     const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int chunks,
@@ -248,22 +67,35 @@ __global__ __launch_bounds__(kStThreads) void permute_weight_scatter_kernel(
   }
 }
 
-template <int INTERP, bool WEIGHTED, int NS, bool BF16>
-__global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
-    const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
-    const float* __restrict__ Ws, float* __restrict__ img, int Cg, int H, int W, int Cp, int K,
-    int P, int chunks, PixelTiling pt) {
-  __shared__ float region[kCC * (kRegionCap + 1)];
-  __shared__ int tc_e[4 * kTapRows * 32];
-  __shared__ float tc_co[4 * kTapRows * 32];
-  __shared__ int tc_rs[4 * (kTapKMax + 1)];
-  __shared__ int tc_ns[4 * kTapKMax];
+// ---------------------------------------------------------------------------
+// planned_gemm_scatter.  A 256-thread workgroup owns one 2-D tile of 128 map
+// pixels of one batch element; each of its 4 waves owns 32 of the pixels.  The
+// pixel-side operand of a lane's pixel (all Cp <= 2*NS channels) stays in
+// registers as MFMA B fragments for the whole kernel.  For every chunk of kCC
+// image channels and every kernel sample k one 32 x 32 accumulator per wave
+// receives D[c][m] = sum_n W[n,(c,k)] pix[n,m]; each lane then splats its
+// accumulator rows through the plan rows of its pixel (conv_plan.hpp) into the
+// tile's image window in LDS (64-bit compare-and-swap adds on channel pairs;
+// global atomics only for taps outside the window).  After the K samples the
+// window is flushed to the image with one atomic per element and cleared.
+// Window and rows come from the plan: no tap arithmetic here, and the rows of
+// sample k+1 and the first weight fragments of the next block are fetched while
+// sample k is processed.
+// ---------------------------------------------------------------------------
+template <int NS, bool BF16>
+__global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
+    const float* __restrict__ pix, const int* __restrict__ hdr, const int* __restrict__ ns,
+    const int2* __restrict__ taps, const float* __restrict__ Ws, float* __restrict__ img, int Cg,
+    int H, int W, int Cp, int K, int S, int chunks, PixelTiling pt) {
+  // window, channel pairs interleaved: value of (channel c, element e) at
+  // region[((c / 2) * RSp + e) * 2 + c % 2], so two channels share an 8-byte word
+  __shared__ __align__(8) float region[kCC * (kRegionCap + 1)];
   __shared__ int src[kRegionCap];
-  __shared__ int bb[4];
+  __shared__ int ns_l[kPlanKMax];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
-  const int ptile = st_xcd_band(blockIdx.x, pt.tiles_x * pt.tiles_y);
-  const int ty0 = (ptile / pt.tiles_x) * pt.TY(), tx0 = (ptile % pt.tiles_x) << pt.tx_shift;
+  const int tile = st_xcd_band(blockIdx.x, pt.tiles_x * pt.tiles_y);
+  const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
   const int p_local = wave * 32 + (lane & 31);
   const int oy = ty0 + (p_local >> pt.tx_shift), ox = tx0 + (p_local & (pt.TX() - 1));
   const bool pix_ok = oy < pt.OH && ox < pt.OW;
@@ -272,14 +104,22 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
   const size_t HW = (size_t)H * W;
   float* img_b = img + (size_t)blockIdx.y * Cg * HW;
   const float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
-  const int q = WEIGHTED ? P : 1;
-  constexpr int NT = Taps2D<INTERP>::N;
 
-  const Region rg = find_region<INTERP, WEIGHTED>(map, wts, pt, ty0, tx0, oy, ox, pix_ok, K, P, H,
-                                                  W, bb, tc_ns);
+  Region rg;
+  rg.ry0 = hdr[tile * 8 + 0];
+  rg.rx0 = hdr[tile * 8 + 1];
+  rg.RH = hdr[tile * 8 + 2];
+  rg.RW = hdr[tile * 8 + 3];
+  rg.RS = rg.RH * rg.RW;
+  rg.RSp = rg.RS | 1;
   build_region_lut(rg, H, W, src);
-  const TapCache tc = build_tap_cache<INTERP, WEIGHTED>(map, wts, pt, oy, ox, pix_ok, K, P, H, W,
-                                                        rg, tc_ns, tc_e, tc_co, tc_rs);
+  for (int k = tid; k < K; k += kStThreads) ns_l[k] = ns[(size_t)tile * K + k];
+  // plan rows of this tile: uniform base, 32-bit lane offsets
+  const char* tile_taps = reinterpret_cast<const char*>(taps + (size_t)tile * K * S * 128);
+  auto plan_row = [&](int k, int r) -> int2 {
+    const char* row = tile_taps + (size_t)(k * S + r) * (128 * sizeof(int2));
+    return *reinterpret_cast<const int2*>(row + (unsigned)p_local * (unsigned)sizeof(int2));
+  };
 
   // pixel-side operand, resident in registers.  fp32: step s holds channel 2*s + half;
   // bf16: fragment t holds channels 16*t + 8*half + 0..7, two per register.
@@ -306,49 +146,88 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
   for (int e = tid; e < kCC * rg.RSp; e += kStThreads) region[e] = 0.0f;
   __syncthreads();
 
+  // rows of the first sample
+  int2 cur[4];
+  int cur_n = ns_l[0];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) cur[r] = (r < cur_n) ? plan_row(0, r) : make_int2(0, 0);
+
+  // this lane's 16-byte weight fragments of block (k, chunk); fp32: fragment g at [g * 64],
+  // bf16: fragment pair t at [t * 128], [t * 128 + 1]
+  auto weight_block = [&](int k, int chunk) -> const float4* {
+    const float4* blk = reinterpret_cast<const float4*>(Ws + ((size_t)k * chunks + chunk) * NS * 64);
+    return blk + (BF16 ? (half * 32 + (lane & 31)) * 2 : half * 32 + (lane & 31));
+  };
+  constexpr int kPre = 4;
+  float4 wpre[kPre];
+  {
+    const float4* w0 = weight_block(0, 0);
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) wpre[i] = BF16 ? w0[(i >> 1) * 128 + (i & 1)] : w0[i * 64];
+  }
+
   for (int chunk = 0; chunk < chunks; ++chunk) {
     const int c0 = chunk * kCC;
     for (int k = 0; k < K; ++k) {
+      // ---- rows of the next sample (of the next chunk's first sample after the last one)
+      const int kn = (k + 1 < K) ? k + 1 : 0;
+      const int nxt_n = ns_l[kn];
+      int2 nxt[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) nxt[r] = (r < nxt_n) ? plan_row(kn, r) : make_int2(0, 0);
+
       floatx16 acc;
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-      const float4* wp = reinterpret_cast<const float4*>(
-                             Ws + ((size_t)k * chunks + chunk) * NS * 64) + half * 32 + (lane & 31);
+      // weights: 16-byte fragments; the first kPre of a block were fetched during the
+      // previous sample's splat, the rest arrive while the first MFMAs run
+      const float4* wblk = weight_block(k, chunk);
       if constexpr (BF16) {
-        // per fragment t: 64 lanes x 8 floats = 128 float4; this lane's pair starts at
-        // (half * 32 + lane % 32) * 2
-        const float4* wb = reinterpret_cast<const float4*>(
-                               Ws + ((size_t)k * chunks + chunk) * NS * 64) +
-                           (half * 32 + (lane & 31)) * 2;
+        float4 w[NS / 4];
+#pragma unroll
+        for (int i = 0; i < NS / 4; ++i) w[i] = (i < kPre) ? wpre[i] : wblk[(i >> 1) * 128 + (i & 1)];
 #pragma unroll
         for (int t = 0; t < NS / 8; ++t) {
-          const float4 lo = wb[t * 128], hi = wb[t * 128 + 1];
+          const float4 lo = w[2 * t], hi = w[2 * t + 1];
           const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
           acc = mfma_bf16(pack_bf16x8(f), bfrag16[t], acc);
         }
       } else {
 #pragma unroll
         for (int g = 0; g < NS / 4; ++g) {
-          const float4 a = wp[g * 64];
+          const float4 a = (g < kPre) ? wpre[g] : wblk[g * 64];
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bfrag[4 * g + 0], acc, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bfrag[4 * g + 1], acc, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bfrag[4 * g + 2], acc, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc, 0, 0, 0);
         }
       }
+      // first fragments of the next block (next sample, or first sample of the next chunk)
+      {
+        const int ck = (k + 1 < K) ? chunk : min(chunk + 1, chunks - 1);
+        const float4* wn = weight_block(kn, ck);
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) wpre[i] = BF16 ? wn[(i >> 1) * 128 + (i & 1)] : wn[i * 64];
+      }
       // splat: accumulator register v of this lane is channel c0 + row(v), pixel m
       auto splat = [&](int e, float co) {
         if (co != 0.0f) {
           if (e >= 0) {
-            float* dst = region + (4 * half) * rg.RSp + e;
-            int offs[16];
-            float vals[16];
+            // registers v = 4q + 2pr, +1 are channels 8q + 4*half + 2pr, +1: pair 4q + 2*half + pr
+            float2* dst = reinterpret_cast<float2*>(region) + (2 * half) * rg.RSp + e;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              offs[v] = (8 * (v >> 2) + (v & 3)) * rg.RSp;
-              vals[v] = co * acc[v];
+            for (int hv = 0; hv < 2; ++hv) {   // two batches of 4 pairs keep the register count down
+              int offs[4];
+              float va[4], vb[4];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                const int q = 2 * hv + (u >> 1), pr = u & 1;
+                offs[u] = (4 * q + pr) * rg.RSp;
+                va[u] = co * acc[4 * q + 2 * pr];
+                vb[u] = co * acc[4 * q + 2 * pr + 1];
+              }
+              lds_add_f32x2_batch<4>(dst, offs, va, vb);
             }
-            lds_add_f32_batch<16>(dst, offs, vals);
           } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -358,34 +237,33 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
           }
         }
       };
-      if (k < tc.kc) {
-        const int r1 = tc.rs[k + 1];
-        for (int r = tc.rs[k]; r < r1; ++r) splat(tc.e[r * 32 + (lane & 31)], tc.co[r * 32 + (lane & 31)]);
-      } else if (pix_ok) {
-        const size_t sbase = ((size_t)m * K + k) * q;
-        Taps2D<INTERP> t;
-        for (int p = 0; p < q; ++p) {
-          t.set(map[(sbase + p) * 2], map[(sbase + p) * 2 + 1], H, W,
-                WEIGHTED ? wts[sbase + p] : 1.0f);
 #pragma unroll
-          for (int i = 0; i < NT; ++i)
-            if (__any(t.w[i] != 0.0f)) splat(rg.encode(t.y[i], t.x[i], W), t.w[i]);
-        }
+      for (int r = 0; r < 4; ++r)
+        if (r < cur_n) splat(cur[r].x, __int_as_float(cur[r].y));
+      for (int r = 4; r < cur_n; ++r) {
+        const int2 ec = plan_row(k, r);
+        splat(ec.x, __int_as_float(ec.y));
       }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) cur[r] = nxt[r];
+      cur_n = nxt_n;
     }
     // flush this chunk's window to the image and clear it
     __syncthreads();
     {
-      constexpr int PER_WAVE = kCC / 4;
+      constexpr int PAIRS = kCC / 8;   // channel pairs per wave
+      float2* r2 = reinterpret_cast<float2*>(region);
       for (int e = lane; e < rg.RS; e += 64) {
         const int o = src[e];
 #pragma unroll
-        for (int j = 0; j < PER_WAVE; ++j) {
-          const int cl = wave * PER_WAVE + j;
-          const float v = region[cl * rg.RSp + e];
-          region[cl * rg.RSp + e] = 0.0f;
-          if (o >= 0 && c0 + cl < Cg && v != 0.0f)
-            atomic_add_noret(img_b + (size_t)(c0 + cl) * HW + o, v);
+        for (int j = 0; j < PAIRS; ++j) {
+          const int pc = wave * PAIRS + j, cl = 2 * pc;
+          const float2 v = r2[pc * rg.RSp + e];
+          r2[pc * rg.RSp + e] = make_float2(0.0f, 0.0f);
+          if (o >= 0 && c0 + cl < Cg && v.x != 0.0f)
+            atomic_add_noret(img_b + (size_t)(c0 + cl) * HW + o, v.x);
+          if (o >= 0 && c0 + cl + 1 < Cg && v.y != 0.0f)
+            atomic_add_noret(img_b + (size_t)(c0 + cl + 1) * HW + o, v.y);
         }
       }
     }
@@ -396,59 +274,20 @@ __global__ __launch_bounds__(kStThreads) void staged_gemm_scatter_kernel(
 // ---------------------------------------------------------------------------
 // Host side.
 // ---------------------------------------------------------------------------
-static PixelTiling make_tiling(const ConvGeom& g) {
-  PixelTiling pt;
-  pt.OW = g.OW;
-  pt.OH = g.M / g.OW;
-  pt.tx_shift = (pt.OH >= 8) ? 4 : (pt.OH >= 4 ? 5 : (pt.OH >= 2 ? 6 : 7));
-  pt.tiles_x = (int)ceil_div(pt.OW, pt.TX());
-  pt.tiles_y = (int)ceil_div(pt.OH, pt.TY());
-  return pt;
-}
-
-bool staged_supported(const ConvGeom& g) {
-  return g.OW >= 1 && g.M % g.OW == 0 && g.B <= 65535;
-}
-
-bool scatter_staged_supported(const ConvGeom& g) { return staged_supported(g) && g.Cp <= 128; }
-
 size_t staged_workspace_bytes(const ConvGeom& g) {
   const size_t CgP = (size_t)(g.Cg + kCC - 1) / kCC * kCC;
   const size_t CpP = (size_t)(g.Cp + 127) / 128 * 128;
   return (size_t)g.K * CgP * CpP * sizeof(float);
 }
 
-int staged_gather_gemm(const ConvGeom& g, const float* img, const float* map, const float* wts,
-                       const float* Wm, const float* bias, float* pix, float* workspace,
-                       hipStream_t stream) {
-  const PixelTiling pt = make_tiling(g);
-  const int NB = g.Cp > 64 ? 4 : (g.Cp > 32 ? 2 : 1);
-  const int TN = NB * 32;
-  const int n_tiles = (int)ceil_div(g.Cp, TN);
-  const int CgP = (int)ceil_div(g.Cg, kCC) * kCC;
-  {
-    const size_t total = (size_t)g.K * CgP * n_tiles * TN;
-    const int blocks = (int)std::min<size_t>((total + kStThreads - 1) / kStThreads, 2048);
-    launch(permute_weight_gather_kernel, dim3(blocks), dim3(kStThreads), stream, Wm, workspace,
-           g.Cp, g.Cg, g.K, CgP, n_tiles, NB);
-    SDK_LAUNCH_CHECK("permute_weight_gather");
-  }
-  const dim3 grid((unsigned)(pt.tiles_x * pt.tiles_y * n_tiles), (unsigned)g.B);
-#define SG(NBv)                                                                                 \
-  SDK_DISPATCH_INTERP(g.interp, g.P,                                                            \
-                      (launch(staged_gather_gemm_kernel<INTERP, WEIGHTED, NBv>, grid,           \
-                              dim3(kStThreads), stream, img, map, wts, (const float*)workspace, \
-                              bias, pix, g.Cg, g.H, g.W, g.Cp, g.K, g.P, CgP, n_tiles, pt)))
-  if (NB == 4) SG(4); else if (NB == 2) SG(2); else SG(1);
-#undef SG
-  SDK_LAUNCH_CHECK("staged_gather_gemm");
-  return SDK_OK;
+bool planned_scatter_supported(const ConvGeom& g) {
+  return plan_supported(g) && g.Cp <= 128 && g.B <= 65535;
 }
 
-int staged_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
-                        const float* wts, const float* Wm, float* img, float* workspace,
-                        hipStream_t stream) {
-  const PixelTiling pt = make_tiling(g);
+// workspace: permuted weights (staged_workspace_bytes, 256-byte aligned) followed by the plan
+int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
+                         const float* wts, const float* Wm, float* img, float* workspace,
+                         hipStream_t stream) {
   const int NS = g.Cp > 64 ? 64 : (g.Cp > 32 ? 32 : 16);   // MFMA steps: 2 channels each
   const int chunks = (int)ceil_div(g.Cg, kCC);
   {
@@ -458,16 +297,19 @@ int staged_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const fl
            g.Cp, g.Cg, g.K, chunks, NS, bf16 ? 1 : 0);
     SDK_LAUNCH_CHECK("permute_weight_scatter");
   }
-  const dim3 grid((unsigned)(pt.tiles_x * pt.tiles_y), (unsigned)g.B);
-#define SS(NSv, BFv)                                                                                  \
-  SDK_DISPATCH_INTERP(g.interp, g.P,                                                             \
-                      (launch(staged_gemm_scatter_kernel<INTERP, WEIGHTED, NSv, BFv>, grid,      \
-                              dim3(kStThreads), stream, pix, map, wts, (const float*)workspace,  \
-                              img, g.Cg, g.H, g.W, g.Cp, g.K, g.P, chunks, pt)))
-  if (bf16) { if (NS == 64) SS(64, true); else if (NS == 32) SS(32, true); else SS(16, true); }
-  else { if (NS == 64) SS(64, false); else if (NS == 32) SS(32, false); else SS(16, false); }
-#undef SS
-  SDK_LAUNCH_CHECK("staged_gemm_scatter");
+  Plan plan;
+  char* plan_ws = reinterpret_cast<char*>(workspace) + ((staged_workspace_bytes(g) + 255) & ~(size_t)255);
+  int rc = build_plan(g, map, wts, plan_ws, stream, &plan);
+  if (rc) return rc;
+  const dim3 grid((unsigned)plan.tiles, (unsigned)g.B);
+#define PS(NSv, BFv)                                                                             \
+  launch(planned_gemm_scatter_kernel<NSv, BFv>, grid, dim3(kStThreads), stream, pix, plan.hdr,   \
+         plan.ns, plan.taps, (const float*)workspace, img, g.Cg, g.H, g.W, g.Cp, g.K, plan.S,    \
+         chunks, plan.pt)
+  if (bf16) { if (NS == 64) PS(64, true); else if (NS == 32) PS(32, true); else PS(16, true); }
+  else { if (NS == 64) PS(64, false); else if (NS == 32) PS(32, false); else PS(16, false); }
+#undef PS
+  SDK_LAUNCH_CHECK("planned_gemm_scatter");
   return SDK_OK;
 }
 

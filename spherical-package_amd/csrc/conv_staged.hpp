@@ -1,4 +1,4 @@
-// Building blocks of the LDS-staged convolution kernels (conv_staged.hip):
+// Building blocks of the LDS-staged convolution kernels (conv_staged.hip, conv_plan.hip):
 // 2-D taps, the per-workgroup image region and its addressing.
 //
 // A workgroup owns a small 2-D tile of map pixels.  The union of everything its
@@ -20,8 +20,6 @@ namespace sdk {
 
 constexpr int kCC = 32;          // channels staged per region chunk
 constexpr int kRegionCap = 288;  // region elements per channel (kCC * 289 * 4 B = 36 KB)
-constexpr int kTapRows = 40;     // tap-cache rows per wave (each row: one tap of 32 pixels)
-constexpr int kTapKMax = 64;     // kernel samples the tap cache can index
 
 // Up to four taps of one sample point as (row, column, coefficient).  A tap that
 // is out of range or has zero weight gets coefficient 0 (and row = column = 0).
@@ -140,155 +138,6 @@ __device__ __forceinline__ Region choose_region(int dy0, int dy1, int dx0, int d
   r.RS = r.RH * r.RW;
   r.RSp = r.RS | 1;
   return r;
-}
-
-// Determines the region of this workgroup's tile: bounding box, relative to an
-// anchor near the tile, of every active tap of every sample (pass over all K
-// samples and points), clipped to the region capacity.  `bb` is 4 ints of LDS.
-// p_local: this lane's pixel inside the tile (0..127); both half-waves of a wave
-// own the same 32 pixels and split the K samples by parity.
-template <int INTERP, bool WEIGHTED>
-__device__ __forceinline__ Region find_region(const float* __restrict__ map,
-                                              const float* __restrict__ wts, const PixelTiling& pt,
-                                              int ty0, int tx0, int oy, int ox, bool pix_ok,
-                                              int K, int P, int H, int W, int* bb,
-                                              int* ns /* [4][kTapKMax] or nullptr */) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int q = WEIGHTED ? P : 1;
-  // anchor: centre-ish sample of the tile's first pixel (same value in every thread)
-  const size_t s0 = (((size_t)ty0 * pt.OW + tx0) * K + K / 2) * q;
-  const float axf = map[s0 * 2], ayf = map[s0 * 2 + 1];
-  const int ax = wrap_index(to_int_clamped(round_t(axf)), W);
-  const int ay = min(max(to_int_clamped(round_t(ayf)), 0), H - 1);
-  if (threadIdx.x == 0) {
-    bb[0] = INT_MAX;
-    bb[1] = INT_MIN;
-    bb[2] = INT_MAX;
-    bb[3] = INT_MIN;
-  }
-  __syncthreads();
-  int dy0 = INT_MAX, dy1 = INT_MIN, dx0 = INT_MAX, dx1 = INT_MIN;
-  {
-    const size_t base = ((size_t)oy * pt.OW + ox) * K;
-    Taps2D<INTERP> t;
-    for (int k = lane >> 5; k < K; k += 2) {
-      int cnt = 0;
-      if (pix_ok) {
-        for (int p = 0; p < q; ++p) {
-          const size_t s = (base + k) * q + p;
-          t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
-#pragma unroll
-          for (int i = 0; i < Taps2D<INTERP>::N; ++i) {
-            if (t.w[i] != 0.0f) {
-              const int dy = t.y[i] - ay;
-              int dx = t.x[i] - ax;
-              dx += (dx > W / 2) ? -W : ((dx < -(W / 2)) ? W : 0);
-              dy0 = min(dy0, dy);
-              dy1 = max(dy1, dy);
-              dx0 = min(dx0, dx);
-              dx1 = max(dx1, dx);
-              ++cnt;
-            }
-          }
-        }
-      }
-      if (ns != nullptr && k < kTapKMax) {
-        // most active taps of sample k among the 32 pixels of this half-wave (= of the wave)
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) cnt = max(cnt, __shfl_xor(cnt, o, 64));
-        if ((lane & 31) == 0) ns[wave * kTapKMax + k] = cnt;
-      }
-    }
-  }
-  dy0 = wave_min(dy0);
-  dy1 = wave_max(dy1);
-  dx0 = wave_min(dx0);
-  dx1 = wave_max(dx1);
-  if (lane == 0) {
-    atomicMin(&bb[0], dy0);
-    atomicMax(&bb[1], dy1);
-    atomicMin(&bb[2], dx0);
-    atomicMax(&bb[3], dx1);
-  }
-  __syncthreads();
-  dy0 = bb[0];
-  dy1 = bb[1];
-  dx0 = bb[2];
-  dx1 = bb[3];
-  return choose_region(dy0, dy1, dx0, dx1, ay, ax, pt.TY(), pt.TX(), W);
-}
-
-// Per-wave cache of encoded taps: for kernel sample k < kc, rows rs[k] .. rs[k+1]-1
-// each hold one (encoded index, coefficient) pair for the wave's 32 pixels; a
-// pixel with fewer active taps than the wave's maximum is padded with
-// coefficient 0.  Built once per workgroup from the counts find_region() left in
-// `ns`; samples that do not fit (k >= kc) are evaluated on the fly by the caller.
-struct TapCache {
-  const int* e;     // [kTapRows][32] for this wave
-  const float* co;  // [kTapRows][32]
-  const int* rs;    // [kTapKMax + 1] row starts for this wave
-  int kc;           // samples cached
-};
-
-template <int INTERP, bool WEIGHTED>
-__device__ __forceinline__ TapCache build_tap_cache(const float* __restrict__ map,
-                                                    const float* __restrict__ wts,
-                                                    const PixelTiling& pt, int oy, int ox,
-                                                    bool pix_ok, int K, int P, int H, int W,
-                                                    const Region& rg, const int* ns, int* tc_e,
-                                                    float* tc_co, int* rs_all) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int* e_w = tc_e + wave * kTapRows * 32;
-  float* co_w = tc_co + wave * kTapRows * 32;
-  int* rs = rs_all + wave * (kTapKMax + 1);
-  // row starts (every lane computes the same values; lane 0 publishes them)
-  int kc = 0, rows = 0;
-  const int kmax = min(K, kTapKMax);
-  for (int k = 0; k < kmax; ++k) {
-    const int n = ns[wave * kTapKMax + k];
-    if (rows + n > kTapRows) break;
-    if (lane == 0) rs[k] = rows;
-    rows += n;
-    kc = k + 1;
-  }
-  if (lane == 0) rs[kc] = rows;
-  const int q = WEIGHTED ? P : 1;
-  const size_t base = ((size_t)oy * pt.OW + ox) * K;
-  const int px = lane & 31;
-  Taps2D<INTERP> t;
-  int start = 0;
-  for (int k = 0; k < kc; ++k) {
-    const int n = ns[wave * kTapKMax + k];
-    if ((k & 1) == (lane >> 5)) {   // the two half-waves split the samples by parity
-      int cnt = 0;
-      if (pix_ok) {
-        for (int p = 0; p < q; ++p) {
-          const size_t s = (base + k) * q + p;
-          t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
-#pragma unroll
-          for (int i = 0; i < Taps2D<INTERP>::N; ++i) {
-            if (t.w[i] != 0.0f) {
-              e_w[(start + cnt) * 32 + px] = rg.encode(t.y[i], t.x[i], W);
-              co_w[(start + cnt) * 32 + px] = t.w[i];
-              ++cnt;
-            }
-          }
-        }
-      }
-      for (; cnt < n; ++cnt) {
-        e_w[(start + cnt) * 32 + px] = 0;
-        co_w[(start + cnt) * 32 + px] = 0.0f;
-      }
-    }
-    start += n;
-  }
-  __syncthreads();
-  TapCache tc;
-  tc.e = e_w;
-  tc.co = co_w;
-  tc.rs = rs;
-  tc.kc = kc;
-  return tc;
 }
 
 // src[e], e < RS: flat offset inside one image plane of region element e, or -1

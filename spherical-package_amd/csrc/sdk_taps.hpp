@@ -36,8 +36,11 @@ __device__ __forceinline__ void lds_add_f32(float* addr, float v) {
 }
 
 // N independent float adds into LDS: all loads, then all compare-and-swaps, are
-// issued back to back so their latencies overlap; an add whose swap lost a race
-// is redone with the single-word loop.
+// issued back to back so their latencies overlap.  A swap that lost a race (two
+// lanes of the wave, or another wave, hit the same word) is repeated with the
+// value the failed swap returned as the new expectation, again all pending
+// words of the lane in one batch; one extra round settles the common case of
+// two lanes sharing a word.
 template <int N>
 __device__ __forceinline__ void lds_add_f32_batch(float* base, const int (&offs)[N],
                                                   const float (&vals)[N]) {
@@ -53,10 +56,56 @@ __device__ __forceinline__ void lds_add_f32_batch(float* base, const int (&offs)
   bool lost = false;
 #pragma unroll
   for (int i = 0; i < N; ++i) lost |= got[i] != old[i];
-  if (lost) {
+  while (lost) {
 #pragma unroll
-    for (int i = 0; i < N; ++i)
-      if (got[i] != old[i]) lds_add_f32(base + offs[i], vals[i]);
+    for (int i = 0; i < N; ++i) {
+      if (got[i] != old[i]) {
+        old[i] = got[i];
+        got[i] = atomicCAS(reinterpret_cast<int*>(base + offs[i]), old[i],
+                           __float_as_int(__int_as_float(old[i]) + vals[i]));
+      }
+    }
+    lost = false;
+#pragma unroll
+    for (int i = 0; i < N; ++i) lost |= got[i] != old[i];
+  }
+}
+
+// The same for pairs of floats that share an aligned 8-byte word: one 64-bit
+// compare-and-swap adds both, which halves the LDS instructions per value.
+__device__ __forceinline__ unsigned long long add_pair(unsigned long long w, float a, float b) {
+  const float lo = __uint_as_float((unsigned)w) + a;
+  const float hi = __uint_as_float((unsigned)(w >> 32)) + b;
+  return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32);
+}
+
+template <int N>
+__device__ __forceinline__ void lds_add_f32x2_batch(float2* base, const int (&offs)[N],
+                                                    const float (&va)[N], const float (&vb)[N]) {
+  unsigned long long old[N], got[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+    old[i] = __hip_atomic_load(reinterpret_cast<unsigned long long*>(base + offs[i]),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+    got[i] = atomicCAS(reinterpret_cast<unsigned long long*>(base + offs[i]), old[i],
+                       add_pair(old[i], va[i], vb[i]));
+  bool lost = false;
+#pragma unroll
+  for (int i = 0; i < N; ++i) lost |= got[i] != old[i];
+  while (lost) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (got[i] != old[i]) {
+        old[i] = got[i];
+        got[i] = atomicCAS(reinterpret_cast<unsigned long long*>(base + offs[i]), old[i],
+                           add_pair(old[i], va[i], vb[i]));
+      }
+    }
+    lost = false;
+#pragma unroll
+    for (int i = 0; i < N; ++i) lost |= got[i] != old[i];
   }
 }
 
