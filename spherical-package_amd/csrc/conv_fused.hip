@@ -33,7 +33,7 @@ namespace sdk {
 
 constexpr int kThreads = 256;
 constexpr int kKC = 32;         // reduction rows staged per step
-constexpr int kMaxSlots = 64;   // tap slots per pixel and kernel sample (points * taps)
+constexpr int kMaxSlots = 32;   // tap slots per pixel and kernel sample (points * taps); LDS: 2 KB per slot at 256 pixels
 
 __host__ __device__ constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
 

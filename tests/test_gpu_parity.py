@@ -241,6 +241,73 @@ def test_fused_conv_tile_edges(ops, oracle, tc):
     assert relerr(_n(gb), wb) <= 1e-4
 
 
+def _coherent_map(rng, OH, OW, K, P, H, W, dtype, scale=1.0, jitter=0.45):
+    """Locally coherent map: pixel (y, x) samples around (x, y) * scale * (W/OW, H/OH) with a
+    ring of K offsets, as a convolution-style map does; a few samples fall outside the image."""
+    ys, xs = np.meshgrid(np.arange(OH), np.arange(OW), indexing="ij")
+    ang = 2 * np.pi * np.arange(K) / max(K, 1)
+    rad = 1.0 + (np.arange(K) % 3)
+    cx = xs[..., None] * (scale * W / OW) + rad * np.cos(ang)
+    cy = ys[..., None] * (scale * H / OH) + rad * np.sin(ang)
+    if P:
+        cx = cx[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
+        cy = cy[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
+    xy = np.stack([cx, cy], -1) + rng.uniform(-jitter, jitter, cx.shape + (2,))
+    sel = rng.uniform(size=cx.shape) < 0.2
+    xy[sel] = np.round(xy[sel])          # exact pixel centres: zero-weight taps are dropped
+    return np.ascontiguousarray(xy.astype(dtype))
+
+
+# (Cin, Cout, H, W, OH, OW, K, P, interp, scale)
+PLAN_CASES = [
+    (40, 72, 24, 40, 24, 40, 9, 0, 1, 1.0),     # windows cover the taps; ragged tiles
+    (32, 128, 20, 36, 20, 36, 9, 4, 2, 1.0),    # weighted bispherical, wrap at the seam
+    (16, 24, 16, 24, 32, 48, 4, 0, 1, 0.5),     # up-sampling map: many pixels share a target
+    (24, 16, 32, 48, 16, 24, 11, 0, 0, 1.0),    # two blocks of kernel samples (K > 9), nearest
+    (8, 8, 12, 20, 12, 18, 25, 0, 1, 1.0),      # three blocks of kernel samples, OW % 4 != 0
+    (64, 64, 1, 700, 1, 700, 7, 0, 0, 1.0),     # one-row vertex list
+    (20, 20, 40, 3, 40, 3, 5, 0, 1, 1.0),       # narrow grid
+    (12, 140, 9, 50, 3, 50, 3, 2, 1, 1.0),      # few rows; more than 128 pixel-side channels
+    (8, 8, 10, 10, 10, 10, 2, 10, 1, 1.0),      # 40 tap slots per sample: generic path
+    (8, 8, 10, 10, 10, 10, 2, 10, 0, 1.0),      # 10 slots, nearest weighted
+]
+
+
+@pytest.mark.parametrize("tc", PLAN_CASES, ids=lambda t: "x".join(map(str, t)))
+def test_fused_conv_coherent_maps(ops, oracle, tc):
+    """Maps with the locality the LDS-window kernels are built for, at shapes that hit their
+    tiling, blocking and fallback branches; conv and transposed conv, forward and backward."""
+    Cin, Cout, H, W, OH, OW, K, P, interp, scale = tc
+    dt = np.float32
+    rng = np.random.default_rng(11 + int(sum(tc)))
+    B = 2
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    m = _coherent_map(rng, OH, OW, K, P, H, W, dt, scale)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if P else None
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), K, interp))
+    assert relerr(got, oracle.mapped_conv_forward(x, m, wt, b, K, interp, iw)) <= 1e-5
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+    bt = rng.standard_normal(Cin).astype(dt)
+    gt = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), _t(iw), _t(wtt), _t(bt), H, W, K,
+                                                interp))
+    assert relerr(got, oracle.mapped_transposed_conv_forward(xt, m, wtt, bt, H, W, K, interp,
+                                                             iw)) <= 1e-4
+    gi, gw, gb = ops.mapped_transposed_conv_backward(_t(gt), _t(m), _t(iw), _t(xt), _t(wtt),
+                                                     _t(bt), K, interp)
+    wi, ww, wb = oracle.mapped_transposed_conv_backward(gt, m, xt, wtt, bt, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+
+
 @pytest.fixture
 def bf16_compute(ops):
     ops.set_conv_compute("bf16")
