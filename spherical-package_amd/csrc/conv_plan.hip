@@ -139,12 +139,12 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
 // v_mfma_f32_32x32x16_bf16: instruction t contracts m = 16t + 8h + 0..7.
 // ---------------------------------------------------------------------------
 constexpr int kColLd = 68;            // column tile row stride (floats): 16-byte rows, 4-bank skew
-constexpr int kRegionLd = kRegionCap + 16;  // largest window stride, see region_stride()
+constexpr int kRegE = 36;             // window element stride (floats): 32 channels + 4 of skew
 constexpr int kRowCap = 36;           // plan rows of one half held in LDS at a time
 
-// Window stride: a multiple of 32 plus 16, so the two channel groups a half-wave
-// reads in one ds_read (channels 4j and 4j+1) fall on disjoint bank halves.
-__device__ __forceinline__ int region_stride(int RS) { return ((RS + 31) & ~31) + 16; }
+// Window layout: region[e * kRegE + c], channels fastest.  A lane reads or writes the 8
+// channels of its group for one element as two 16-byte accesses; 8 lanes on consecutive
+// elements are 144 bytes apart and cover all 32 banks once.
 
 template <int KB, bool BF16>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW, int Cg,
     int H, int W, int Cp, int K, int S, PixelTiling pt, int tiles,
     int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
-  __shared__ __align__(16) float region[kCC * kRegionLd];
+  __shared__ __align__(16) float region[kRegionCap * kRegE];
   __shared__ __align__(16) float colT[2][kCC * kColLd];
   __shared__ __align__(16) int2 prow[kRowCap * 64];
   __shared__ int src[kRegionCap];
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     rg.RH = hdr[tile * 8 + 2];
     rg.RW = hdr[tile * 8 + 3];
     rg.RS = rg.RH * rg.RW;
-    rg.RSp = region_stride(rg.RS);
+    rg.RSp = rg.RS;
     // plan rows of this tile and sample block: uniform base, 32-bit lane offsets
     const char* tile_taps = reinterpret_cast<const char*>(taps + ((size_t)tile * K + k0) * S * 128);
 
@@ -222,23 +222,26 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
       const char* cbase = reinterpret_cast<const char*>(
           img_b + (size_t)min(c0 + wave * PER_WAVE, Cg - 1) * HW);
       const unsigned plane = (unsigned)HW * 4u;
+      float v[ITER][PER_WAVE];
 #pragma unroll
-      for (int j = 0; j < PER_WAVE; ++j) {
-        const bool c_ok = c0 + wave * PER_WAVE + j < Cg;
-        float v[ITER];
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        const int o = e < rg.RS ? src[e] : -1;
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) {
-          const int e = lane + 64 * it;
-          const int o = e < rg.RS ? src[e] : -1;
-          const bool ok = o >= 0 && c_ok;
+        for (int j = 0; j < PER_WAVE; ++j) {
+          const bool ok = o >= 0 && c0 + wave * PER_WAVE + j < Cg;
           const float d = *reinterpret_cast<const float*>(
               cbase + (ok ? (unsigned)j * plane + (unsigned)o * 4u : 0u));
-          v[it] = ok ? d : 0.0f;
+          v[it][j] = ok ? d : 0.0f;
         }
+      }
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) {
-          const int e = lane + 64 * it;
-          if (e < rg.RS) region[(wave * PER_WAVE + j) * rg.RSp + e] = v[it];
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        if (e < rg.RS) {
+          float4* dst = reinterpret_cast<float4*>(region + e * kRegE + wave * PER_WAVE);
+          dst[0] = make_float4(v[it][0], v[it][1], v[it][2], v[it][3]);
+          dst[1] = make_float4(v[it][4], v[it][5], v[it][6], v[it][7]);
         }
       }
     }
@@ -305,7 +308,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 #pragma unroll 1
         for (int kk = kk_beg; kk < kk_end; ++kk) {
           const int nrows = ns_l[kk];
-          // ---- gather: column values of pixel m_local, channels 4j + cg
+          // ---- gather: column values of pixel m_local, channels 8*cg + j
           float col[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j) col[j] = 0.0f;
@@ -314,17 +317,18 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
             // some lane's tap lies outside the window: that lane reads the image directly
             // (uniform base, 32-bit byte offsets; 32 planes of < 2^24 elements fit)
             const bool out = e < 0 && co != 0.0f;
-            const float* rp = region + cg * rg.RSp + (e >= 0 ? e : 0);
+            const float4* rp = reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);
+            const float4 l0 = rp[0], l1 = rp[1];
+            const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
             const char* gbase = reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
             const unsigned plane = (unsigned)HW * 4u;
-            const unsigned o0 = out ? (unsigned)cg * plane + (unsigned)(-e - 1) * 4u : 0u;
+            const unsigned o0 = out ? (unsigned)(8 * cg) * plane + (unsigned)(-e - 1) * 4u : 0u;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              const bool g_ok = out && c0 + 4 * j + cg < Cg;
+              const bool g_ok = out && c0 + 8 * cg + j < Cg;
               const float dg =
-                  *reinterpret_cast<const float*>(gbase + (g_ok ? o0 + 4u * j * plane : 0u));
-              const float dl = rp[4 * j * rg.RSp];
-              col[j] += co * (e >= 0 ? dl : (g_ok ? dg : 0.0f));
+                  *reinterpret_cast<const float*>(gbase + (g_ok ? o0 + (unsigned)j * plane : 0u));
+              col[j] += co * (e >= 0 ? dl[j] : (g_ok ? dg : 0.0f));
             }
           };
           for (int r = 0; r < nrows; r += 2) {
@@ -333,14 +337,13 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
             const int2 ec1 = (r + 1 < nrows) ? prow[(row0 + r + 1) * 64 + m_local] : make_int2(0, 0);
             const float co0 = __int_as_float(ec0.y), co1 = __int_as_float(ec1.y);
             if (__all((ec0.x >= 0 || co0 == 0.0f) && (ec1.x >= 0 || co1 == 0.0f))) {
-              const float* rp0 = region + cg * rg.RSp + (ec0.x >= 0 ? ec0.x : 0);
-              const float* rp1 = region + cg * rg.RSp + (ec1.x >= 0 ? ec1.x : 0);
-              float d0[8], d1[8];
-#pragma unroll
-              for (int j = 0; j < 8; ++j) {
-                d0[j] = rp0[4 * j * rg.RSp];
-                d1[j] = rp1[4 * j * rg.RSp];
-              }
+              const float4* rp0 = reinterpret_cast<const float4*>(
+                  region + (ec0.x >= 0 ? ec0.x : 0) * kRegE + 8 * cg);
+              const float4* rp1 = reinterpret_cast<const float4*>(
+                  region + (ec1.x >= 0 ? ec1.x : 0) * kRegE + 8 * cg);
+              const float4 a0 = rp0[0], a1 = rp0[1], b0 = rp1[0], b1 = rp1[1];
+              const float d0[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+              const float d1[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
               for (int j = 0; j < 8; ++j) {
                 col[j] += co0 * d0[j];
@@ -354,26 +357,28 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
           row0 += nrows;
           float* ct = colT[buf];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) ct[(4 * j + cg) * kColLd + m_local] = col[j];
+          for (int j = 0; j < 8; ++j) ct[(8 * cg + j) * kColLd + (m_local ^ ((cg & 1) << 4))] = col[j];
           __syncthreads();
 
           // ---- D[n][c] += A[n][m] * col[c][m]; one copy of this block per accumulator
+          // rows of channel group cg = nl / 8 were written with pixel bit 4 flipped by cg
           const float* bt = ct + nl * kColLd;
+          const int sw = ((nl >> 3) & 1) << 4;
           auto mma = [&](floatx16& d) {
             if constexpr (BF16) {
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
-                const float4 lo = *reinterpret_cast<const float4*>(bt + 16 * t + 8 * h);
-                const float4 hi = *reinterpret_cast<const float4*>(bt + 16 * t + 8 * h + 4);
+                const float4 lo = *reinterpret_cast<const float4*>(bt + ((16 * t + 8 * h) ^ sw));
+                const float4 hi = *reinterpret_cast<const float4*>(bt + ((16 * t + 8 * h + 4) ^ sw));
                 const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
                 d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
               }
             } else {
-              float4 b = *reinterpret_cast<const float4*>(bt + 4 * h);
+              float4 b = *reinterpret_cast<const float4*>(bt + ((4 * h) ^ sw));
 #pragma unroll
               for (int g = 0; g < 8; ++g) {
                 float4 bn = b;
-                if (g < 7) bn = *reinterpret_cast<const float4*>(bt + 8 * (g + 1) + 4 * h);
+                if (g < 7) bn = *reinterpret_cast<const float4*>(bt + ((8 * (g + 1) + 4 * h) ^ sw));
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 0], b.x, d, 0, 0, 0);
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 1], b.y, d, 0, 0, 0);
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 2], b.z, d, 0, 0, 0);
