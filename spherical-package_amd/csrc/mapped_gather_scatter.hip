@@ -20,6 +20,18 @@ namespace sdk {
 constexpr int kBlock = 256;  // 4 wavefronts
 constexpr int kPC = 8;       // planes per thread
 
+// Pixel block of this workgroup.  Workgroup ids go round-robin over the 8 XCDs, each with
+// its own L2; grid.x is 8 * per_xcd and XCD x walks the contiguous band of pixel blocks
+// [x * per_xcd, (x + 1) * per_xcd) in order, so neighbouring map rows, which read the same
+// image rows, meet in one L2 shortly after each other.  Blocks past the last pixel do nothing.
+__device__ __forceinline__ int banded_pixel_block() {
+  const int per_xcd = gridDim.x >> 3;
+  return (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+inline unsigned banded_grid_x(int64_t pixels) {
+  return 8u * (unsigned)ceil_div(ceil_div(pixels, kBlock), 8);
+}
+
 // ---------------------------------------------------------------------------
 // Fill kernels (scatter targets start from zero; hipMemsetAsync is avoided so
 // that callers may capture these entry points into a HIP graph).
@@ -65,7 +77,7 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
     const T* __restrict__ image, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ out, int planes, int H, int W, int MP, int P) {
-  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= MP) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
@@ -88,7 +100,7 @@ template <typename T, int INTERP, bool WEIGHTED, bool ONES>
 __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ out, int planes, int H, int W, int MP, int P) {
-  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= MP) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
@@ -121,7 +133,7 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void mapped_im2col_kernel(
     const T* __restrict__ im, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ col, int planes, int H, int W, int M, int K, int P) {
-  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= M) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
@@ -142,7 +154,7 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void mapped_col2im_kernel(
     const T* __restrict__ col, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ im, int planes, int H, int W, int M, int K, int P) {
-  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= M) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
@@ -168,7 +180,7 @@ __global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ out, int64_t* __restrict__ idx, int planes, int H, int W, int M, int K,
     int P) {
-  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= M) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
@@ -243,7 +255,7 @@ template <typename T>
 static int launch_resample_from_map(const T* image, const T* map, const T* wts, T* out,
                                     int64_t planes, int H, int W, int MP, int P, int interp,
                                     hipStream_t stream) {
-  const dim3 grid((unsigned)ceil_div(MP, kBlock), (unsigned)ceil_div(planes, kPC));
+  const dim3 grid(banded_grid_x(MP), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((resample_from_map_kernel<T, INTERP, WEIGHTED>), grid,
                                           dim3(kBlock), stream, image, map, wts, out,
@@ -258,7 +270,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
                                   hipStream_t stream) {
   int rc = zero_fill(out, sizeof(T) * (size_t)planes * H * W, stream);
   if (rc != SDK_OK) return rc;
-  const dim3 grid((unsigned)ceil_div(MP, kBlock), (unsigned)ceil_div(planes, kPC));
+  const dim3 grid(banded_grid_x(MP), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, false>),
                                           grid, dim3(kBlock), stream, in, map, wts, out,
@@ -267,7 +279,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
   if (wsum) {
     rc = zero_fill(wsum, sizeof(T) * (size_t)H * W, stream);
     if (rc != SDK_OK) return rc;
-    const dim3 g1((unsigned)ceil_div(MP, kBlock), 1);
+    const dim3 g1(banded_grid_x(MP), 1);
     SDK_DISPATCH_INTERP(interp, P,
                         (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, true>),
                                             g1, dim3(kBlock), stream, (const T*)nullptr, map,
@@ -281,7 +293,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
 template <typename T>
 int launch_mapped_im2col(const T* im, const T* map, const T* wts, T* col, int64_t planes, int H,
                          int W, int M, int K, int P, int interp, hipStream_t stream) {
-  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((mapped_im2col_kernel<T, INTERP, WEIGHTED>), grid,
                                           dim3(kBlock), stream, im, map, wts, col, (int)planes,
@@ -294,7 +306,7 @@ int launch_mapped_im2col(const T* im, const T* map, const T* wts, T* col, int64_
 template <typename T>
 int launch_mapped_col2im(const T* col, const T* map, const T* wts, T* im, int64_t planes, int H,
                          int W, int M, int K, int P, int interp, hipStream_t stream) {
-  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((mapped_col2im_kernel<T, INTERP, WEIGHTED>), grid,
                                           dim3(kBlock), stream, col, map, wts, im, (int)planes,
@@ -447,7 +459,7 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
   if (rc) return rc;
   const int64_t planes = batch * channels;
   if (planes == 0) return SDK_OK;
-  const dim3 grid((unsigned)ceil_div(M, kBlock), (unsigned)ceil_div(planes, kPC));
+  const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_DTYPE(
       dtype,
       SDK_DISPATCH_INTERP(interp, num_interp_pts,
