@@ -85,7 +85,7 @@ def _conv_entry_points(torch, ops, x, m, iw, w, b, g, K, interp, compute):
     OH, OW = m.shape[:2]
     P = 0 if iw is None else int(iw.shape[-1])
     mode = {"native": _capi.SDK_COMPUTE_NATIVE, "bf16": _capi.SDK_COMPUTE_BF16}[compute]
-    nws = _capi.load().sdk_mapped_conv_workspace_bytes(B, Cin, Cout, OH, OW, K, P, interp, 0, mode)
+    nws = _capi.load().sdk_mapped_conv_workspace_bytes(B, Cin, Cout, H, W, OH, OW, K, P, interp, 0, mode)
     ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=x.device)
     out = torch.empty(B, Cout, OH, OW, device=x.device)
     gi, gw = torch.empty_like(x), torch.empty_like(w)

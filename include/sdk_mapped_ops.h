@@ -168,12 +168,15 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
  * ask sdk_mapped_conv_workspace_bytes() (same arguments for the forward,
  * backward and transposed entry points of one layer call; map_height x map_width
  * is the grid of the sample map: OH x OW, resp. IH x IW for the transposed
- * layer) and pass at least that many bytes, 256-byte aligned.  Besides the
+ * layer; image_height x image_width is the image the map points into: the
+ * input of a mapped convolution, the output of a transposed one) and pass at
+ * least that many bytes, 256-byte aligned.  Besides the
  * weights the scratch holds the call's tap plan (the sample map resolved into
  * window indices and coefficients), up to
  * 8 * map pixels * kernel_size * points * taps-per-point bytes.
  * ------------------------------------------------------------------------- */
 size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
+                                       int64_t image_height, int64_t image_width,
                                        int64_t map_height, int64_t map_width,
                                        int64_t kernel_size,
                                        int32_t num_interp_pts, int32_t interp, int32_t dtype,

@@ -55,7 +55,7 @@ def load():
     lib.sdk_last_error.restype = ctypes.c_char_p
     lib.sdk_version.argtypes = []
     lib.sdk_version.restype = ctypes.c_int
-    lib.sdk_mapped_conv_workspace_bytes.argtypes = [_i64] * 6 + [_i32] * 4
+    lib.sdk_mapped_conv_workspace_bytes.argtypes = [_i64] * 8 + [_i32] * 4
     lib.sdk_mapped_conv_workspace_bytes.restype = _sz
     _lib = lib
     return lib

@@ -79,9 +79,10 @@ def _npts(sample_map, interp_weights, map_rank_unweighted):
     return int(interp_weights.shape[-1])
 
 
-def _workspace(ref, batch, cin, cout, map_h, map_w, K, P, interp):
+def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
     n = _capi.load().sdk_mapped_conv_workspace_bytes(
-        batch, cin, cout, map_h, map_w, K, P, interp, _DTYPES[ref.dtype], _compute_mode)
+        batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp, _DTYPES[ref.dtype],
+        _compute_mode)
     if n == 0:
         return None, 0
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
@@ -226,7 +227,7 @@ def mapped_conv_forward(x, sample_map, interp_weights, weight, bias, kernel_size
     OH, OW = sample_map.shape[:2]
     out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
-        ws, nws = _workspace(x, B, Cin, Cout, OH, OW, K, P, int(interp))
+        ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         _capi.call("sdk_mapped_conv_forward", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
                    _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B, Cin, H, W, Cout, OH,
                    OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode, _stream(x))
@@ -249,7 +250,7 @@ def mapped_conv_backward(grad_output, sample_map, interp_weights, x, weight, bia
     gb = torch.empty((Cout,), dtype=x.dtype, device=x.device)
     dt = _DTYPES[x.dtype]
     with torch.cuda.device(x.device):
-        ws, nws = _workspace(x, B, Cin, Cout, OH, OW, K, P, int(interp))
+        ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
         _capi.call("sdk_mapped_conv_backward_input", _ptr(grad_output), _ptr(sample_map),
@@ -273,7 +274,7 @@ def mapped_transposed_conv_forward(x, sample_map, interp_weights, weight, bias, 
     OH, OW = int(out_h), int(out_w)
     out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
-        ws, nws = _workspace(x, B, Cin, Cout, IH, IW, K, P, int(interp))
+        ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         _capi.call("sdk_mapped_transposed_conv_forward", _ptr(x), _ptr(sample_map),
                    _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B,
                    Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype],
@@ -295,7 +296,7 @@ def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, 
     gb = torch.empty((Cout,), dtype=x.dtype, device=x.device)
     dt = _DTYPES[x.dtype]
     with torch.cuda.device(x.device):
-        ws, nws = _workspace(x, B, Cin, Cout, IH, IW, K, P, int(interp))
+        ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
         _capi.call("sdk_mapped_transposed_conv_backward_input", _ptr(grad_output),

@@ -92,17 +92,20 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
 extern "C" {
 
 size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
+                                       int64_t image_height, int64_t image_width,
                                        int64_t map_height, int64_t map_width,
                                        int64_t kernel_size, int32_t num_interp_pts,
                                        int32_t interp, int32_t dtype, int32_t compute) {
   if (map_height < 1 || map_width < 1 || map_height * map_width >= ((int64_t)1 << 31)) return 0;
+  if (image_height < 1 || image_width < 1 || image_height * image_width >= ((int64_t)1 << 31))
+    return 0;
   const int64_t gather_pixels = map_height * map_width;
   // Upper bound over the conv (gather side = in_channels) and transposed conv
   // (gather side = out_channels) roles, so one query serves a whole layer call.
-  ConvGeom a{batch, (int)in_channels, 1, 1, (int)out_channels, (int)gather_pixels,
-             (int)kernel_size, num_interp_pts, interp, (int)map_width};
-  ConvGeom b{batch, (int)out_channels, 1, 1, (int)in_channels, (int)gather_pixels,
-             (int)kernel_size, num_interp_pts, interp, (int)map_width};
+  ConvGeom a{batch, (int)in_channels, (int)image_height, (int)image_width, (int)out_channels,
+             (int)gather_pixels, (int)kernel_size, num_interp_pts, interp, (int)map_width};
+  ConvGeom b{batch, (int)out_channels, (int)image_height, (int)image_width, (int)in_channels,
+             (int)gather_pixels, (int)kernel_size, num_interp_pts, interp, (int)map_width};
   if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(a) &&
       fused_supported(b))
     return align256(std::max(fused_workspace_bytes(a), fused_workspace_bytes(b)));

@@ -198,12 +198,21 @@ __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
 // gather_gemm.  Workgroup tile: TN pixel-side channels x TM pixels, TN*TM = 16384.
 // grid.x = pixel tiles * n tiles, grid.y = batch.
 // LDS: Bs[kKC][TM] column tile, As[kKC][TN] weight tile, tap table.
+//
+// INV: the tap lists do not come from the sample map but from an inverse map
+// (conv_inverse.hip): rows inv_off / inv_co [(pixel tile * K + k) * slots + s][TM] and
+// their count inv_ns[pixel tile * K + k].  The kernel does nothing unless *gate == 0.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int TN, int TM, bool BF16>
+template <int INTERP, bool WEIGHTED, int TN, int TM, bool BF16, bool INV = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wg, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
-    int H, int W, int Cp, int M, int K, int P, int CgP, int CpP, int slots, int m_tiles) {
+    int H, int W, int Cp, int M, int K, int P, int CgP, int CpP, int slots, int m_tiles,
+    const int* __restrict__ inv_off = nullptr, const float* __restrict__ inv_co = nullptr,
+    const int* __restrict__ inv_ns = nullptr, const int* __restrict__ gate = nullptr) {
+  if constexpr (INV) {
+    if (*gate != 0) return;
+  }
   extern __shared__ __align__(16) unsigned char smem[];
   float* Bs = reinterpret_cast<float*>(smem);             // [kKC][TM]
   float* As = Bs + kKC * TM;                               // [kKC][TN]
@@ -227,7 +236,19 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   zero_acc(acc);
 
   for (int k = 0; k < K; ++k) {
-    build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    if constexpr (INV) {
+      const size_t rows = ((size_t)(tile / n_tiles) * K + k) * slots * TM;
+      if (tid == 0) *smax = min(inv_ns[(size_t)(tile / n_tiles) * K + k], slots);
+      __syncthreads();
+      for (int e = tid; e < *smax * TM; e += kThreads) {
+        const float co = inv_co[rows + e];
+        tap_co[e] = co;
+        tap_off[e] = co != 0.0f ? inv_off[rows + e] : 0;
+      }
+      __syncthreads();
+    } else {
+      build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    }
     const int ns = *smax;
     for (int c0 = 0; c0 < CgP; c0 += kKC) {
       // ---- gather kKC column rows (channels c0.., sample k) for TM pixels
@@ -498,10 +519,15 @@ bool fused_supported(const ConvGeom& g) {
   return true;
 }
 
+static bool inverse_candidate(const ConvGeom& g);
+static size_t inverse_bytes(const ConvGeom& g);
+
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
   size_t need = std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
+  if (planned_scatter_supported(g) && inverse_candidate(g))
+    need = ((need + 255) & ~(size_t)255) + inverse_bytes(g);
   return need;
 }
 
@@ -549,10 +575,169 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                                         gather_gemm_kernel<INTERP, WEIGHTED, TNv, TMv, BFv>, grid, \
                                         smem, stream, img, map, wts, (const float*)workspace, \
                                         bias, pix, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP,  \
-                                        CpP, slots, m_tiles)))
+                                        CpP, slots, m_tiles, (const int*)nullptr,             \
+                                        (const float*)nullptr, (const int*)nullptr,           \
+                                        (const int*)nullptr)))
   if (bf16) { if (narrow) GG(64, 256, true); else GG(128, 128, true); }
   else { if (narrow) GG(64, 256, false); else GG(128, 128, false); }
 #undef GG
+  return rc;
+}
+
+
+// ---------------------------------------------------------------------------
+// Inverse map: the scatter  img[u] += co * v[m, k]  over all taps (m, k) -> u, regrouped by
+// target u, so that gemm_scatter can run as gather_gemm over the pixel-side tensor with no
+// atomics.  Rows: for target tile t (TM consecutive image elements), sample k, slot s < kInvSlots:
+// source pixel inv_off[((t*K + k)*kInvSlots + s)*TM + u % TM] and coefficient inv_co[...] (0 = empty).
+// cnt[u*K + k] counts the sources of (u, k); *gate counts taps that found no free slot: the
+// inverse is usable only if it stays 0.
+// ---------------------------------------------------------------------------
+constexpr int kInvSlots = 8;
+
+template <int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kThreads) void inverse_fill_kernel(
+    const float* __restrict__ map, const float* __restrict__ wts, int M, int K, int P, int H, int W,
+    int TM, int* __restrict__ cnt, int* __restrict__ inv_off, float* __restrict__ inv_co,
+    int* __restrict__ gate) {
+  const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= (size_t)M * K) return;
+  const int m = (int)(i / K), k = (int)(i % K);
+  const int q = WEIGHTED ? P : 1;
+  PointTaps<float, INTERP> t;
+  for (int p = 0; p < q; ++p) {
+    const size_t s = i * q + p;
+    t.set(map[s * 2], map[s * 2 + 1], H, W);
+    const float wt = WEIGHTED ? wts[s] : 1.0f;
+#pragma unroll
+    for (int j = 0; j < PointTaps<float, INTERP>::N; ++j) {
+      const float co = WEIGHTED ? wt * t.w[j] : t.w[j];
+      if (t.off[j] >= 0 && co != 0.0f) {
+        const int u = t.off[j];
+        const int slot = atomicAdd(&cnt[(size_t)u * K + k], 1);
+        if (slot < kInvSlots) {
+          const size_t e = (((size_t)(u / TM) * K + k) * kInvSlots + slot) * TM + u % TM;
+          inv_off[e] = m;
+          inv_co[e] = co;
+        } else {
+          atomicAdd(gate, 1);
+        }
+      }
+    }
+  }
+}
+
+// ns[t*K + k] = largest source count of any target of tile t for sample k (capped at the slots)
+__global__ __launch_bounds__(kThreads) void inverse_rows_kernel(const int* __restrict__ cnt, int HW,
+                                                                int K, int TM,
+                                                                int* __restrict__ ns) {
+  __shared__ int mx[256];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  for (int k = tid; k < K; k += kThreads) mx[k] = 0;
+  __syncthreads();
+  for (int e = tid; e < TM * K; e += kThreads) {
+    const int u = t * TM + e / K, k = e % K;   // cnt rows of a tile are contiguous: coalesced
+    if (u < HW) {
+      const int c = cnt[(size_t)u * K + k];
+      if (c > 0) atomicMax(&mx[k], min(c, kInvSlots));
+    }
+  }
+  __syncthreads();
+  for (int k = tid; k < K; k += kThreads) ns[(size_t)t * K + k] = mx[k];
+}
+
+struct InverseMap {
+  int TM, tiles;
+  int* gate;
+  int* cnt;
+  int* ns;
+  int* off;
+  float* co;
+  float* weights;   // Ws[k][n][c] copy for the gather kernel
+};
+
+static bool inverse_candidate(const ConvGeom& g) {
+  // one tap per sample (nearest, unweighted): inverse lists are as short as the map is
+  // injective; K <= 256 for the row-count kernel; the pixel side is gathered with 32-bit offsets
+  return g.P == 0 && g.interp != 1 && g.interp != 2 && g.K <= 256 && g.M <= (1 << 24);
+}
+
+static int inverse_tm(const ConvGeom& g) { return g.Cg <= 64 ? 256 : 128; }
+
+static void inverse_layout(const ConvGeom& g, size_t (&off)[7]) {
+  const size_t HW = (size_t)g.H * g.W, TM = inverse_tm(g), tiles = (HW + TM - 1) / TM;
+  const size_t rows = tiles * g.K * kInvSlots * TM;
+  const int TN = g.Cg <= 64 ? 64 : 128;
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  off[0] = 0;                                  // gate
+  off[1] = 256;                                // cnt
+  off[2] = off[1] + up(HW * g.K * 4);          // co   (gate, cnt, co are cleared together)
+  off[3] = off[2] + up(rows * 4);              // off
+  off[4] = off[3] + up(rows * 4);              // ns
+  off[5] = off[4] + up(tiles * g.K * 4);       // weights
+  off[6] = off[5] + up((size_t)g.K * round_up(g.Cp, kKC) * round_up(g.Cg, TN) * 4);
+}
+
+static size_t inverse_bytes(const ConvGeom& g) {
+  size_t off[7];
+  inverse_layout(g, off);
+  return off[6];
+}
+
+static int build_inverse(const ConvGeom& g, const float* map, const float* wts, char* ws,
+                         hipStream_t stream, InverseMap* inv) {
+  size_t off[7];
+  inverse_layout(g, off);
+  const int HW = g.H * g.W;
+  inv->TM = inverse_tm(g);
+  inv->tiles = (int)ceil_div(HW, inv->TM);
+  inv->gate = reinterpret_cast<int*>(ws + off[0]);
+  inv->cnt = reinterpret_cast<int*>(ws + off[1]);
+  inv->co = reinterpret_cast<float*>(ws + off[2]);
+  inv->off = reinterpret_cast<int*>(ws + off[3]);
+  inv->ns = reinterpret_cast<int*>(ws + off[4]);
+  inv->weights = reinterpret_cast<float*>(ws + off[5]);
+  int rc = zero_fill(ws, off[3], stream);
+  if (rc) return rc;
+  const int64_t total = (int64_t)g.M * g.K;
+  if (ceil_div(total, kThreads) >= ((int64_t)1 << 31))
+    return fail(SDK_ERR_UNSUPPORTED, "inverse map: too many samples");
+  SDK_DISPATCH_INTERP(g.interp, g.P,
+                      (launch(inverse_fill_kernel<INTERP, WEIGHTED>,
+                              dim3((unsigned)ceil_div(total, kThreads)), dim3(kThreads), stream, map,
+                              wts, g.M, g.K, g.P, g.H, g.W, inv->TM, inv->cnt, inv->off, inv->co,
+                              inv->gate)));
+  SDK_LAUNCH_CHECK("inverse_fill");
+  launch(inverse_rows_kernel, dim3((unsigned)inv->tiles), dim3(kThreads), stream,
+         (const int*)inv->cnt, HW, g.K, inv->TM, inv->ns);
+  SDK_LAUNCH_CHECK("inverse_rows");
+  return SDK_OK;
+}
+
+// img[b] = Ws^T x gather(pix[b]) + bias over the inverse map; does nothing if *inv.gate != 0.
+static int inverse_gather_gemm(const ConvGeom& g, bool bf16, const InverseMap& inv,
+                               const float* pix, const float* Wm, const float* bias, float* img,
+                               hipStream_t stream) {
+  // roles in the gather kernel: gathered tensor = pix (Cp channels, planes of M elements),
+  // output = img (Cg channels, H*W elements), weights Ws[k][n][c] with c contiguous
+  const bool narrow = g.Cg <= 64;
+  const int TN = narrow ? 64 : 128, TM = inv.TM;
+  const int CoutP = round_up(g.Cg, TN), CinP = round_up(g.Cp, kKC);
+  int rc = relayout(g, Wm, inv.weights, CinP, CoutP, false, stream);
+  if (rc) return rc;
+  const int HW = g.H * g.W;
+  const int m_tiles = inv.tiles, n_tiles = CoutP / TN;
+  const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
+  const size_t smem = sizeof(float) * (kKC * TM + kKC * TN) + (size_t)kInvSlots * TM * 8 + 16;
+#define IG(TNv, TMv, BFv)                                                                        \
+  rc = launch_smem("inverse_gather_gemm", gather_gemm_kernel<0, false, TNv, TMv, BFv, true>, grid, \
+                   smem, stream, pix, (const float*)nullptr, (const float*)nullptr,              \
+                   (const float*)inv.weights, bias, img, g.Cp, 1, g.M, g.Cg, HW, g.K, 0, CinP,   \
+                   CoutP, kInvSlots, m_tiles, (const int*)inv.off, (const float*)inv.co,         \
+                   (const int*)inv.ns, (const int*)inv.gate)
+  if (bf16) { if (narrow) IG(64, 256, true); else IG(128, 128, true); }
+  else { if (narrow) IG(64, 256, false); else IG(128, 128, false); }
+#undef IG
   return rc;
 }
 
@@ -562,8 +747,23 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
-  if (planned_scatter_supported(g))
-    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, stream);
+  if (planned_scatter_supported(g)) {
+    const int* gate = nullptr;
+    if (inverse_candidate(g)) {
+      // One tap per sample: try the scatter as a gather over the inverse map.  The inverse
+      // is built on the device; if a target collects more sources than its rows hold, the
+      // gather kernel exits at once and the scatter kernel below runs instead (and vice versa).
+      const size_t base = ((staged_workspace_bytes(g) + 255) & ~(size_t)255) + plan_bytes(g);
+      char* inv_ws = reinterpret_cast<char*>(workspace) + ((base + 255) & ~(size_t)255);
+      InverseMap inv;
+      rc = build_inverse(g, map, wts, inv_ws, stream, &inv);
+      if (rc) return rc;
+      rc = inverse_gather_gemm(g, bf16, inv, pix, Wm, bias, img, stream);
+      if (rc) return rc;
+      gate = inv.gate;
+    }
+    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream);
+  }
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;

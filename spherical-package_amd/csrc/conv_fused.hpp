@@ -25,10 +25,11 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
 // Bytes of the permuted weight copy the plan-driven scatter kernel reads.
 size_t staged_workspace_bytes(const ConvGeom& g);
 
-// Plan-driven variant (conv_plan.hpp); workspace = permuted weights + plan.
+// Plan-driven variant (conv_plan.hpp); workspace = permuted weights + plan.  With a gate
+// (device counter) the kernel runs only if *gate != 0.
 bool planned_scatter_supported(const ConvGeom& g);
 int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
                          const float* wts, const float* Wm, float* img, float* workspace,
-                         hipStream_t stream);
+                         const int* gate, hipStream_t stream);
 
 }  // namespace sdk

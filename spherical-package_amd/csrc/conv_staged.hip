@@ -86,7 +86,8 @@ template <int NS, bool BF16>
 __global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
     const float* __restrict__ pix, const int* __restrict__ hdr, const int* __restrict__ ns,
     const int2* __restrict__ taps, const float* __restrict__ Ws, float* __restrict__ img, int Cg,
-    int H, int W, int Cp, int K, int S, int chunks, PixelTiling pt) {
+    int H, int W, int Cp, int K, int S, int chunks, PixelTiling pt, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;   // another kernel has done the work
   // window, channel pairs interleaved: value of (channel c, element e) at
   // region[((c / 2) * RSp + e) * 2 + c % 2], so two channels share an 8-byte word
   __shared__ __align__(8) float region[kCC * (kRegionCap + 1)];
@@ -287,7 +288,7 @@ bool planned_scatter_supported(const ConvGeom& g) {
 // workspace: permuted weights (staged_workspace_bytes, 256-byte aligned) followed by the plan
 int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
                          const float* wts, const float* Wm, float* img, float* workspace,
-                         hipStream_t stream) {
+                         const int* gate, hipStream_t stream) {
   const int NS = g.Cp > 64 ? 64 : (g.Cp > 32 ? 32 : 16);   // MFMA steps: 2 channels each
   const int chunks = (int)ceil_div(g.Cg, kCC);
   {
@@ -305,7 +306,7 @@ int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const f
 #define PS(NSv, BFv)                                                                             \
   launch(planned_gemm_scatter_kernel<NSv, BFv>, grid, dim3(kStThreads), stream, pix, plan.hdr,   \
          plan.ns, plan.taps, (const float*)workspace, img, g.Cg, g.H, g.W, g.Cp, g.K, plan.S,    \
-         chunks, plan.pt)
+         chunks, plan.pt, gate)
   if (bf16) { if (NS == 64) PS(64, true); else if (NS == 32) PS(32, true); else PS(16, true); }
   else { if (NS == 64) PS(64, false); else if (NS == 32) PS(32, false); else PS(16, false); }
 #undef PS

@@ -308,6 +308,34 @@ def test_fused_conv_coherent_maps(ops, oracle, tc):
     assert relerr(_n(gw), ww) <= 1e-4
 
 
+@pytest.mark.parametrize("crowded", [False, True], ids=["injective", "crowded"])
+def test_nearest_scatter_inverse_map_and_its_fallback(ops, oracle, crowded):
+    """Nearest unweighted maps run the scatter contractions as a gather over the inverse map
+    when every (target, sample) pair has at most 8 sources; a crowded map (a quarter of the
+    pixels sample one spot) must take the atomic scatter kernel instead.  Same results."""
+    dt = np.float32
+    rng = np.random.default_rng(99 + crowded)
+    B, Cin, Cout, H, W, OH, OW, K = 2, 24, 40, 14, 30, 14, 30, 5
+    m = _coherent_map(rng, OH, OW, K, 0, H, W, dt)
+    if crowded:
+        sel = rng.uniform(size=(OH, OW, K)) < 0.25
+        m[sel] = np.array([7.2, 3.9], dtype=dt)
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), None, _t(x), _t(wt), _t(b), K, 0)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, 0, None)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+    bt = rng.standard_normal(Cin).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), None, _t(wtt), _t(bt), H, W, K, 0))
+    assert relerr(got, oracle.mapped_transposed_conv_forward(xt, m, wtt, bt, H, W, K, 0,
+                                                             None)) <= 1e-4
+
+
 @pytest.fixture
 def bf16_compute(ops):
     ops.set_conv_compute("bf16")
