@@ -94,12 +94,19 @@ int sdk_resample_from_map(const void* image, const void* sample_map, const void*
  * Replaces `_resample.resample_to_map` / `_weighted_resample.weighted_resample_to_map`
  * (ext_modules/include/layers/resample_layer.h:40-60,
  *  ext_modules/include/layers/weighted_resample_layer.h:49-74;
- *  device side include/cuda/resample.cuh:14-47, :87-124). */
+ *  device side include/cuda/resample.cuh:14-47, :87-124).
+ *
+ * workspace (optional, may be NULL): sdk_resample_to_map_workspace_bytes() bytes of device
+ * scratch.  With it the map is first inverted on the device (per target pixel the list of
+ * (source pixel, weight) pairs, up to 16); the scatter then runs as a gather without float
+ * atomics and without the zero fill.  If a target collects more than 16 sources the call
+ * falls back, on the device, to the atomic scatter. */
+size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_t dtype);
 int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
-                        void* out, void* weight_sum, int64_t batch, int64_t channels,
-                        int64_t map_height, int64_t map_width, int64_t height, int64_t width,
-                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                        sdk_stream_t stream);
+                        void* out, void* weight_sum, void* workspace, size_t workspace_bytes,
+                        int64_t batch, int64_t channels, int64_t map_height, int64_t map_width,
+                        int64_t height, int64_t width, int32_t num_interp_pts, int32_t interp,
+                        int32_t dtype, sdk_stream_t stream);
 
 /* data[p, i] /= (weight_sum[i] + eps) for p < planes, i < plane_size, in place.
  * The reference does this in Python for its weighted splat

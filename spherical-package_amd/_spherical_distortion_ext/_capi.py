@@ -18,7 +18,7 @@ _vp, _i64, _i32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c
 _CONV_DIMS = [_i64] * 8 + [_i32] * 4 + [_vp]
 SIGNATURES = {
     "sdk_resample_from_map": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
-    "sdk_resample_to_map": [_vp] * 5 + [_i64] * 6 + [_i32] * 3 + [_vp],
+    "sdk_resample_to_map": [_vp] * 6 + [_sz] + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_normalize_by_weight_sum": [_vp, _vp, ctypes.c_double, _i64, _i64, _i32, _vp],
     "sdk_mapped_im2col": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
@@ -32,7 +32,8 @@ SIGNATURES = {
     "sdk_mapped_transposed_conv_backward_input": [_vp] * 6 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_weight": [_vp] * 6 + [_sz] + _CONV_DIMS,
 }
-OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes")
+OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes",
+                 "sdk_resample_to_map_workspace_bytes")
 
 _lib = None
 
@@ -57,6 +58,8 @@ def load():
     lib.sdk_version.restype = ctypes.c_int
     lib.sdk_mapped_conv_workspace_bytes.argtypes = [_i64] * 8 + [_i32] * 4
     lib.sdk_mapped_conv_workspace_bytes.restype = _sz
+    lib.sdk_resample_to_map_workspace_bytes.argtypes = [_i64, _i64, _i32]
+    lib.sdk_resample_to_map_workspace_bytes.restype = _sz
     _lib = lib
     return lib
 

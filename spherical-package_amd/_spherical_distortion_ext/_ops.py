@@ -88,6 +88,14 @@ def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
 
 
+def _scatter_workspace(ref, out_h, out_w):
+    n = _capi.load().sdk_resample_to_map_workspace_bytes(int(out_h), int(out_w),
+                                                         _DTYPES[ref.dtype])
+    if n == 0:
+        return None, 0
+    return torch.empty(n, dtype=torch.uint8, device=ref.device), n
+
+
 # --------------------------------------------------------------------------- resample
 def resample_from_map(x, sample_map, interp_weights, interp):
     _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
@@ -110,9 +118,10 @@ def resample_to_map(x, sample_map, interp_weights, out_h, out_w, interp):
                            % (tuple(sample_map.shape[:2]), (MH, MW)))
     out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
+        ws, nws = _scatter_workspace(x, out_h, out_w)
         _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
-                   _ptr(out), ctypes.c_void_p(0), B, C, MH, MW, int(out_h), int(out_w), P,
-                   int(interp), _DTYPES[x.dtype], _stream(x))
+                   _ptr(out), ctypes.c_void_p(0), _ptr(ws), nws, B, C, MH, MW, int(out_h),
+                   int(out_w), P, int(interp), _DTYPES[x.dtype], _stream(x))
     return out
 
 
@@ -126,9 +135,10 @@ def resample_to_map_normalized(x, sample_map, interp_weights, out_h, out_w, inte
     out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     wsum = torch.empty((int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
+        ws, nws = _scatter_workspace(x, out_h, out_w)
         _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
-                   _ptr(out), _ptr(wsum), B, C, MH, MW, int(out_h), int(out_w), P, int(interp),
-                   _DTYPES[x.dtype], _stream(x))
+                   _ptr(out), _ptr(wsum), _ptr(ws), nws, B, C, MH, MW, int(out_h), int(out_w), P,
+                   int(interp), _DTYPES[x.dtype], _stream(x))
         _capi.call("sdk_normalize_by_weight_sum", _ptr(out), _ptr(wsum), float(eps), B * C,
                    int(out_h) * int(out_w), _DTYPES[x.dtype], _stream(x))
     return out, wsum

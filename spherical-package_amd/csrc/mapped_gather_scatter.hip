@@ -36,34 +36,43 @@ inline unsigned banded_grid_x(int64_t pixels) {
 // Fill kernels (scatter targets start from zero; hipMemsetAsync is avoided so
 // that callers may capture these entry points into a HIP graph).
 // ---------------------------------------------------------------------------
+// gate: optional device flag; a gated kernel runs only if *gate != 0.
 template <typename T>
-__global__ __launch_bounds__(kBlock) void fill_kernel(T* __restrict__ p, size_t n, T v) {
+__global__ __launch_bounds__(kBlock) void fill_kernel(T* __restrict__ p, size_t n, T v,
+                                                      const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const size_t stride = (size_t)gridDim.x * kBlock;
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) p[i] = v;
 }
 
 // 16-byte stores for the bulk of a zero fill.
-__global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p, size_t n16) {
+__global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p, size_t n16,
+                                                        const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const size_t stride = (size_t)gridDim.x * kBlock;
   const uint4 z = make_uint4(0, 0, 0, 0);
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) p[i] = z;
 }
 
+static int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream) {
+  return zero_fill_gated(ptr, bytes, stream, nullptr);
+}
+static int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate) {
   if (bytes == 0) return SDK_OK;
   // ptr comes from a framework allocator (>= 256-byte aligned) and all element
   // sizes divide 16, so only a tail of < 16 bytes needs the scalar kernel.
   const size_t n16 = ((uintptr_t)ptr % 16 == 0) ? bytes / 16 : 0;
   if (n16) {
     const int blocks = (int)std::min<size_t>(ceil_div((int64_t)n16, kBlock), 256 * 16);
-    launch(zero16_kernel, dim3(blocks), dim3(kBlock), stream, (uint4*)ptr, n16);
+    launch(zero16_kernel, dim3(blocks), dim3(kBlock), stream, (uint4*)ptr, n16, gate);
   }
   const size_t done = n16 * 16;
   if (done < bytes) {
     const size_t rest = bytes - done;
     const int blocks = (int)std::min<size_t>(ceil_div((int64_t)rest, kBlock), 256 * 16);
     launch(fill_kernel<unsigned char>, dim3(blocks), dim3(kBlock), stream,
-                       (unsigned char*)ptr + done, rest, (unsigned char)0);
+                       (unsigned char*)ptr + done, rest, (unsigned char)0, gate);
   }
   SDK_LAUNCH_CHECK("zero_fill");
   return SDK_OK;
@@ -99,7 +108,8 @@ __global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
 template <typename T, int INTERP, bool WEIGHTED, bool ONES>
 __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
-    T* __restrict__ out, int planes, int H, int W, int MP, int P) {
+    T* __restrict__ out, int planes, int H, int W, int MP, int P, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= MP) return;
   const int plane0 = blockIdx.y * kPC;
@@ -113,6 +123,73 @@ __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
   scatter_sample<T, INTERP, WEIGHTED, kPC>(out + (size_t)plane0 * HW, HW, np,
                                            map + (size_t)pix * q * 2,
                                            WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W, val);
+}
+
+
+// ---------------------------------------------------------------------------
+// resample_to_map as a gather over the inverted map.  inverse_fill: one thread per map
+// pixel appends (pixel, tap weight) to the list of every image pixel its taps hit
+// (slot = atomic counter per target; lists are [slot][target], kInvSlots long); taps that
+// find their list full raise *gate, which switches the call to the atomic scatter above.
+// inverse_gather: one thread per image pixel and 8 planes sums its list.
+// ---------------------------------------------------------------------------
+constexpr int kInvSlots = 16;
+
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void resample_inverse_fill_kernel(
+    const T* __restrict__ map, const T* __restrict__ wts, int H, int W, int MP, int P,
+    int* __restrict__ cnt, int* __restrict__ src, T* __restrict__ co, int* __restrict__ gate) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  if (pix >= MP) return;
+  const int q = WEIGHTED ? P : 1;
+  const size_t HW = (size_t)H * W;
+  PointTaps<T, INTERP> t;
+  for (int p = 0; p < q; ++p) {
+    const size_t s = (size_t)pix * q + p;
+    t.set(map[s * 2], map[s * 2 + 1], H, W);
+    const T wt = WEIGHTED ? wts[s] : T(1);
+#pragma unroll
+    for (int i = 0; i < PointTaps<T, INTERP>::N; ++i) {
+      if (t.off[i] >= 0) {
+        const int u = t.off[i];
+        const int slot = atomicAdd(&cnt[u], 1);
+        if (slot < kInvSlots) {
+          src[(size_t)slot * HW + u] = pix;
+          co[(size_t)slot * HW + u] = INTERP == 0 ? wt : t.w[i] * wt;
+        } else {
+          atomicAdd(gate, 1);
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
+    const T* __restrict__ in, const int* __restrict__ cnt, const int* __restrict__ src,
+    const T* __restrict__ co, T* __restrict__ out, T* __restrict__ wsum, int planes, int HW,
+    int MP, const int* __restrict__ gate) {
+  if (*gate != 0) return;
+  const int u = banded_pixel_block() * kBlock + threadIdx.x;
+  if (u >= HW) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const int n = min(cnt[u], kInvSlots);
+  T acc[kPC];
+#pragma unroll
+  for (int j = 0; j < kPC; ++j) acc[j] = T(0);
+  T wtot = T(0);
+  for (int s = 0; s < n; ++s) {
+    const int m = src[(size_t)s * HW + u];
+    const T c = co[(size_t)s * HW + u];
+    wtot += c;
+#pragma unroll
+    for (int j = 0; j < kPC; ++j) acc[j] += c * in[(size_t)(plane0 + (j < np ? j : 0)) * MP + m];
+  }
+#pragma unroll
+  for (int j = 0; j < kPC; ++j)
+    if (j < np) out[(size_t)(plane0 + j) * HW + u] = acc[j];
+  if (wsum != nullptr && blockIdx.y == 0) wsum[u] = wtot;
 }
 
 template <typename T>
@@ -264,26 +341,61 @@ static int launch_resample_from_map(const T* image, const T* map, const T* wts, 
   return SDK_OK;
 }
 
+static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  off[0] = 0;                                   // gate (first int), then cnt: cleared together
+  off[1] = 256;                                 // cnt
+  off[2] = off[1] + up((size_t)HW * 4);         // src
+  off[3] = off[2] + up((size_t)HW * kInvSlots * 4);   // co
+  return off[3] + up((size_t)HW * kInvSlots * esz);
+}
+
 template <typename T>
 static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
-                                  int64_t planes, int H, int W, int MP, int P, int interp,
-                                  hipStream_t stream) {
-  int rc = zero_fill(out, sizeof(T) * (size_t)planes * H * W, stream);
+                                  void* workspace, size_t workspace_bytes, int64_t planes, int H,
+                                  int W, int MP, int P, int interp, hipStream_t stream) {
+  const int HW = H * W;
+  const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
+  size_t off[4];
+  if (workspace != nullptr && workspace_bytes >= inverse_layout(HW, sizeof(T), off)) {
+    char* ws = static_cast<char*>(workspace);
+    int* g = reinterpret_cast<int*>(ws + off[0]);
+    int* cnt = reinterpret_cast<int*>(ws + off[1]);
+    int* src = reinterpret_cast<int*>(ws + off[2]);
+    T* co = reinterpret_cast<T*>(ws + off[3]);
+    int rc = zero_fill(ws, off[2], stream);
+    if (rc != SDK_OK) return rc;
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((resample_inverse_fill_kernel<T, INTERP, WEIGHTED>),
+                                dim3((unsigned)ceil_div(MP, kBlock)), dim3(kBlock), stream, map,
+                                wts, H, W, MP, P, cnt, src, co, g)));
+    SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
+    if (planes > 0 || wsum) {
+      const dim3 gridg(banded_grid_x(HW), (unsigned)std::max<int64_t>(1, ceil_div(planes, kPC)));
+      launch(resample_inverse_gather_kernel<T>, gridg, dim3(kBlock), stream, in, (const int*)cnt,
+             (const int*)src, (const T*)co, out, wsum, (int)planes, HW, MP, (const int*)g);
+      SDK_LAUNCH_CHECK("resample_to_map(inverse gather)");
+    }
+    gate = g;
+  }
+  int rc = zero_fill_gated(out, sizeof(T) * (size_t)planes * H * W, stream, gate);
   if (rc != SDK_OK) return rc;
   const dim3 grid(banded_grid_x(MP), (unsigned)ceil_div(planes, kPC));
-  SDK_DISPATCH_INTERP(interp, P,
-                      (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, false>),
-                                          grid, dim3(kBlock), stream, in, map, wts, out,
-                                          (int)planes, H, W, MP, P)));
-  SDK_LAUNCH_CHECK("resample_to_map");
+  if (planes > 0) {
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, false>), grid,
+                                dim3(kBlock), stream, in, map, wts, out, (int)planes, H, W, MP, P,
+                                gate)));
+    SDK_LAUNCH_CHECK("resample_to_map");
+  }
   if (wsum) {
-    rc = zero_fill(wsum, sizeof(T) * (size_t)H * W, stream);
+    rc = zero_fill_gated(wsum, sizeof(T) * (size_t)H * W, stream, gate);
     if (rc != SDK_OK) return rc;
     const dim3 g1(banded_grid_x(MP), 1);
     SDK_DISPATCH_INTERP(interp, P,
-                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, true>),
-                                            g1, dim3(kBlock), stream, (const T*)nullptr, map,
-                                            wts, wsum, 1, H, W, MP, P)));
+                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, true>), g1,
+                                dim3(kBlock), stream, (const T*)nullptr, map, wts, wsum, 1, H, W,
+                                MP, P, gate)));
     SDK_LAUNCH_CHECK("resample_to_map(weight_sum)");
   }
   return SDK_OK;
@@ -358,11 +470,17 @@ int sdk_resample_from_map(const void* image, const void* sample_map, const void*
   return SDK_OK;
 }
 
+size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_t dtype) {
+  if (height < 1 || width < 1 || height * width >= ((int64_t)1 << 31)) return 0;
+  size_t off[4];
+  return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off);
+}
+
 int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
-                        void* out, void* weight_sum, int64_t batch, int64_t channels,
-                        int64_t map_height, int64_t map_width, int64_t height, int64_t width,
-                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                        sdk_stream_t stream) {
+                        void* out, void* weight_sum, void* workspace, size_t workspace_bytes,
+                        int64_t batch, int64_t channels, int64_t map_height, int64_t map_width,
+                        int64_t height, int64_t width, int32_t num_interp_pts, int32_t interp,
+                        int32_t dtype, sdk_stream_t stream) {
   SDK_REQUIRE(input && sample_map && out, "resample_to_map: NULL pointer");
   SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
               "resample_to_map: weighted map needs interp_weights");
@@ -377,9 +495,9 @@ int sdk_resample_to_map(const void* input, const void* sample_map, const void* i
   if (planes == 0 && !weight_sum) return SDK_OK;
   SDK_DISPATCH_DTYPE(dtype, return launch_resample_to_map<T>(
                                 (const T*)input, (const T*)sample_map, (const T*)interp_weights,
-                                (T*)out, (T*)weight_sum, planes, (int)height, (int)width,
-                                (int)(map_height * map_width), num_interp_pts, interp,
-                                (hipStream_t)stream));
+                                (T*)out, (T*)weight_sum, workspace, workspace_bytes, planes,
+                                (int)height, (int)width, (int)(map_height * map_width),
+                                num_interp_pts, interp, (hipStream_t)stream));
   return SDK_OK;
 }
 

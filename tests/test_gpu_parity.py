@@ -76,6 +76,34 @@ def test_resample_both_directions(ops, oracle, case):
     assert relerr(_n(gotn), want / (ones + dt(1e-12))) <= 10 * BWD_TOL[dt]
 
 
+@pytest.mark.parametrize("interp,weighted", [(0, False), (1, False), (2, True)])
+def test_resample_to_map_crowded_targets_and_no_workspace(ops, oracle, interp, weighted):
+    """The scatter direction runs as a gather over the inverted map while every image pixel has
+    at most 16 sources.  A map that sends a third of its pixels to one spot must fall back to
+    the atomic scatter on the device, and a call without workspace must take it directly."""
+    from _spherical_distortion_ext import _capi
+    dt = np.float32
+    rng = np.random.default_rng(300 + interp)
+    B, C, H, W, MH, MW, P = 2, 3, 21, 33, 19, 27, 2
+    m = _coords(rng, (MH, MW, P) if weighted else (MH, MW), H, W, dt)
+    sel = rng.uniform(size=m.shape[:-1]) < 0.33
+    m[sel] = np.array([11.3, 7.6], dtype=dt)
+    iw = rng.uniform(0.1, 1, (MH, MW, P)).astype(dt) if weighted else None
+    y = rng.standard_normal((B, C, MH, MW)).astype(dt)
+    want = oracle.resample_to_map(y, m, H, W, interp, iw)
+    ones = oracle.resample_to_map(np.ones((1, 1, MH, MW), dt), m, H, W, interp, iw)[0, 0]
+    gotn, wsum = ops.resample_to_map_normalized(_t(y), _t(m), _t(iw), H, W, interp, 1e-12)
+    assert relerr(_n(wsum), ones) <= 1e-4
+    assert relerr(_n(gotn), want / (ones + dt(1e-12))) <= 1e-3
+    assert relerr(_n(ops.resample_to_map(_t(y), _t(m), _t(iw), H, W, interp)), want) <= 1e-4
+    # the same call through the C ABI without workspace
+    ty, tm, tw = _t(y), _t(m), _t(iw)
+    out = torch.empty((B, C, H, W), dtype=torch.float32, device=DEV)
+    _capi.call("sdk_resample_to_map", ops._ptr(ty), ops._ptr(tm), ops._ptr(tw), ops._ptr(out),
+               None, None, 0, B, C, MH, MW, H, W, P if weighted else 0, interp, 0, ops._stream(ty))
+    assert relerr(_n(out), want) <= 1e-4
+
+
 @pytest.mark.parametrize("case", CASES, ids=_ids)
 def test_im2col_col2im(ops, oracle, case):
     interp, weighted, dt = case
