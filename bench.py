@@ -265,7 +265,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); "
-                 "multi-GPU sharding is described in DESIGN.md, not built")
+                 "the path shards over the batch (only grad_weight / grad_bias would need an "
+                 "all-reduce), which is not built")
 
     import torch
     from _spherical_distortion_ext import _ops as ops
