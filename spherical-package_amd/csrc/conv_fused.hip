@@ -159,6 +159,60 @@ __device__ __forceinline__ void mfma_chunk_any(const float* __restrict__ As, int
     mfma_chunk(As, lda, a_base, Bs, ldb, b_base, rows, acc);
 }
 
+// The same contraction over operand tiles stored with the reduction index contiguous:
+// At[i][kLdK], Bt[j][kLdK] (kKC values per row, 4 floats of skew).  Lane half h contracts
+// rows 16h + 0..15 (fp32, four per 16-byte read) or 16t + 8h + 0..7 (bf16, instruction t),
+// so every operand fragment arrives as a 16-byte LDS read: a quarter of the LDS
+// instructions of mfma_chunk().
+constexpr int kLdK = kKC + 4;
+
+template <bool BF16>
+__device__ __forceinline__ void mfma_chunk_kc(const float* __restrict__ At, int a_base,
+                                              const float* __restrict__ Bt, int b_base,
+                                              floatx16 (&acc)[2][2]) {
+  const int lane = threadIdx.x & 63;
+  const int lk = lane >> 5, lj = lane & 31;
+  const float* a0p = At + (a_base + lj) * kLdK;
+  const float* a1p = a0p + 32 * kLdK;
+  const float* b0p = Bt + (b_base + lj) * kLdK;
+  const float* b1p = b0p + 32 * kLdK;
+  if constexpr (BF16) {
+#pragma unroll
+    for (int t = 0; t < kKC / 16; ++t) {
+      const int o = 16 * t + 8 * lk;
+      auto frag = [&](const float* p) {
+        const float4 lo = *reinterpret_cast<const float4*>(p + o);
+        const float4 hi = *reinterpret_cast<const float4*>(p + o + 4);
+        const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        return pack_bf16x8(f);
+      };
+      const Bf16Frag a0 = frag(a0p), a1 = frag(a1p), b0 = frag(b0p), b1 = frag(b1p);
+      acc[0][0] = mfma_bf16(a0, b0, acc[0][0]);
+      acc[0][1] = mfma_bf16(a0, b1, acc[0][1]);
+      acc[1][0] = mfma_bf16(a1, b0, acc[1][0]);
+      acc[1][1] = mfma_bf16(a1, b1, acc[1][1]);
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < kKC / 8; ++q) {
+      const int o = (kKC / 2) * lk + 4 * q;
+      const float4 a0 = *reinterpret_cast<const float4*>(a0p + o);
+      const float4 a1 = *reinterpret_cast<const float4*>(a1p + o);
+      const float4 b0 = *reinterpret_cast<const float4*>(b0p + o);
+      const float4 b1 = *reinterpret_cast<const float4*>(b1p + o);
+      const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+      const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[i], bv0[i], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[i], bv1[i], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[i], bv0[i], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[i], bv1[i], acc[1][1], 0, 0, 0);
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ void zero_acc(floatx16 (&acc)[2][2]) {
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -170,8 +224,11 @@ __device__ __forceinline__ void zero_acc(floatx16 (&acc)[2][2]) {
 
 // ---------------------------------------------------------------------------
 // Weight re-layout (once per call, a few hundred KB): from Wm[Cp][Cg*K] to
-//   Wg[k][c][n]  (n contiguous, padded to CgP x CpP)   for gather_gemm
-//   Ws[k][n][c]  (c contiguous, padded to CpP x CgP)   for gemm_scatter
+//   Wg[k][c][n]  (n contiguous, padded to CgP x CpP)   (n_fastest = 1)
+//   Ws[k][n][c]  (c contiguous, padded to CpP x CgP)   for gemm_scatter (n_fastest = 0)
+//   Wk[k][c / kKC][n][c % kKC]  (rows of kKC reduction values)  for gather_gemm (n_fastest = 2)
+//   Wt[k][n / kKC][c][n % kKC]  (the same with the roles of n and c exchanged: CpP pads c,
+//                                CgP pads n)                for the inverse gather (n_fastest = 3)
 // Padding is zero so the hot loops need no channel guards on the weight side.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
@@ -181,7 +238,20 @@ __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
   for (size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x; e < total;
        e += (size_t)gridDim.x * kThreads) {
     int n, c, k;
-    if (n_fastest) {
+    if (n_fastest >= 2) {
+      int red = (int)(e % kKC);
+      const int row = (int)((e / kKC) % CpP);
+      const size_t rest = e / ((size_t)kKC * CpP);   // k * (CgP / kKC) + chunk
+      red += (int)(rest % (CgP / kKC)) * kKC;
+      k = (int)(rest / (CgP / kKC));
+      if (n_fastest == 2) {
+        n = row;
+        c = red;
+      } else {
+        n = red;
+        c = row;
+      }
+    } else if (n_fastest) {
       n = (int)(e % CpP);
       c = (int)((e / CpP) % CgP);
       k = (int)(e / ((size_t)CpP * CgP));
@@ -214,9 +284,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     if (*gate != 0) return;
   }
   extern __shared__ __align__(16) unsigned char smem[];
-  float* Bs = reinterpret_cast<float*>(smem);             // [kKC][TM]
-  float* As = Bs + kKC * TM;                               // [kKC][TN]
-  int* tap_off = reinterpret_cast<int*>(As + kKC * TN);    // [slots][TM]
+  float* Bs = reinterpret_cast<float*>(smem);             // [TM][kLdK] columns, reduction index contiguous
+  float* As = Bs + TM * kLdK;                              // [TN][kLdK] weights
+  int* tap_off = reinterpret_cast<int*>(As + TN * kLdK);   // [slots][TM]
   float* tap_co = reinterpret_cast<float*>(tap_off + slots * TM);
   int* smax = reinterpret_cast<int*>(tap_co + slots * TM);
 
@@ -282,15 +352,18 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
         }
       }
 #pragma unroll
-      for (int j = 0; j < RPT; ++j) Bs[(gpart * RPT + j) * TM + gm] = col[j];
-      // ---- weight tile As[r][n] = Wg[k][c0 + r][n0 + n]
-      const float4* src = reinterpret_cast<const float4*>(Wg + ((size_t)k * CgP + c0) * CpP + n0);
-      for (int e = tid; e < kKC * TN / 4; e += kThreads) {
-        const int r = e / (TN / 4), n4 = e % (TN / 4);
-        reinterpret_cast<float4*>(As)[e] = src[(size_t)r * (CpP / 4) + n4];
+      for (int j = 0; j < RPT; j += 4)
+        *reinterpret_cast<float4*>(Bs + gm * kLdK + gpart * RPT + j) =
+            make_float4(col[j], col[j + 1], col[j + 2], col[j + 3]);
+      // ---- weight tile As[n][r] = Wk[k][c0 / kKC][n0 + n][r]
+      const float4* src = reinterpret_cast<const float4*>(
+          Wg + (((size_t)k * (CgP / kKC) + c0 / kKC) * CpP + n0) * kKC);
+      for (int e = tid; e < TN * kKC / 4; e += kThreads) {
+        const int n = e / (kKC / 4), r4 = e % (kKC / 4);
+        *reinterpret_cast<float4*>(As + n * kLdK + 4 * r4) = src[e];
       }
       __syncthreads();
-      mfma_chunk_any<BF16>(As, TN, a_base, Bs, TM, b_base, kKC, acc);
+      mfma_chunk_kc<BF16>(As, a_base, Bs, b_base, acc);
       __syncthreads();
     }
   }
@@ -532,11 +605,11 @@ size_t fused_workspace_bytes(const ConvGeom& g) {
 }
 
 static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
-                    bool n_fastest, hipStream_t stream) {
+                    int n_fastest, hipStream_t stream) {
   const size_t total = (size_t)g.K * CpP * CgP;
   const int blocks = (int)std::min<size_t>((total + kThreads - 1) / kThreads, 2048);
   launch(relayout_weight_kernel, dim3(blocks), dim3(kThreads), stream, Wm, out, g.Cp, g.Cg, g.K,
-         CpP, CgP, n_fastest ? 1 : 0);
+         CpP, CgP, n_fastest);
   SDK_LAUNCH_CHECK("relayout_weight");
   return SDK_OK;
 }
@@ -564,11 +637,11 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
   const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
   const int CpP = round_up(g.Cp, TN), CgP = round_up(g.Cg, kKC);
-  int rc = relayout(g, Wm, workspace, CpP, CgP, true, stream);
+  int rc = relayout(g, Wm, workspace, CpP, CgP, 2, stream);
   if (rc) return rc;
   const int m_tiles = (int)ceil_div(g.M, TM), n_tiles = CpP / TN;
   const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
-  const size_t smem = sizeof(float) * (kKC * TM + kKC * TN) + (size_t)slots * TM * 8 + 16;
+  const size_t smem = sizeof(float) * kLdK * (TM + TN) + (size_t)slots * TM * 8 + 16;
 #define GG(TNv, TMv, BFv)                                                                          \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                          \
                       (rc = launch_smem("gather_gemm",                                        \
@@ -723,12 +796,12 @@ static int inverse_gather_gemm(const ConvGeom& g, bool bf16, const InverseMap& i
   const bool narrow = g.Cg <= 64;
   const int TN = narrow ? 64 : 128, TM = inv.TM;
   const int CoutP = round_up(g.Cg, TN), CinP = round_up(g.Cp, kKC);
-  int rc = relayout(g, Wm, inv.weights, CinP, CoutP, false, stream);
+  int rc = relayout(g, Wm, inv.weights, CoutP, CinP, 3, stream);
   if (rc) return rc;
   const int HW = g.H * g.W;
   const int m_tiles = inv.tiles, n_tiles = CoutP / TN;
   const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
-  const size_t smem = sizeof(float) * (kKC * TM + kKC * TN) + (size_t)kInvSlots * TM * 8 + 16;
+  const size_t smem = sizeof(float) * kLdK * (TM + TN) + (size_t)kInvSlots * TM * 8 + 16;
 #define IG(TNv, TMv, BFv)                                                                        \
   rc = launch_smem("inverse_gather_gemm", gather_gemm_kernel<0, false, TNv, TMv, BFv, true>, grid, \
                    smem, stream, pix, (const float*)nullptr, (const float*)nullptr,              \
