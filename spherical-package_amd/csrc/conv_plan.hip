@@ -15,8 +15,13 @@ constexpr int kPlThreads = 256;
 // ---------------------------------------------------------------------------
 // Plan construction: one workgroup per tile.  Thread = (pixel of the tile,
 // parity of the kernel sample).  Pass 1 finds the bounding box of all active
-// taps and the per-sample row counts, pass 2 writes the encoded rows.
+// taps and the per-sample row counts, pass 2 writes the encoded rows.  When the
+// tile's part of the map (128 pixels x K samples x points, 12 bytes each with
+// the point weights) fits kPlanStage bytes it is first copied to LDS with
+// coalesced reads; both passes then read LDS instead of striding through HBM.
 // ---------------------------------------------------------------------------
+constexpr int kPlanStage = 56 * 1024;
+
 template <int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     const float* __restrict__ map, const float* __restrict__ wts, PixelTiling pt, int K, int P,
@@ -24,6 +29,7 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     int2* __restrict__ taps) {
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
+  __shared__ __align__(8) float stage[kPlanStage / sizeof(float)];
   const int tid = threadIdx.x, lane = tid & 63;
   const int tile = blockIdx.x;
   const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
@@ -38,6 +44,41 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
   const int ax = wrap_index(to_int_clamped(round_t(map[s0 * 2])), W);
   const int ay = min(max(to_int_clamped(round_t(map[s0 * 2 + 1])), 0), H - 1);
 
+  // ---- stage the tile's coordinates (and point weights): per tile pixel K*q (x, y) pairs
+  const int per_pix = K * q;   // samples x points of one pixel
+  const bool staged = (size_t)128 * per_pix * (WEIGHTED ? 12 : 8) <= (size_t)kPlanStage;
+  float* st_xy = stage;                      // [128][per_pix][2]
+  float* st_w = stage + 128 * per_pix * 2;   // [128][per_pix]
+  if (staged) {
+    const int run = per_pix * 2;   // floats per pixel
+    for (int i = tid; i < 128 * run; i += kPlThreads) {
+      const int pl = i / run, o = i - pl * run;
+      const int py = ty0 + (pl >> pt.tx_shift), px = tx0 + (pl & (pt.TX() - 1));
+      st_xy[i] = (py < pt.OH && px < pt.OW) ? map[((size_t)py * pt.OW + px) * run + o] : 0.0f;
+    }
+    if constexpr (WEIGHTED) {
+      for (int i = tid; i < 128 * per_pix; i += kPlThreads) {
+        const int pl = i / per_pix, o = i - pl * per_pix;
+        const int py = ty0 + (pl >> pt.tx_shift), px = tx0 + (pl & (pt.TX() - 1));
+        st_w[i] = (py < pt.OH && px < pt.OW) ? wts[((size_t)py * pt.OW + px) * per_pix + o] : 0.0f;
+      }
+    }
+  }
+  // sample point (x, y, weight) of this thread's pixel
+  auto point = [&](int k, int pp, float& x, float& y, float& w) {
+    if (staged) {
+      const int o = p * per_pix + k * q + pp;
+      x = st_xy[2 * o];
+      y = st_xy[2 * o + 1];
+      w = WEIGHTED ? st_w[o] : 1.0f;
+    } else {
+      const size_t sidx = (((size_t)oy * pt.OW + ox) * K + k) * q + pp;
+      x = map[sidx * 2];
+      y = map[sidx * 2 + 1];
+      w = WEIGHTED ? wts[sidx] : 1.0f;
+    }
+  };
+
   for (int k = tid; k < K; k += kPlThreads) ns_l[k] = 0;
   if (tid == 0) {
     bb[0] = INT_MAX;
@@ -47,15 +88,15 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
   }
   __syncthreads();
 
-  const size_t base = ((size_t)oy * pt.OW + ox) * K;
   Taps2D<INTERP> t;
   int dy0 = INT_MAX, dy1 = INT_MIN, dx0 = INT_MAX, dx1 = INT_MIN;
   for (int k = kpar; k < K; k += 2) {
     int cnt = 0;
     if (pix_ok) {
       for (int pp = 0; pp < q; ++pp) {
-        const size_t s = (base + k) * q + pp;
-        t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
+        float sx, sy, sw;
+        point(k, pp, sx, sy, sw);
+        t.set(sx, sy, H, W, sw);
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
           if (t.w[i] != 0.0f) {
@@ -100,8 +141,9 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     int cnt = 0;
     if (pix_ok) {
       for (int pp = 0; pp < q; ++pp) {
-        const size_t s = (base + k) * q + pp;
-        t.set(map[s * 2], map[s * 2 + 1], H, W, WEIGHTED ? wts[s] : 1.0f);
+        float sx, sy, sw;
+        point(k, pp, sx, sy, sw);
+        t.set(sx, sy, H, W, sw);
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
           if (t.w[i] != 0.0f) {
