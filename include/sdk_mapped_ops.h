@@ -233,6 +233,21 @@ int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_
 int sdk_bias_grad(const void* grad_output, void* grad_bias, int64_t batch, int64_t channels,
                   int64_t pixels, int32_t dtype, sdk_stream_t stream);
 
+/* All three gradients of one layer call: grad_input, grad_weight and grad_bias as the
+ * three entry points above compute them, with the map resolved once for both contractions.
+ * Replaces `_mapped_convolution.mapped_conv_backward` /
+ * `_weighted_mapped_convolution.weighted_mapped_conv_backward`, which return the three
+ * tensors from one call (ext_modules/include/layers/mapped_convolution_layer.h:89-134,
+ *  weighted_mapped_convolution_layer.h:103-153). */
+int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
+                             const void* interp_weights, const void* input, const void* weight,
+                             void* grad_input, void* grad_weight, void* grad_bias,
+                             void* workspace, size_t workspace_bytes, int64_t batch,
+                             int64_t in_channels, int64_t height, int64_t width,
+                             int64_t out_channels, int64_t out_height, int64_t out_width,
+                             int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                             int32_t dtype, int32_t compute, sdk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mapped transposed convolution.  weight [Cin, Cout, K]; bias [Cout];
  * input [B,Cin,IH,IW]; sample_map [IH,IW,K,(P,)2] pointing into the
@@ -273,6 +288,20 @@ int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const vo
                                                int64_t kernel_size, int32_t num_interp_pts,
                                                int32_t interp, int32_t dtype, int32_t compute,
                                                sdk_stream_t stream);
+
+/* All three gradients of one transposed layer call.  Replaces
+ * `_mapped_transposed_convolution.mapped_transposed_conv_backward` and its weighted twin
+ * (ext_modules/include/layers/mapped_transposed_convolution_layer.h:92-140). */
+int sdk_mapped_transposed_conv_backward(const void* grad_output, const void* sample_map,
+                                        const void* interp_weights, const void* input,
+                                        const void* weight, void* grad_input, void* grad_weight,
+                                        void* grad_bias, void* workspace, size_t workspace_bytes,
+                                        int64_t batch, int64_t in_channels, int64_t in_height,
+                                        int64_t in_width, int64_t out_channels,
+                                        int64_t out_height, int64_t out_width,
+                                        int64_t kernel_size, int32_t num_interp_pts,
+                                        int32_t interp, int32_t dtype, int32_t compute,
+                                        sdk_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -28,6 +28,8 @@ SIGNATURES = {
     "sdk_mapped_conv_backward_input": [_vp] * 6 + [_sz] + _CONV_DIMS,
     "sdk_mapped_conv_backward_weight": [_vp] * 6 + [_sz] + _CONV_DIMS,
     "sdk_bias_grad": [_vp, _vp, _i64, _i64, _i64, _i32, _vp],
+    "sdk_mapped_conv_backward": [_vp] * 9 + [_sz] + _CONV_DIMS,
+    "sdk_mapped_transposed_conv_backward": [_vp] * 9 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_forward": [_vp] * 7 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_input": [_vp] * 6 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_weight": [_vp] * 6 + [_sz] + _CONV_DIMS,

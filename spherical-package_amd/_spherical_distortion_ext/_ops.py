@@ -263,11 +263,9 @@ def mapped_conv_backward(grad_output, sample_map, interp_weights, x, weight, bia
         ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
-        _capi.call("sdk_mapped_conv_backward_input", _ptr(grad_output), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(weight), _ptr(gi), _ptr(ws), nws, *dims)
-        _capi.call("sdk_mapped_conv_backward_weight", _ptr(grad_output), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(x), _ptr(gw), _ptr(ws), nws, *dims)
-        _capi.call("sdk_bias_grad", _ptr(grad_output), _ptr(gb), B, Cout, OH * OW, dt, s)
+        _capi.call("sdk_mapped_conv_backward", _ptr(grad_output), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
+                   _ptr(ws), nws, *dims)
     return gi, gw, gb
 
 
@@ -309,13 +307,9 @@ def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, 
         ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
-        _capi.call("sdk_mapped_transposed_conv_backward_input", _ptr(grad_output),
-                   _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(gi), _ptr(ws), nws,
-                   *dims)
-        _capi.call("sdk_mapped_transposed_conv_backward_weight", _ptr(grad_output),
-                   _ptr(sample_map), _ptr(interp_weights), _ptr(x), _ptr(gw), _ptr(ws), nws,
-                   *dims)
-        _capi.call("sdk_bias_grad", _ptr(grad_output), _ptr(gb), B, Cout, OH * OW, dt, s)
+        _capi.call("sdk_mapped_transposed_conv_backward", _ptr(grad_output), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
+                   _ptr(ws), nws, *dims)
     return gi, gw, gb
 
 

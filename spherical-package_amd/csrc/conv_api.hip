@@ -48,7 +48,7 @@ enum Op { GATHER_GEMM, GEMM_SCATTER, GATHER_WGRAD };
 // a: pixel-side tensor for GEMM_SCATTER / GATHER_WGRAD inputs, image otherwise (see call sites).
 int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, const void* in0,
         const void* map, const void* wts, const void* in1, const void* bias, void* out, void* ws,
-        size_t ws_bytes, hipStream_t stream) {
+        size_t ws_bytes, hipStream_t stream, SharedPlan* shared = nullptr) {
   if (g.B == 0 && op != GATHER_WGRAD) return SDK_OK;
   if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(g)) {
     int rc = check_workspace(what, fused_workspace_bytes(g), ws, ws_bytes);
@@ -61,10 +61,10 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
                                  (const float*)bias, (float*)out, (float*)ws, stream);
       case GEMM_SCATTER:
         return fused_gemm_scatter(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                  (const float*)bias, (float*)out, (float*)ws, stream);
+                                  (const float*)bias, (float*)out, (float*)ws, stream, shared);
       case GATHER_WGRAD:
         return fused_gather_wgrad(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                  (float*)out, (float*)ws, stream);
+                                  (float*)out, (float*)ws, stream, shared);
     }
   }
   if (compute == SDK_COMPUTE_BF16)
@@ -241,6 +241,60 @@ int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const vo
              (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GATHER_WGRAD, g, dtype, compute, input, sample_map, interp_weights,
              grad_output, nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
+                             const void* interp_weights, const void* input, const void* weight,
+                             void* grad_input, void* grad_weight, void* grad_bias,
+                             void* workspace, size_t workspace_bytes, int64_t batch,
+                             int64_t in_channels, int64_t height, int64_t width,
+                             int64_t out_channels, int64_t out_height, int64_t out_width,
+                             int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                             int32_t dtype, int32_t compute, sdk_stream_t stream) {
+  const char* what = "mapped_conv_backward";
+  SDK_REQUIRE(grad_output && sample_map && input && weight && grad_input && grad_weight &&
+                  grad_bias,
+              "%s: NULL pointer", what);
+  SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
+  const int64_t M = out_height * out_width;
+  int rc = check_common(what, batch, in_channels, height, width, out_channels, M, kernel_size,
+                        num_interp_pts, interp_weights, dtype, compute);
+  if (rc) return rc;
+  ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
+             (int)kernel_size, num_interp_pts, interp, (int)out_width};
+  SharedPlan shared;   // the tap plan of the map is built once for both contractions
+  rc = run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
+           nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared);
+  if (rc) return rc;
+  rc = run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
+           nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, &shared);
+  if (rc) return rc;
+  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, stream);
+}
+
+int sdk_mapped_transposed_conv_backward(const void* grad_output, const void* sample_map,
+                                        const void* interp_weights, const void* input,
+                                        const void* weight, void* grad_input, void* grad_weight,
+                                        void* grad_bias, void* workspace, size_t workspace_bytes,
+                                        int64_t batch, int64_t in_channels, int64_t in_height,
+                                        int64_t in_width, int64_t out_channels,
+                                        int64_t out_height, int64_t out_width,
+                                        int64_t kernel_size, int32_t num_interp_pts,
+                                        int32_t interp, int32_t dtype, int32_t compute,
+                                        sdk_stream_t stream) {
+  int rc = sdk_mapped_transposed_conv_backward_input(
+      grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes,
+      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
+      num_interp_pts, interp, dtype, compute, stream);
+  if (rc) return rc;
+  rc = sdk_mapped_transposed_conv_backward_weight(
+      grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes,
+      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
+      num_interp_pts, interp, dtype, compute, stream);
+  if (rc) return rc;
+  SDK_REQUIRE(grad_bias, "mapped_transposed_conv_backward: NULL pointer");
+  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype,
+                       stream);
 }
 
 }  // extern "C"

@@ -816,7 +816,7 @@ static int inverse_gather_gemm(const ConvGeom& g, bool bf16, const InverseMap& i
 
 int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* Wm, const float* bias, float* img,
-                       float* workspace, hipStream_t stream) {
+                       float* workspace, hipStream_t stream, SharedPlan* shared) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
   if (rc) return rc;
@@ -835,7 +835,7 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
       if (rc) return rc;
       gate = inv.gate;
     }
-    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream);
+    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream, shared);
   }
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
@@ -861,12 +861,14 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
 
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* img, float* gW, float* workspace,
-                       hipStream_t stream) {
+                       hipStream_t stream, const SharedPlan* shared) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
   if (planned_wgrad_supported(g)) {
+    if (shared != nullptr && shared->valid)
+      return planned_wgrad(g, bf16, shared->plan, pix, img, gW, stream);
     Plan plan;
     rc = build_plan(g, map, wts, workspace, stream, &plan);
     if (rc) return rc;

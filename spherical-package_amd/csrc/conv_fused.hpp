@@ -3,8 +3,16 @@
 #include <hip/hip_runtime.h>
 
 #include "conv_internal.hpp"
+#include "conv_plan.hpp"
 
 namespace sdk {
+
+// A tap plan handed from one contraction of a call to the next (backward-input builds it,
+// backward-weight of the same call reuses it).
+struct SharedPlan {
+  bool valid = false;
+  Plan plan;
+};
 
 // True when the fused kernels cover this geometry.
 bool fused_supported(const ConvGeom& g);
@@ -15,12 +23,14 @@ size_t fused_workspace_bytes(const ConvGeom& g);
 int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
                       const float* wts, const float* Wm, const float* bias, float* pix,
                       float* workspace, hipStream_t stream);
+// shared (optional): gemm_scatter stores the plan it built there; gather_wgrad uses a valid one
+// instead of building its own (same map, weights and geometry, same workspace still alive).
 int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* Wm, const float* bias, float* img,
-                       float* workspace, hipStream_t stream);
+                       float* workspace, hipStream_t stream, SharedPlan* shared = nullptr);
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* img, float* gW, float* workspace,
-                       hipStream_t stream);
+                       hipStream_t stream, const SharedPlan* shared = nullptr);
 
 // Bytes of the permuted weight copy the plan-driven scatter kernel reads.
 size_t staged_workspace_bytes(const ConvGeom& g);
@@ -30,6 +40,6 @@ size_t staged_workspace_bytes(const ConvGeom& g);
 bool planned_scatter_supported(const ConvGeom& g);
 int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
                          const float* wts, const float* Wm, float* img, float* workspace,
-                         const int* gate, hipStream_t stream);
+                         const int* gate, hipStream_t stream, SharedPlan* shared = nullptr);
 
 }  // namespace sdk

@@ -288,7 +288,7 @@ bool planned_scatter_supported(const ConvGeom& g) {
 // workspace: permuted weights (staged_workspace_bytes, 256-byte aligned) followed by the plan
 int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const float* map,
                          const float* wts, const float* Wm, float* img, float* workspace,
-                         const int* gate, hipStream_t stream) {
+                         const int* gate, hipStream_t stream, SharedPlan* shared) {
   const int NS = g.Cp > 64 ? 64 : (g.Cp > 32 ? 32 : 16);   // MFMA steps: 2 channels each
   const int chunks = (int)ceil_div(g.Cg, kCC);
   {
@@ -302,6 +302,10 @@ int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const f
   char* plan_ws = reinterpret_cast<char*>(workspace) + ((staged_workspace_bytes(g) + 255) & ~(size_t)255);
   int rc = build_plan(g, map, wts, plan_ws, stream, &plan);
   if (rc) return rc;
+  if (shared != nullptr) {
+    shared->plan = plan;
+    shared->valid = true;
+  }
   const dim3 grid((unsigned)plan.tiles, (unsigned)g.B);
 #define PS(NSv, BFv)                                                                             \
   launch(planned_gemm_scatter_kernel<NSv, BFv>, grid, dim3(kStThreads), stream, pix, plan.hdr,   \
