@@ -195,22 +195,41 @@ SDK_INSTANTIATE(float)
 SDK_INSTANTIATE(double)
 
 // ---------------------------------------------------------------------------
-// grad_bias[c] = sum_{b,i} gout[b,c,i].  grid (C, S): every block reduces one
-// slice of channel c and adds its partial sum atomically.
+// grad_bias[c] = sum_{b,i} gout[b,c,i].  grid (C, B * slices): every block reduces one
+// contiguous slice of one plane (b, c), with 16-byte loads where the slice allows, and adds
+// its partial sum atomically.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void bias_grad_kernel(const T* __restrict__ gout,
-                                                        T* __restrict__ gbias, int B, int C,
-                                                        int M, int per_block) {
+                                                        T* __restrict__ gbias, int C, int M,
+                                                        int slices, int per_block) {
   const int c = blockIdx.x;
-  const int64_t total = (int64_t)B * M;
-  const int64_t beg = (int64_t)blockIdx.y * per_block;
-  const int64_t end = min(total, beg + per_block);
+  const int b = blockIdx.y / slices, sl = blockIdx.y % slices;
+  const int beg = sl * per_block, end = min(M, beg + per_block);
+  const T* p = gout + ((size_t)b * C + c) * M;
+  constexpr int V = 16 / (int)sizeof(T);   // elements per 16-byte load
   T acc = T(0);
-  for (int64_t e = beg + threadIdx.x; e < end; e += 256) {
-    const int64_t b = e / M, i = e % M;
-    acc += gout[(b * C + c) * (int64_t)M + i];
+  int e = beg;
+  if (((reinterpret_cast<uintptr_t>(p) + (size_t)beg * sizeof(T)) & 15) == 0) {
+    T a0 = T(0), a1 = T(0), a2 = T(0), a3 = T(0);
+    const int nv = (end - beg) / V;
+    for (int i = threadIdx.x; i < nv; i += 256) {
+      if constexpr (V == 4) {
+        const float4 v = reinterpret_cast<const float4*>(p + beg)[i];
+        a0 += v.x;
+        a1 += v.y;
+        a2 += v.z;
+        a3 += v.w;
+      } else {
+        const double2 v = reinterpret_cast<const double2*>(p + beg)[i];
+        a0 += v.x;
+        a1 += v.y;
+      }
+    }
+    acc = (a0 + a1) + (a2 + a3);
+    e = beg + nv * V;
   }
+  for (int i = e + threadIdx.x; i < end; i += 256) acc += p[i];
   // wave64 butterfly, then one LDS slot per wave
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
   __shared__ T part[4];
@@ -224,15 +243,16 @@ int launch_bias_grad(const T* gout, T* gbias, int64_t B, int64_t C, int64_t M,
                      hipStream_t stream) {
   int rc = zero_fill(gbias, sizeof(T) * (size_t)C, stream);
   if (rc) return rc;
-  const int64_t total = B * M;
-  if (total == 0 || C == 0) return SDK_OK;
-  int64_t slices = std::min<int64_t>(std::max<int64_t>(1, ceil_div(4096, C)),
-                                     ceil_div(total, 4096));
-  slices = std::min<int64_t>(slices, 65535);
-  const int per_block = (int)ceil_div(total, slices);
-  slices = ceil_div(total, per_block);
-  launch(bias_grad_kernel<T>, dim3((unsigned)C, (unsigned)slices), dim3(256),
-                     stream, gout, gbias, (int)B, (int)C, (int)M, per_block);
+  if (B * M == 0 || C == 0) return SDK_OK;
+  // about 8192 blocks overall, at least 4096 elements each; slices of a multiple of 4 elements
+  int64_t slices = std::min<int64_t>(std::max<int64_t>(1, ceil_div(8192, C * B)),
+                                     std::max<int64_t>(1, M / 4096));
+  int64_t per_block = ceil_div(ceil_div(M, slices), 4) * 4;
+  slices = ceil_div(M, per_block);
+  if (B * slices > 65535)
+    return fail(SDK_ERR_UNSUPPORTED, "bias_grad: batch %lld too large", (long long)B);
+  launch(bias_grad_kernel<T>, dim3((unsigned)C, (unsigned)(B * slices)), dim3(256), stream, gout,
+         gbias, (int)C, (int)M, (int)slices, (int)per_block);
   SDK_LAUNCH_CHECK("bias_grad");
   return SDK_OK;
 }
