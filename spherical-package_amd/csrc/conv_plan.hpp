@@ -17,7 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include "conv_internal.hpp"
-#include "conv_staged.hpp"
+#include "conv_window.hpp"
 
 namespace sdk {
 

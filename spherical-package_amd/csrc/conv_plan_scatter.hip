@@ -10,7 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include "conv_fused.hpp"
-#include "conv_staged.hpp"
+#include "conv_window.hpp"
 #include "conv_plan.hpp"
 #include "sdk_host.hpp"
 #include "sdk_mfma.hpp"

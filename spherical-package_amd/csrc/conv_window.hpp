@@ -1,4 +1,4 @@
-// Building blocks of the LDS-staged convolution kernels (conv_staged.hip, conv_plan.hip):
+// Building blocks of the LDS-staged convolution kernels (conv_plan_scatter.hip, conv_plan.hip):
 // 2-D taps, the per-workgroup image region and its addressing.
 //
 // A workgroup owns a small 2-D tile of map pixels.  The union of everything its

@@ -298,6 +298,7 @@ PLAN_CASES = [
     (12, 140, 9, 50, 3, 50, 3, 2, 1, 1.0),      # few rows; more than 128 pixel-side channels
     (8, 8, 10, 10, 10, 10, 2, 10, 1, 1.0),      # 40 tap slots per sample: generic path
     (8, 8, 10, 10, 10, 10, 2, 10, 0, 1.0),      # 10 slots, nearest weighted
+    (4, 6, 6, 7, 6, 7, 260, 0, 1, 1.0),         # more kernel samples than a plan holds
 ]
 
 
