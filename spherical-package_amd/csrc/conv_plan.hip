@@ -188,7 +188,10 @@ constexpr int kRowCap = 36;           // plan rows of one half held in LDS at a 
 // channels of its group for one element as two 16-byte accesses; 8 lanes on consecutive
 // elements are 144 bytes apart and cover all 32 banks once.
 
-template <int KB, bool BF16>
+// NW: 32-row blocks of pixel-side channels per workgroup (4, 2 or 1).  With NW < 4 the waves
+// also split the 64 pixels of a half tile (4 / NW ways), so narrow layers waste no MFMAs on
+// padding; waves that share rows add their partial sums to gW independently.
+template <int KB, bool BF16, int NW>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW, int Cg,
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
   const int cc = (kind / (kblocks * n_tiles)) % c_chunks;
   const int batch = kind / (kblocks * n_tiles * c_chunks);
   const int k0 = kb * KB, kcount = min(KB, K - k0);
-  const int c0 = cc * kCC, n0 = nt * 128;
+  const int c0 = cc * kCC, n0 = nt * (32 * NW);
   const int M = pt.OH * pt.OW;
   const size_t HW = (size_t)H * W;
   const float* img_b = img + ((size_t)batch * Cg) * HW;
@@ -223,7 +226,11 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
   const int px16 = lane & 15, cg = lane >> 4;
   const int m_local = wave * 16 + px16;
   const int nl = lane & 31, h = lane >> 5;
-  const int n_row = n0 + 32 * wave + nl;
+  constexpr int PSPLIT = 4 / NW;         // waves sharing a row block split the pixels
+  constexpr int PXW = 64 / PSPLIT;       // pixels of a half tile per wave
+  const int nbw = wave % NW;             // this wave's row block
+  const int poff = (wave / NW) * PXW;    // ... and its first pixel inside a half tile
+  const int n_row = n0 + 32 * nbw + nl;
   const bool n_ok = n_row < Cp;
   const float* pix_row = pix_b + (size_t)(n_ok ? n_row : 0) * M;
 
@@ -292,14 +299,14 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
       // ---- A fragments of this lane's row n for the 64 pixels of the half
-      float afrag[BF16 ? 1 : 32];
-      Bf16Frag afrag16[BF16 ? 4 : 1];
+      float afrag[BF16 ? 1 : PXW / 2];
+      Bf16Frag afrag16[BF16 ? PXW / 16 : 1];
       {
-        constexpr int GROUPS = BF16 ? 4 : 8;   // groups of 8 consecutive pixels per lane half ...
-        constexpr int RUN = BF16 ? 8 : 4;      // ... of which this lane holds RUN
+        constexpr int GROUPS = BF16 ? PXW / 16 : PXW / 8;   // groups of pixels per lane half ...
+        constexpr int RUN = BF16 ? 8 : 4;                   // ... of which this lane holds RUN
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
-          const int p0 = half * 64 + (BF16 ? 16 * g + 8 * h : 8 * g + 4 * h);
+          const int p0 = half * 64 + poff + (BF16 ? 16 * g + 8 * h : 8 * g + 4 * h);
           float f[RUN];
           if (vec4) {
             const int m0 = pixel_index(p0);
@@ -409,18 +416,19 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
           auto mma = [&](floatx16& d) {
             if constexpr (BF16) {
 #pragma unroll
-              for (int t = 0; t < 4; ++t) {
-                const float4 lo = *reinterpret_cast<const float4*>(bt + ((16 * t + 8 * h) ^ sw));
-                const float4 hi = *reinterpret_cast<const float4*>(bt + ((16 * t + 8 * h + 4) ^ sw));
+              for (int t = 0; t < PXW / 16; ++t) {
+                const float4 lo = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h) ^ sw));
+                const float4 hi = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h + 4) ^ sw));
                 const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
                 d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
               }
             } else {
-              float4 b = *reinterpret_cast<const float4*>(bt + ((4 * h) ^ sw));
+              float4 b = *reinterpret_cast<const float4*>(bt + ((poff + 4 * h) ^ sw));
 #pragma unroll
-              for (int g = 0; g < 8; ++g) {
+              for (int g = 0; g < PXW / 8; ++g) {
                 float4 bn = b;
-                if (g < 7) bn = *reinterpret_cast<const float4*>(bt + ((8 * (g + 1) + 4 * h) ^ sw));
+                if (g < PXW / 8 - 1)
+                  bn = *reinterpret_cast<const float4*>(bt + ((poff + 8 * (g + 1) + 4 * h) ^ sw));
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 0], b.x, d, 0, 0, 0);
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 1], b.y, d, 0, 0, 0);
                 d = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * g + 2], b.z, d, 0, 0, 0);
@@ -447,7 +455,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
       if (kk < kcount) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int n = n0 + 32 * wave + 8 * (v >> 2) + 4 * h + (v & 3);
+          const int n = n0 + 32 * nbw + 8 * (v >> 2) + 4 * h + (v & 3);
           if (n < Cp)
             atomic_add_noret(gW + (size_t)n * Cg * K + (size_t)c * K + k0 + kk, acc[kk][v]);
         }
@@ -525,7 +533,8 @@ int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* p
   const int per = (int)ceil_div(g.K, kblocks);
   const int KB = per <= 1 ? 1 : (per <= 4 ? 4 : (per <= 7 ? 7 : 9));
   const int kb_count = (int)ceil_div(g.K, KB);
-  const int c_chunks = (int)ceil_div(g.Cg, kCC), n_tiles = (int)ceil_div(g.Cp, 128);
+  const int NW = g.Cp > 64 ? 4 : (g.Cp > 32 ? 2 : 1);
+  const int c_chunks = (int)ceil_div(g.Cg, kCC), n_tiles = (int)ceil_div(g.Cp, 32 * NW);
   const int64_t kinds = (int64_t)c_chunks * n_tiles * kb_count * g.B;
   // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall
   int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, kinds), 8) * 8);
@@ -538,16 +547,21 @@ int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* p
   const int vec4 = (g.OW % 4 == 0 && TX >= (bf16 ? 8 : 4) &&
                     reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)slots);
+#define PW3(KBv, BFv, NWv)                                                                      \
+  launch(planned_wgrad_kernel<KBv, BFv, NWv>, grid, dim3(kPlThreads), stream, pix, img,         \
+         plan.hdr, plan.ns, plan.taps, gW, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt,          \
+         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4)
 #define PW(KBv, BFv)                                                                            \
-  launch(planned_wgrad_kernel<KBv, BFv>, grid, dim3(kPlThreads), stream, pix, img, plan.hdr,    \
-         plan.ns, plan.taps, gW, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, plan.tiles,        \
-         groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4)
+  do {                                                                                          \
+    if (NW == 4) PW3(KBv, BFv, 4); else if (NW == 2) PW3(KBv, BFv, 2); else PW3(KBv, BFv, 1);   \
+  } while (0)
   if (bf16) {
     if (KB == 1) PW(1, true); else if (KB == 4) PW(4, true); else if (KB == 7) PW(7, true); else PW(9, true);
   } else {
     if (KB == 1) PW(1, false); else if (KB == 4) PW(4, false); else if (KB == 7) PW(7, false); else PW(9, false);
   }
 #undef PW
+#undef PW3
   SDK_LAUNCH_CHECK("planned_wgrad");
   return SDK_OK;
 }
