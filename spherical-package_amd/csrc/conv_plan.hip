@@ -191,6 +191,12 @@ constexpr int kRowCap = 36;           // plan rows of one half held in LDS at a 
 // NW: 32-row blocks of pixel-side channels per workgroup (4, 2 or 1).  With NW < 4 the waves
 // also split the 64 pixels of a half tile (4 / NW ways), so narrow layers waste no MFMAs on
 // padding; waves that share rows add their partial sums to gW independently.
+// Workgroup barrier that orders LDS traffic only: global loads issued before it may still be
+// in flight afterwards (__syncthreads() would wait for them too).
+__device__ __forceinline__ void lds_only_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int KB, bool BF16, int NW>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
@@ -354,6 +360,15 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
         __syncthreads();
 
         int row0 = 0;
+        // Image values of the next sample's first row, for lanes whose tap lies outside the
+        // window: requested one sample ahead so that they arrive during the MFMAs (maps without
+        // locality, e.g. mesh neighbourhoods, have all their taps there).
+        // (The variant with nine fp32 accumulators of 128 rows has no registers left for it.)
+        constexpr bool PRE = !(KB == 9 && NW == 4 && !BF16);
+        float pre[8];
+        bool pre_valid = false;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pre[j] = 0.0f;
 #pragma unroll 1
         for (int kk = kk_beg; kk < kk_end; ++kk) {
           const int nrows = ns_l[kk];
@@ -380,7 +395,23 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
               col[j] += co * (e >= 0 ? dl[j] : (g_ok ? dg : 0.0f));
             }
           };
-          for (int r = 0; r < nrows; r += 2) {
+          int r_first = 0;
+          if (PRE && pre_valid) {   // first row: outside lanes use the values requested a sample ago
+            const int2 ec = prow[row0 * 64 + m_local];
+            const int e = ec.x;
+            const float co = __int_as_float(ec.y);
+            const bool out = e < 0 && co != 0.0f;
+            const float4* rp = reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);
+            const float4 l0 = rp[0], l1 = rp[1];
+            const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const bool g_ok = out && c0 + 8 * cg + j < Cg;
+              col[j] += co * (e >= 0 ? dl[j] : (g_ok ? pre[j] : 0.0f));
+            }
+            r_first = 1;
+          }
+          for (int r = r_first; r < nrows; r += 2) {
             // two rows per step so that their LDS reads overlap
             const int2 ec0 = prow[(row0 + r) * 64 + m_local];
             const int2 ec1 = (r + 1 < nrows) ? prow[(row0 + r + 1) * 64 + m_local] : make_int2(0, 0);
@@ -404,10 +435,27 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
             }
           }
           row0 += nrows;
+          // ---- request the outside values of the next sample's first row
+          pre_valid = false;
+          if (PRE && kk + 1 < kk_end && ns_l[kk + 1] > 0) {
+            const int2 ec = prow[row0 * 64 + m_local];
+            const bool out = ec.x < 0 && __int_as_float(ec.y) != 0.0f;
+            if (__any(out)) {
+              const char* gbase = reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
+              const unsigned plane = (unsigned)HW * 4u;
+              const unsigned o0 = out ? (unsigned)(8 * cg) * plane + (unsigned)(-ec.x - 1) * 4u : 0u;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const bool g_ok = out && c0 + 8 * cg + j < Cg;
+                pre[j] = *reinterpret_cast<const float*>(gbase + (g_ok ? o0 + (unsigned)j * plane : 0u));
+              }
+              pre_valid = true;
+            }
+          }
           float* ct = colT[buf];
 #pragma unroll
           for (int j = 0; j < 8; ++j) ct[(8 * cg + j) * kColLd + (m_local ^ ((cg & 1) << 4))] = col[j];
-          __syncthreads();
+          lds_only_barrier();   // the requests above stay in flight
 
           // ---- D[n][c] += A[n][m] * col[c][m]; one copy of this block per accumulator
           // rows of channel group cg = nl / 8 were written with pixel bit 4 flipped by cg
