@@ -153,18 +153,31 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
                         int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
                         int32_t dtype, sdk_stream_t stream);
 
-/* grad_input [B,C,H,W] (zero-filled by the call) receives grad_output[b,c,oy,ox]
+/* grad_input [B,C,H,W] (fully written by the call) receives grad_output[b,c,oy,ox]
  * splatted at the sample the stored index names, with the same interpolation.
  * Negative or out-of-range indices contribute nothing.
+ *
+ * `workspace` is optional device scratch of sdk_mapped_max_unpool_workspace_bytes()
+ * bytes (it depends on the input plane and the element size only).  With it the
+ * call inverts the sample map once and runs as a gather: every input pixel sums
+ * the pooled pixels whose index names a sample that reaches it, and is written
+ * once with a plain store.  Without it (NULL, or too small), or when the map or
+ * the indices do not fit that scheme (more than 32 taps reach one input pixel,
+ * the pooled pixels that can reach one tile of the input are spread too far
+ * apart, or an index names a sample of another pooled pixel than its own), the
+ * call zero-fills grad_input and scatters with atomic adds, as the reference
+ * does; the choice is made on the device, the result is the same.
  * Replaces `_mapped_max_pooling.mapped_max_unpool` /
  * `_weighted_mapped_max_pooling.weighted_mapped_max_unpool`
  * (ext_modules/include/layers/mapped_max_pooling_layer.h:64-88,
  *  weighted_mapped_max_pooling_layer.h:68-99; body common/mapped_max_pool.h:60-78, :136-171). */
+size_t sdk_mapped_max_unpool_workspace_bytes(int64_t height, int64_t width, int32_t dtype);
 int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,
-                          const void* interp_weights, void* grad_input, int64_t batch,
-                          int64_t channels, int64_t height, int64_t width, int64_t out_height,
-                          int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
-                          int32_t interp, int32_t dtype, sdk_stream_t stream);
+                          const void* interp_weights, void* grad_input, void* workspace,
+                          size_t workspace_bytes, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t out_height, int64_t out_width,
+                          int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                          int32_t dtype, sdk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Mapped convolution.  weight [Cout, Cin, K]; bias [Cout];

@@ -88,9 +88,8 @@ def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
 
 
-def _scatter_workspace(ref, out_h, out_w):
-    n = _capi.load().sdk_resample_to_map_workspace_bytes(int(out_h), int(out_w),
-                                                         _DTYPES[ref.dtype])
+def _scatter_workspace(ref, out_h, out_w, query="sdk_resample_to_map_workspace_bytes"):
+    n = getattr(_capi.load(), query)(int(out_h), int(out_w), _DTYPES[ref.dtype])
     if n == 0:
         return None, 0
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
@@ -176,6 +175,16 @@ def mapped_col2im(col, sample_map, interp_weights, height, width, interp):
 
 
 # --------------------------------------------------------------------------- pooling
+_UNPOOL_WORKSPACE = True
+
+
+def set_unpool_workspace(enabled):
+    """mapped_max_unpool with (default) or without the scratch buffer that lets the call run
+    as a gather; without it the call is the zero fill + atomic scatter."""
+    global _UNPOOL_WORKSPACE
+    _UNPOOL_WORKSPACE = bool(enabled)
+
+
 def mapped_max_pool(x, sample_map, interp_weights, kernel_size, interp):
     _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
     P = _npts(sample_map, interp_weights, 4)
@@ -207,8 +216,13 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, i
     gin = torch.empty((B, C, int(in_h), int(in_w)), dtype=grad_output.dtype,
                       device=grad_output.device)
     with torch.cuda.device(grad_output.device):
+        ws, nws = _scatter_workspace(grad_output, in_h, in_w,
+                                     "sdk_mapped_max_unpool_workspace_bytes")
+        if not _UNPOOL_WORKSPACE:
+            ws, nws = None, 0
         _capi.call("sdk_mapped_max_unpool", _ptr(grad_output), _ptr(idx_mask), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(gin), B, C, int(in_h), int(in_w), OH, OW,
+                   _ptr(interp_weights), _ptr(gin), _ptr(ws), nws, B, C, int(in_h), int(in_w),
+                   OH, OW,
                    int(kernel_size), P, int(interp), _DTYPES[grad_output.dtype],
                    _stream(grad_output))
     return gin

@@ -299,16 +299,239 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void mapped_max_unpool_kernel(
     const T* __restrict__ gout, const int64_t* __restrict__ idx, const T* __restrict__ map,
     const T* __restrict__ wts, T* __restrict__ gin, size_t total, int H, int W, int M, int P,
-    int64_t map_elems) {
-  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= total) return;
-  const size_t plane = i / (size_t)M;
-  const int64_t s = idx[i];
+    int64_t map_elems, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const int q = WEIGHTED ? P : 1;
-  if (s < 0 || s + 2 * q > map_elems) return;
-  const T val[1] = {gout[i]};
-  scatter_sample<T, INTERP, WEIGHTED, 1>(gin + plane * (size_t)H * W, 0, 1, map + s,
-                                         WEIGHTED ? wts + s / 2 : nullptr, P, H, W, val);
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / (size_t)M;
+    const int64_t s = idx[i];
+    if (s < 0 || s + 2 * q > map_elems) continue;
+    const T val[1] = {gout[i]};
+    scatter_sample<T, INTERP, WEIGHTED, 1>(gin + plane * (size_t)H * W, 0, 1, map + s,
+                                           WEIGHTED ? wts + s / 2 : nullptr, P, H, W, val);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Unpool by image tile.  A workgroup owns a tile of kUpTile image pixels and a group of
+// planes, accumulates the tile in LDS and writes every pixel of it exactly once with a
+// plain store: no zero fill of the image, no global atomics.  It has to look at every
+// pooled pixel that can reach the tile, whichever sample wins: the map alone fixes that
+// set, and two small kernels find, per tile, the window of the pooled grid that holds it
+// (rows x columns, columns wrap modulo the pooled width):
+//   unpool_anchor:  one thread per (pooled pixel, sample); every tile a tap of the sample
+//       falls into records that pooled pixel (any one of them serves as the anchor).
+//   unpool_window:  the same walk; the tile's window grows to hold the pooled pixel,
+//       measured from the anchor so that a window may straddle the seam.
+//   unpool_tiles:   per pass of up to kUpPlanes planes: clear the LDS tile; every thread
+//       takes pooled pixels of the window (coalesced index and gradient reads), reads the
+//       winning sample's coordinates from the map and adds the taps that fall inside the
+//       tile to LDS; then the tile is stored.  Windows of neighbouring tiles overlap, so a
+//       pooled pixel is read by every tile it can reach, and adds only what lands there.
+// *gate is raised, and the call falls back to zero fill + atomic scatter, when a window is
+// larger than kUpWindow pooled pixels (an incoherent map) or an index names a sample of
+// another pooled pixel than its own (mapped_max_pool never writes one, but the scatter
+// accepts it): such a sample may reach tiles whose windows do not hold the pixel.
+// ---------------------------------------------------------------------------
+constexpr int kUpTile = 1024;     // image pixels per workgroup (4 per thread); 2^10, see tile_of
+constexpr int kUpWindow = 8192;   // pooled pixels a tile may have to look at
+constexpr int kUpBytes = 16384;   // LDS of the tile accumulators: kUpTile x planes per pass
+
+struct UnpoolTiling {
+  int H, W, tw_shift, tiles_x, tiles_y;
+  __host__ __device__ int TW() const { return 1 << tw_shift; }
+  __host__ __device__ int TH() const { return kUpTile >> tw_shift; }
+  __device__ int tile_of(int y, int x) const {
+    return (y >> (10 - tw_shift)) * tiles_x + (x >> tw_shift);   // TH = kUpTile >> tw_shift
+  }
+};
+
+__device__ __forceinline__ int wave_min_int(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_max_int(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Per tile, 8 ints (cleared before the analysis): [0] anchor pooled pixel + 1 (0: nothing
+// reaches the tile), [1..4] window extent around the anchor: rows up, rows down, columns
+// left, columns right.
+template <typename T, int INTERP, bool WEIGHTED, bool GROW>
+__global__ __launch_bounds__(kBlock) void unpool_window_kernel(
+    const T* __restrict__ map, int64_t samples, int P, int K, int OW, UnpoolTiling ut,
+    int* __restrict__ win) {
+  int64_t smp = (int64_t)blockIdx.x * kBlock + threadIdx.x;   // pooled pixel * K + k
+  const bool in_range = smp < samples;   // lanes past the end walk the last sample, mute
+  smp = in_range ? smp : samples - 1;
+  const int q = WEIGHTED ? P : 1;
+  const int o = (int)(smp / K);
+  PointTaps<T, INTERP> t;
+  for (int p = 0; p < q; ++p) {
+    const size_t s = (size_t)smp * q + p;
+    t.set(map[s * 2], map[s * 2 + 1], ut.H, ut.W);
+#pragma unroll
+    for (int i = 0; i < PointTaps<T, INTERP>::N; ++i) {
+      const bool hit = in_range && t.off[i] >= 0;
+      const int tile = hit ? ut.tile_of(t.ty[i], t.tx[i]) : -1;
+      if constexpr (!GROW) {
+        if (hit) win[(size_t)tile * 8] = o + 1;
+      } else {
+        // lanes of a wave mostly hit one tile: one lane speaks for all lanes of a tile
+        int dy = 0, dx = 0;
+        if (hit) {
+          const int a = win[(size_t)tile * 8] - 1;
+          dy = o / OW - a / OW;
+          dx = o % OW - a % OW;
+          dx += (dx > OW / 2) ? -OW : ((dx < -(OW / 2)) ? OW : 0);
+        }
+        bool todo = hit;
+        while (__any(todo)) {
+          const int pick = wave_min_int(todo ? tile : INT_MAX);   // smallest pending tile
+          const bool mine = todo && tile == pick;
+          const int up = wave_max_int(mine ? -dy : INT_MIN), down = wave_max_int(mine ? dy : INT_MIN);
+          const int left = wave_max_int(mine ? -dx : INT_MIN), right = wave_max_int(mine ? dx : INT_MIN);
+          if (mine) todo = false;
+          if ((threadIdx.x & 63) == 0) {
+            int* w = win + (size_t)pick * 8;
+            if (up > w[1]) atomicMax(&w[1], up);
+            if (down > w[2]) atomicMax(&w[2], down);
+            if (left > w[3]) atomicMax(&w[3], left);
+            if (right > w[4]) atomicMax(&w[4], right);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
+    const T* __restrict__ gout, const int64_t* __restrict__ idx, const T* __restrict__ map,
+    const T* __restrict__ wts, const int* __restrict__ win, T* __restrict__ gin,
+    int* __restrict__ gate, UnpoolTiling ut, int planes, int planes_per_group, int M, int OW,
+    int K, int P, int64_t map_elems) {
+  if (*gate != 0) return;
+  constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));   // planes per pass
+  __shared__ T acc[PLMAX * kUpTile];
+  const int tid = threadIdx.x, tile = blockIdx.x;
+  const size_t HW = (size_t)ut.H * ut.W;
+  const int p_begin = blockIdx.y * planes_per_group;
+  const int p_end = min(planes, p_begin + planes_per_group);
+  const int ty0 = (tile / ut.tiles_x) * ut.TH(), tx0 = (tile % ut.tiles_x) << ut.tw_shift;
+  const int q = WEIGHTED ? P : 1;
+  const int twoq = 2 * q;
+  // window of pooled pixels
+  const int* w = win + (size_t)tile * 8;
+  const int anchor = w[0] - 1;
+  int WH = 0, WW = 0, wy0 = 0, wx0 = 0;
+  if (anchor >= 0) {
+    const int ay = anchor / OW, ax = anchor % OW;
+    WH = w[1] + w[2] + 1;
+    const bool full = w[3] + w[4] + 1 >= OW;   // all around: columns as they are
+    WW = full ? OW : w[3] + w[4] + 1;
+    wy0 = ay - w[1];
+    wx0 = full ? 0 : ax - w[3];
+    wx0 += wx0 < 0 ? OW : 0;
+  }
+  if ((int64_t)WH * WW > kUpWindow) {
+    if (tid == 0) atomicAdd(gate, 1);
+    return;
+  }
+  const int WN = WH * WW;
+  const float rcp_ww = WW > 0 ? 1.0f / (float)WW : 0.0f;
+  const int per_pixel = K * twoq;   // map elements of one pooled pixel
+  // the thread's 4 image pixels: waves own 4 consecutive 64-pixel runs of the tile
+  int u[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int L = (((tid >> 6) * 4 + j) << 6) + (tid & 63);
+    const int y = ty0 + (L >> ut.tw_shift), x = tx0 + (L & (ut.TW() - 1));
+    u[j] = (y < ut.H && x < ut.W) ? y * ut.W + x : -1;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int pl = 0; pl < PLMAX; ++pl)
+      acc[pl * kUpTile + (((tid >> 6) * 4 + j) << 6) + (tid & 63)] = T(0);
+  __syncthreads();
+  for (int p0 = p_begin; p0 < p_end; p0 += PLMAX) {
+    const int np = min(PLMAX, p_end - p0);
+    // ---- pooled pixels of the window: a thread takes one at a time and walks the planes
+    // of the pass, so the position arithmetic is shared and PLMAX independent (index,
+    // gradient) pairs, then their map reads, are in flight together
+    for (int o = tid; o < WN; o += kBlock) {
+      const int r = (int)(((float)o + 0.5f) * rcp_ww);    // o / WW (o < 2^13: exact)
+      int ox = wx0 + (o - r * WW);
+      ox -= ox >= OW ? OW : 0;
+      const int m = (wy0 + r) * OW + ox;
+      const int first = m * per_pixel;   // map element of the pixel's first sample
+      const size_t at = (size_t)p0 * M + m;
+      int sv[PLMAX];
+      T gv[PLMAX];
+      bool live[PLMAX];
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        const bool on = pl < np;
+        const int64_t s64 = on ? idx[at + (size_t)pl * M] : (int64_t)-1;
+        gv[pl] = on ? gout[at + (size_t)pl * M] : T(0);
+        live[pl] = s64 >= 0 && s64 + twoq <= map_elems;   // others contribute nothing
+        sv[pl] = (int)s64;                                  // map_elems < 2^31
+      }
+      T cx[PLMAX], cy[PLMAX];
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        if (live[pl]) {
+          const int d = sv[pl] - first;
+          if (d < 0 || d >= per_pixel || d % twoq != 0) {   // not a sample of this pixel
+            atomicAdd(gate, 1);
+            live[pl] = false;
+          }
+        }
+        cx[pl] = live[pl] ? map[sv[pl]] : T(0);
+        cy[pl] = live[pl] ? map[sv[pl] + 1] : T(0);
+      }
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        if (!live[pl]) continue;
+        T* a = acc + pl * kUpTile;
+        PointTaps<T, INTERP> taps;
+        for (int p = 0; p < q; ++p) {
+          T v = gv[pl];
+          if (p == 0) {
+            taps.set(cx[pl], cy[pl], ut.H, ut.W);
+          } else {
+            taps.set(map[sv[pl] + 2 * p], map[sv[pl] + 2 * p + 1], ut.H, ut.W);
+          }
+          if constexpr (WEIGHTED) v = wts[sv[pl] / 2 + p] * v;
+#pragma unroll
+          for (int n = 0; n < PointTaps<T, INTERP>::N; ++n) {
+            const int ry = taps.ty[n] - ty0, rx = taps.tx[n] - tx0;
+            if (taps.off[n] >= 0 && (unsigned)ry < (unsigned)ut.TH() &&
+                (unsigned)rx < (unsigned)ut.TW())
+              lds_add(a + (ry << ut.tw_shift) + rx, INTERP == 0 ? v : taps.w[n] * v);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // store the tile and clear it for the next pass
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        T* cell = acc + pl * kUpTile + (((tid >> 6) * 4 + j) << 6) + (tid & 63);
+        const T v = *cell;
+        *cell = T(0);
+        if (u[j] >= 0 && pl < np) gin[(size_t)(p0 + pl) * HW + u[j]] = v;
+      }
+    }
+    __syncthreads();
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -398,6 +621,80 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
                                 MP, P, gate)));
     SDK_LAUNCH_CHECK("resample_to_map(weight_sum)");
   }
+  return SDK_OK;
+}
+
+static UnpoolTiling unpool_tiling(int H, int W) {
+  UnpoolTiling ut;
+  ut.H = H;
+  ut.W = W;
+  ut.tw_shift = 6;
+  while ((kUpTile >> ut.tw_shift) > H && ut.tw_shift < 10) ++ut.tw_shift;   // flat images: wider tiles
+  while (ut.tw_shift > 0 && (1 << (ut.tw_shift - 1)) >= W) --ut.tw_shift;   // narrow ones: taller
+  ut.tiles_x = (int)ceil_div(W, ut.TW());
+  ut.tiles_y = (int)ceil_div(H, ut.TH());
+  return ut;
+}
+
+// Workspace of the tiled unpool: gate (first 256 bytes) and the tile windows, cleared together.
+static size_t unpool_layout(const UnpoolTiling& ut) {
+  return 256 + (size_t)ut.tiles_x * ut.tiles_y * 8 * sizeof(int);
+}
+
+template <typename T>
+static int launch_unpool(const T* gout, const int64_t* indices, const T* map, const T* wts, T* gin,
+                         void* workspace, size_t workspace_bytes, int64_t planes, int H, int W,
+                         int OH, int OW, int K, int P, int interp, hipStream_t stream) {
+  const int64_t HW = (int64_t)H * W, M = (int64_t)OH * OW;
+  const int q = pts(P);
+  const size_t total = (size_t)planes * M;
+  const int64_t map_elems = M * K * q * 2;
+  const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
+  const UnpoolTiling ut = unpool_tiling(H, W);
+  const int64_t tiles = (int64_t)ut.tiles_x * ut.tiles_y;
+  constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));
+  // plane groups: many short workgroups (the kernel is bound by instruction issue and by the
+  // latency of each workgroup's few dependent loads; one or two passes each measured best)
+  int64_t groups = std::max<int64_t>(1, std::min<int64_t>(ceil_div(planes, PLMAX),
+                                                          ceil_div(16384, tiles)));
+  const int64_t per_group = ceil_div(ceil_div(planes, groups), PLMAX) * PLMAX;
+  groups = ceil_div(planes, per_group);
+  if (workspace != nullptr && workspace_bytes >= unpool_layout(ut) &&
+      map_elems < ((int64_t)1 << 31) &&
+      tiles < ((int64_t)1 << 27) && groups <= 65535) {
+    char* ws = static_cast<char*>(workspace);
+    int* g = reinterpret_cast<int*>(ws);
+    int* win = reinterpret_cast<int*>(ws + 256);
+    int rc = zero_fill(ws, unpool_layout(ut), stream);
+    if (rc != SDK_OK) return rc;
+    const int64_t samples = M * K;
+    const dim3 grid_s((unsigned)ceil_div(samples, kBlock));
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((unpool_window_kernel<T, INTERP, WEIGHTED, false>), grid_s,
+                                dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+    SDK_LAUNCH_CHECK("mapped_max_unpool(anchors)");
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((unpool_window_kernel<T, INTERP, WEIGHTED, true>), grid_s,
+                                dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+    SDK_LAUNCH_CHECK("mapped_max_unpool(windows)");
+    const dim3 grid_t((unsigned)tiles, (unsigned)groups);
+    SDK_DISPATCH_INTERP(interp, P,
+                        (launch((unpool_tiles_kernel<T, INTERP, WEIGHTED>), grid_t, dim3(kBlock),
+                                stream, gout, indices, map, wts, (const int*)win, gin, g, ut,
+                                (int)planes, (int)per_group, (int)M, OW, K, P, map_elems)));
+    SDK_LAUNCH_CHECK("mapped_max_unpool(tiles)");
+    gate = g;
+  }
+  int rc = zero_fill_gated(gin, sizeof(T) * (size_t)planes * HW, stream, gate);
+  if (rc != SDK_OK) return rc;
+  // as a fallback (seldom run): fewer workgroups, each striding over the elements
+  const int64_t blocks = ceil_div((int64_t)total, kBlock);
+  const dim3 grid_el((unsigned)(gate != nullptr ? std::min<int64_t>(blocks, 4096) : blocks));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((mapped_max_unpool_kernel<T, INTERP, WEIGHTED>), grid_el,
+                              dim3(kBlock), stream, gout, indices, map, wts, gin, total, H, W,
+                              (int)M, P, map_elems, gate)));
+  SDK_LAUNCH_CHECK("mapped_max_unpool");
   return SDK_OK;
 }
 
@@ -591,11 +888,18 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
   return SDK_OK;
 }
 
+size_t sdk_mapped_max_unpool_workspace_bytes(int64_t height, int64_t width, int32_t dtype) {
+  if (height < 1 || width < 1 || height * width >= ((int64_t)1 << 31)) return 0;
+  (void)dtype;
+  return unpool_layout(unpool_tiling((int)height, (int)width));
+}
+
 int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,
-                          const void* interp_weights, void* grad_input, int64_t batch,
-                          int64_t channels, int64_t height, int64_t width, int64_t out_height,
-                          int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
-                          int32_t interp, int32_t dtype, sdk_stream_t stream) {
+                          const void* interp_weights, void* grad_input, void* workspace,
+                          size_t workspace_bytes, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t out_height, int64_t out_width,
+                          int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                          int32_t dtype, sdk_stream_t stream) {
   SDK_REQUIRE(indices, "mapped_max_unpool: NULL indices");
   SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_unpool: bad pooled size");
   const int64_t M = out_height * out_width;
@@ -604,25 +908,14 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
   if (rc) return rc;
   const int64_t planes = batch * channels;
   if (planes == 0) return SDK_OK;
-  const size_t esz = dtype == SDK_F64 ? 8 : 4;
-  rc = zero_fill(grad_input, esz * (size_t)planes * height * width, (hipStream_t)stream);
-  if (rc) return rc;
-  const size_t total = (size_t)planes * M;
-  const int64_t map_elems = M * kernel_size * pts(num_interp_pts) * 2;
-  SDK_REQUIRE(ceil_div((int64_t)total, kBlock) < ((int64_t)1 << 31),
+  SDK_REQUIRE(ceil_div(planes * M, kBlock) < ((int64_t)1 << 31),
               "mapped_max_unpool: too many elements");
-  const dim3 grid((unsigned)ceil_div((int64_t)total, kBlock));
-  SDK_DISPATCH_DTYPE(
-      dtype,
-      SDK_DISPATCH_INTERP(interp, num_interp_pts,
-                          (launch((mapped_max_unpool_kernel<T, INTERP, WEIGHTED>),
-                                              grid, dim3(kBlock), (hipStream_t)stream,
-                                              (const T*)grad_output, indices,
-                                              (const T*)sample_map, (const T*)interp_weights,
-                                              (T*)grad_input, total, (int)height, (int)width,
-                                              (int)M, num_interp_pts, map_elems))));
-  SDK_LAUNCH_CHECK("mapped_max_unpool");
-  return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_unpool<T>(
+                                (const T*)grad_output, indices, (const T*)sample_map,
+                                (const T*)interp_weights, (T*)grad_input, workspace,
+                                workspace_bytes, planes, (int)height, (int)width, (int)out_height,
+                                (int)out_width, (int)kernel_size, num_interp_pts, interp,
+                                (hipStream_t)stream));
 }
 
 }  // extern "C"

@@ -35,6 +35,19 @@ __device__ __forceinline__ void lds_add_f32(float* addr, float v) {
   }
 }
 
+__device__ __forceinline__ void lds_add_f64(double* addr, double v) {
+  unsigned long long* ip = reinterpret_cast<unsigned long long*>(addr);
+  unsigned long long old = __hip_atomic_load(ip, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  while (true) {
+    const unsigned long long assumed = old;
+    old = atomicCAS(ip, assumed, (unsigned long long)__double_as_longlong(
+                                     __longlong_as_double((long long)assumed) + v));
+    if (old == assumed) break;
+  }
+}
+__device__ __forceinline__ void lds_add(float* addr, float v) { lds_add_f32(addr, v); }
+__device__ __forceinline__ void lds_add(double* addr, double v) { lds_add_f64(addr, v); }
+
 // N independent float adds into LDS: all loads, then all compare-and-swaps, are
 // issued back to back so their latencies overlap.  A swap that lost a race (two
 // lanes of the wave, or another wave, hit the same word) is repeated with the
@@ -134,6 +147,7 @@ template <typename T, int INTERP>
 struct PointTaps {
   static constexpr int N = (INTERP == 0) ? 1 : 4;
   int off[N];  // element offset inside one H x W plane, or -1 (inactive tap)
+  int ty[N], tx[N];  // row and column of the tap (meaningful where off >= 0)
   T w[N];
 
   __device__ __forceinline__ void set(T x, T y, int H, int W) {
@@ -142,6 +156,8 @@ struct PointTaps {
       const int yi = to_int_clamped(round_t(y));
       const bool ok = (unsigned)xi < (unsigned)W && (unsigned)yi < (unsigned)H;
       off[0] = ok ? yi * W + xi : -1;
+      ty[0] = yi;
+      tx[0] = xi;
       w[0] = T(1);
     } else {
       const T fx = floor_t(x), fy = floor_t(y);
@@ -167,6 +183,10 @@ struct PointTaps {
       w[2] = D * B;
       w[3] = D * C;
       const int r1 = y1 * W, r2 = r1 + W;
+      ty[0] = ty[1] = y1;
+      ty[2] = ty[3] = y1 + 1;
+      tx[0] = tx[2] = c1;
+      tx[1] = tx[3] = c2;
       off[0] = (x1ok && y1ok && w[0] != T(0)) ? r1 + c1 : -1;
       off[1] = (x2ok && y1ok && w[1] != T(0)) ? r1 + c2 : -1;
       off[2] = (x1ok && y2ok && w[2] != T(0)) ? r2 + c1 : -1;

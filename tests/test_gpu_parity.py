@@ -161,6 +161,111 @@ def test_pool_ties_nan_and_no_winner(ops, oracle):
     assert got.reshape(-1).tolist() == [2, 0, 0, 0, 0, 0, 0, 0]  # -1 and out-of-image drop out
 
 
+def _unpool_capi(ops, g, idx, m, iw, H, W, K, P, interp, with_workspace):
+    """mapped_max_unpool through the C ABI; returns (grad_input, gate) where gate is the
+    workspace's first word after the call: 0 = the gather ran, > 0 = the call fell back to the
+    atomic scatter, None = no workspace was passed."""
+    from _spherical_distortion_ext import _capi
+    tg, tm, tw = _t(g), _t(m), _t(iw)
+    B, C, OH, OW = g.shape
+    dtype = 0 if g.dtype == np.float32 else 1
+    out = torch.full((B, C, H, W), 7.0, dtype=tg.dtype, device=DEV)   # must be overwritten
+    ws, nws = None, 0
+    if with_workspace:
+        nws = _capi.load().sdk_mapped_max_unpool_workspace_bytes(H, W, dtype)
+        assert nws > 0
+        ws = torch.empty(nws, dtype=torch.uint8, device=DEV)
+    _capi.call("sdk_mapped_max_unpool", ops._ptr(tg), ops._ptr(idx), ops._ptr(tm), ops._ptr(tw),
+               ops._ptr(out), ops._ptr(ws), nws, B, C, H, W, OH, OW, K, P, interp, dtype,
+               ops._stream(tg))
+    gate = int(ws[:4].view(torch.int32)[0]) if with_workspace else None
+    return _n(out), gate
+
+
+UNPOOL_CASES = [
+    # (H, W, OH, OW, K, P, interp, dtype, scale)
+    (40, 150, 20, 75, 9, 0, 0, np.float32, 1.0),    # strided nearest map over 3 x 3 image tiles
+    (40, 150, 20, 75, 9, 0, 1, np.float32, 1.0),    # bilinear: four candidates per sample
+    (33, 70, 16, 35, 5, 2, 2, np.float32, 1.0),     # weighted, columns wrap at the seam
+    (1, 3000, 1, 1500, 7, 0, 0, np.float32, 1.0),   # one-row vertex list, flat tiles
+    (40, 150, 20, 75, 9, 0, 0, np.float64, 1.0),
+    (50, 20, 25, 10, 3, 2, 1, np.float64, 1.0),     # narrow image, tall tiles
+]
+
+
+@pytest.mark.parametrize("tc", UNPOOL_CASES, ids=lambda c: "H%dW%d_K%dP%d_i%d_%s" % (
+    c[0], c[1], c[4], c[5], c[6], np.dtype(c[7]).name))
+def test_unpool_by_image_tile(ops, oracle, tc):
+    """Coherent maps: the call with workspace runs tile by tile (gate stays 0) and agrees with
+    the oracle and with the atomic scatter of the call without workspace."""
+    H, W, OH, OW, K, P, interp, dt, scale = tc
+    rng = np.random.default_rng(900 + H + K + interp)
+    B, C = 2, 5
+    m = _coherent_map(rng, OH, OW, K, P, H, W, dt, scale)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if P else None
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    _, idx = ops.mapped_max_pool(_t(x), _t(m), _t(iw), K, interp)
+    g = rng.standard_normal((B, C, OH, OW)).astype(dt)
+    want = oracle.mapped_max_unpool(g, _n(idx), m, H, W, K, interp, iw)
+    got, gate = _unpool_capi(ops, g, idx, m, iw, H, W, K, P, interp, True)
+    assert gate == 0
+    assert relerr(got, want) <= BWD_TOL[dt]
+    plain, _ = _unpool_capi(ops, g, idx, m, iw, H, W, K, P, interp, False)
+    assert relerr(plain, want) <= BWD_TOL[dt]
+
+
+def test_unpool_falls_back_to_the_scatter(ops, oracle):
+    """Indices the pooling never writes and scattered maps raise the gate on the device; the
+    result is the oracle's either way."""
+    rng = np.random.default_rng(77)
+    B, C, H, W, OH, OW, K = 2, 3, 24, 40, 12, 20, 9
+    m = _coherent_map(rng, OH, OW, K, 0, H, W, np.float32)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    _, idx = ops.mapped_max_pool(_t(x), _t(m), None, K, 0)
+    g = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
+    # (a) an index that names a sample of another pooled pixel, a negative one, one past the end
+    # of the map (the reference would read outside the map there; here it contributes nothing,
+    # like a negative one, which is how the oracle is asked)
+    idx_np = _n(idx).copy()
+    idx_np[0, 0, 3, 4] = idx_np[0, 0, 7, 9]
+    idx_np[1, 2, 0, 0] = -1
+    idx_dev = idx_np.copy()
+    idx_np[1, 1, 5, 5] = -1
+    idx_dev[1, 1, 5, 5] = OH * OW * K * 2 + 10
+    want = oracle.mapped_max_unpool(g, idx_np, m, H, W, K, 0)
+    got, gate = _unpool_capi(ops, g, _t(idx_dev), m, None, H, W, K, 0, 0, True)
+    assert gate > 0
+    assert relerr(got, want) <= 1e-4
+    # the same without the foreign index: negative / out-of-range ones alone do not fall back
+    idx_np[0, 0, 3, 4] = idx_dev[0, 0, 3, 4] = _n(idx)[0, 0, 3, 4]
+    want = oracle.mapped_max_unpool(g, idx_np, m, H, W, K, 0)
+    got, gate = _unpool_capi(ops, g, _t(idx_dev), m, None, H, W, K, 0, 0, True)
+    assert gate == 0
+    assert relerr(got, want) <= 1e-4
+    plain, _ = _unpool_capi(ops, g, _t(idx_dev), m, None, H, W, K, 0, 0, False)
+    assert relerr(plain, want) <= 1e-4
+    # (b) every sample of every pixel hits one of two image pixels: heavy collisions inside
+    # one tile, still no fallback
+    mc = np.zeros((OH, OW, K, 2), np.float32)
+    mc[..., 0] = rng.integers(5, 7, (OH, OW, K))
+    mc[..., 1] = 3
+    _, idx_c = ops.mapped_max_pool(_t(x), _t(mc), None, K, 0)
+    want = oracle.mapped_max_unpool(g, _n(idx_c), mc, H, W, K, 0)
+    got, gate = _unpool_capi(ops, g, idx_c, mc, None, H, W, K, 0, 0, True)
+    assert gate == 0
+    assert relerr(got, want) <= 1e-4
+    # (c) a scattered map: every tile would have to look at the whole pooled grid, which is
+    # larger than a tile's window may be
+    OH2, OW2 = 100, 120
+    ms = _coords(rng, (OH2, OW2, 3), H, W, np.float32)
+    _, idx_s = ops.mapped_max_pool(_t(x), _t(ms), None, 3, 0)
+    g2 = rng.standard_normal((B, C, OH2, OW2)).astype(np.float32)
+    want = oracle.mapped_max_unpool(g2, _n(idx_s), ms, H, W, 3, 0)
+    got, gate = _unpool_capi(ops, g2, idx_s, ms, None, H, W, 3, 0, 0, True)
+    assert gate > 0
+    assert relerr(got, want) <= 1e-4
+
+
 CONV_CASES = [(i, wgt, dt) for i in (0, 1, 2) for wgt in (False, True)
               for dt in (np.float32, np.float64)]
 
