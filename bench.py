@@ -64,6 +64,16 @@ class Timer:
         return float(np.mean(ms)), float(np.min(ms))
 
 
+def _measured_traffic(kernel):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
+    a copy kernel of known size); kept with the profile summaries, None when not measured."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(kernel)
+
+
 def _roof(bound, work, ms, traffic=None, peak=None):
     if bound == "hbm":
         peak = HBM_PEAK_GBS
@@ -126,12 +136,32 @@ def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
     parts = {}
     for name, fn in calls.items():
         t, _ = timer.run(fn, max(3, steps // 2), 1)
-        parts[name] = dict(ms=t, **(_roof("mfma", flops, t, peak=peak) if name != "bias_grad"
-                                    else _roof("hbm", _nbytes(g), t)))
+        traffic = _measured_traffic("mapped_conv_" + name) if compute == "native" else None
+        parts[name] = dict(ms=t, **(_roof("mfma", flops, t, traffic=traffic, peak=peak)
+                                    if name != "bias_grad" else _roof("hbm", _nbytes(g), t)))
     del keep
     dominant = max(("forward", "backward_input", "backward_weight"), key=lambda n: parts[n]["ms"])
     return {"ms_per_step": ms, "ms_min": ms_min, "images_per_s": B / (ms * 1e-3),
             "flops_per_contraction": flops, "parts": parts, "dominant": dominant}
+
+
+def bench_conv1(torch, ops, timer, steps, warmup):
+    """Configuration 1 (x [1,3,64,128] -> 16 channels, bilinear, K = 9): 7 MFLOP and 2 MB, bound by
+    launch latency, so it is reported in microseconds per call and not against a roofline."""
+    import workloads
+    cfg = workloads.config1()
+    dev = "cuda:0"
+    x, m, w, b, g = (torch.from_numpy(cfg[k]).to(dev) for k in
+                     ("x", "sample_map", "weight", "bias", "grad_output"))
+    K, interp = cfg["kernel_size"], cfg["interp"]
+    ms_f, _ = timer.run(lambda: ops.mapped_conv_forward(x, m, None, w, b, K, interp), steps, warmup)
+
+    def step():
+        ops.mapped_conv_forward(x, m, None, w, b, K, interp)
+        ops.mapped_conv_backward(g, m, None, x, w, b, K, interp)
+    ms_s, _ = timer.run(step, steps, warmup)
+    return {"conv1_latency": {"forward_us": round(ms_f * 1e3, 1),
+                              "forward_backward_us": round(ms_s * 1e3, 1)}}
 
 
 def bench_resample2(torch, ops, timer, steps, warmup):
@@ -147,8 +177,10 @@ def bench_resample2(torch, ops, timer, steps, warmup):
                         steps, warmup)
     gather_bytes = _nbytes(x, m, patches)
     scatter_bytes = _nbytes(patches, m, x) + H * W * 4.0
-    return {"gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g)),
-            "scatter_normalise": dict(ms=ms_s, **_roof("hbm", scatter_bytes, ms_s))}
+    return {"gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,
+                                            traffic=_measured_traffic("resample_from_map"))),
+            "scatter_normalise": dict(ms=ms_s, **_roof("hbm", scatter_bytes, ms_s,
+                                                       traffic=_measured_traffic("resample_to_map")))}
 
 
 def bench_pool3(torch, ops, timer, steps, warmup):
@@ -165,8 +197,10 @@ def bench_pool3(torch, ops, timer, steps, warmup):
     ms_b, _ = timer.run(lambda: ops.mapped_max_unpool(g, idx, m, None, H, W, K, 0), steps, warmup)
     fwd_bytes = _nbytes(x, m, val, idx)
     bwd_bytes = _nbytes(g, idx, m, x)
-    return {"pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f)),
-            "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b)),
+    return {"pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f,
+                                                  traffic=_measured_traffic("mapped_max_pool"))),
+            "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b,
+                                                   traffic=_measured_traffic("mapped_max_unpool"))),
             "no_winner_outputs": int((idx < 0).sum().item())}
 
 
@@ -195,16 +229,6 @@ def bench_ico5(torch, ops, timer, steps, warmup):
                                                    peak=MFMA_FP32_TFLOPS)),
             "transposed_conv_forward": dict(ms=ms_t, **_roof("mfma", tflops, ms_t,
                                                              peak=MFMA_FP32_TFLOPS))}
-
-
-def _measured_traffic(kernel):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
-    a copy kernel of known size); kept with the profile summaries, None when not measured."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if not os.path.exists(path):
-        return None
-    with open(path) as f:
-        return json.load(f).get(kernel)
 
 
 def cpu_baseline(budget_s=12.0):
@@ -260,7 +284,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--only", default="", help="comma list of: conv4,conv4_bf16,resample2,pool3,ico5")
+    ap.add_argument("--only", default="", help="comma list of: conv4,conv4_bf16,conv1,resample2,pool3,ico5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -291,6 +315,8 @@ def main():
         except RuntimeError as e:
             kernels["conv4_bf16"] = {"error": str(e)[:200]}
         torch.cuda.empty_cache()
+    if want("conv1"):
+        kernels.update(bench_conv1(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
     if want("resample2"):
         kernels.update(bench_resample2(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
     if want("pool3"):

@@ -194,14 +194,20 @@ __global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
           acc = mfma_bf16(pack_bf16x8(f), bfrag16[t], acc);
         }
       } else {
+        // two independent accumulator chains (even / odd step groups), summed at the end
+        floatx16 acc2;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc2[v] = 0.0f;
 #pragma unroll
         for (int g = 0; g < NS / 4; ++g) {
           const float4 a = (g < kPre) ? wpre[g] : wblk[g * 64];
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bfrag[4 * g + 0], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bfrag[4 * g + 1], acc, 0, 0, 0);
+          acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bfrag[4 * g + 1], acc2, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bfrag[4 * g + 2], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc, 0, 0, 0);
+          acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bfrag[4 * g + 3], acc2, 0, 0, 0);
         }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] += acc2[v];
       }
       // first fragments of the next block (next sample, or first sample of the next chunk)
       {
