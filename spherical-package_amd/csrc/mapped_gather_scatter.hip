@@ -347,65 +347,78 @@ struct UnpoolTiling {
   }
 };
 
-__device__ __forceinline__ int wave_min_int(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
-  return v;
-}
-__device__ __forceinline__ int wave_max_int(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
-  return v;
-}
-
 // Per tile, 8 ints (cleared before the analysis): [0] anchor pooled pixel + 1 (0: nothing
 // reaches the tile), [1..4] window extent around the anchor: rows up, rows down, columns
 // left, columns right.
+// A workgroup's samples reach a handful of tiles: their extents are first merged in a small
+// LDS table (kWinSlots tiles, open addressing) and reach global memory once per tile and
+// workgroup; a sample that finds the table full goes to global memory directly.
+constexpr int kWinSlots = 8;
+
+__device__ __forceinline__ void grow_window(int* w, int up, int down, int left, int right) {
+  if (up > w[1]) atomicMax(&w[1], up);
+  if (down > w[2]) atomicMax(&w[2], down);
+  if (left > w[3]) atomicMax(&w[3], left);
+  if (right > w[4]) atomicMax(&w[4], right);
+}
+
 template <typename T, int INTERP, bool WEIGHTED, bool GROW>
 __global__ __launch_bounds__(kBlock) void unpool_window_kernel(
     const T* __restrict__ map, int64_t samples, int P, int K, int OW, UnpoolTiling ut,
     int* __restrict__ win) {
-  int64_t smp = (int64_t)blockIdx.x * kBlock + threadIdx.x;   // pooled pixel * K + k
-  const bool in_range = smp < samples;   // lanes past the end walk the last sample, mute
-  smp = in_range ? smp : samples - 1;
-  const int q = WEIGHTED ? P : 1;
-  const int o = (int)(smp / K);
-  PointTaps<T, INTERP> t;
-  for (int p = 0; p < q; ++p) {
-    const size_t s = (size_t)smp * q + p;
-    t.set(map[s * 2], map[s * 2 + 1], ut.H, ut.W);
+  __shared__ int s_tile[kWinSlots];
+  __shared__ int s_ext[kWinSlots][4];
+  if (GROW) {
+    if (threadIdx.x < kWinSlots) {
+      s_tile[threadIdx.x] = -1;
+      s_ext[threadIdx.x][0] = s_ext[threadIdx.x][1] = 0;
+      s_ext[threadIdx.x][2] = s_ext[threadIdx.x][3] = 0;
+    }
+    __syncthreads();
+  }
+  const int64_t smp = (int64_t)blockIdx.x * kBlock + threadIdx.x;   // pooled pixel * K + k
+  if (smp < samples) {
+    const int q = WEIGHTED ? P : 1;
+    const int o = (int)(smp / K);
+    PointTaps<T, INTERP> t;
+    for (int p = 0; p < q; ++p) {
+      const size_t s = (size_t)smp * q + p;
+      t.set(map[s * 2], map[s * 2 + 1], ut.H, ut.W);
 #pragma unroll
-    for (int i = 0; i < PointTaps<T, INTERP>::N; ++i) {
-      const bool hit = in_range && t.off[i] >= 0;
-      const int tile = hit ? ut.tile_of(t.ty[i], t.tx[i]) : -1;
-      if constexpr (!GROW) {
-        if (hit) win[(size_t)tile * 8] = o + 1;
-      } else {
-        // lanes of a wave mostly hit one tile: one lane speaks for all lanes of a tile
-        int dy = 0, dx = 0;
-        if (hit) {
-          const int a = win[(size_t)tile * 8] - 1;
-          dy = o / OW - a / OW;
-          dx = o % OW - a % OW;
+      for (int i = 0; i < PointTaps<T, INTERP>::N; ++i) {
+        if (t.off[i] < 0) continue;
+        const int tile = ut.tile_of(t.ty[i], t.tx[i]);
+        int* w = win + (size_t)tile * 8;
+        if constexpr (!GROW) {
+          w[0] = o + 1;
+        } else {
+          const int a = w[0] - 1;
+          const int dy = o / OW - a / OW;
+          int dx = o % OW - a % OW;
           dx += (dx > OW / 2) ? -OW : ((dx < -(OW / 2)) ? OW : 0);
-        }
-        bool todo = hit;
-        while (__any(todo)) {
-          const int pick = wave_min_int(todo ? tile : INT_MAX);   // smallest pending tile
-          const bool mine = todo && tile == pick;
-          const int up = wave_max_int(mine ? -dy : INT_MIN), down = wave_max_int(mine ? dy : INT_MIN);
-          const int left = wave_max_int(mine ? -dx : INT_MIN), right = wave_max_int(mine ? dx : INT_MIN);
-          if (mine) todo = false;
-          if ((threadIdx.x & 63) == 0) {
-            int* w = win + (size_t)pick * 8;
-            if (up > w[1]) atomicMax(&w[1], up);
-            if (down > w[2]) atomicMax(&w[2], down);
-            if (left > w[3]) atomicMax(&w[3], left);
-            if (right > w[4]) atomicMax(&w[4], right);
+          int slot = -1;
+          for (int probe = 0; probe < kWinSlots && slot < 0; ++probe) {
+            const int h = (tile + probe) & (kWinSlots - 1);
+            const int seen = atomicCAS(&s_tile[h], -1, tile);
+            if (seen == -1 || seen == tile) slot = h;
+          }
+          if (slot >= 0) {
+            if (-dy > s_ext[slot][0]) atomicMax(&s_ext[slot][0], -dy);
+            if (dy > s_ext[slot][1]) atomicMax(&s_ext[slot][1], dy);
+            if (-dx > s_ext[slot][2]) atomicMax(&s_ext[slot][2], -dx);
+            if (dx > s_ext[slot][3]) atomicMax(&s_ext[slot][3], dx);
+          } else {
+            grow_window(w, -dy, dy, -dx, dx);
           }
         }
       }
     }
+  }
+  if (GROW) {
+    __syncthreads();
+    if (threadIdx.x < kWinSlots && s_tile[threadIdx.x] >= 0)
+      grow_window(win + (size_t)s_tile[threadIdx.x] * 8, s_ext[threadIdx.x][0],
+                  s_ext[threadIdx.x][1], s_ext[threadIdx.x][2], s_ext[threadIdx.x][3]);
   }
 }
 
