@@ -1,0 +1,150 @@
+"""Seeded sweep over random small geometries: every entry-point family against the CPU oracle
+with shapes, channel counts, kernel sizes, interpolation, point counts and map character
+(locally coherent or scattered) drawn per seed.  The fixed cases of test_gpu_parity.py pin known
+corners; this sweep looks for the ones nobody thought of (tile remainders, channel paddings,
+plan / inverse-map / tiled-unpool paths and their fallbacks meeting odd sizes).
+Tolerances as everywhere: nearest gather and pooling bit-exact, float32 forward 1e-5, float32
+backward 1e-4, norm-relative.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import relerr
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FWD, BWD = 1e-5, 1e-4
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from _spherical_distortion_ext import _ops
+    return _ops
+
+
+def _t(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _n(t):
+    return t.detach().cpu().numpy()
+
+
+def _map(rng, grid, K, P, H, W, coherent):
+    """[*grid, K, (P,) 2] float32 map into an H x W image; about one sample in ten lands outside."""
+    shape = tuple(grid) + (K,) + ((P,) if P else ())
+    if coherent:
+        gy, gx = np.meshgrid(np.arange(grid[0]), np.arange(grid[1]), indexing="ij")
+        cx = gx * (W / grid[1])
+        cy = gy * (H / grid[0])
+        ang = 2 * np.pi * np.arange(K) / K
+        rad = 0.8 + (np.arange(K) % 3)
+        x = cx[..., None] + rad * np.cos(ang)
+        y = cy[..., None] + rad * np.sin(ang)
+        if P:
+            x = x[..., None] + rng.uniform(-1, 1, shape)
+            y = y[..., None] + rng.uniform(-1, 1, shape)
+        x = x + rng.uniform(-0.4, 0.4, shape)
+        y = y + rng.uniform(-0.4, 0.4, shape)
+    else:
+        x = rng.uniform(-1.5, W + 0.5, shape)
+        y = rng.uniform(-1.5, H + 0.5, shape)
+    snap = rng.uniform(size=shape) < 0.25          # exact pixel centres: zero-weight taps
+    x = np.where(snap, np.round(x), x)
+    y = np.where(snap, np.round(y), y)
+    return np.ascontiguousarray(np.stack([x, y], -1).astype(np.float32))
+
+
+def _geometry(seed):
+    rng = np.random.default_rng(5000 + seed)
+    interp = int(rng.integers(0, 3))
+    P = int(rng.choice([0, 0, 1, 2, 4]))
+    K = int(rng.choice([1, 2, 3, 5, 7, 9, 10]))
+    H, W = int(rng.integers(1, 40)), int(rng.integers(2, 70))
+    OH, OW = int(rng.integers(1, 30)), int(rng.integers(1, 50))
+    if rng.uniform() < 0.2:                         # vertex lists: one-row images
+        H, OH = 1, 1
+        W, OW = int(rng.integers(50, 600)), int(rng.integers(50, 600))
+    coherent = bool(rng.uniform() < 0.7)
+    return rng, interp, P, K, H, W, OH, OW, coherent
+
+
+def _conv_case(seed):
+    rng, interp, P, K, H, W, OH, OW, coherent = _geometry(seed)
+    B = int(rng.integers(1, 4))
+    Cin, Cout = int(rng.choice([1, 3, 8, 17, 32, 40, 64, 130])), int(rng.choice([1, 4, 16, 33, 64, 96, 136]))
+    m = _map(rng, (OH, OW), K, P, H, W, coherent)
+    iw = rng.uniform(0.1, 1, m.shape[:-1]).astype(np.float32) if P else None
+    x = rng.standard_normal((B, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(np.float32)
+    return rng, interp, K, H, W, OH, OW, B, Cin, Cout, m, iw, x, w, b, g
+
+
+@pytest.mark.parametrize("seed", range(100, 116))
+def test_convolution_bf16_operands(ops, oracle, seed):
+    """The bf16 compute mode (operands rounded to bf16, fp32 accumulation) on the same sweep:
+    1e-2 norm-relative against the float32 oracle."""
+    rng, interp, K, H, W, OH, OW, B, Cin, Cout, m, iw, x, w, b, g = _conv_case(seed)
+    ops.set_conv_compute("bf16")
+    try:
+        y = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(w), _t(b), K, interp))
+        gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(w), _t(b), K, interp)
+        gi, gw, gb = _n(gi), _n(gw), _n(gb)
+    finally:
+        ops.set_conv_compute("native")
+    assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= 1e-2
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
+    assert relerr(gi, wi) <= 1e-2 and relerr(gw, ww) <= 1e-2 and relerr(gb, wb) <= 1e-4
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_convolution_and_transposed(ops, oracle, seed):
+    rng, interp, K, H, W, OH, OW, B, Cin, Cout, m, iw, x, w, b, g = _conv_case(seed)
+    y = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(w), _t(b), K, interp))
+    assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= FWD
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(w), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and relerr(_n(gb), wb) <= BWD
+    # the transposed layer over the same map: input on the map's grid, output on the image
+    xt = rng.standard_normal((B, Cin, OH, OW)).astype(np.float32)
+    wt = (rng.standard_normal((Cin, Cout, K)) / np.sqrt(Cin * K)).astype(np.float32)
+    yt = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), _t(iw), _t(wt), _t(b), H, W, K, interp))
+    want = oracle.mapped_transposed_conv_forward(xt, m, wt, b, H, W, K, interp, iw)
+    assert relerr(yt, want) <= BWD
+    gt = rng.standard_normal(want.shape).astype(np.float32)
+    gi, gw, gb = ops.mapped_transposed_conv_backward(_t(gt), _t(m), _t(iw), _t(xt), _t(wt), _t(b),
+                                                     K, interp)
+    wi, ww, wb = oracle.mapped_transposed_conv_backward(gt, m, xt, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and relerr(_n(gb), wb) <= BWD
+
+
+@pytest.mark.parametrize("seed", range(40, 76))
+def test_pooling_and_resampling(ops, oracle, seed):
+    rng, interp, P, K, H, W, OH, OW, coherent = _geometry(seed)
+    B, C = int(rng.integers(1, 4)), int(rng.choice([1, 3, 7, 9, 20]))
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    # pooling
+    m = _map(rng, (OH, OW), K, P, H, W, coherent)
+    iw = rng.uniform(0.1, 1, m.shape[:-1]).astype(np.float32) if P else None
+    val, idx = ops.mapped_max_pool(_t(x), _t(m), _t(iw), K, interp)
+    wval, widx = oracle.mapped_max_pool(x, m, K, interp, iw)
+    assert np.array_equal(_n(idx), widx)
+    assert np.array_equal(_n(val), wval)
+    g = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
+    want = oracle.mapped_max_unpool(g, widx, m, H, W, K, interp, iw)
+    assert relerr(_n(ops.mapped_max_unpool(_t(g), idx, _t(m), _t(iw), H, W, K, interp)), want) <= BWD
+    # resampling over a map without the sample axis
+    mr = np.ascontiguousarray(m[:, :, 0])
+    iwr = None if iw is None else np.ascontiguousarray(iw[:, :, 0])
+    got = _n(ops.resample_from_map(_t(x), _t(mr), _t(iwr), interp))
+    wantr = oracle.resample_from_map(x, mr, interp, iwr)
+    if interp == 0 and not P:
+        assert np.array_equal(got, wantr)
+    else:
+        assert relerr(got, wantr) <= FWD
+    y = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
+    back = _n(ops.resample_to_map(_t(y), _t(mr), _t(iwr), H, W, interp))
+    assert relerr(back, oracle.resample_to_map(y, mr, H, W, interp, iwr)) <= BWD
