@@ -666,7 +666,7 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
 // cnt[u*K + k] counts the sources of (u, k); *gate counts taps that found no free slot: the
 // inverse is usable only if it stays 0.
 // ---------------------------------------------------------------------------
-constexpr int kInvSlots = 8;
+constexpr int kInvSlots = 16;
 
 template <int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kThreads) void inverse_fill_kernel(
@@ -730,9 +730,10 @@ struct InverseMap {
 };
 
 static bool inverse_candidate(const ConvGeom& g) {
-  // one tap per sample (nearest, unweighted): inverse lists are as short as the map is
-  // injective; K <= 256 for the row-count kernel; the pixel side is gathered with 32-bit offsets
-  return g.P == 0 && g.interp != 1 && g.interp != 2 && g.K <= 256 && g.M <= (1 << 24);
+  // Inverse lists are as short as the map is injective per sample: one source per target for a
+  // one-to-one map, about as many as a sample has taps for a map of unit scale.  K <= 256 for
+  // the row-count kernel; the pixel side is gathered with 32-bit offsets.
+  return g.K <= 256 && g.M <= (1 << 24);
 }
 
 static int inverse_tm(const ConvGeom& g) { return g.Cg <= 64 ? 256 : 128; }
@@ -818,14 +819,13 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                        const float* wts, const float* Wm, const float* bias, float* img,
                        float* workspace, hipStream_t stream, SharedPlan* shared) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
-  int rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
-  if (rc) return rc;
+  int rc = SDK_OK;
   if (planned_scatter_supported(g)) {
     const int* gate = nullptr;
     if (inverse_candidate(g)) {
-      // One tap per sample: try the scatter as a gather over the inverse map.  The inverse
-      // is built on the device; if a target collects more sources than its rows hold, the
-      // gather kernel exits at once and the scatter kernel below runs instead (and vice versa).
+      // Try the scatter as a gather over the inverse map.  The inverse is built on the device;
+      // if a target collects more sources than its rows hold, the gather kernel exits at once
+      // and the fill and the scatter kernel below run instead (and vice versa).
       const size_t base = ((staged_workspace_bytes(g) + 255) & ~(size_t)255) + plan_bytes(g);
       char* inv_ws = reinterpret_cast<char*>(workspace) + ((base + 255) & ~(size_t)255);
       InverseMap inv;
@@ -835,8 +835,12 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
       if (rc) return rc;
       gate = inv.gate;
     }
+    rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream, gate);
+    if (rc) return rc;
     return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream, shared);
   }
+  rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+  if (rc) return rc;
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;

@@ -105,7 +105,8 @@ static int gemm_strided(const T* A, const T* B, T* C, const T* row_bias, int m, 
 template <typename T>
 __global__ __launch_bounds__(256) void plane_fill_kernel(T* __restrict__ dst,
                                                          const T* __restrict__ bias, int C,
-                                                         size_t n) {
+                                                         size_t n, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const size_t plane = blockIdx.y;
   const T v = bias ? bias[plane % C] : T(0);
   T* p = dst + plane * n;
@@ -114,17 +115,19 @@ __global__ __launch_bounds__(256) void plane_fill_kernel(T* __restrict__ dst,
 }
 
 template <typename T>
-int plane_fill(T* dst, const T* bias, int64_t planes, int C, size_t n, hipStream_t stream) {
+int plane_fill(T* dst, const T* bias, int64_t planes, int C, size_t n, hipStream_t stream,
+               const int* gate) {
   if (planes == 0 || n == 0) return SDK_OK;
-  if (!bias) return zero_fill(dst, sizeof(T) * (size_t)planes * n, stream);
+  if (!bias) return zero_fill_gated(dst, sizeof(T) * (size_t)planes * n, stream, gate);
   if (planes > 65535) return fail(SDK_ERR_UNSUPPORTED, "plane_fill: too many planes");
   const dim3 grid((unsigned)std::min<int64_t>(ceil_div((int64_t)n, 256), 64), (unsigned)planes);
-  launch(plane_fill_kernel<T>, grid, dim3(256), stream, dst, bias, C, n);
+  launch(plane_fill_kernel<T>, grid, dim3(256), stream, dst, bias, C, n, gate);
   SDK_LAUNCH_CHECK("plane_fill");
   return SDK_OK;
 }
-template int plane_fill<float>(float*, const float*, int64_t, int, size_t, hipStream_t);
-template int plane_fill<double>(double*, const double*, int64_t, int, size_t, hipStream_t);
+template int plane_fill<float>(float*, const float*, int64_t, int, size_t, hipStream_t, const int*);
+template int plane_fill<double>(double*, const double*, int64_t, int, size_t, hipStream_t,
+                                const int*);
 
 template <typename T>
 int generic_gather_gemm(const ConvGeom& g, const T* img, const T* map, const T* wts, const T* Wm,

@@ -8,6 +8,8 @@
 namespace sdk {
 
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream);
+// gate: optional device flag; with one, the fill runs only if *gate != 0.
+int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
 
 // Batched mapped im2col / col2im over `planes` image planes (see
 // mapped_gather_scatter.hip).  col2im accumulates onto what `im` holds.
@@ -18,9 +20,11 @@ template <typename T>
 int launch_mapped_col2im(const T* col, const T* map, const T* wts, T* im, int64_t planes, int H,
                          int W, int M, int K, int P, int interp, hipStream_t stream);
 
-// dst[(b*C + c)*n + i] = bias ? bias[c] : 0 for `planes` = B*C planes of n elements.
+// dst[(b*C + c)*n + i] = bias ? bias[c] : 0 for `planes` = B*C planes of n elements; with a gate
+// (device flag) only if *gate != 0.
 template <typename T>
-int plane_fill(T* dst, const T* bias, int64_t planes, int C, size_t n, hipStream_t stream);
+int plane_fill(T* dst, const T* bias, int64_t planes, int C, size_t n, hipStream_t stream,
+               const int* gate = nullptr);
 
 // Geometry of one convolution-shaped call, shared by the generic and the fused
 // drivers.  "gather side" is the image the sample map points into, "pixel side"

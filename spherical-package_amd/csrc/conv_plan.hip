@@ -26,7 +26,8 @@ template <int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     const float* __restrict__ map, const float* __restrict__ wts, PixelTiling pt, int K, int P,
     int H, int W, int S, int* __restrict__ hdr, int* __restrict__ ns_out,
-    int2* __restrict__ taps) {
+    int2* __restrict__ taps, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
   __shared__ __align__(8) float stage[kPlanStage / sizeof(float)];
@@ -548,7 +549,7 @@ size_t plan_bytes(const ConvGeom& g) {
 }
 
 int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-               hipStream_t stream, Plan* plan) {
+               hipStream_t stream, Plan* plan, const int* gate) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
   const int S = plan_slots(g);
@@ -560,7 +561,7 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
   SDK_DISPATCH_INTERP(g.interp, g.P,
                       (launch(plan_kernel<INTERP, WEIGHTED>, dim3((unsigned)tiles),
                               dim3(kPlThreads), stream, map, wts, pt, g.K, g.P, g.H, g.W, S, hdr,
-                              ns, taps)));
+                              ns, taps, gate)));
   SDK_LAUNCH_CHECK("plan");
   plan->pt = pt;
   plan->tiles = (int)tiles;

@@ -36,8 +36,10 @@ bool plan_supported(const ConvGeom& g);
 size_t plan_bytes(const ConvGeom& g);
 
 // Builds the plan of (g, map, wts) in `workspace` (plan_bytes(g) bytes, 16-byte aligned).
+// gate: optional device flag; with one, the plan is built only if *gate != 0 (its only reader
+// is gated the same way).
 int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-               hipStream_t stream, Plan* plan);
+               hipStream_t stream, Plan* plan, const int* gate = nullptr);
 
 // gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
 bool planned_wgrad_supported(const ConvGeom& g);

@@ -306,7 +306,9 @@ int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const f
   }
   Plan plan;
   char* plan_ws = reinterpret_cast<char*>(workspace) + ((staged_workspace_bytes(g) + 255) & ~(size_t)255);
-  int rc = build_plan(g, map, wts, plan_ws, stream, &plan);
+  // a plan that only this (gated) kernel reads is built under the same gate; one that is
+  // handed on to the weight gradient is built in any case
+  int rc = build_plan(g, map, wts, plan_ws, stream, &plan, shared != nullptr ? nullptr : gate);
   if (rc) return rc;
   if (shared != nullptr) {
     shared->plan = plan;

@@ -54,11 +54,11 @@ __global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p, s
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) p[i] = z;
 }
 
-static int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
+int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream) {
   return zero_fill_gated(ptr, bytes, stream, nullptr);
 }
-static int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate) {
+int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate) {
   if (bytes == 0) return SDK_OK;
   // ptr comes from a framework allocator (>= 256-byte aligned) and all element
   // sizes divide 16, so only a tail of < 16 bytes needs the scalar kernel.
