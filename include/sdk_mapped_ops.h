@@ -108,6 +108,19 @@ int sdk_resample_to_map(const void* input, const void* sample_map, const void* i
                         int64_t height, int64_t width, int32_t num_interp_pts, int32_t interp,
                         int32_t dtype, sdk_stream_t stream);
 
+/* sdk_resample_to_map followed by sdk_normalize_by_weight_sum in one call:
+ * out[b,c] = splat(input[b,c]) / (weight_sum + eps), weight_sum [H,W] (required) = the splat of
+ * an all-ones plane.  With the workspace the division happens where the splat is gathered, so
+ * `out` is written once.  Replaces the reference's splat + weight-sum splat + division
+ * (layers/functional/sphere_ops.py:74-80, eps 1e-12; resample entry points as above). */
+int sdk_resample_to_map_normalized(const void* input, const void* sample_map,
+                                   const void* interp_weights, void* out, void* weight_sum,
+                                   void* workspace, size_t workspace_bytes, double eps,
+                                   int64_t batch, int64_t channels, int64_t map_height,
+                                   int64_t map_width, int64_t height, int64_t width,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   sdk_stream_t stream);
+
 /* data[p, i] /= (weight_sum[i] + eps) for p < planes, i < plane_size, in place.
  * The reference does this in Python for its weighted splat
  * (layers/functional/sphere_ops.py:74-80, eps 1e-12). */

@@ -19,6 +19,8 @@ _CONV_DIMS = [_i64] * 8 + [_i32] * 4 + [_vp]
 SIGNATURES = {
     "sdk_resample_from_map": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_resample_to_map": [_vp] * 6 + [_sz] + [_i64] * 6 + [_i32] * 3 + [_vp],
+    "sdk_resample_to_map_normalized": [_vp] * 6 + [_sz, ctypes.c_double] + [_i64] * 6 + [_i32] * 3
+                                      + [_vp],
     "sdk_normalize_by_weight_sum": [_vp, _vp, ctypes.c_double, _i64, _i64, _i32, _vp],
     "sdk_mapped_im2col": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],

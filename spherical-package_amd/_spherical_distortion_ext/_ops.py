@@ -135,11 +135,9 @@ def resample_to_map_normalized(x, sample_map, interp_weights, out_h, out_w, inte
     wsum = torch.empty((int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         ws, nws = _scatter_workspace(x, out_h, out_w)
-        _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
-                   _ptr(out), _ptr(wsum), _ptr(ws), nws, B, C, MH, MW, int(out_h), int(out_w), P,
-                   int(interp), _DTYPES[x.dtype], _stream(x))
-        _capi.call("sdk_normalize_by_weight_sum", _ptr(out), _ptr(wsum), float(eps), B * C,
-                   int(out_h) * int(out_w), _DTYPES[x.dtype], _stream(x))
+        _capi.call("sdk_resample_to_map_normalized", _ptr(x), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(out), _ptr(wsum), _ptr(ws), nws, float(eps), B, C,
+                   MH, MW, int(out_h), int(out_w), P, int(interp), _DTYPES[x.dtype], _stream(x))
     return out, wsum
 
 

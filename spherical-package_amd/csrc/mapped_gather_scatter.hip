@@ -110,26 +110,45 @@ __global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
 // resample_to_map (scatter).  Body: common/resample.h:11-31, :55-82.
 // ONES: the input is an implicit all-ones plane (weight-sum pass).
 // ---------------------------------------------------------------------------
-template <typename T, int INTERP, bool WEIGHTED, bool ONES>
+template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
-    T* __restrict__ out, int planes, int H, int W, int MP, int P, const int* __restrict__ gate) {
+    T* __restrict__ out, T* __restrict__ wsum, int planes, int H, int W, int MP, int P,
+    const int* __restrict__ gate) {
   if (gate != nullptr && *gate == 0) return;
   const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= MP) return;
-  const int plane0 = blockIdx.y * kPC;
-  const int np = min(kPC, planes - plane0);
   const size_t HW = (size_t)H * W;
   const int q = WEIGHTED ? P : 1;
+  const T* coords = map + (size_t)pix * q * 2;
+  const T* pw = WEIGHTED ? wts + (size_t)pix * q : nullptr;
+  const int chunks = (planes + kPC - 1) / kPC;
+  if ((int)blockIdx.y >= chunks) {   // the extra row of the grid: the weight-sum plane
+    const T one[1] = {T(1)};
+    scatter_sample<T, INTERP, WEIGHTED, 1>(wsum, 0, 1, coords, pw, P, H, W, one);
+    return;
+  }
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
   T val[kPC];
 #pragma unroll
-  for (int j = 0; j < kPC; ++j)
-    val[j] = ONES ? T(1) : (j < np ? in[(size_t)(plane0 + j) * MP + pix] : T(0));
-  scatter_sample<T, INTERP, WEIGHTED, kPC>(out + (size_t)plane0 * HW, HW, np,
-                                           map + (size_t)pix * q * 2,
-                                           WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W, val);
+  for (int j = 0; j < kPC; ++j) val[j] = j < np ? in[(size_t)(plane0 + j) * MP + pix] : T(0);
+  scatter_sample<T, INTERP, WEIGHTED, kPC>(out + (size_t)plane0 * HW, HW, np, coords, pw, P, H, W,
+                                           val);
 }
 
+// Zero fill of two buffers in one launch (16-byte aligned, sizes in 16-byte units).
+__global__ __launch_bounds__(kBlock) void zero16_pair_kernel(uint4* __restrict__ a, size_t na,
+                                                             uint4* __restrict__ b, size_t nb,
+                                                             const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < na + nb; i += stride) {
+    if (i < na) a[i] = z;
+    else b[i - na] = z;
+  }
+}
 
 // ---------------------------------------------------------------------------
 // resample_to_map as a gather over the inverted map.  inverse_fill: one thread per map
@@ -173,7 +192,7 @@ template <typename T, int PC>
 __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
     const T* __restrict__ in, const int* __restrict__ cnt, const int* __restrict__ src,
     const T* __restrict__ co, T* __restrict__ out, T* __restrict__ wsum, int planes, int HW,
-    int MP, const int* __restrict__ gate) {
+    int MP, const int* __restrict__ gate, int normalize, T eps) {
   if (*gate != 0) return;
   const int u = banded_pixel_block() * kBlock + threadIdx.x;
   if (u >= HW) return;
@@ -191,16 +210,20 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
 #pragma unroll
     for (int j = 0; j < PC; ++j) acc[j] += c * in[(size_t)(plane0 + (j < np ? j : 0)) * MP + m];
   }
+  // normalised: the weight sum of the pixel is the sum of its list, no second pass needed
+  const T den = wtot + eps;
 #pragma unroll
   for (int j = 0; j < PC; ++j)
-    if (j < np) out[(size_t)(plane0 + j) * HW + u] = acc[j];
+    if (j < np) out[(size_t)(plane0 + j) * HW + u] = normalize ? acc[j] / den : acc[j];
   if (wsum != nullptr && blockIdx.y == 0) wsum[u] = wtot;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void normalize_kernel(T* __restrict__ data,
                                                            const T* __restrict__ wsum, T eps,
-                                                           size_t plane_size, size_t total) {
+                                                           size_t plane_size, size_t total,
+                                                           const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
   const size_t stride = (size_t)gridDim.x * kBlock;
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride)
     data[i] = data[i] / (wsum[i % plane_size] + eps);
@@ -563,9 +586,9 @@ static int check_plane(int64_t h, int64_t w, const char* what) {
 }
 
 static int check_grid_y(int64_t planes, const char* what) {
-  if (ceil_div(planes, kPC) > 65535)
+  if (ceil_div(planes, kPC) > 65534)   // one grid row is kept for a weight-sum plane
     return fail(SDK_ERR_UNSUPPORTED, "%s: batch*channels = %lld exceeds %d", what,
-                (long long)planes, 65535 * kPC);
+                (long long)planes, 65534 * kPC);
   return SDK_OK;
 }
 
@@ -598,7 +621,8 @@ static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
 template <typename T>
 static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
                                   void* workspace, size_t workspace_bytes, int64_t planes, int H,
-                                  int W, int MP, int P, int interp, hipStream_t stream) {
+                                  int W, int MP, int P, int interp, hipStream_t stream,
+                                  bool normalize = false, double eps = 0.0) {
   const int HW = H * W;
   const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
   size_t off[4];
@@ -621,32 +645,41 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
   launch(resample_inverse_gather_kernel<T, PCv>,                                                 \
          dim3(banded_grid_x(HW), (unsigned)std::max<int64_t>(1, ceil_div(planes, PCv))),         \
          dim3(kBlock), stream, in, (const int*)cnt, (const int*)src, (const T*)co, out, wsum,    \
-         (int)planes, HW, MP, (const int*)g)
+         (int)planes, HW, MP, (const int*)g, normalize ? 1 : 0, (T)eps)
       if (pc == 8) RIG(8); else if (pc == 4) RIG(4); else RIG(2);
 #undef RIG
       SDK_LAUNCH_CHECK("resample_to_map(inverse gather)");
     }
     gate = g;
   }
-  int rc = zero_fill_gated(out, sizeof(T) * (size_t)planes * H * W, stream, gate);
-  if (rc != SDK_OK) return rc;
-  const dim3 grid(banded_grid_x(MP), (unsigned)ceil_div(planes, kPC));
-  if (planes > 0) {
+  // the scatter: fills, then one launch for all planes and (an extra grid row) the weight sum
+  const size_t out_bytes = sizeof(T) * (size_t)planes * H * W, sum_bytes = sizeof(T) * (size_t)H * W;
+  if (wsum && out_bytes % 16 == 0 && sum_bytes % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+      (uintptr_t)wsum % 16 == 0) {
+    const size_t n16 = (out_bytes + sum_bytes) / 16;
+    const int blocks = (int)std::min<size_t>(ceil_div((int64_t)n16, kBlock), 256 * 16);
+    launch(zero16_pair_kernel, dim3(blocks), dim3(kBlock), stream, (uint4*)out, out_bytes / 16,
+           (uint4*)wsum, sum_bytes / 16, gate);
+    SDK_LAUNCH_CHECK("resample_to_map(fill)");
+  } else {
+    int rc = zero_fill_gated(out, out_bytes, stream, gate);
+    if (rc != SDK_OK) return rc;
+    if (wsum) rc = zero_fill_gated(wsum, sum_bytes, stream, gate);
+    if (rc != SDK_OK) return rc;
+  }
+  if (planes > 0 || wsum) {
+    const dim3 grid(banded_grid_x(MP), (unsigned)(ceil_div(planes, kPC) + (wsum ? 1 : 0)));
     SDK_DISPATCH_INTERP(interp, P,
-                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, false>), grid,
-                                dim3(kBlock), stream, in, map, wts, out, (int)planes, H, W, MP, P,
-                                gate)));
+                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED>), grid, dim3(kBlock),
+                                stream, in, map, wts, out, wsum, (int)planes, H, W, MP, P, gate)));
     SDK_LAUNCH_CHECK("resample_to_map");
   }
-  if (wsum) {
-    rc = zero_fill_gated(wsum, sizeof(T) * (size_t)H * W, stream, gate);
-    if (rc != SDK_OK) return rc;
-    const dim3 g1(banded_grid_x(MP), 1);
-    SDK_DISPATCH_INTERP(interp, P,
-                        (launch((resample_to_map_kernel<T, INTERP, WEIGHTED, true>), g1,
-                                dim3(kBlock), stream, (const T*)nullptr, map, wts, wsum, 1, H, W,
-                                MP, P, gate)));
-    SDK_LAUNCH_CHECK("resample_to_map(weight_sum)");
+  if (normalize && planes > 0) {   // scatter path only: the gather has divided already
+    const size_t total = (size_t)planes * HW;
+    const int blocks = (int)std::min<int64_t>(ceil_div((int64_t)total, kBlock), 256 * 16);
+    launch(normalize_kernel<T>, dim3(blocks), dim3(kBlock), stream, out, (const T*)wsum, (T)eps,
+           (size_t)HW, total, gate);
+    SDK_LAUNCH_CHECK("resample_to_map(normalise)");
   }
   return SDK_OK;
 }
@@ -800,12 +833,15 @@ size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_
   return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off);
 }
 
-int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
-                        void* out, void* weight_sum, void* workspace, size_t workspace_bytes,
-                        int64_t batch, int64_t channels, int64_t map_height, int64_t map_width,
-                        int64_t height, int64_t width, int32_t num_interp_pts, int32_t interp,
-                        int32_t dtype, sdk_stream_t stream) {
+static int resample_to_map_entry(const void* input, const void* sample_map,
+                                 const void* interp_weights, void* out, void* weight_sum,
+                                 void* workspace, size_t workspace_bytes, int64_t batch,
+                                 int64_t channels, int64_t map_height, int64_t map_width,
+                                 int64_t height, int64_t width, int32_t num_interp_pts,
+                                 int32_t interp, int32_t dtype, sdk_stream_t stream,
+                                 bool normalize, double eps) {
   SDK_REQUIRE(input && sample_map && out, "resample_to_map: NULL pointer");
+  SDK_REQUIRE(!normalize || weight_sum, "resample_to_map_normalized: NULL weight_sum");
   SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
               "resample_to_map: weighted map needs interp_weights");
   SDK_REQUIRE(batch >= 0 && channels >= 0, "resample_to_map: negative size");
@@ -821,8 +857,30 @@ int sdk_resample_to_map(const void* input, const void* sample_map, const void* i
                                 (const T*)input, (const T*)sample_map, (const T*)interp_weights,
                                 (T*)out, (T*)weight_sum, workspace, workspace_bytes, planes,
                                 (int)height, (int)width, (int)(map_height * map_width),
-                                num_interp_pts, interp, (hipStream_t)stream));
+                                num_interp_pts, interp, (hipStream_t)stream, normalize, eps));
   return SDK_OK;
+}
+
+int sdk_resample_to_map(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, void* weight_sum, void* workspace, size_t workspace_bytes,
+                        int64_t batch, int64_t channels, int64_t map_height, int64_t map_width,
+                        int64_t height, int64_t width, int32_t num_interp_pts, int32_t interp,
+                        int32_t dtype, sdk_stream_t stream) {
+  return resample_to_map_entry(input, sample_map, interp_weights, out, weight_sum, workspace,
+                               workspace_bytes, batch, channels, map_height, map_width, height,
+                               width, num_interp_pts, interp, dtype, stream, false, 0.0);
+}
+
+int sdk_resample_to_map_normalized(const void* input, const void* sample_map,
+                                   const void* interp_weights, void* out, void* weight_sum,
+                                   void* workspace, size_t workspace_bytes, double eps,
+                                   int64_t batch, int64_t channels, int64_t map_height,
+                                   int64_t map_width, int64_t height, int64_t width,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   sdk_stream_t stream) {
+  return resample_to_map_entry(input, sample_map, interp_weights, out, weight_sum, workspace,
+                               workspace_bytes, batch, channels, map_height, map_width, height,
+                               width, num_interp_pts, interp, dtype, stream, true, eps);
 }
 
 int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, int64_t planes,
@@ -835,7 +893,7 @@ int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, 
   SDK_DISPATCH_DTYPE(dtype, (launch(normalize_kernel<T>, dim3(blocks), dim3(kBlock),
                                                 (hipStream_t)stream, (T*)data,
                                                 (const T*)weight_sum, (T)eps, (size_t)plane_size,
-                                                total)));
+                                                total, (const int*)nullptr)));
   SDK_LAUNCH_CHECK("normalize_by_weight_sum");
   return SDK_OK;
 }

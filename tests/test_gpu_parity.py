@@ -102,6 +102,13 @@ def test_resample_to_map_crowded_targets_and_no_workspace(ops, oracle, interp, w
     _capi.call("sdk_resample_to_map", ops._ptr(ty), ops._ptr(tm), ops._ptr(tw), ops._ptr(out),
                None, None, 0, B, C, MH, MW, H, W, P if weighted else 0, interp, 0, ops._stream(ty))
     assert relerr(_n(out), want) <= 1e-4
+    # ... and the normalised variant without workspace: scatter, weight-sum scatter, division
+    wsum2 = torch.empty((H, W), dtype=torch.float32, device=DEV)
+    _capi.call("sdk_resample_to_map_normalized", ops._ptr(ty), ops._ptr(tm), ops._ptr(tw),
+               ops._ptr(out), ops._ptr(wsum2), None, 0, 1e-12, B, C, MH, MW, H, W,
+               P if weighted else 0, interp, 0, ops._stream(ty))
+    assert relerr(_n(wsum2), ones) <= 1e-4
+    assert relerr(_n(out), want / (ones + dt(1e-12))) <= 1e-3
 
 
 @pytest.mark.parametrize("case", CASES, ids=_ids)
