@@ -27,6 +27,14 @@ def _t(a):
     return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
 
 
+def _bias_grad_ok(got, want, g, tol=BWD):
+    """grad_bias is a plain sum of thousands of signed values: its float32 rounding error scales
+    with the sum of magnitudes, not with the (possibly cancelled) result, so a channel whose sum
+    nearly cancels is compared against 1 % of sum |g| rather than against |sum g|."""
+    scale = max(np.abs(want).max(), 1e-2 * np.abs(g).sum(axis=(0, 2, 3)).max())
+    return np.abs(np.asarray(got, np.float64) - want).max() <= tol * scale
+
+
 def _n(t):
     return t.detach().cpu().numpy()
 
@@ -97,7 +105,7 @@ def test_convolution_bf16_operands(ops, oracle, seed):
         ops.set_conv_compute("native")
     assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= 1e-2
     wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
-    assert relerr(gi, wi) <= 1e-2 and relerr(gw, ww) <= 1e-2 and relerr(gb, wb) <= 1e-4
+    assert relerr(gi, wi) <= 1e-2 and relerr(gw, ww) <= 1e-2 and _bias_grad_ok(gb, wb, g)
 
 
 @pytest.mark.parametrize("seed", range(40))
@@ -107,7 +115,7 @@ def test_convolution_and_transposed(ops, oracle, seed):
     assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= FWD
     gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(w), _t(b), K, interp)
     wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
-    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and relerr(_n(gb), wb) <= BWD
+    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and _bias_grad_ok(_n(gb), wb, g)
     # the transposed layer over the same map: input on the map's grid, output on the image
     xt = rng.standard_normal((B, Cin, OH, OW)).astype(np.float32)
     wt = (rng.standard_normal((Cin, Cout, K)) / np.sqrt(Cin * K)).astype(np.float32)
@@ -118,7 +126,7 @@ def test_convolution_and_transposed(ops, oracle, seed):
     gi, gw, gb = ops.mapped_transposed_conv_backward(_t(gt), _t(m), _t(iw), _t(xt), _t(wt), _t(b),
                                                      K, interp)
     wi, ww, wb = oracle.mapped_transposed_conv_backward(gt, m, xt, wt, b, K, interp, iw)
-    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and relerr(_n(gb), wb) <= BWD
+    assert relerr(_n(gi), wi) <= BWD and relerr(_n(gw), ww) <= BWD and _bias_grad_ok(_n(gb), wb, gt)
 
 
 @pytest.mark.parametrize("seed", range(40, 76))
