@@ -197,10 +197,16 @@ def bench_pool3(torch, ops, timer, steps, warmup):
     ms_b, _ = timer.run(lambda: ops.mapped_max_unpool(g, idx, m, None, H, W, K, 0), steps, warmup)
     fwd_bytes = _nbytes(x, m, val, idx)
     bwd_bytes = _nbytes(g, idx, m, x)
+    # average pooling on the same input and map: no index tensor on either side
+    ms_af, _ = timer.run(lambda: ops.mapped_avg_pool(x, m, None, K, 0), steps, warmup)
+    ms_ab, _ = timer.run(lambda: ops.mapped_avg_unpool(g, m, None, H, W, K, 0), steps, warmup)
+    avg_bytes = _nbytes(x, m, val)
     return {"pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f,
                                                   traffic=_measured_traffic("mapped_max_pool"))),
             "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b,
                                                    traffic=_measured_traffic("mapped_max_unpool"))),
+            "avg_pool_forward": dict(ms=ms_af, **_roof("hbm", avg_bytes, ms_af)),
+            "avg_pool_backward": dict(ms=ms_ab, **_roof("hbm", avg_bytes, ms_ab)),
             "no_winner_outputs": int((idx < 0).sum().item())}
 
 

@@ -166,6 +166,30 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
                         int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
                         int32_t dtype, sdk_stream_t stream);
 
+/* Mapped average pool: out[b,c,oy,ox] = (sum over the K samples of the interpolated input) / K,
+ * summed in ascending sample order.  Replaces `_mapped_avg_pooling.mapped_avg_pool` /
+ * `_weighted_mapped_avg_pooling.weighted_mapped_avg_pool`
+ * (ext_modules/include/layers/mapped_avg_pooling_layer.h, weighted_mapped_avg_pooling_layer.h;
+ *  body common/mapped_avg_pool.h:13-40, :70-105). */
+int sdk_mapped_avg_pool(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                        int64_t out_height, int64_t out_width, int64_t kernel_size,
+                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                        sdk_stream_t stream);
+
+/* Its adjoint: grad_input [B,C,H,W] (fully written by the call) receives grad_output / K
+ * splatted at every one of the K samples of its pixel.  `workspace` as for
+ * sdk_resample_to_map (sdk_resample_to_map_workspace_bytes(height, width, dtype)): with it the
+ * splat runs as a gather over the inverted map, without it (NULL, 0) with float atomics.
+ * Replaces `_mapped_avg_pooling.mapped_avg_unpool` / `weighted_mapped_avg_unpool`
+ * (same headers; body common/mapped_avg_pool.h:42-68, :107-140). */
+int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
+                          const void* interp_weights, void* grad_input, void* workspace,
+                          size_t workspace_bytes, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t out_height, int64_t out_width,
+                          int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                          int32_t dtype, sdk_stream_t stream);
+
 /* grad_input [B,C,H,W] (fully written by the call) receives grad_output[b,c,oy,ox]
  * splatted at the sample the stored index names, with the same interpolation.
  * Negative or out-of-range indices contribute nothing.

@@ -156,6 +156,28 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, in_h, in_w, kernel_size
     return out
 
 
+def mapped_avg_pool(x, sample_map, kernel_size, interp, interp_weights=None):
+    x = _c(x); m = _c(sample_map, x.dtype); w = _c(interp_weights, x.dtype)
+    B, C, H, W = x.shape
+    OH, OW = m.shape[:2]
+    out = np.empty((B, C, OH, OW), x.dtype)
+    _check(lib().sdk_oracle_mapped_avg_pool(
+        _p(x), _p(m), _p(w), _p(out), *_i64(B, C, H, W, OH, OW, kernel_size),
+        *_i32(_num_pts(m, w), int(interp), _dt(x))))
+    return out
+
+
+def mapped_avg_unpool(grad_output, sample_map, in_h, in_w, kernel_size, interp,
+                      interp_weights=None):
+    g = _c(grad_output); m = _c(sample_map, g.dtype); w = _c(interp_weights, g.dtype)
+    B, C, OH, OW = g.shape
+    out = np.empty((B, C, in_h, in_w), g.dtype)
+    _check(lib().sdk_oracle_mapped_avg_unpool(
+        _p(g), _p(m), _p(w), _p(out), *_i64(B, C, in_h, in_w, OH, OW, kernel_size),
+        *_i32(_num_pts(m, w), int(interp), _dt(g))))
+    return out
+
+
 def mapped_conv_forward(x, sample_map, weight, bias, kernel_size, interp,
                         interp_weights=None):
     x = _c(x); m = _c(sample_map, x.dtype); w = _c(interp_weights, x.dtype)

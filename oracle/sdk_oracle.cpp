@@ -23,6 +23,8 @@
 //       + F.conv2d special case + compiled-reference fixtures
 //   max pool values: reference known-answer vectors; argmax index encoding and
 //       the CPU initial-value quirk: compiled-reference fixtures.
+//   average pool / unpool: reference known-answer vector (tests/test_mapped_pooling.py:110-132)
+//       + "mean over k of the pinned im2col rows" + adjoint identity.
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -433,6 +435,46 @@ void max_unpool(const T* gout, const int64_t* idx, const T* map, const T* wts, T
   }
 }
 
+// ---------------------------------------------------------------------------
+// Mapped average pool and its adjoint.  common/mapped_avg_pool.h:13-40 (:70-105
+// weighted): the K samples are summed in ascending order and the sum is divided
+// by K; :42-68 (:107-140 weighted): every sample of a pooled pixel receives
+// grad / K (divided first, then splatted).
+// ---------------------------------------------------------------------------
+template <typename T>
+void avg_pool(const T* x, const T* map, const T* wts, T* out, int64_t B, int64_t C, int64_t H,
+              int64_t W, int64_t OH, int64_t OW, int64_t K, int P, int interp) {
+  const int64_t M = OH * OW, q = pts(P);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < B * C * M; ++i) {
+    const int64_t pix = i % M, plane = i / M;
+    T accum = T(0);
+    for (int64_t k = 0; k < K; ++k) {
+      const int64_t s = (pix * K + k) * q;
+      accum += gather_sample(x + plane * H * W, map + s * 2, wts ? wts + s : nullptr, P, H, W,
+                             interp);
+    }
+    out[i] = accum / T(K);
+  }
+}
+
+template <typename T>
+void avg_unpool(const T* gout, const T* map, const T* wts, T* gin, int64_t B, int64_t C,
+                int64_t H, int64_t W, int64_t OH, int64_t OW, int64_t K, int P, int interp) {
+  const int64_t M = OH * OW, q = pts(P);
+  std::memset(gin, 0, sizeof(T) * B * C * H * W);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < B * C * M; ++i) {
+    const int64_t pix = i % M, plane = i / M;
+    const T value = gout[i] / T(K);
+    for (int64_t k = 0; k < K; ++k) {
+      const int64_t s = (pix * K + k) * q;
+      scatter_sample(value, gin + plane * H * W, map + s * 2, wts ? wts + s : nullptr, P, H, W,
+                     interp);
+    }
+  }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -492,6 +534,20 @@ int sdk_oracle_mapped_max_unpool(const void* gout, const int64_t* idx, const voi
                                  int interp, int dtype) {
   DISPATCH(dtype, max_unpool<T>((const T*)gout, idx, (const T*)map, (const T*)wts, (T*)gin, B,
                                  C, H, W, OH, OW, K, P, interp));
+}
+
+int sdk_oracle_mapped_avg_pool(const void* x, const void* map, const void* wts, void* out,
+                               int64_t B, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                               int64_t K, int P, int interp, int dtype) {
+  DISPATCH(dtype, avg_pool<T>((const T*)x, (const T*)map, (const T*)wts, (T*)out, B, C, H, W, OH,
+                               OW, K, P, interp));
+}
+
+int sdk_oracle_mapped_avg_unpool(const void* gout, const void* map, const void* wts, void* gin,
+                                 int64_t B, int64_t C, int64_t H, int64_t W, int64_t OH,
+                                 int64_t OW, int64_t K, int P, int interp, int dtype) {
+  DISPATCH(dtype, avg_unpool<T>((const T*)gout, (const T*)map, (const T*)wts, (T*)gin, B, C, H, W,
+                                 OH, OW, K, P, interp));
 }
 
 int sdk_oracle_mapped_conv_forward(const void* x, const void* map, const void* wts,

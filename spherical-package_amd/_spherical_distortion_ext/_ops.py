@@ -226,6 +226,40 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, i
     return gin
 
 
+def mapped_avg_pool(x, sample_map, interp_weights, kernel_size, interp):
+    _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, H, W = x.shape
+    OH, OW, K = sample_map.shape[:3]
+    if K != int(kernel_size):
+        raise RuntimeError("kernel_size %d does not match sample_map %s"
+                           % (int(kernel_size), tuple(sample_map.shape)))
+    out = torch.empty((B, C, OH, OW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_mapped_avg_pool", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(out), B, C, H, W, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _stream(x))
+    return out
+
+
+def mapped_avg_unpool(grad_output, sample_map, interp_weights, in_h, in_w, kernel_size, interp):
+    _check(grad_output, grad_output=grad_output, sample_map=sample_map,
+           interp_weights=interp_weights)
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, OH, OW = grad_output.shape
+    if tuple(sample_map.shape[:3]) != (OH, OW, int(kernel_size)):
+        raise RuntimeError("sample_map %s does not match grad_output %s / kernel_size %d"
+                           % (tuple(sample_map.shape), tuple(grad_output.shape), int(kernel_size)))
+    gin = torch.empty((B, C, int(in_h), int(in_w)), dtype=grad_output.dtype,
+                      device=grad_output.device)
+    with torch.cuda.device(grad_output.device):
+        ws, nws = _scatter_workspace(grad_output, in_h, in_w)
+        _capi.call("sdk_mapped_avg_unpool", _ptr(grad_output), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(gin), _ptr(ws), nws, B, C, int(in_h), int(in_w),
+                   OH, OW, int(kernel_size), P, int(interp), _DTYPES[grad_output.dtype],
+                   _stream(grad_output))
+    return gin
+
+
 # --------------------------------------------------------------------------- convolution
 def _conv_dims(x_shape, weight, sample_map, kernel_size, transposed):
     K = int(kernel_size)
@@ -348,6 +382,12 @@ _SCHEMAS = (
     ("mapped_max_unpool",
      "(Tensor grad_output, Tensor idx_mask, Tensor sample_map, Tensor? interp_weights, int in_h,"
      " int in_w, int kernel_size, int interp) -> Tensor", mapped_max_unpool),
+    ("mapped_avg_pool",
+     "(Tensor x, Tensor sample_map, Tensor? interp_weights, int kernel_size, int interp)"
+     " -> Tensor", mapped_avg_pool),
+    ("mapped_avg_unpool",
+     "(Tensor grad_output, Tensor sample_map, Tensor? interp_weights, int in_h, int in_w,"
+     " int kernel_size, int interp) -> Tensor", mapped_avg_unpool),
     ("mapped_conv_forward",
      "(Tensor x, Tensor sample_map, Tensor? interp_weights, Tensor weight, Tensor bias,"
      " int kernel_size, int interp) -> Tensor", mapped_conv_forward),

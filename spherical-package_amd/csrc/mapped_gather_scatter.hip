@@ -114,7 +114,7 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ out, T* __restrict__ wsum, int planes, int H, int W, int MP, int P,
-    const int* __restrict__ gate) {
+    const int* __restrict__ gate, int group) {
   if (gate != nullptr && *gate == 0) return;
   const int pix = banded_pixel_block() * kBlock + threadIdx.x;
   if (pix >= MP) return;
@@ -130,9 +130,16 @@ __global__ __launch_bounds__(kBlock) void resample_to_map_kernel(
   }
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
+  // group > 1 (average unpooling): `group` consecutive map entries are the samples of one
+  // source pixel, each of which receives the pixel's value divided by `group`
+  const int src = group > 1 ? pix / group : pix;
+  const size_t in_plane = group > 1 ? (size_t)(MP / group) : (size_t)MP;
   T val[kPC];
 #pragma unroll
-  for (int j = 0; j < kPC; ++j) val[j] = j < np ? in[(size_t)(plane0 + j) * MP + pix] : T(0);
+  for (int j = 0; j < kPC; ++j) {
+    val[j] = j < np ? in[(size_t)(plane0 + j) * in_plane + src] : T(0);
+    if (group > 1) val[j] = val[j] / T(group);
+  }
   scatter_sample<T, INTERP, WEIGHTED, kPC>(out + (size_t)plane0 * HW, HW, np, coords, pw, P, H, W,
                                            val);
 }
@@ -192,11 +199,12 @@ template <typename T, int PC>
 __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
     const T* __restrict__ in, const int* __restrict__ cnt, const int* __restrict__ src,
     const T* __restrict__ co, T* __restrict__ out, T* __restrict__ wsum, int planes, int HW,
-    int MP, const int* __restrict__ gate, int normalize, T eps) {
+    int MP, const int* __restrict__ gate, int normalize, T eps, int group) {
   if (*gate != 0) return;
   const int u = banded_pixel_block() * kBlock + threadIdx.x;
   if (u >= HW) return;
   const int plane0 = blockIdx.y * PC;
+  const size_t in_plane = group > 1 ? (size_t)(MP / group) : (size_t)MP;
   const int np = min(PC, planes - plane0);
   const int n = min(cnt[u], kInvSlots);
   T acc[PC];
@@ -204,11 +212,16 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
   for (int j = 0; j < PC; ++j) acc[j] = T(0);
   T wtot = T(0);
   for (int s = 0; s < n; ++s) {
-    const int m = src[(size_t)s * HW + u];
+    int m = src[(size_t)s * HW + u];
+    if (group > 1) m /= group;   // map entry -> source pixel (average unpooling)
     const T c = co[(size_t)s * HW + u];
     wtot += c;
 #pragma unroll
-    for (int j = 0; j < PC; ++j) acc[j] += c * in[(size_t)(plane0 + (j < np ? j : 0)) * MP + m];
+    for (int j = 0; j < PC; ++j) {
+      T v = in[(size_t)(plane0 + (j < np ? j : 0)) * in_plane + m];
+      if (group > 1) v = v / T(group);
+      acc[j] += c * v;
+    }
   }
   // normalised: the weight sum of the pixel is the sum of its list, no second pass needed
   const T den = wtot + eps;
@@ -318,6 +331,35 @@ __global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
       idx[o] = best_k[j] < 0 ? (int64_t)-1
                              : (int64_t)(((size_t)pix * K + best_k[j]) * q * 2);
     }
+}
+
+// Average pool: body common/mapped_avg_pool.h:13-40, :70-105 (sum of the K samples in
+// ascending order, divided by K).  Its adjoint (:42-68, :107-140: every sample of a pixel
+// receives grad / K) is the resample scatter over the map read as [pixels * K] entries.
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_avg_pool_kernel(
+    const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
+    T* __restrict__ out, int planes, int H, int W, int M, int K, int P) {
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
+  if (pix >= M) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t HW = (size_t)H * W;
+  const int q = WEIGHTED ? P : 1;
+  T sum[kPC];
+#pragma unroll
+  for (int j = 0; j < kPC; ++j) sum[j] = T(0);
+  for (int k = 0; k < K; ++k) {
+    const size_t s = ((size_t)pix * K + k) * q;
+    T v[kPC];
+    gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                            WEIGHTED ? wts + s : nullptr, P, H, W, v);
+#pragma unroll
+    for (int j = 0; j < kPC; ++j) sum[j] += v[j];
+  }
+#pragma unroll
+  for (int j = 0; j < kPC; ++j)
+    if (j < np) out[(size_t)(plane0 + j) * M + pix] = sum[j] / T(K);
 }
 
 // Unpool: body common/mapped_max_pool.h:60-78, :136-171.  One thread per pooled
@@ -622,7 +664,7 @@ template <typename T>
 static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
                                   void* workspace, size_t workspace_bytes, int64_t planes, int H,
                                   int W, int MP, int P, int interp, hipStream_t stream,
-                                  bool normalize = false, double eps = 0.0) {
+                                  bool normalize = false, double eps = 0.0, int group = 1) {
   const int HW = H * W;
   const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
   size_t off[4];
@@ -645,7 +687,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
   launch(resample_inverse_gather_kernel<T, PCv>,                                                 \
          dim3(banded_grid_x(HW), (unsigned)std::max<int64_t>(1, ceil_div(planes, PCv))),         \
          dim3(kBlock), stream, in, (const int*)cnt, (const int*)src, (const T*)co, out, wsum,    \
-         (int)planes, HW, MP, (const int*)g, normalize ? 1 : 0, (T)eps)
+         (int)planes, HW, MP, (const int*)g, normalize ? 1 : 0, (T)eps, group)
       if (pc == 8) RIG(8); else if (pc == 4) RIG(4); else RIG(2);
 #undef RIG
       SDK_LAUNCH_CHECK("resample_to_map(inverse gather)");
@@ -671,7 +713,8 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
     const dim3 grid(banded_grid_x(MP), (unsigned)(ceil_div(planes, kPC) + (wsum ? 1 : 0)));
     SDK_DISPATCH_INTERP(interp, P,
                         (launch((resample_to_map_kernel<T, INTERP, WEIGHTED>), grid, dim3(kBlock),
-                                stream, in, map, wts, out, wsum, (int)planes, H, W, MP, P, gate)));
+                                stream, in, map, wts, out, wsum, (int)planes, H, W, MP, P, gate,
+                                group)));
     SDK_LAUNCH_CHECK("resample_to_map");
   }
   if (normalize && planes > 0) {   // scatter path only: the gather has divided already
@@ -970,6 +1013,54 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
                                               (int)planes, (int)height, (int)width, (int)M,
                                               (int)kernel_size, num_interp_pts))));
   SDK_LAUNCH_CHECK("mapped_max_pool");
+  return SDK_OK;
+}
+
+int sdk_mapped_avg_pool(const void* input, const void* sample_map, const void* interp_weights,
+                        void* out, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                        int64_t out_height, int64_t out_width, int64_t kernel_size,
+                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                        sdk_stream_t stream) {
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_avg_pool: bad output size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(input, sample_map, interp_weights, out, batch, channels, height, width, M,
+                        kernel_size, num_interp_pts, "mapped_avg_pool");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
+  SDK_DISPATCH_DTYPE(
+      dtype,
+      SDK_DISPATCH_INTERP(interp, num_interp_pts,
+                          (launch((mapped_avg_pool_kernel<T, INTERP, WEIGHTED>), grid,
+                                  dim3(kBlock), (hipStream_t)stream, (const T*)input,
+                                  (const T*)sample_map, (const T*)interp_weights, (T*)out,
+                                  (int)planes, (int)height, (int)width, (int)M, (int)kernel_size,
+                                  num_interp_pts))));
+  SDK_LAUNCH_CHECK("mapped_avg_pool");
+  return SDK_OK;
+}
+
+int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
+                          const void* interp_weights, void* grad_input, void* workspace,
+                          size_t workspace_bytes, int64_t batch, int64_t channels, int64_t height,
+                          int64_t width, int64_t out_height, int64_t out_width,
+                          int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                          int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_avg_unpool: bad pooled size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(grad_output, sample_map, interp_weights, grad_input, batch, channels,
+                        height, width, M, kernel_size, num_interp_pts, "mapped_avg_unpool");
+  if (rc) return rc;
+  SDK_REQUIRE(M * kernel_size < ((int64_t)1 << 31), "mapped_avg_unpool: too many samples");
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_resample_to_map<T>(
+                                (const T*)grad_output, (const T*)sample_map,
+                                (const T*)interp_weights, (T*)grad_input, (T*)nullptr, workspace,
+                                workspace_bytes, planes, (int)height, (int)width,
+                                (int)(M * kernel_size), num_interp_pts, interp,
+                                (hipStream_t)stream, false, 0.0, (int)kernel_size));
   return SDK_OK;
 }
 

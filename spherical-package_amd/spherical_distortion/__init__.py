@@ -3,7 +3,7 @@
 Mirrors the part of the reference's `spherical_distortion` package (its
 `layers/` directory, reference setup.py:211-228) that sits on the mapped
 operation path: `nn.MappedConvolution`, `nn.MappedTransposedConvolution`,
-`nn.MappedMaxPool`, `nn.Resample`, `nn.Unresample` and the matching
+`nn.MappedMaxPool`, `nn.MappedAvgPool`, `nn.MappedAvgUnpool`, `nn.Resample`, `nn.Unresample` and the matching
 `functional` entry points, with the reference's names, signatures, parameter
 shapes, initialisation and argument checks.  The arithmetic is done by the
 gfx950 HIP kernels behind `_spherical_distortion_ext`.

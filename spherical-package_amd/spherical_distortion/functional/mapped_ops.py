@@ -6,10 +6,12 @@ weighted and unweighted extension modules, same gradient tuple arity.
 """
 import torch
 
+import _spherical_distortion_ext._mapped_avg_pooling as _mapped_avg_pool
 import _spherical_distortion_ext._mapped_convolution as _mapped_conv
 import _spherical_distortion_ext._mapped_max_pooling as _mapped_max_pool
 import _spherical_distortion_ext._mapped_transposed_convolution as _mapped_transposed_conv
 import _spherical_distortion_ext._resample as _resample
+import _spherical_distortion_ext._weighted_mapped_avg_pooling as _weighted_mapped_avg_pool
 import _spherical_distortion_ext._weighted_mapped_convolution as _weighted_mapped_conv
 import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mapped_max_pool
 import _spherical_distortion_ext._weighted_mapped_transposed_convolution as _weighted_mapped_transposed_conv
@@ -112,6 +114,61 @@ class MappedMaxPoolFunction(torch.autograd.Function):
         return grad_input, None, None, None, None
 
 
+def _avg_pool(input, sample_map, interp_weights, kernel_size, interp):
+    if interp_weights is None:
+        return _mapped_avg_pool.mapped_avg_pool(input, sample_map, kernel_size, interp)
+    return _weighted_mapped_avg_pool.weighted_mapped_avg_pool(input, sample_map, interp_weights,
+                                                              kernel_size, interp)
+
+
+def _avg_unpool(input, sample_map, interp_weights, height, width, kernel_size, interp):
+    if interp_weights is None:
+        return _mapped_avg_pool.mapped_avg_unpool(input, sample_map, height, width, kernel_size,
+                                                  interp)
+    return _weighted_mapped_avg_pool.weighted_mapped_avg_unpool(
+        input, sample_map, interp_weights, height, width, kernel_size, interp)
+
+
+class MappedAvgPoolFunction(torch.autograd.Function):
+    """Forward mean of the K samples, backward its adjoint
+    (layers/functional/mapped_pooling.py:10-57)."""
+
+    @staticmethod
+    def forward(ctx, input, sample_map, kernel_size, interp, interp_weights=None):
+        ctx.save_for_backward(sample_map, interp_weights)
+        ctx.in_hw = (int(input.shape[2]), int(input.shape[3]))
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = InterpolationType(interp)
+        return _avg_pool(input, sample_map, interp_weights, ctx.kernel_size, ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        sample_map, interp_weights = ctx.saved_tensors
+        grad = _avg_unpool(grad_output.contiguous(), sample_map, interp_weights, ctx.in_hw[0],
+                           ctx.in_hw[1], ctx.kernel_size, ctx.interp)
+        return grad, None, None, None, None
+
+
+class MappedAvgUnpoolFunction(torch.autograd.Function):
+    """Forward the adjoint of average pooling onto an oh x ow image, backward the pooling
+    (layers/functional/mapped_pooling.py:60-103)."""
+
+    @staticmethod
+    def forward(ctx, input, oh, ow, sample_map, kernel_size, interp, interp_weights=None):
+        ctx.save_for_backward(sample_map, interp_weights)
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = InterpolationType(interp)
+        return _avg_unpool(input, sample_map, interp_weights, int(oh), int(ow), ctx.kernel_size,
+                           ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        sample_map, interp_weights = ctx.saved_tensors
+        grad = _avg_pool(grad_output.contiguous(), sample_map, interp_weights, ctx.kernel_size,
+                         ctx.interp)
+        return grad, None, None, None, None, None, None
+
+
 class ResampleFunction(torch.autograd.Function):
     """Forward scatter, backward gather (layers/functional/resample.py:11-48)."""
 
@@ -186,6 +243,20 @@ def mapped_max_pool(input, sample_map, kernel_size, interp, interp_weights=None)
     """-> (pooled, idx_mask); layers/functional/mapped_pooling.py:225-232."""
     check_args(input, sample_map, interp_weights, None, kernel_size)
     return MappedMaxPoolFunction.apply(input, sample_map, kernel_size, interp, interp_weights)
+
+
+def mapped_avg_pool(input, sample_map, kernel_size, interp, interp_weights=None):
+    """layers/functional/mapped_pooling.py:202-209."""
+    check_args(input, sample_map, interp_weights, None, kernel_size)
+    return MappedAvgPoolFunction.apply(input, sample_map, kernel_size, interp, interp_weights)
+
+
+def mapped_avg_unpool(input, oh, ow, sample_map, kernel_size, interp, interp_weights=None):
+    """layers/functional/mapped_pooling.py:212-222."""
+    check_args(input, sample_map, interp_weights, None, kernel_size)
+    check_input_map_shape(input, sample_map)
+    return MappedAvgUnpoolFunction.apply(input, oh, ow, sample_map, kernel_size, interp,
+                                         interp_weights)
 
 
 def _with_batch_dim(input):

@@ -1,3 +1,3 @@
 from .modules import (MappedConvolution, MappedTransposedConvolution, MappedMaxPool,  # noqa: F401
-                      Resample, Unresample)
+                      MappedAvgPool, MappedAvgUnpool, Resample, Unresample)
 from ..layer_utils import InterpolationType  # noqa: F401

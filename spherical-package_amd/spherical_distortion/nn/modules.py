@@ -92,6 +92,32 @@ class MappedMaxPool(nn.Module):
         return (pooled, idx_mask) if self.return_indices else pooled
 
 
+class MappedAvgPool(nn.Module):
+    """(mapped_avg_pooling_layer.py:7-19)."""
+
+    def __init__(self, kernel_size, interpolation=InterpolationType.BILINEAR):
+        super().__init__()
+        self.kernel_size = kernel_size
+        self.interp = interpolation
+
+    def forward(self, x, sample_map, interp_weights=None):
+        return F.mapped_avg_pool(x, sample_map, self.kernel_size, self.interp, interp_weights)
+
+
+class MappedAvgUnpool(nn.Module):
+    """x on the map's grid is spread, divided by the kernel size, over the samples of each of
+    its pixels in an oh x ow image (mapped_avg_pooling_layer.py:22-44)."""
+
+    def __init__(self, kernel_size, interpolation=InterpolationType.BILINEAR):
+        super().__init__()
+        self.kernel_size = kernel_size
+        self.interp = interpolation
+
+    def forward(self, x, oh, ow, sample_map, interp_weights=None):
+        return F.mapped_avg_unpool(x, oh, ow, sample_map, self.kernel_size, self.interp,
+                                   interp_weights)
+
+
 class Resample(nn.Module):
     """Scatter: integer input locations go to the real-valued output locations
     the map gives (resample_layer.py:13-32)."""

@@ -152,6 +152,31 @@ def test_max_pool_and_unpool(ops, oracle, case):
     assert relerr(got, want) <= BWD_TOL[dt]
 
 
+@pytest.mark.parametrize("case", CASES, ids=_ids)
+def test_avg_pool_and_unpool(ops, oracle, case):
+    interp, weighted, dt = case
+    rng = np.random.default_rng(350 + interp)
+    B, C, H, W, OH, OW, K, P = 2, 9, 21, 27, 10, 13, 5, 2
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if weighted else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if weighted else None
+    got = _n(ops.mapped_avg_pool(_t(x), _t(m), _t(iw), K, interp))
+    want = oracle.mapped_avg_pool(x, m, K, interp, iw)
+    assert np.array_equal(got, want) or relerr(got, want) <= FWD_TOL[dt]
+    g = rng.standard_normal((B, C, OH, OW)).astype(dt)
+    got = _n(ops.mapped_avg_unpool(_t(g), _t(m), _t(iw), H, W, K, interp))
+    want = oracle.mapped_avg_unpool(g, m, H, W, K, interp, iw)
+    assert relerr(got, want) <= BWD_TOL[dt]
+    # without workspace (float atomics) through the C ABI
+    from _spherical_distortion_ext import _capi
+    tg, tm, tw = _t(g), _t(m), _t(iw)
+    out = torch.empty((B, C, H, W), dtype=tg.dtype, device=DEV)
+    _capi.call("sdk_mapped_avg_unpool", ops._ptr(tg), ops._ptr(tm), ops._ptr(tw), ops._ptr(out),
+               None, 0, B, C, H, W, OH, OW, K, P if weighted else 0, interp,
+               0 if dt == np.float32 else 1, ops._stream(tg))
+    assert relerr(_n(out), want) <= BWD_TOL[dt]
+
+
 def test_pool_ties_nan_and_no_winner(ops, oracle):
     """First maximum wins; NaN never wins; a window below -FLT_MAX has index -1."""
     x = np.zeros((1, 1, 2, 4), np.float32)

@@ -144,6 +144,11 @@ def test_pooling_and_resampling(ops, oracle, seed):
     g = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
     want = oracle.mapped_max_unpool(g, widx, m, H, W, K, interp, iw)
     assert relerr(_n(ops.mapped_max_unpool(_t(g), idx, _t(m), _t(iw), H, W, K, interp)), want) <= BWD
+    # average pooling over the same map
+    got = _n(ops.mapped_avg_pool(_t(x), _t(m), _t(iw), K, interp))
+    assert relerr(got, oracle.mapped_avg_pool(x, m, K, interp, iw)) <= FWD
+    back = _n(ops.mapped_avg_unpool(_t(g), _t(m), _t(iw), H, W, K, interp))
+    assert relerr(back, oracle.mapped_avg_unpool(g, m, H, W, K, interp, iw)) <= BWD
     # resampling over a map without the sample axis
     mr = np.ascontiguousarray(m[:, :, 0])
     iwr = None if iw is None else np.ascontiguousarray(iw[:, :, 0])

@@ -70,6 +70,28 @@ def test_mapped_max_pool(known_answers, case):
     np.testing.assert_allclose(out, np.broadcast_to(np.array(c["expected"]), out.shape), rtol=1e-7)
 
 
+def test_mapped_avg_pool(known_answers):
+    """tests/test_mapped_pooling.py:110-132 of the reference, and the unpool module on the same
+    map (forward of the adjoint, gradcheck)."""
+    from spherical_distortion.nn import MappedAvgPool, MappedAvgUnpool
+    c = known_answers["mapped_avg_pool"][0]
+    bs, _, _, K, _ = _sizes(known_answers)
+    x = _t(ka_input(c["input"], bs, 1)).requires_grad_(True)
+    m = _t(ka_kernel_map(known_answers, c["map"]))
+    out = _run(MappedAvgPool(kernel_size=K).double().to(DEV), (x, m))
+    want = np.array(c["expected"], np.float64)
+    np.testing.assert_allclose(out, np.broadcast_to(want, out.shape), rtol=1e-12)
+    y = torch.rand(bs, 1, *m.shape[:2], dtype=torch.float64, device=DEV, requires_grad=True)
+    layer = MappedAvgUnpool(kernel_size=K).double().to(DEV)
+    h, w = x.shape[2:]
+    spread = layer(y, h, w, m)
+    assert spread.shape == (bs, 1, h, w)
+    assert gradcheck(lambda t: layer(t, h, w, m), (y,))
+    # adjoint of the pooling: <pool(x), y> = <x, unpool(y)>
+    pooled = MappedAvgPool(kernel_size=K).double().to(DEV)(x.detach(), m)
+    assert abs(float((pooled * y.detach()).sum()) - float((x.detach() * spread.detach()).sum())) < 1e-9
+
+
 @pytest.mark.parametrize("case", range(10))
 def test_unresample(known_answers, case):
     from spherical_distortion.nn import InterpolationType, Unresample

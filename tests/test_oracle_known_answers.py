@@ -59,6 +59,17 @@ def test_mapped_max_pool_values(oracle, known_answers, case, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_mapped_avg_pool_values(oracle, known_answers, dtype):
+    c = known_answers["mapped_avg_pool"][0]
+    bs, _, _, K, _ = _sizes(known_answers)
+    x = ka_input(c["input"], bs, 1, dtype)
+    m = ka_kernel_map(known_answers, c["map"], dtype)
+    out = oracle.mapped_avg_pool(x, m, K, BILINEAR)
+    want = np.array(c["expected"], np.float64)
+    np.testing.assert_allclose(out, np.broadcast_to(want, out.shape), rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("case", range(10))
 def test_unresample(oracle, known_answers, case, dtype):
     c = known_answers["unresample"][case]

@@ -242,3 +242,31 @@ def test_transposed_forward_is_conv_backward_input(oracle):
     gi, _, _ = oracle.mapped_conv_backward(x, m, np.zeros((b, cout, oh, ow)), wt, np.zeros(cin),
                                            k, 1)
     np.testing.assert_allclose(out, gi, atol=1e-12)
+
+
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_avg_pool_is_the_mean_of_im2col_rows_and_unpool_its_adjoint(oracle, interp, weighted):
+    """Average pooling is pinned through functions pinned above: its value is the mean over k of
+    the im2col rows (summed in ascending k, then divided), and the unpool is its exact adjoint,
+    i.e. col2im of grad / K repeated over the K samples."""
+    rng = np.random.default_rng(40 + interp)
+    b, c, h, w, oh, ow, k, p = 2, 3, 9, 11, 5, 7, 4, 2
+    x = rng.standard_normal((b, c, h, w))
+    m = np.stack([rng.uniform(-1.5, w + 0.5, (oh, ow, k, p) if weighted else (oh, ow, k)),
+                  rng.uniform(-1.5, h + 0.5, (oh, ow, k, p) if weighted else (oh, ow, k))], -1)
+    iw = rng.uniform(0.1, 1, (oh, ow, k, p)) if weighted else None
+    got = oracle.mapped_avg_pool(x, m, k, interp, iw)
+    col = np.stack([oracle.mapped_im2col(x[i], m, interp, iw) for i in range(b)])
+    col = col.reshape(b, c, k, oh, ow)
+    want = np.zeros((b, c, oh, ow))
+    for kk in range(k):
+        want = want + col[:, :, kk]
+    want = want / k
+    assert np.array_equal(got, want)
+    g = rng.standard_normal((b, c, oh, ow))
+    back = oracle.mapped_avg_unpool(g, m, h, w, k, interp, iw)
+    assert abs((got * g).sum() - (x * back).sum()) <= 1e-10 * np.abs(got * g).sum()
+    cols = np.repeat((g / k)[:, :, None], k, axis=2).reshape(b, c * k, oh * ow)
+    via = np.stack([oracle.mapped_col2im(cols[i], m, h, w, interp, iw) for i in range(b)])
+    assert relerr(back, via) <= 1e-13
