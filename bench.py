@@ -177,7 +177,19 @@ def bench_resample2(torch, ops, timer, steps, warmup):
                         steps, warmup)
     gather_bytes = _nbytes(x, m, patches)
     scatter_bytes = _nbytes(patches, m, x) + H * W * 4.0
-    return {"gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,
+    # the UV way back: every image pixel reads its face's patch at (u, v); and its adjoint
+    quad = torch.from_numpy(cfg["quad_idx"]).to(dev)
+    uv = torch.from_numpy(cfg["tex_uv"]).to(dev)
+    B, C = x.shape[:2]
+    NT, TP = m.shape[0], cfg["patch"]
+    tex = patches.view(B, C, NT, TP, TP)
+    ms_uf, _ = timer.run(lambda: ops.resample_from_uv_maps(tex, quad, uv, 1), steps, warmup)
+    ms_ub, _ = timer.run(lambda: ops.resample_to_uv_maps(x, quad, uv, NT, TP, TP, 1), steps,
+                         warmup)
+    uv_bytes = _nbytes(tex, quad, uv, x)
+    return {"uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf)),
+            "uv_scatter": dict(ms=ms_ub, **_roof("hbm", uv_bytes, ms_ub)),
+            "gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,
                                             traffic=_measured_traffic("resample_from_map"))),
             "scatter_normalise": dict(ms=ms_s, **_roof("hbm", scatter_bytes, ms_s,
                                                        traffic=_measured_traffic("resample_to_map")))}

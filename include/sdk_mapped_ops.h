@@ -128,6 +128,41 @@ int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, 
                                 int64_t plane_size, int32_t dtype, sdk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * UV resampling (tangent images back to one image).
+ * textures [B,C,NT,TH,TW]; quad_idx [H,W] int64 names, per image pixel, one of the NT textures;
+ * tex_uv [H,W,2] = (u, v) in that texture's pixel coordinates (x first).  Interpolation taps stay
+ * inside the named texture (bispherical wraps u within TW).  A quad_idx outside [0, NT)
+ * contributes nothing (the reference reads out of bounds there).
+ * ------------------------------------------------------------------------- */
+
+/* Gather: out[b,c,y,x] = interp(textures[b,c,quad_idx[y,x]], tex_uv[y,x]).  out [B,C,H,W].
+ * Replaces `_uv_resample.resample_from_uv_maps`
+ * (ext_modules/include/layers/uv_resample_layer.h:76-99; body
+ *  ext_modules/include/common/resample.h:132-158; host loop src/cpp/uv_resample_layer.cpp:41-72). */
+int sdk_resample_from_uv_maps(const void* textures, const int64_t* quad_idx, const void* tex_uv,
+                              void* out, int64_t batch, int64_t channels, int64_t num_textures,
+                              int64_t tex_height, int64_t tex_width, int64_t height,
+                              int64_t width, int32_t interp, int32_t dtype, sdk_stream_t stream);
+
+/* Its adjoint: textures (zero-filled) accumulate input[b,c,y,x] at (quad_idx, tex_uv)[y,x].
+ * input [B,C,H,W]; textures [B,C,NT,TH,TW].  Replaces `_uv_resample.resample_to_uv_maps`
+ * (uv_resample_layer.h:48-74; body common/resample.h:160-187; src/cpp/uv_resample_layer.cpp:7-39).
+ * workspace (optional, may be NULL): sdk_resample_to_uv_maps_workspace_bytes() bytes of device
+ * scratch (4 bytes per image pixel + 12 per texture).  With it the image pixels are bucketed by
+ * texture on the device and every texture is summed in on-chip memory and written once, without
+ * atomics in memory and without a zero fill; the query returns 0 (and the call then needs no
+ * workspace) when a texture does not fit there (TH*TW*sizeof > 64 KiB).  Without it: zero fill
+ * and atomic adds. */
+size_t sdk_resample_to_uv_maps_workspace_bytes(int64_t num_textures, int64_t tex_height,
+                                               int64_t tex_width, int64_t height, int64_t width,
+                                               int32_t dtype);
+int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const void* tex_uv,
+                            void* textures, void* workspace, size_t workspace_bytes,
+                            int64_t batch, int64_t channels, int64_t num_textures,
+                            int64_t tex_height, int64_t tex_width, int64_t height, int64_t width,
+                            int32_t interp, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Mapped im2col / col2im (batched).
  * col[b, c*K + k, pix] with pix = y_out*OW + x_out, out_pixels = OH*OW.
  * sample_map [OH,OW,K,(P,)2].

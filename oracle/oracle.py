@@ -178,6 +178,28 @@ def mapped_avg_unpool(grad_output, sample_map, in_h, in_w, kernel_size, interp,
     return out
 
 
+def resample_from_uv_maps(textures, quad_idx, tex_uv, interp):
+    """textures [B,C,NT,TH,TW], quad_idx [H,W] int64, tex_uv [H,W,2] -> [B,C,H,W]."""
+    t = _c(textures); q = _c(quad_idx, np.int64); uv = _c(tex_uv, t.dtype)
+    B, C, NT, TH, TW = t.shape
+    H, W = q.shape
+    out = np.empty((B, C, H, W), t.dtype)
+    _check(lib().sdk_oracle_resample_from_uv_maps(
+        _p(t), _p(q), _p(uv), _p(out), *_i64(B, C, NT, TH, TW, H, W), *_i32(int(interp), _dt(t))))
+    return out
+
+
+def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp):
+    """x [B,C,H,W] -> [B,C,NT,TH,TW]: the adjoint of resample_from_uv_maps."""
+    x = _c(x); q = _c(quad_idx, np.int64); uv = _c(tex_uv, x.dtype)
+    B, C, H, W = x.shape
+    out = np.empty((B, C, num_textures, tex_h, tex_w), x.dtype)
+    _check(lib().sdk_oracle_resample_to_uv_maps(
+        _p(x), _p(q), _p(uv), _p(out), *_i64(B, C, num_textures, tex_h, tex_w, H, W),
+        *_i32(int(interp), _dt(x))))
+    return out
+
+
 def mapped_conv_forward(x, sample_map, weight, bias, kernel_size, interp,
                         interp_weights=None):
     x = _c(x); m = _c(sample_map, x.dtype); w = _c(interp_weights, x.dtype)

@@ -24,7 +24,10 @@
 //   max pool values: reference known-answer vectors; argmax index encoding and
 //       the CPU initial-value quirk: compiled-reference fixtures.
 //   average pool / unpool: reference known-answer vector (tests/test_mapped_pooling.py:110-132)
-//       + "mean over k of the pinned im2col rows" + adjoint identity.
+//       + "mean over k of the pinned im2col rows" + adjoint identity + compiled-reference
+//       fixtures (weighted, nearest, bispherical).
+//   UV resampling: compiled-reference fixtures + "per texture it is the pinned gather" +
+//       adjoint identity (the reference's test-suite holds no vector for it).
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -189,6 +192,41 @@ void resample_to_map(const T* in, const T* map, const T* wts, T* out, int64_t B,
       scatter_sample(in_b[i], out_b + c * H * W, map + pix * q * 2,
                      wts ? wts + pix * q : nullptr, P, H, W, interp);
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// UV resampling.  Per image pixel: texture quad[y,x] of plane c (plane = NT textures of
+// TH x TW), point uv[y,x] interpolated inside that texture alone.
+// common/resample.h:132-158 (gather), :160-187 (adjoint); loops cpp/resample.h:124-166;
+// batch loops and zero fill src/cpp/uv_resample_layer.cpp:7-72.
+// A texture index outside [0, NT) is skipped (the reference would index out of bounds).
+// ---------------------------------------------------------------------------
+template <typename T>
+void resample_from_uv(const T* tex, const int64_t* quad, const T* uv, T* out, int64_t B,
+                      int64_t C, int64_t NT, int64_t TH, int64_t TW, int64_t H, int64_t W,
+                      int interp) {
+  const int64_t hw = H * W, thw = TH * TW;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < B * C * hw; ++i) {
+    const int64_t pix = i % hw, plane = i / hw, t = quad[pix];
+    out[i] = (t < 0 || t >= NT) ? T(0)
+                                : gather_point(tex + (plane * NT + t) * thw, uv[pix * 2],
+                                               uv[pix * 2 + 1], TH, TW, interp);
+  }
+}
+
+template <typename T>
+void resample_to_uv(const T* in, const int64_t* quad, const T* uv, T* tex, int64_t B, int64_t C,
+                    int64_t NT, int64_t TH, int64_t TW, int64_t H, int64_t W, int interp) {
+  const int64_t hw = H * W, thw = TH * TW;
+  std::memset(tex, 0, sizeof(T) * B * C * NT * thw);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < B * C * hw; ++i) {
+    const int64_t pix = i % hw, plane = i / hw, t = quad[pix];
+    if (t < 0 || t >= NT) continue;
+    scatter_point(in[i], tex + (plane * NT + t) * thw, uv[pix * 2], uv[pix * 2 + 1], TH, TW,
+                  interp);
   }
 }
 
@@ -548,6 +586,20 @@ int sdk_oracle_mapped_avg_unpool(const void* gout, const void* map, const void* 
                                  int64_t OW, int64_t K, int P, int interp, int dtype) {
   DISPATCH(dtype, avg_unpool<T>((const T*)gout, (const T*)map, (const T*)wts, (T*)gin, B, C, H, W,
                                  OH, OW, K, P, interp));
+}
+
+int sdk_oracle_resample_from_uv_maps(const void* tex, const int64_t* quad, const void* uv,
+                                     void* out, int64_t B, int64_t C, int64_t NT, int64_t TH,
+                                     int64_t TW, int64_t H, int64_t W, int interp, int dtype) {
+  DISPATCH(dtype, resample_from_uv<T>((const T*)tex, quad, (const T*)uv, (T*)out, B, C, NT, TH,
+                                       TW, H, W, interp));
+}
+
+int sdk_oracle_resample_to_uv_maps(const void* in, const int64_t* quad, const void* uv, void* tex,
+                                   int64_t B, int64_t C, int64_t NT, int64_t TH, int64_t TW,
+                                   int64_t H, int64_t W, int interp, int dtype) {
+  DISPATCH(dtype, resample_to_uv<T>((const T*)in, quad, (const T*)uv, (T*)tex, B, C, NT, TH, TW,
+                                     H, W, interp));
 }
 
 int sdk_oracle_mapped_conv_forward(const void* x, const void* map, const void* wts,

@@ -9,7 +9,8 @@ kernels in libsdk_mapped_ops.so:
     _enums, _resample, _weighted_resample, _mapped_convolution,
     _weighted_mapped_convolution, _mapped_transposed_convolution,
     _weighted_mapped_transposed_convolution, _mapped_max_pooling,
-    _weighted_mapped_max_pooling, _mapped_avg_pooling, _weighted_mapped_avg_pooling
+    _weighted_mapped_max_pooling, _mapped_avg_pooling, _weighted_mapped_avg_pooling,
+    _uv_resample
 
 Importing the package loads the library and registers the operators; it raises
 ImportError when the library has not been built.

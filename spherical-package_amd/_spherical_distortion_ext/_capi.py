@@ -22,6 +22,8 @@ SIGNATURES = {
     "sdk_resample_to_map_normalized": [_vp] * 6 + [_sz, ctypes.c_double] + [_i64] * 6 + [_i32] * 3
                                       + [_vp],
     "sdk_normalize_by_weight_sum": [_vp, _vp, ctypes.c_double, _i64, _i64, _i32, _vp],
+    "sdk_resample_from_uv_maps": [_vp] * 4 + [_i64] * 7 + [_i32] * 2 + [_vp],
+    "sdk_resample_to_uv_maps": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 2 + [_vp],
     "sdk_mapped_im2col": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_pool": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],
@@ -39,7 +41,8 @@ SIGNATURES = {
     "sdk_mapped_transposed_conv_backward_weight": [_vp] * 6 + [_sz] + _CONV_DIMS,
 }
 OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes",
-                 "sdk_resample_to_map_workspace_bytes", "sdk_mapped_max_unpool_workspace_bytes")
+                 "sdk_resample_to_map_workspace_bytes", "sdk_mapped_max_unpool_workspace_bytes",
+                 "sdk_resample_to_uv_maps_workspace_bytes")
 
 _lib = None
 
@@ -68,6 +71,8 @@ def load():
     lib.sdk_resample_to_map_workspace_bytes.restype = _sz
     lib.sdk_mapped_max_unpool_workspace_bytes.argtypes = [_i64, _i64, _i32]
     lib.sdk_mapped_max_unpool_workspace_bytes.restype = _sz
+    lib.sdk_resample_to_uv_maps_workspace_bytes.argtypes = [_i64] * 5 + [_i32]
+    lib.sdk_resample_to_uv_maps_workspace_bytes.restype = _sz
     _lib = lib
     return lib
 

@@ -51,7 +51,7 @@ def _check(ref, **tensors):
             raise RuntimeError("%s must be contiguous" % name)
         if not t.is_cuda or t.device != ref.device:
             raise RuntimeError("%s must be a CUDA tensor on %s" % (name, ref.device))
-        if t.dtype != ref.dtype and name != "idx_mask":
+        if t.dtype != ref.dtype and name not in ("idx_mask", "quad_idx"):
             raise RuntimeError("%s must have dtype %s (got %s)" % (name, ref.dtype, t.dtype))
 
 
@@ -359,6 +359,49 @@ def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, 
     return gi, gw, gb
 
 
+# --------------------------------------------------------------------------- UV resample
+def _uv_dims(quad_idx, tex_uv):
+    if quad_idx.dtype != torch.int64 or quad_idx.dim() != 2:
+        raise RuntimeError("quad_idx must be a 2-D int64 tensor, got %s %s"
+                           % (quad_idx.dtype, tuple(quad_idx.shape)))
+    if tuple(tex_uv.shape) != tuple(quad_idx.shape) + (2,):
+        raise RuntimeError("tex_uv %s must be quad_idx %s + (2,)"
+                           % (tuple(tex_uv.shape), tuple(quad_idx.shape)))
+    return int(quad_idx.shape[0]), int(quad_idx.shape[1])
+
+
+def resample_from_uv_maps(textures, quad_idx, tex_uv, interp):
+    _check(textures, textures=textures, quad_idx=quad_idx, tex_uv=tex_uv)
+    if textures.dim() != 5:
+        raise RuntimeError("textures must be [B, C, T, TH, TW], got %s" % (tuple(textures.shape),))
+    H, W = _uv_dims(quad_idx, tex_uv)
+    B, C, NT, TH, TW = textures.shape
+    out = torch.empty((B, C, H, W), dtype=textures.dtype, device=textures.device)
+    with torch.cuda.device(textures.device):
+        _capi.call("sdk_resample_from_uv_maps", _ptr(textures), _ptr(quad_idx), _ptr(tex_uv),
+                   _ptr(out), B, C, NT, TH, TW, H, W, int(interp), _DTYPES[textures.dtype],
+                   _stream(textures))
+    return out
+
+
+def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp):
+    _check(x, x=x, quad_idx=quad_idx, tex_uv=tex_uv)
+    H, W = _uv_dims(quad_idx, tex_uv)
+    if x.dim() != 4 or tuple(x.shape[2:]) != (H, W):
+        raise RuntimeError("input %s must be [B, C, %d, %d]" % (tuple(x.shape), H, W))
+    B, C = x.shape[:2]
+    NT, TH, TW = int(num_textures), int(tex_h), int(tex_w)
+    out = torch.empty((B, C, NT, TH, TW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        nws = _capi.load().sdk_resample_to_uv_maps_workspace_bytes(NT, TH, TW, H, W,
+                                                                   _DTYPES[x.dtype])
+        ws = torch.empty(nws, dtype=torch.uint8, device=x.device) if nws else None
+        _capi.call("sdk_resample_to_uv_maps", _ptr(x), _ptr(quad_idx), _ptr(tex_uv), _ptr(out),
+                   _ptr(ws), nws, B, C, NT, TH, TW, H, W, int(interp), _DTYPES[x.dtype],
+                   _stream(x))
+    return out
+
+
 # --------------------------------------------------------------------------- registration
 _SCHEMAS = (
     ("resample_from_map",
@@ -370,6 +413,12 @@ _SCHEMAS = (
     ("resample_to_map_normalized",
      "(Tensor x, Tensor sample_map, Tensor? interp_weights, int out_h, int out_w, int interp,"
      " float eps) -> (Tensor, Tensor)", resample_to_map_normalized),
+    ("resample_from_uv_maps",
+     "(Tensor textures, Tensor quad_idx, Tensor tex_uv, int interp) -> Tensor",
+     resample_from_uv_maps),
+    ("resample_to_uv_maps",
+     "(Tensor x, Tensor quad_idx, Tensor tex_uv, int num_textures, int tex_h, int tex_w,"
+     " int interp) -> Tensor", resample_to_uv_maps),
     ("mapped_im2col",
      "(Tensor x, Tensor sample_map, Tensor? interp_weights, int interp) -> Tensor",
      mapped_im2col),

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cfloat>
+#include <climits>
 
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
@@ -240,6 +241,215 @@ __global__ __launch_bounds__(kBlock) void normalize_kernel(T* __restrict__ data,
   const size_t stride = (size_t)gridDim.x * kBlock;
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride)
     data[i] = data[i] / (wsum[i % plane_size] + eps);
+}
+
+// ---------------------------------------------------------------------------
+// UV resampling: every pixel of the image names one of NT textures (quad) and a point (u, v) in
+// that texture's TH x TW plane; taps never leave the named texture.  Bodies:
+// common/resample.h:132-158 (gather), :160-187 (its adjoint).  A texture index outside
+// [0, NT) contributes nothing (the reference reads out of bounds there).
+// ---------------------------------------------------------------------------
+template <typename T, int INTERP, int PC>
+__global__ __launch_bounds__(kBlock) void uv_gather_kernel(
+    const T* __restrict__ textures, const int64_t* __restrict__ quad, const T* __restrict__ uv,
+    T* __restrict__ out, int planes, int NT, int TH, int TW, int MP) {
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
+  if (pix >= MP) return;
+  const int plane0 = blockIdx.y * PC;
+  const int np = min(PC, planes - plane0);
+  const size_t THW = (size_t)TH * TW, stride = THW * NT;
+  const long long q = quad[pix];
+  T acc[PC];
+  if (q >= 0 && q < NT) {
+    gather_sample<T, INTERP, false, PC>(textures + (size_t)plane0 * stride + (size_t)q * THW,
+                                        stride, np, uv + (size_t)pix * 2, nullptr, 0, TH, TW, acc);
+  } else {
+#pragma unroll
+    for (int j = 0; j < PC; ++j) acc[j] = T(0);
+  }
+#pragma unroll
+  for (int j = 0; j < PC; ++j)
+    if (j < np) out[(size_t)(plane0 + j) * MP + pix] = acc[j];
+}
+
+template <typename T, int INTERP>
+__global__ __launch_bounds__(kBlock) void uv_scatter_kernel(
+    const T* __restrict__ in, const int64_t* __restrict__ quad, const T* __restrict__ uv,
+    T* __restrict__ textures, int planes, int NT, int TH, int TW, int MP,
+    const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
+  if (pix >= MP) return;
+  const long long q = quad[pix];
+  if (q < 0 || q >= NT) return;
+  const int plane0 = blockIdx.y * kPC;
+  const int np = min(kPC, planes - plane0);
+  const size_t THW = (size_t)TH * TW, stride = THW * NT;
+  T val[kPC];
+#pragma unroll
+  for (int j = 0; j < kPC; ++j) val[j] = j < np ? in[(size_t)(plane0 + j) * MP + pix] : T(0);
+  scatter_sample<T, INTERP, false, kPC>(textures + (size_t)plane0 * stride + (size_t)q * THW,
+                                        stride, np, uv + (size_t)pix * 2, nullptr, 0, TH, TW, val);
+}
+
+// ---------------------------------------------------------------------------
+// The adjoint by texture.  A texture is small (TH x TW texels fit in LDS) and receives many
+// image pixels per texel, often hundreds near the poles of an equirectangular image, so neither
+// atomics in memory nor a bounded inverse list suit it.  Instead the image pixels are bucketed
+// by texture (count, scan, fill: a counting sort of pixel indices, keyed by quad), and one
+// workgroup per (texture, plane chunk) sums its bucket into an LDS copy of the texture and
+// writes that out with plain stores, zeros included, so no fill of the output is needed.
+//
+// Lanes own consecutive bucket entries, which are consecutive image pixels of one row wherever
+// the map is coherent; these hit the same texel in runs.  Each run is summed across lanes first
+// (segmented scan over shuffles) and only its last lane adds to LDS, which keeps the
+// compare-and-swap adds nearly free of collisions.
+// ---------------------------------------------------------------------------
+constexpr int kUvMaxTextures = 1 << 20;
+constexpr int kUvLdsBytes = 64 * 1024;
+
+// Runs of equal keys over the lanes of a wave: distance of each lane to the first lane of its
+// run and whether it is the last one.  `same` = this lane continues the run of the lane below.
+struct LaneRuns {
+  int dist;
+  bool tail;
+  __device__ __forceinline__ LaneRuns(bool same) {
+    const int lane = threadIdx.x & 63;
+    const unsigned long long heads = __ballot(lane == 0 || !same);
+    const unsigned long long upto = heads & (~0ull >> (63 - lane));
+    dist = lane - (63 - __clzll((long long)upto));
+    tail = lane == 63 || (((heads >> 1) >> lane) & 1ull);
+  }
+  // inclusive sum of v over the lanes of the run up to this one
+  template <typename T>
+  __device__ __forceinline__ T sum(T v) const {
+    for (int d = 1; d < 64; d <<= 1) {
+      if (!__any(dist >= d)) break;
+      const T below = __shfl_up(v, d);
+      if (dist >= d) v += below;
+    }
+    return v;
+  }
+};
+
+__global__ __launch_bounds__(kBlock) void uv_count_kernel(const int64_t* __restrict__ quad,
+                                                          int NT, int MP,
+                                                          int* __restrict__ count) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const long long q = pix < MP ? quad[pix] : -1;
+  const bool ok = q >= 0 && q < NT;
+  const int t = ok ? (int)q : -1;
+  const int below = __shfl_up(t, 1);
+  const LaneRuns runs(below == t);
+  if (ok && runs.tail) atomicAdd(&count[t], runs.dist + 1);
+}
+
+// offset[t] = cursor[t] = number of pixels in textures below t; offset[NT] = all of them.
+__global__ __launch_bounds__(kBlock) void uv_scan_kernel(const int* __restrict__ count, int NT,
+                                                         int* __restrict__ offset,
+                                                         int* __restrict__ cursor) {
+  __shared__ int part[kBlock];
+  int carry = 0;
+  for (int base = 0; base < NT; base += kBlock) {
+    const int i = base + threadIdx.x;
+    const int c = i < NT ? count[i] : 0;
+    part[threadIdx.x] = c;
+    __syncthreads();
+    for (int d = 1; d < kBlock; d <<= 1) {
+      const int add = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+      __syncthreads();
+      part[threadIdx.x] += add;
+      __syncthreads();
+    }
+    const int incl = part[threadIdx.x];
+    if (i < NT) {
+      offset[i] = carry + incl - c;
+      cursor[i] = carry + incl - c;
+    }
+    carry += part[kBlock - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) offset[NT] = carry;
+}
+
+__global__ __launch_bounds__(kBlock) void uv_fill_kernel(const int64_t* __restrict__ quad, int NT,
+                                                         int MP, int* __restrict__ cursor,
+                                                         int* __restrict__ list) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;
+  const long long q = pix < MP ? quad[pix] : -1;
+  const bool ok = q >= 0 && q < NT;
+  const int t = ok ? (int)q : -1;
+  const int below = __shfl_up(t, 1);
+  const LaneRuns runs(below == t);
+  // the last lane of a run reserves the run's slots; the others read the start from it
+  int start = 0;
+  if (ok && runs.tail) start = atomicAdd(&cursor[t], runs.dist + 1);
+  const int lane = threadIdx.x & 63;
+  // lane of this run's tail: the next run's head minus one
+  const unsigned long long tails = __ballot(runs.tail);
+  const int tail_lane = __ffsll((long long)(tails & (~0ull << lane))) - 1;
+  start = __shfl(start, tail_lane);
+  if (ok) list[start + runs.dist] = pix;
+}
+
+template <typename T, int INTERP, int PL>
+__global__ __launch_bounds__(kBlock) void uv_texture_scatter_kernel(
+    const T* __restrict__ in, const T* __restrict__ uv, const int* __restrict__ offset,
+    const int* __restrict__ list, T* __restrict__ textures, int planes, int NT, int TH, int TW,
+    int MP) {
+  extern __shared__ __align__(16) unsigned char uv_lds[];
+  T* acc = reinterpret_cast<T*>(uv_lds);             // [PL][TH * TW]
+  const int THW = TH * TW;
+  const int t = blockIdx.x;
+  const int plane0 = blockIdx.y * PL;
+  const int np = min(PL, planes - plane0);
+  // segment of the texture's bucket this workgroup sums (gridDim.z > 1: several workgroups
+  // share a texture and add their sums to the zero-filled output)
+  const int lo0 = offset[t], hi0 = offset[t + 1];
+  const int per = (hi0 - lo0 + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int lo = lo0 + (int)blockIdx.z * per, hi = min(hi0, lo + per);
+  for (int i = threadIdx.x; i < PL * THW; i += kBlock) acc[i] = T(0);
+  __syncthreads();
+  constexpr int N = PointTaps<T, INTERP>::N;
+  for (int base = lo; base < hi; base += kBlock) {   // uniform trip count over the workgroup
+    const int e = base + threadIdx.x;
+    const bool live = e < hi;
+    const int pix = live ? list[e] : 0;
+    PointTaps<T, INTERP> taps;
+    taps.set(live ? uv[(size_t)pix * 2] : T(0), live ? uv[(size_t)pix * 2 + 1] : T(0), TH, TW);
+    T val[PL];
+#pragma unroll
+    for (int j = 0; j < PL; ++j)
+      val[j] = (live && j < np) ? in[(size_t)(plane0 + j) * MP + pix] : T(0);
+    // lanes whose first tap is the same texel form a run: all their taps coincide
+    const int ky = live ? taps.ty[0] : INT_MIN, kx = live ? taps.tx[0] : (int)threadIdx.x;
+    const int by = __shfl_up(ky, 1), bx = __shfl_up(kx, 1);
+    const LaneRuns runs(by == ky && bx == kx);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const T w = taps.off[i] >= 0 ? (INTERP == 0 ? T(1) : taps.w[i]) : T(0);
+      const bool inside = (unsigned)taps.ty[i] < (unsigned)TH && (unsigned)taps.tx[i] < (unsigned)TW;
+      const int o = inside ? taps.ty[i] * TW + taps.tx[i] : 0;
+#pragma unroll
+      for (int j = 0; j < PL; ++j) {
+        const T total = runs.sum(w * val[j]);
+        if (live && runs.tail && inside && total != T(0)) lds_add(acc + j * THW + o, total);
+      }
+    }
+  }
+  __syncthreads();
+  const size_t stride = (size_t)NT * THW;
+  for (int i = threadIdx.x; i < THW; i += kBlock) {
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      if (j < np) {
+        T* dst = textures + (size_t)(plane0 + j) * stride + (size_t)t * THW + i;
+        const T v = acc[j * THW + i];
+        if (gridDim.z == 1) *dst = v;
+        else if (v != T(0)) atomicAdd(dst, v);
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -727,6 +937,105 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
   return SDK_OK;
 }
 
+// INTERP alone (UV maps carry no interpolation weights); same mapping of the enum as
+// SDK_DISPATCH_INTERP.
+#define SDK_DISPATCH_INTERP_ONLY(interp, CALL)                  \
+  do {                                                          \
+    if ((interp) == 1) { constexpr int INTERP = 1; CALL; }      \
+    else if ((interp) == 2) { constexpr int INTERP = 2; CALL; } \
+    else { constexpr int INTERP = 0; CALL; }                    \
+  } while (0)
+
+template <typename T>
+static int launch_uv_gather(const T* textures, const int64_t* quad, const T* uv, T* out,
+                            int64_t planes, int NT, int TH, int TW, int MP, int interp,
+                            hipStream_t stream) {
+  const int pc = planes_per_thread(planes);
+#define UVG(PCv)                                                                              \
+  SDK_DISPATCH_INTERP_ONLY(interp,                                                            \
+                           (launch((uv_gather_kernel<T, INTERP, PCv>),                        \
+                                   dim3(banded_grid_x(MP), (unsigned)ceil_div(planes, PCv)),  \
+                                   dim3(kBlock), stream, textures, quad, uv, out, (int)planes, \
+                                   NT, TH, TW, MP)))
+  if (pc >= 8) UVG(8); else if (pc >= 4) UVG(4); else UVG(2);
+#undef UVG
+  SDK_LAUNCH_CHECK("resample_from_uv_maps");
+  return SDK_OK;
+}
+
+// Workspace of the adjoint by texture: count | offset (NT + 1) | cursor | bucket (MP pixels).
+static size_t uv_layout(int64_t NT, int64_t MP, size_t (&off)[4]) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  off[0] = 0;                                  // count
+  off[1] = off[0] + up((size_t)NT * 4);        // offset
+  off[2] = off[1] + up((size_t)(NT + 1) * 4);  // cursor
+  off[3] = off[2] + up((size_t)NT * 4);        // bucket
+  return off[3] + up((size_t)MP * 4);
+}
+
+static bool uv_by_texture_fits(int64_t NT, int64_t THW, size_t esz) {
+  return NT <= kUvMaxTextures && THW * (int64_t)esz <= kUvLdsBytes;
+}
+
+// The adjoint: with a workspace (and textures that fit in LDS) by texture, see
+// uv_texture_scatter_kernel; otherwise a zero fill and atomic adds in memory.
+template <typename T>
+static int launch_uv_scatter(const T* in, const int64_t* quad, const T* uv, T* textures,
+                             void* workspace, size_t workspace_bytes, int64_t planes, int NT,
+                             int TH, int TW, int MP, int interp, hipStream_t stream) {
+  const int THW = TH * TW;
+  size_t off[4];
+  if (workspace != nullptr && uv_by_texture_fits(NT, THW, sizeof(T)) &&
+      workspace_bytes >= uv_layout(NT, MP, off)) {
+    char* ws = static_cast<char*>(workspace);
+    int* count = reinterpret_cast<int*>(ws + off[0]);
+    int* offset = reinterpret_cast<int*>(ws + off[1]);
+    int* cursor = reinterpret_cast<int*>(ws + off[2]);
+    int* list = reinterpret_cast<int*>(ws + off[3]);
+    int rc = zero_fill(count, off[1], stream);
+    if (rc != SDK_OK) return rc;
+    const dim3 pixel_grid((unsigned)ceil_div(MP, kBlock));
+    launch(uv_count_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, count);
+    launch(uv_scan_kernel, dim3(1), dim3(kBlock), stream, (const int*)count, NT, offset, cursor);
+    launch(uv_fill_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, cursor, list);
+    SDK_LAUNCH_CHECK("resample_to_uv_maps(bucket)");
+    // planes per workgroup: as many as LDS holds while the grid still fills the GPU; few
+    // textures: several workgroups share one and add their parts to a zero-filled output
+    int pl = 1;
+    while (pl < 4 && (size_t)(2 * pl) * THW * sizeof(T) <= (size_t)kUvLdsBytes &&
+           (int64_t)NT * ceil_div(planes, 2 * pl) >= 1024)
+      pl *= 2;
+    const int64_t groups = (int64_t)NT * ceil_div(planes, pl);
+    const int split = (int)std::min<int64_t>(64, std::max<int64_t>(1, 512 / groups));
+    if (ceil_div(planes, pl) > 65535)
+      return fail(SDK_ERR_UNSUPPORTED, "resample_to_uv_maps: batch*channels = %lld too large",
+                  (long long)planes);
+    if (split > 1) {
+      rc = zero_fill(textures, sizeof(T) * (size_t)planes * NT * THW, stream);
+      if (rc != SDK_OK) return rc;
+    }
+    const dim3 grid((unsigned)NT, (unsigned)ceil_div(planes, pl), (unsigned)split);
+#define UVS(PLv)                                                                              \
+  SDK_DISPATCH_INTERP_ONLY(interp, (uv_texture_scatter_kernel<T, INTERP, PLv>                 \
+                                    <<<grid, dim3(kBlock), (size_t)PLv * THW * sizeof(T), stream>>>( \
+                                        in, uv, (const int*)offset, (const int*)list, textures, \
+                                        (int)planes, NT, TH, TW, MP)))
+    if (pl == 4) UVS(4); else if (pl == 2) UVS(2); else UVS(1);
+#undef UVS
+    SDK_LAUNCH_CHECK("resample_to_uv_maps(by texture)");
+    return SDK_OK;
+  }
+  int rc = zero_fill(textures, sizeof(T) * (size_t)planes * NT * THW, stream);
+  if (rc != SDK_OK) return rc;
+  SDK_DISPATCH_INTERP_ONLY(interp,
+                           (launch((uv_scatter_kernel<T, INTERP>),
+                                   dim3(banded_grid_x(MP), (unsigned)ceil_div(planes, kPC)),
+                                   dim3(kBlock), stream, in, quad, uv, textures, (int)planes, NT,
+                                   TH, TW, MP, (const int*)nullptr)));
+  SDK_LAUNCH_CHECK("resample_to_uv_maps");
+  return SDK_OK;
+}
+
 static UnpoolTiling unpool_tiling(int H, int W) {
   UnpoolTiling ut;
   ut.H = H;
@@ -924,6 +1233,69 @@ int sdk_resample_to_map_normalized(const void* input, const void* sample_map,
   return resample_to_map_entry(input, sample_map, interp_weights, out, weight_sum, workspace,
                                workspace_bytes, batch, channels, map_height, map_width, height,
                                width, num_interp_pts, interp, dtype, stream, true, eps);
+}
+
+static int check_uv(const void* a, const void* quad, const void* uv, const void* b,
+                    int64_t batch, int64_t channels, int64_t num_textures, int64_t tex_height,
+                    int64_t tex_width, int64_t height, int64_t width, const char* what) {
+  if (batch < 0 || channels < 0) return fail(SDK_ERR_INVALID_ARGUMENT, "%s: negative size", what);
+  // an empty batch has no tensors to point at
+  if (batch * channels > 0 && (!a || !quad || !uv || !b))
+    return fail(SDK_ERR_INVALID_ARGUMENT, "%s: NULL pointer", what);
+  if (num_textures < 1 || num_textures >= ((int64_t)1 << 31))
+    return fail(SDK_ERR_INVALID_ARGUMENT, "%s: num_textures = %lld", what, (long long)num_textures);
+  int rc = check_plane(tex_height, tex_width, what);
+  if (rc) return rc;
+  rc = check_plane(num_textures * tex_height, tex_width, what);   // all texels of one plane
+  if (rc) return rc;
+  rc = check_plane(height, width, what);
+  if (rc) return rc;
+  return check_grid_y(batch * channels, what);
+}
+
+int sdk_resample_from_uv_maps(const void* textures, const int64_t* quad_idx, const void* tex_uv,
+                              void* out, int64_t batch, int64_t channels, int64_t num_textures,
+                              int64_t tex_height, int64_t tex_width, int64_t height,
+                              int64_t width, int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  int rc = check_uv(textures, quad_idx, tex_uv, out, batch, channels, num_textures, tex_height,
+                    tex_width, height, width, "resample_from_uv_maps");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_uv_gather<T>(
+                                (const T*)textures, quad_idx, (const T*)tex_uv, (T*)out, planes,
+                                (int)num_textures, (int)tex_height, (int)tex_width,
+                                (int)(height * width), interp, (hipStream_t)stream));
+  return SDK_OK;
+}
+
+size_t sdk_resample_to_uv_maps_workspace_bytes(int64_t num_textures, int64_t tex_height,
+                                               int64_t tex_width, int64_t height, int64_t width,
+                                               int32_t dtype) {
+  if (num_textures < 1 || tex_height < 1 || tex_width < 1 || height < 1 || width < 1 ||
+      height * width >= ((int64_t)1 << 31))
+    return 0;
+  if (!uv_by_texture_fits(num_textures, tex_height * tex_width, dtype == SDK_F64 ? 8 : 4)) return 0;
+  size_t off[4];
+  return uv_layout(num_textures, height * width, off);
+}
+
+int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const void* tex_uv,
+                            void* textures, void* workspace, size_t workspace_bytes,
+                            int64_t batch, int64_t channels, int64_t num_textures,
+                            int64_t tex_height, int64_t tex_width, int64_t height, int64_t width,
+                            int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  int rc = check_uv(input, quad_idx, tex_uv, textures, batch, channels, num_textures, tex_height,
+                    tex_width, height, width, "resample_to_uv_maps");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_uv_scatter<T>(
+                                (const T*)input, quad_idx, (const T*)tex_uv, (T*)textures,
+                                workspace, workspace_bytes, planes, (int)num_textures,
+                                (int)tex_height, (int)tex_width, (int)(height * width), interp,
+                                (hipStream_t)stream));
+  return SDK_OK;
 }
 
 int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, int64_t planes,

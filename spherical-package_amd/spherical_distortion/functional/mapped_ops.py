@@ -11,6 +11,7 @@ import _spherical_distortion_ext._mapped_convolution as _mapped_conv
 import _spherical_distortion_ext._mapped_max_pooling as _mapped_max_pool
 import _spherical_distortion_ext._mapped_transposed_convolution as _mapped_transposed_conv
 import _spherical_distortion_ext._resample as _resample
+import _spherical_distortion_ext._uv_resample as _uv_resample
 import _spherical_distortion_ext._weighted_mapped_avg_pooling as _weighted_mapped_avg_pool
 import _spherical_distortion_ext._weighted_mapped_convolution as _weighted_mapped_conv
 import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mapped_max_pool
@@ -220,6 +221,26 @@ class UnresampleFunction(torch.autograd.Function):
         return grad, None, None, None
 
 
+class UVResampleFunction(torch.autograd.Function):
+    """Forward gather from a stack of textures, backward the splat into it
+    (layers/functional/resample.py:86-110)."""
+
+    @staticmethod
+    def forward(ctx, input, quad_idx, tex_uv, interp):
+        ctx.save_for_backward(quad_idx, tex_uv)
+        ctx.interp = InterpolationType(interp)
+        ctx.tex_shape = tuple(int(v) for v in input.shape[-3:])
+        return _uv_resample.resample_from_uv_maps(input, quad_idx, tex_uv, ctx.interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        quad_idx, tex_uv = ctx.saved_tensors
+        grad = _uv_resample.resample_to_uv_maps(grad_output.contiguous(), quad_idx, tex_uv,
+                                                ctx.tex_shape[0], ctx.tex_shape[1],
+                                                ctx.tex_shape[2], ctx.interp)
+        return grad, None, None, None
+
+
 # ----------------------------------------------------------------------------- entry points
 def mapped_convolution(input, weight, bias, sample_map, kernel_size, interp,
                        interp_weights=None):
@@ -280,4 +301,15 @@ def unresample(input, sample_map, interp, interp_weights=None):
     batched, added = _with_batch_dim(input)
     check_args(batched, sample_map, interp_weights, None, None)
     out = UnresampleFunction.apply(batched, sample_map, interp, interp_weights)
+    return out.squeeze(0) if added else out
+
+
+def uv_resample(input, quad_idx, tex_uv, interp):
+    """[B, C, T, TH, TW] (or [C, T, TH, TW]) textures -> [B, C, H, W] image: pixel (y, x) reads
+    texture quad_idx[y, x] at tex_uv[y, x] (layers/functional/resample.py:192-209)."""
+    assert input.dim() in [4, 5], \
+        'Input must have 4 or 5 dimensions (input.dim() == {})'.format(input.dim())
+    added = input.dim() == 4
+    out = UVResampleFunction.apply(input.unsqueeze(0) if added else input, quad_idx, tex_uv,
+                                   interp)
     return out.squeeze(0) if added else out

@@ -1,3 +1,3 @@
 from .modules import (MappedConvolution, MappedTransposedConvolution, MappedMaxPool,  # noqa: F401
-                      MappedAvgPool, MappedAvgUnpool, Resample, Unresample)
+                      MappedAvgPool, MappedAvgUnpool, Resample, Unresample, UVResample)
 from ..layer_utils import InterpolationType  # noqa: F401

@@ -140,3 +140,19 @@ class Unresample(nn.Module):
 
     def forward(self, x, sample_map, interp_weights=None):
         return F.unresample(x, sample_map, self.interp, interp_weights)
+
+
+class UVResample(nn.Module):
+    """Tangent images (a stack of textures) back to one image: the resampling step of the
+    reference's TangentImagesToEquirectangular (layers/nn/tangent_image_layer.py:42-70), with
+    the per-pixel texture index and UV coordinates handed in as tensors instead of being
+    generated from an icosphere in the constructor."""
+
+    def __init__(self, quad_idx, tex_uv, interpolation=InterpolationType.BILINEAR):
+        super().__init__()
+        self.register_buffer('quad', quad_idx)
+        self.register_buffer('uv', tex_uv)
+        self.interp = interpolation
+
+    def forward(self, x):
+        return F.uv_resample(x, self.quad, self.uv, self.interp)

@@ -270,3 +270,62 @@ def test_avg_pool_is_the_mean_of_im2col_rows_and_unpool_its_adjoint(oracle, inte
     cols = np.repeat((g / k)[:, :, None], k, axis=2).reshape(b, c * k, oh * ow)
     via = np.stack([oracle.mapped_col2im(cols[i], m, h, w, interp, iw) for i in range(b)])
     assert relerr(back, via) <= 1e-13
+
+
+# ----------------------------------------------------------------------------- average pooling
+# and UV resampling against the compiled reference (tests/golden/ref_fixtures_avg_uv.npz)
+@pytest.fixture(scope="module")
+def fx2():
+    return np.load(os.path.join(GOLDEN_DIR, "ref_fixtures_avg_uv.npz"))
+
+
+@pytest.mark.parametrize("d", ["f64", "f32"])
+@pytest.mark.parametrize("interp", [0, 1, 2])
+class TestAvgPoolAndUVAgainstCompiledReference:
+    @pytest.mark.parametrize("weighted", [False, True])
+    def test_avg_pool_and_unpool(self, oracle, fx2, d, interp, weighted):
+        pre = "%s/i%d/%s" % (d, interp, "w" if weighted else "")
+        m = _in(fx2, d, "m_w" if weighted else "m_u")
+        iw = _in(fx2, d, "iw") if weighted else None
+        x, g = _in(fx2, d, "x"), _in(fx2, d, "g")
+        assert np.array_equal(oracle.mapped_avg_pool(x, m, K, interp, iw), fx2[pre + "avg_pool"])
+        back = oracle.mapped_avg_unpool(g, m, x.shape[2], x.shape[3], K, interp, iw)
+        assert relerr(back, fx2[pre + "avg_unpool"]) <= TOL[d]
+
+    def test_uv_gather_is_bit_exact_and_its_adjoint(self, oracle, fx2, d, interp):
+        pre = "%s/i%d/" % (d, interp)
+        tex, quad, uv, x = (_in(fx2, d, n) for n in ("tex", "quad", "uv", "x"))
+        assert np.array_equal(oracle.resample_from_uv_maps(tex, quad, uv, interp),
+                              fx2[pre + "from_uv"])
+        nt, th, tw = tex.shape[2:]
+        back = oracle.resample_to_uv_maps(x, quad, uv, nt, th, tw, interp)
+        assert relerr(back, fx2[pre + "to_uv"]) <= TOL[d]
+
+
+@pytest.mark.parametrize("interp", [0, 1, 2])
+def test_uv_resampling_is_the_plain_gather_per_texture(oracle, interp):
+    """A UV gather reads, for each pixel, what resample_from_map (pinned above) reads from the
+    named texture alone; taps never cross into a neighbouring texture.  The other direction is
+    its adjoint, and texture indices outside the range contribute nothing."""
+    rng = np.random.default_rng(70 + interp)
+    b, c, nt, th, tw, h, w = 2, 3, 6, 5, 8, 9, 13
+    tex = rng.standard_normal((b, c, nt, th, tw))
+    quad = rng.integers(0, nt, (h, w))
+    uv = np.stack([rng.uniform(-1.5, tw + 0.5, (h, w)), rng.uniform(-1.5, th + 0.5, (h, w))], -1)
+    got = oracle.resample_from_uv_maps(tex, quad, uv, interp)
+    want = np.zeros((b, c, h, w))
+    for t in range(nt):
+        per = oracle.resample_from_map(np.ascontiguousarray(tex[:, :, t]), uv, interp)
+        want = np.where(quad == t, per, want)
+    assert np.array_equal(got, want)
+    y = rng.standard_normal((b, c, h, w))
+    back = oracle.resample_to_uv_maps(y, quad, uv, nt, th, tw, interp)
+    assert abs((got * y).sum() - (tex * back).sum()) <= 1e-10 * np.abs(got * y).sum()
+    bad = quad.copy()
+    bad[::2, ::3] = nt
+    bad[1::2, ::4] = -1
+    masked = np.where((bad >= 0) & (bad < nt), got, 0.0)
+    assert np.array_equal(oracle.resample_from_uv_maps(tex, bad, uv, interp), masked)
+    ok = ((bad >= 0) & (bad < nt)).astype(np.float64)
+    assert relerr(oracle.resample_to_uv_maps(y, bad, uv, nt, th, tw, interp),
+                  oracle.resample_to_uv_maps(y * ok, quad, uv, nt, th, tw, interp)) <= 1e-13

@@ -160,6 +160,34 @@ def tangent_patch_map(H, W, level=1, patch=64, dtype=np.float32):
     return np.ascontiguousarray(m.astype(dtype))
 
 
+def tangent_uv_map(H, W, level=1, patch=64, dtype=np.float32):
+    """The way back from tangent_patch_map's patches: for every pixel of the H x W
+    equirectangular image the face whose centre is nearest on the sphere (quad [H, W] int64) and
+    the pixel's gnomonic projection onto that face's tangent plane in patch pixel coordinates
+    (uv [H, W, 2], x first; 0 .. patch-1 spans the patch)."""
+    v, f = icosphere(level)
+    centres = v[f].mean(1)
+    centres /= np.linalg.norm(centres, axis=1, keepdims=True)
+    ang = np.arccos(np.clip((centres * v[f[:, 0]]).sum(1), -1, 1)).max()
+    half = math.tan(ang)
+    lon = (np.arange(W) * (2 * math.pi / W) - math.pi)[None, :]
+    lat = (np.arange(H) * (math.pi / (H - 1)) - math.pi / 2)[:, None]
+    # inverse of: lon = atan2(z, x), lat = atan2(-y, hypot(x, z))
+    d = np.stack(np.broadcast_arrays(np.cos(lat) * np.cos(lon), -np.sin(lat),
+                                     np.cos(lat) * np.sin(lon)), -1)
+    quad = np.argmax(d.reshape(-1, 3) @ centres.T, axis=1).reshape(H, W)
+    lon0 = np.arctan2(centres[:, 2], centres[:, 0])[quad]
+    lat0 = np.arctan2(-centres[:, 1], np.hypot(centres[:, 0], centres[:, 2]))[quad]
+    dl = lon - lon0
+    cosc = np.sin(lat0) * np.sin(lat) + np.cos(lat0) * np.cos(lat) * np.cos(dl)
+    dx = np.cos(lat) * np.sin(dl) / cosc
+    dy = (np.cos(lat0) * np.sin(lat) - np.sin(lat0) * np.cos(lat) * np.cos(dl)) / cosc
+    u = (dx + half) / (2 * half) * (patch - 1)
+    w_ = (-dy + half) / (2 * half) * (patch - 1)
+    uv = np.stack([u, w_], -1).astype(dtype)
+    return np.ascontiguousarray(quad.astype(np.int64)), np.ascontiguousarray(uv)
+
+
 # ----------------------------------------------------------------------------- configurations
 def _rng(cfg):
     return np.random.default_rng(1234 + cfg)
@@ -183,10 +211,13 @@ def config1(dtype=np.float32):
 
 
 def config2(batch=4, H=512, W=1024, patch=64, dtype=np.float32):
-    """Tangent-image resampling: gather [B,3,H,W] onto 80 patches, scatter back."""
+    """Tangent-image resampling: gather [B,3,H,W] onto 80 patches, scatter back; and the UV
+    way back: every image pixel reads its nearest face's patch at (u, v)."""
     rng = _rng(2)
+    quad, uv = tangent_uv_map(H, W, 1, patch, dtype)
     return dict(x=rng.uniform(0, 1, (batch, 3, H, W)).astype(dtype),
-                sample_map=tangent_patch_map(H, W, 1, patch, dtype), out_shape=(H, W), interp=1)
+                sample_map=tangent_patch_map(H, W, 1, patch, dtype), out_shape=(H, W), interp=1,
+                quad_idx=quad, tex_uv=uv, patch=patch)
 
 
 def config3(batch=8, channels=64, H=256, W=512, dtype=np.float32):
