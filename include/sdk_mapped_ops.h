@@ -148,9 +148,9 @@ int sdk_resample_from_uv_maps(const void* textures, const int64_t* quad_idx, con
  * input [B,C,H,W]; textures [B,C,NT,TH,TW].  Replaces `_uv_resample.resample_to_uv_maps`
  * (uv_resample_layer.h:48-74; body common/resample.h:160-187; src/cpp/uv_resample_layer.cpp:7-39).
  * workspace (optional, may be NULL): sdk_resample_to_uv_maps_workspace_bytes() bytes of device
- * scratch (4 bytes per image pixel + 12 per texture).  With it the image pixels are bucketed by
- * texture on the device and every texture is summed in on-chip memory and written once, without
- * atomics in memory and without a zero fill; the query returns 0 (and the call then needs no
+ * scratch (4 bytes per image pixel + at most 260 per texture).  With it the image pixels are
+ * bucketed by texture on the device and every texture is summed in on-chip memory and written
+ * once, without atomics in memory and without a zero fill; the query returns 0 (and the call then needs no
  * workspace) when a texture does not fit there (TH*TW*sizeof > 64 KiB).  Without it: zero fill
  * and atomic adds. */
 size_t sdk_resample_to_uv_maps_workspace_bytes(int64_t num_textures, int64_t tex_height,

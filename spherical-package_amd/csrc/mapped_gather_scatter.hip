@@ -332,8 +332,11 @@ struct LaneRuns {
   }
 };
 
+// count / cursor are kept in R copies ([R][NT]; a workgroup uses copy blockIdx % R), so that
+// neighbouring workgroups, which mostly see the same texture, do not queue on one address.
+// A texture's bucket is the concatenation of its R parts.
 __global__ __launch_bounds__(kBlock) void uv_count_kernel(const int64_t* __restrict__ quad,
-                                                          int NT, int MP,
+                                                          int NT, int MP, int R,
                                                           int* __restrict__ count) {
   const int pix = blockIdx.x * kBlock + threadIdx.x;
   const long long q = pix < MP ? quad[pix] : -1;
@@ -341,39 +344,43 @@ __global__ __launch_bounds__(kBlock) void uv_count_kernel(const int64_t* __restr
   const int t = ok ? (int)q : -1;
   const int below = __shfl_up(t, 1);
   const LaneRuns runs(below == t);
-  if (ok && runs.tail) atomicAdd(&count[t], runs.dist + 1);
+  if (ok && runs.tail) atomicAdd(&count[(size_t)(blockIdx.x % R) * NT + t], runs.dist + 1);
 }
 
-// offset[t] = cursor[t] = number of pixels in textures below t; offset[NT] = all of them.
+// Exclusive scan in bucket order (texture-major, copy-minor): cursor[r][t] = first slot of part
+// r of texture t; offset[t] = first slot of texture t, offset[NT] = number of pixels listed.
+// One workgroup; every thread owns a contiguous strip of the NT * R counters, so the counters
+// are read in one sweep of independent loads.
 __global__ __launch_bounds__(kBlock) void uv_scan_kernel(const int* __restrict__ count, int NT,
-                                                         int* __restrict__ offset,
+                                                         int R, int* __restrict__ offset,
                                                          int* __restrict__ cursor) {
-  __shared__ int part[kBlock];
-  int carry = 0;
-  for (int base = 0; base < NT; base += kBlock) {
-    const int i = base + threadIdx.x;
-    const int c = i < NT ? count[i] : 0;
-    part[threadIdx.x] = c;
-    __syncthreads();
-    for (int d = 1; d < kBlock; d <<= 1) {
-      const int add = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
-      __syncthreads();
-      part[threadIdx.x] += add;
-      __syncthreads();
-    }
-    const int incl = part[threadIdx.x];
-    if (i < NT) {
-      offset[i] = carry + incl - c;
-      cursor[i] = carry + incl - c;
-    }
-    carry += part[kBlock - 1];
-    __syncthreads();
+  __shared__ int wave_total[kBlock / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = NT * R;
+  const int strip = (n + kBlock - 1) / kBlock;
+  const int first = threadIdx.x * strip, last = min(n, first + strip);
+  int mine = 0;
+  for (int i = first; i < last; ++i) mine += count[(size_t)(i % R) * NT + i / R];
+  int incl = mine;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int below = __shfl_up(incl, d);
+    if (lane >= d) incl += below;
   }
-  if (threadIdx.x == 0) offset[NT] = carry;
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int run = incl - mine;
+  for (int w = 0; w < wave; ++w) run += wave_total[w];
+  for (int i = first; i < last; ++i) {
+    const int t = i / R, r = i - t * R;
+    cursor[(size_t)r * NT + t] = run;
+    if (r == 0) offset[t] = run;
+    run += count[(size_t)r * NT + t];
+  }
+  if (threadIdx.x == kBlock - 1) offset[NT] = run;
 }
 
 __global__ __launch_bounds__(kBlock) void uv_fill_kernel(const int64_t* __restrict__ quad, int NT,
-                                                         int MP, int* __restrict__ cursor,
+                                                         int MP, int R, int* __restrict__ cursor,
                                                          int* __restrict__ list) {
   const int pix = blockIdx.x * kBlock + threadIdx.x;
   const long long q = pix < MP ? quad[pix] : -1;
@@ -383,17 +390,19 @@ __global__ __launch_bounds__(kBlock) void uv_fill_kernel(const int64_t* __restri
   const LaneRuns runs(below == t);
   // the last lane of a run reserves the run's slots; the others read the start from it
   int start = 0;
-  if (ok && runs.tail) start = atomicAdd(&cursor[t], runs.dist + 1);
+  if (ok && runs.tail)
+    start = atomicAdd(&cursor[(size_t)(blockIdx.x % R) * NT + t], runs.dist + 1);
   const int lane = threadIdx.x & 63;
-  // lane of this run's tail: the next run's head minus one
   const unsigned long long tails = __ballot(runs.tail);
   const int tail_lane = __ffsll((long long)(tails & (~0ull << lane))) - 1;
   start = __shfl(start, tail_lane);
   if (ok) list[start + runs.dist] = pix;
 }
 
+constexpr int kUvBlock = 1024;   // 16 waves: a long bucket (a polar face) takes few rounds
+
 template <typename T, int INTERP, int PL>
-__global__ __launch_bounds__(kBlock) void uv_texture_scatter_kernel(
+__global__ __launch_bounds__(kUvBlock) void uv_texture_scatter_kernel(
     const T* __restrict__ in, const T* __restrict__ uv, const int* __restrict__ offset,
     const int* __restrict__ list, T* __restrict__ textures, int planes, int NT, int TH, int TW,
     int MP) {
@@ -408,19 +417,32 @@ __global__ __launch_bounds__(kBlock) void uv_texture_scatter_kernel(
   const int lo0 = offset[t], hi0 = offset[t + 1];
   const int per = (hi0 - lo0 + (int)gridDim.z - 1) / (int)gridDim.z;
   const int lo = lo0 + (int)blockIdx.z * per, hi = min(hi0, lo + per);
-  for (int i = threadIdx.x; i < PL * THW; i += kBlock) acc[i] = T(0);
+  for (int i = threadIdx.x; i < PL * THW; i += kUvBlock) acc[i] = T(0);
   __syncthreads();
   constexpr int N = PointTaps<T, INTERP>::N;
-  for (int base = lo; base < hi; base += kBlock) {   // uniform trip count over the workgroup
-    const int e = base + threadIdx.x;
-    const bool live = e < hi;
-    const int pix = live ? list[e] : 0;
-    PointTaps<T, INTERP> taps;
-    taps.set(live ? uv[(size_t)pix * 2] : T(0), live ? uv[(size_t)pix * 2 + 1] : T(0), TH, TW);
-    T val[PL];
+  // this round's pixel, point and values are loaded during the round before
+  int e = lo + (int)threadIdx.x;
+  int pix = e < hi ? list[e] : 0;
+  T pu = uv[(size_t)pix * 2], pv = uv[(size_t)pix * 2 + 1];
+  T val[PL];
 #pragma unroll
-    for (int j = 0; j < PL; ++j)
-      val[j] = (live && j < np) ? in[(size_t)(plane0 + j) * MP + pix] : T(0);
+  for (int j = 0; j < PL; ++j) val[j] = in[(size_t)(plane0 + (j < np ? j : 0)) * MP + pix];
+  int pix_next = e + kUvBlock < hi ? list[e + kUvBlock] : 0;
+  for (int base = lo; base < hi; base += kUvBlock) {   // uniform trip count over the workgroup
+    const bool live = e < hi;
+    PointTaps<T, INTERP> taps;
+    taps.set(pu, pv, TH, TW);
+    T cur[PL];
+#pragma unroll
+    for (int j = 0; j < PL; ++j) cur[j] = (live && j < np) ? val[j] : T(0);
+    // next round's loads
+    e += kUvBlock;
+    pix = pix_next;
+    pu = uv[(size_t)pix * 2];
+    pv = uv[(size_t)pix * 2 + 1];
+#pragma unroll
+    for (int j = 0; j < PL; ++j) val[j] = in[(size_t)(plane0 + (j < np ? j : 0)) * MP + pix];
+    pix_next = e + kUvBlock < hi ? list[e + kUvBlock] : 0;
     // lanes whose first tap is the same texel form a run: all their taps coincide
     const int ky = live ? taps.ty[0] : INT_MIN, kx = live ? taps.tx[0] : (int)threadIdx.x;
     const int by = __shfl_up(ky, 1), bx = __shfl_up(kx, 1);
@@ -432,14 +454,14 @@ __global__ __launch_bounds__(kBlock) void uv_texture_scatter_kernel(
       const int o = inside ? taps.ty[i] * TW + taps.tx[i] : 0;
 #pragma unroll
       for (int j = 0; j < PL; ++j) {
-        const T total = runs.sum(w * val[j]);
+        const T total = runs.sum(w * cur[j]);
         if (live && runs.tail && inside && total != T(0)) lds_add(acc + j * THW + o, total);
       }
     }
   }
   __syncthreads();
   const size_t stride = (size_t)NT * THW;
-  for (int i = threadIdx.x; i < THW; i += kBlock) {
+  for (int i = threadIdx.x; i < THW; i += kUvBlock) {
 #pragma unroll
     for (int j = 0; j < PL; ++j) {
       if (j < np) {
@@ -963,13 +985,23 @@ static int launch_uv_gather(const T* textures, const int64_t* quad, const T* uv,
   return SDK_OK;
 }
 
-// Workspace of the adjoint by texture: count | offset (NT + 1) | cursor | bucket (MP pixels).
+// Copies of the bucket counters (a power of two; fewer for many textures, whose pixels
+// spread over more addresses anyway and whose scan runs in one workgroup).
+static int uv_counter_copies(int64_t NT) {
+  int r = 32;
+  while (r > 1 && NT * r > 65536) r >>= 1;
+  return r;
+}
+
+// Workspace of the adjoint by texture: count [R][NT] | offset (NT + 1) | cursor [R][NT] |
+// bucket (MP pixels).
 static size_t uv_layout(int64_t NT, int64_t MP, size_t (&off)[4]) {
   auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
-  off[0] = 0;                                  // count
-  off[1] = off[0] + up((size_t)NT * 4);        // offset
-  off[2] = off[1] + up((size_t)(NT + 1) * 4);  // cursor
-  off[3] = off[2] + up((size_t)NT * 4);        // bucket
+  const size_t copies = (size_t)uv_counter_copies(NT);
+  off[0] = 0;                                       // count
+  off[1] = off[0] + up((size_t)NT * copies * 4);    // offset
+  off[2] = off[1] + up((size_t)(NT + 1) * 4);       // cursor
+  off[3] = off[2] + up((size_t)NT * copies * 4);    // bucket
   return off[3] + up((size_t)MP * 4);
 }
 
@@ -995,9 +1027,11 @@ static int launch_uv_scatter(const T* in, const int64_t* quad, const T* uv, T* t
     int rc = zero_fill(count, off[1], stream);
     if (rc != SDK_OK) return rc;
     const dim3 pixel_grid((unsigned)ceil_div(MP, kBlock));
-    launch(uv_count_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, count);
-    launch(uv_scan_kernel, dim3(1), dim3(kBlock), stream, (const int*)count, NT, offset, cursor);
-    launch(uv_fill_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, cursor, list);
+    const int copies = uv_counter_copies(NT);
+    launch(uv_count_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, count);
+    launch(uv_scan_kernel, dim3(1), dim3(kBlock), stream, (const int*)count, NT, copies, offset,
+           cursor);
+    launch(uv_fill_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, cursor, list);
     SDK_LAUNCH_CHECK("resample_to_uv_maps(bucket)");
     // planes per workgroup: as many as LDS holds while the grid still fills the GPU; few
     // textures: several workgroups share one and add their parts to a zero-filled output
@@ -1017,7 +1051,7 @@ static int launch_uv_scatter(const T* in, const int64_t* quad, const T* uv, T* t
     const dim3 grid((unsigned)NT, (unsigned)ceil_div(planes, pl), (unsigned)split);
 #define UVS(PLv)                                                                              \
   SDK_DISPATCH_INTERP_ONLY(interp, (uv_texture_scatter_kernel<T, INTERP, PLv>                 \
-                                    <<<grid, dim3(kBlock), (size_t)PLv * THW * sizeof(T), stream>>>( \
+                                    <<<grid, dim3(kUvBlock), (size_t)PLv * THW * sizeof(T), stream>>>( \
                                         in, uv, (const int*)offset, (const int*)list, textures, \
                                         (int)planes, NT, TH, TW, MP)))
     if (pl == 4) UVS(4); else if (pl == 2) UVS(2); else UVS(1);
