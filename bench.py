@@ -187,7 +187,11 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     ms_ub, _ = timer.run(lambda: ops.resample_to_uv_maps(x, quad, uv, NT, TP, TP, 1), steps,
                          warmup)
     uv_bytes = _nbytes(tex, quad, uv, x)
-    return {"uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf)),
+    # the kernel map of configuration 4's image, generated on the device (bytes = the map)
+    ms_map, _ = timer.run(lambda: ops.equirect_kernel_map(256, 512, 3, 3), steps, warmup)
+    map_bytes = 256 * 512 * 9 * 2 * 4.0
+    return {"map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
+            "uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf)),
             "uv_scatter": dict(ms=ms_ub, **_roof("hbm", uv_bytes, ms_ub)),
             "gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,
                                             traffic=_measured_traffic("resample_from_map"))),

@@ -163,6 +163,39 @@ int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const vo
                             int32_t interp, int32_t dtype, sdk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * Sample maps computed on the device (the reference builds them on the host with tensor
+ * operations).  Maps are written in the layout every entry point above reads: (x, y) pairs in
+ * pixel coordinates of an equirectangular image, lon = -pi + 2 pi x / W, lat = -pi/2 + pi y / (H-1).
+ * ------------------------------------------------------------------------- */
+typedef enum sdk_projection {
+  SDK_MAP_GRID = 0,                   /* pixel grid offsets: layers/util/mapping_functions.py:43-75 */
+  SDK_MAP_INVERSE_GNOMONIC = 1,       /* tangent-plane kernel projected back: :78-120 */
+  SDK_MAP_INVERSE_EQUIRECTANGULAR = 2 /* longitude step widened by 1 / cos(lat): :123-160 */
+} sdk_projection;
+
+/* sample_map [ceil(H/stride), ceil(W/stride), kernel_h*kernel_w, 2]: for every stride-th pixel of an
+ * H x W equirectangular image the kernel_h x kernel_w kernel about it (row-major, sample
+ * (i, j) offset by (j - kernel_w/2, i - kernel_h/2) * dilation image steps), projected as
+ * `projection` says; longitudes wrapped into the image for the two inverse projections.
+ * Replaces `grid_projection_map`, `inverse_gnomonic_projection_map`,
+ * `inverse_equirectangular_projection_map` (layers/util/mapping_functions.py:43-160, with
+ * grids.py:5-25 and conversions.py:24-52). */
+int sdk_equirect_kernel_map(void* sample_map, int64_t height, int64_t width, int64_t kernel_h,
+                            int64_t kernel_w, int64_t stride, int64_t dilation,
+                            int32_t projection, int32_t dtype, sdk_stream_t stream);
+
+/* out [num_points, kernel_h*kernel_w, 2]: a gnomonic kernel_h x kernel_w kernel with angular
+ * steps (res_lon, res_lat) about each of the points lonlat [num_points, 2] (lon, lat), returned
+ * in (lon, lat) when image_height == 0, else in pixel coordinates of an image_height x
+ * image_width equirectangular image.  Replaces `gnomonic_kernel`
+ * (layers/util/icosahedron_functions.py:47-103) followed by `convert_spherical_to_image`
+ * (layers/util/conversions.py:33-52), the pair the tangent-image and icosphere map builders use
+ * (layers/util/tangent_images.py:59-88). */
+int sdk_gnomonic_kernel_at(const void* lonlat, void* out, int64_t num_points, int64_t kernel_h,
+                           int64_t kernel_w, double res_lat, double res_lon, int64_t image_height,
+                           int64_t image_width, int32_t dtype, sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Mapped im2col / col2im (batched).
  * col[b, c*K + k, pix] with pix = y_out*OW + x_out, out_pixels = OH*OW.
  * sample_map [OH,OW,K,(P,)2].

@@ -274,3 +274,31 @@ def mapped_transposed_conv_backward(grad_output, sample_map, x, weight, bias,
 
 def num_threads():
     return int(lib().sdk_oracle_num_threads())
+
+
+GRID, INVERSE_GNOMONIC, INVERSE_EQUIRECTANGULAR = 0, 1, 2
+
+
+def equirect_kernel_map(shape, kernel_size, stride=1, dilation=1, projection=INVERSE_GNOMONIC,
+                        dtype=np.float32):
+    """[ceil(H/stride), ceil(W/stride), kh*kw, 2] kernel map of an H x W equirectangular image
+    (layers/util/mapping_functions.py:43-160)."""
+    H, W = shape
+    kh, kw = kernel_size
+    out = np.empty((-(-H // stride), -(-W // stride), kh * kw, 2), dtype)
+    _check(lib().sdk_oracle_equirect_kernel_map(
+        _p(out), *_i64(H, W, kh, kw, stride, dilation), *_i32(projection, _dt(out))))
+    return out
+
+
+def gnomonic_kernel_at(lonlat, kh, kw, res_lat, res_lon, image_shape=None):
+    """[N, kh*kw, 2] gnomonic kernels about the points lonlat [N, 2], in (lon, lat) or, with
+    image_shape, in equirectangular pixel coordinates
+    (layers/util/icosahedron_functions.py:47-103, layers/util/conversions.py:33-52)."""
+    pts = _c(lonlat)
+    out = np.empty((pts.shape[0], kh * kw, 2), pts.dtype)
+    ih, iw = image_shape if image_shape is not None else (0, 0)
+    _check(lib().sdk_oracle_gnomonic_kernel_at(
+        _p(pts), _p(out), *_i64(pts.shape[0], kh, kw), ctypes.c_double(res_lat),
+        ctypes.c_double(res_lon), *_i64(ih, iw), *_i32(_dt(pts))))
+    return out

@@ -26,6 +26,9 @@
 //   average pool / unpool: reference known-answer vector (tests/test_mapped_pooling.py:110-132)
 //       + "mean over k of the pinned im2col rows" + adjoint identity + compiled-reference
 //       fixtures (weighted, nearest, bispherical).
+//   sample-map generation: closed forms in pixel units (grid, inverse equirectangular), the
+//       forward gnomonic projection of every sample giving back its tangent-plane offset,
+//       centre sample = the pixel, stride = sub-sampling, float32 against float64.
 //   UV resampling: compiled-reference fixtures + "per texture it is the pinned gather" +
 //       adjoint identity (the reference's test-suite holds no vector for it).
 #include <cmath>
@@ -520,6 +523,100 @@ void avg_unpool(const T* gout, const T* map, const T* wts, T* gin, int64_t B, in
 // layout [..., 2]; P >= 1 the weighted layout [..., P, 2] with weights [..., P].
 // Every function returns 0 on success, 1 on an unsupported dtype.
 // ---------------------------------------------------------------------------
+// ---------------------------------------------------------------------------
+// Sample-map generation.  The reference builds its maps with float32 (default dtype) tensor
+// operations; every step below is the corresponding scalar operation in T, in the same order.
+// layers/util/grids.py:5-25 (angular resolution, mesh grid; linspace is evaluated from the
+// nearer end as the tensor library does), layers/util/conversions.py:24-52 (renormalize,
+// spherical -> pixel), layers/util/mapping_functions.py:16-160 (kernel differentials and the
+// three projections), layers/util/icosahedron_functions.py:47-103 (gnomonic kernel about
+// given points).  Python scalars enter a tensor operation rounded to the tensor's type.
+// ---------------------------------------------------------------------------
+const double PI = 3.14159265358979323846;
+
+template <typename T>
+inline T linspace_at(T lo, T hi, int64_t steps, int64_t i) {
+  const T step = (hi - lo) / T(steps - 1);
+  return i < steps / 2 ? lo + step * T(i) : hi - step * T(steps - i - 1);
+}
+
+template <typename T>
+inline T floor_mod(T a, T b) {
+  T m = std::fmod(a, b);
+  if (m != T(0) && ((b < T(0)) != (m < T(0)))) m += b;
+  return m;
+}
+
+template <typename T>
+inline T lon_to_x(T lon, int64_t W) { return T(W) * (lon - T(-PI)) / T(PI - (-PI)); }
+template <typename T>
+inline T lat_to_y(T lat, int64_t H) { return T(H - 1) * (lat - T(-PI / 2)) / T(PI / 2 - (-PI / 2)); }
+
+template <typename T>
+inline void inverse_gnomonic(T lon, T lat, T dx, T dy, T& out_lon, T& out_lat) {
+  const T rho = std::sqrt(dx * dx + dy * dy);
+  const T nu = std::atan(rho);
+  out_lat = std::asin(std::cos(nu) * std::sin(lat) + dy * std::sin(nu) * std::cos(lat) / rho);
+  out_lon = lon + std::atan2(dx * std::sin(nu),
+                             rho * std::cos(lat) * std::cos(nu) - dy * std::sin(lat) * std::sin(nu));
+}
+
+template <typename T>
+void equirect_kernel_map(T* out, int64_t H, int64_t W, int64_t kh, int64_t kw, int64_t stride,
+                         int64_t dilation, int proj) {
+  const int64_t OH = (H + stride - 1) / stride, OW = (W + stride - 1) / stride, K = kh * kw;
+  const double res_lon = 2 * PI / double(W), res_lat = PI / double(H - 1);
+#pragma omp parallel for schedule(static)
+  for (int64_t idx = 0; idx < OH * OW * K; ++idx) {
+    const int64_t k = idx % K, pix = idx / K;
+    const int64_t x = (pix % OW) * stride, y = (pix / OW) * stride;
+    const int64_t ci = k / kw - kh / 2, cj = k % kw - kw / 2;
+    const T dlon = T(double(cj * dilation) * res_lon);
+    const T dlat = T(double(ci * dilation) * -res_lat);
+    const T lon = linspace_at<T>(T(-PI), T(PI), W + 1, x);
+    const T lat = linspace_at<T>(T(-PI / 2), T(PI / 2), H, y);
+    T mlon, mlat;
+    if (proj == 0) {
+      mlat = lat + dlat;
+      mlon = lon + dlon;
+    } else {
+      if (proj == 1) {
+        inverse_gnomonic(lon, lat, dlon, dlat, mlon, mlat);
+        if (k == K / 2) { mlat = lat; mlon = lon; }
+      } else {
+        mlat = lat + dlat;
+        mlon = lon + dlon / std::cos(mlat);
+      }
+      mlon = floor_mod(mlon + T(PI), T(2 * PI)) - T(PI);
+    }
+    out[idx * 2] = lon_to_x(mlon, W);
+    out[idx * 2 + 1] = lat_to_y(mlat, H);
+  }
+}
+
+template <typename T>
+void gnomonic_kernel_at(const T* lonlat, T* out, int64_t n, int64_t kh, int64_t kw,
+                        double res_lat, double res_lon, int64_t img_h, int64_t img_w) {
+  const int64_t K = kh * kw;
+#pragma omp parallel for schedule(static)
+  for (int64_t idx = 0; idx < n * K; ++idx) {
+    const int64_t k = idx % K, p = idx / K, i = k / kw, j = k % kw;
+    T dx = T(double(j - kw / 2) * res_lon);
+    T dy = T(double(i - kh / 2) * res_lat);
+    if (kh % 2 == 0) dy += T(res_lat / 2);
+    if (kw % 2 == 0) dx += T(res_lon / 2);
+    const T lon = lonlat[p * 2], lat = lonlat[p * 2 + 1];
+    T olon, olat;
+    inverse_gnomonic(lon, lat, dx, dy, olon, olat);
+    const bool centre = k == (kh / 2) * kw + kw / 2;
+    if (kh % 2 == 1 && centre) olat = lat;
+    if (kw % 2 == 1 && centre) olon = lon;
+    olon = floor_mod(olon + T(PI), T(2 * PI)) - T(PI);
+    out[idx * 2] = img_h > 0 ? lon_to_x(olon, img_w) : olon;
+    out[idx * 2 + 1] = img_h > 0 ? lat_to_y(olat, img_h) : olat;
+  }
+}
+
 #define DISPATCH(dtype, CALL)                                       \
   do {                                                              \
     if ((dtype) == 0) { using T = float; CALL; return 0; }          \
@@ -600,6 +697,18 @@ int sdk_oracle_resample_to_uv_maps(const void* in, const int64_t* quad, const vo
                                    int64_t H, int64_t W, int interp, int dtype) {
   DISPATCH(dtype, resample_to_uv<T>((const T*)in, quad, (const T*)uv, (T*)tex, B, C, NT, TH, TW,
                                      H, W, interp));
+}
+
+int sdk_oracle_equirect_kernel_map(void* out, int64_t H, int64_t W, int64_t kh, int64_t kw,
+                                   int64_t stride, int64_t dilation, int proj, int dtype) {
+  DISPATCH(dtype, equirect_kernel_map<T>((T*)out, H, W, kh, kw, stride, dilation, proj));
+}
+
+int sdk_oracle_gnomonic_kernel_at(const void* lonlat, void* out, int64_t n, int64_t kh, int64_t kw,
+                                  double res_lat, double res_lon, int64_t img_h, int64_t img_w,
+                                  int dtype) {
+  DISPATCH(dtype, gnomonic_kernel_at<T>((const T*)lonlat, (T*)out, n, kh, kw, res_lat, res_lon,
+                                         img_h, img_w));
 }
 
 int sdk_oracle_mapped_conv_forward(const void* x, const void* map, const void* wts,

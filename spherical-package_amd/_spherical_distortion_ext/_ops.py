@@ -402,6 +402,45 @@ def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp)
     return out
 
 
+# --------------------------------------------------------------------------- map generation
+# Factory functions (no tensor argument to dispatch on): plain Python, not registered operators.
+
+def equirect_kernel_map(height, width, kernel_h, kernel_w, stride=1, dilation=1, projection=1,
+                        dtype=torch.float32, device="cuda"):
+    """[ceil(H/stride), ceil(W/stride), kh*kw, 2] kernel map of an H x W equirectangular image,
+    computed on the device.  projection: 0 grid, 1 inverse gnomonic, 2 inverse equirectangular."""
+    if dtype not in _DTYPES:
+        raise RuntimeError("unsupported dtype %s (float32 and float64 only)" % dtype)
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("this backend runs on the GPU only: device must be a CUDA/HIP device")
+    H, W, s = int(height), int(width), int(stride)
+    if H < 2 or W < 1 or s < 1:
+        raise RuntimeError("image %d x %d (height at least 2), stride %d" % (H, W, s))
+    out = torch.empty((-(-H // s), -(-W // s), int(kernel_h) * int(kernel_w), 2), dtype=dtype,
+                      device=device)
+    with torch.cuda.device(out.device):
+        _capi.call("sdk_equirect_kernel_map", _ptr(out), H, W, int(kernel_h), int(kernel_w), s,
+                   int(dilation), int(projection), _DTYPES[dtype], _stream(out))
+    return out
+
+
+def gnomonic_kernel_at(lonlat, kernel_h, kernel_w, res_lat, res_lon, image_h=0, image_w=0):
+    """[N, kh*kw, 2] gnomonic kernels about the points lonlat [N, 2] (lon, lat): spherical
+    coordinates, or pixel coordinates of an image_h x image_w equirectangular image."""
+    _check(lonlat, lonlat=lonlat)
+    if lonlat.dim() != 2 or lonlat.shape[1] != 2:
+        raise RuntimeError("lonlat must be [N, 2], got %s" % (tuple(lonlat.shape),))
+    n = int(lonlat.shape[0])
+    out = torch.empty((n, int(kernel_h) * int(kernel_w), 2), dtype=lonlat.dtype,
+                      device=lonlat.device)
+    with torch.cuda.device(lonlat.device):
+        _capi.call("sdk_gnomonic_kernel_at", _ptr(lonlat), _ptr(out), n, int(kernel_h),
+                   int(kernel_w), float(res_lat), float(res_lon), int(image_h), int(image_w),
+                   _DTYPES[lonlat.dtype], _stream(lonlat))
+    return out
+
+
 # --------------------------------------------------------------------------- registration
 _SCHEMAS = (
     ("resample_from_map",
