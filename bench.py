@@ -190,7 +190,16 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     # the kernel map of configuration 4's image, generated on the device (bytes = the map)
     ms_map, _ = timer.run(lambda: ops.equirect_kernel_map(256, 512, 3, 3), steps, warmup)
     map_bytes = 256 * 512 * 9 * 2 * 4.0
-    return {"map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
+    # voting resample: a 13-class label image halved in size, four sources per output pixel
+    gen = torch.Generator().manual_seed(7)
+    labels = torch.randint(0, 13, (B, 1, H, W), generator=gen, dtype=torch.int64).to(dev)
+    yy, xx = torch.meshgrid(torch.arange(H) // 2, torch.arange(W) // 2, indexing="ij")
+    vmap = torch.stack([xx, yy], -1).contiguous().to(dev)
+    ms_v, _ = timer.run(lambda: ops.voting_resample_to_map(labels, vmap, H // 2, W // 2, 13),
+                        steps, warmup)
+    vote_bytes = _nbytes(labels, vmap) + B * (H // 2) * (W // 2) * 8.0
+    return {"voting_resample": dict(ms=ms_v, **_roof("hbm", vote_bytes, ms_v)),
+            "map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
             "uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf)),
             "uv_scatter": dict(ms=ms_ub, **_roof("hbm", uv_bytes, ms_ub)),
             "gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,

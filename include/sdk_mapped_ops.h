@@ -163,6 +163,29 @@ int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const vo
                             int32_t interp, int32_t dtype, sdk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * Voting resample (integer labels).  input [B,C,IH,IW] int64 labels in [0, num_candidates);
+ * sample_map [IH,IW,2] int64 (x, y) target of every input pixel; out [B,C,OH,OW] int64 = for
+ * every output pixel the label most of its sources carry (the first such label on a tie, 0
+ * where no source lands).  Targets outside the output and labels outside the range cast no
+ * vote.  With channels > 1 the reference offsets channel c's votes by c*OH*OW histogram elements
+ * instead of c whole histograms, so votes of different channels share cells; that indexing is
+ * reproduced (label images have one channel).  Replaces `_voting_resample.voting_resample_to_map`
+ * (ext_modules/include/layers/voting_resample_layer.h:31-53; body
+ *  core/interpolation.h:249-265, common/resample.h:109-130; histogram + argmax
+ *  src/cpp/voting_resample_layer.cpp:8-37).
+ * workspace (required): at least sdk_voting_resample_workspace_bytes() bytes, 16-byte aligned:
+ * the vote histogram of one batch element, 4 bytes per (channel, output pixel, candidate); a
+ * workspace n times that size lets n batch elements be processed per pass.
+ * ------------------------------------------------------------------------- */
+size_t sdk_voting_resample_workspace_bytes(int64_t channels, int64_t out_height,
+                                           int64_t out_width, int64_t num_candidates);
+int sdk_voting_resample_to_map(const int64_t* input, const int64_t* sample_map, int64_t* out,
+                               void* workspace, size_t workspace_bytes, int64_t batch,
+                               int64_t channels, int64_t in_height, int64_t in_width,
+                               int64_t out_height, int64_t out_width, int64_t num_candidates,
+                               sdk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Sample maps computed on the device (the reference builds them on the host with tensor
  * operations).  Maps are written in the layout every entry point above reads: (x, y) pairs in
  * pixel coordinates of an equirectangular image, lon = -pi + 2 pi x / W, lat = -pi/2 + pi y / (H-1).

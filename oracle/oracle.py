@@ -302,3 +302,14 @@ def gnomonic_kernel_at(lonlat, kh, kw, res_lat, res_lon, image_shape=None):
         _p(pts), _p(out), *_i64(pts.shape[0], kh, kw), ctypes.c_double(res_lat),
         ctypes.c_double(res_lon), *_i64(ih, iw), *_i32(_dt(pts))))
     return out
+
+
+def voting_resample_to_map(labels, sample_map, out_h, out_w, num_candidates):
+    """labels [B,C,IH,IW] int64, sample_map [IH,IW,2] int64 -> [B,C,OH,OW] int64: the label
+    with the most votes per output pixel (src/cpp/voting_resample_layer.cpp:8-37)."""
+    x = _c(labels, np.int64); m = _c(sample_map, np.int64)
+    B, C, IH, IW = x.shape
+    out = np.empty((B, C, out_h, out_w), np.int64)
+    _check(lib().sdk_oracle_voting_resample(_p(x), _p(m), _p(out),
+                                            *_i64(B, C, IH, IW, out_h, out_w, num_candidates)))
+    return out

@@ -19,7 +19,7 @@ MODULES = ("_enums", "_resample", "_weighted_resample", "_mapped_convolution",
            "_weighted_mapped_convolution", "_mapped_transposed_convolution",
            "_weighted_mapped_transposed_convolution", "_mapped_max_pooling",
            "_weighted_mapped_max_pooling", "_mapped_avg_pooling",
-           "_weighted_mapped_avg_pooling", "_uv_resample")
+           "_weighted_mapped_avg_pooling", "_uv_resample", "_voting_resample")
 
 
 def available():

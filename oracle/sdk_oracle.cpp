@@ -29,8 +29,10 @@
 //   sample-map generation: closed forms in pixel units (grid, inverse equirectangular), the
 //       forward gnomonic projection of every sample giving back its tangent-plane offset,
 //       centre sample = the pixel, stride = sub-sampling, float32 against float64.
+//   voting resample: compiled-reference fixtures + brute force with numpy's bincount.
 //   UV resampling: compiled-reference fixtures + "per texture it is the pinned gather" +
 //       adjoint identity (the reference's test-suite holds no vector for it).
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -617,6 +619,38 @@ void gnomonic_kernel_at(const T* lonlat, T* out, int64_t n, int64_t kh, int64_t 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Voting resample.  core/interpolation.h:249-265 (one vote per in-range target),
+// common/resample.h:109-130 (label and target of an input pixel),
+// src/cpp/voting_resample_layer.cpp:8-37 (histogram [C, OH, OW, candidates] per batch element,
+// argmax over the last axis: the first of equal counts).  A label outside the range casts no
+// vote (the reference would write outside its histogram).  The reference offsets channel c's
+// votes by c * OH * OW histogram elements rather than by c whole planes of OH * OW * NC, so
+// with more than one channel the histograms overlap; that indexing is kept as it is (label
+// images have one channel, for which it is the plain vote).
+// ---------------------------------------------------------------------------
+void voting_resample(const int64_t* in, const int64_t* map, int64_t* out, int64_t B, int64_t C,
+                     int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t NC) {
+  std::vector<int64_t> votes((size_t)C * OH * OW * NC);
+  for (int64_t b = 0; b < B; ++b) {
+    std::fill(votes.begin(), votes.end(), 0);
+    for (int64_t i = 0; i < C * IH * IW; ++i) {
+      const int64_t pix = i % (IH * IW), c = i / (IH * IW);
+      const int64_t x = map[pix * 2], y = map[pix * 2 + 1], label = in[b * C * IH * IW + i];
+      if (x < 0 || x > OW - 1 || y < 0 || y > OH - 1 || label < 0 || label >= NC) continue;
+      // the channel's histogram starts c * OH * OW elements in, not c * OH * OW * NC
+      // (common/resample.h:127-129): for C > 1 the channels' histograms overlap
+      ++votes[c * OH * OW + (y * OW + x) * NC + label];
+    }
+    for (int64_t o = 0; o < C * OH * OW; ++o) {
+      int64_t arg = 0;
+      for (int64_t k = 1; k < NC; ++k)
+        if (votes[o * NC + k] > votes[o * NC + arg]) arg = k;
+      out[b * C * OH * OW + o] = arg;
+    }
+  }
+}
+
 #define DISPATCH(dtype, CALL)                                       \
   do {                                                              \
     if ((dtype) == 0) { using T = float; CALL; return 0; }          \
@@ -709,6 +743,13 @@ int sdk_oracle_gnomonic_kernel_at(const void* lonlat, void* out, int64_t n, int6
                                   int dtype) {
   DISPATCH(dtype, gnomonic_kernel_at<T>((const T*)lonlat, (T*)out, n, kh, kw, res_lat, res_lon,
                                          img_h, img_w));
+}
+
+int sdk_oracle_voting_resample(const int64_t* in, const int64_t* map, int64_t* out, int64_t B,
+                               int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                               int64_t NC) {
+  voting_resample(in, map, out, B, C, IH, IW, OH, OW, NC);
+  return 0;
 }
 
 int sdk_oracle_mapped_conv_forward(const void* x, const void* map, const void* wts,

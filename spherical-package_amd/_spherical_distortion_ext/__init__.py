@@ -10,7 +10,7 @@ kernels in libsdk_mapped_ops.so:
     _weighted_mapped_convolution, _mapped_transposed_convolution,
     _weighted_mapped_transposed_convolution, _mapped_max_pooling,
     _weighted_mapped_max_pooling, _mapped_avg_pooling, _weighted_mapped_avg_pooling,
-    _uv_resample
+    _uv_resample, _voting_resample
 
 Importing the package loads the library and registers the operators; it raises
 ImportError when the library has not been built.

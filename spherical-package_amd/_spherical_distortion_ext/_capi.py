@@ -27,6 +27,7 @@ SIGNATURES = {
     "sdk_equirect_kernel_map": [_vp] + [_i64] * 6 + [_i32] * 2 + [_vp],
     "sdk_gnomonic_kernel_at": [_vp, _vp] + [_i64] * 3 + [ctypes.c_double] * 2 + [_i64] * 2
                               + [_i32, _vp],
+    "sdk_voting_resample_to_map": [_vp] * 4 + [_sz] + [_i64] * 7 + [_vp],
     "sdk_mapped_im2col": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_pool": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],
@@ -45,7 +46,7 @@ SIGNATURES = {
 }
 OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes",
                  "sdk_resample_to_map_workspace_bytes", "sdk_mapped_max_unpool_workspace_bytes",
-                 "sdk_resample_to_uv_maps_workspace_bytes")
+                 "sdk_resample_to_uv_maps_workspace_bytes", "sdk_voting_resample_workspace_bytes")
 
 _lib = None
 
@@ -76,6 +77,8 @@ def load():
     lib.sdk_mapped_max_unpool_workspace_bytes.restype = _sz
     lib.sdk_resample_to_uv_maps_workspace_bytes.argtypes = [_i64] * 5 + [_i32]
     lib.sdk_resample_to_uv_maps_workspace_bytes.restype = _sz
+    lib.sdk_voting_resample_workspace_bytes.argtypes = [_i64] * 4
+    lib.sdk_voting_resample_workspace_bytes.restype = _sz
     _lib = lib
     return lib
 

@@ -402,6 +402,32 @@ def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp)
     return out
 
 
+# --------------------------------------------------------------------------- voting resample
+def voting_resample_to_map(labels, sample_map, out_h, out_w, num_candidates):
+    for name, t in (("input", labels), ("sample_map", sample_map)):
+        if not t.is_cuda:
+            raise RuntimeError("this backend runs on the GPU only: %s must be a CUDA/HIP tensor"
+                               % name)
+        if t.dtype != torch.int64:
+            raise RuntimeError("%s must be int64 (got %s)" % (name, t.dtype))
+        if not t.is_contiguous():
+            raise RuntimeError("%s must be contiguous" % name)
+    if labels.dim() != 4 or tuple(sample_map.shape) != tuple(labels.shape[2:]) + (2,):
+        raise RuntimeError("input %s must be [B, C, IH, IW] and sample_map %s [IH, IW, 2]"
+                           % (tuple(labels.shape), tuple(sample_map.shape)))
+    B, C, IH, IW = labels.shape
+    OH, OW, NC = int(out_h), int(out_w), int(num_candidates)
+    out = torch.empty((B, C, OH, OW), dtype=torch.int64, device=labels.device)
+    with torch.cuda.device(labels.device):
+        nws = _capi.load().sdk_voting_resample_workspace_bytes(C, OH, OW, NC)
+        # room for several batch elements per pass, within 256 MiB
+        nws *= max(1, min(B, (256 << 20) // max(nws, 1)))
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=labels.device)
+        _capi.call("sdk_voting_resample_to_map", _ptr(labels), _ptr(sample_map), _ptr(out),
+                   _ptr(ws), nws, B, C, IH, IW, OH, OW, NC, _stream(labels))
+    return out
+
+
 # --------------------------------------------------------------------------- map generation
 # Factory functions (no tensor argument to dispatch on): plain Python, not registered operators.
 
@@ -458,6 +484,9 @@ _SCHEMAS = (
     ("resample_to_uv_maps",
      "(Tensor x, Tensor quad_idx, Tensor tex_uv, int num_textures, int tex_h, int tex_w,"
      " int interp) -> Tensor", resample_to_uv_maps),
+    ("voting_resample_to_map",
+     "(Tensor labels, Tensor sample_map, int out_h, int out_w, int num_candidates) -> Tensor",
+     voting_resample_to_map),
     ("mapped_im2col",
      "(Tensor x, Tensor sample_map, Tensor? interp_weights, int interp) -> Tensor",
      mapped_im2col),

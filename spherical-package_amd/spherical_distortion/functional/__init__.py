@@ -1,6 +1,6 @@
 from .mapped_ops import (mapped_convolution, mapped_transposed_convolution,  # noqa: F401
                          mapped_max_pool, mapped_avg_pool, mapped_avg_unpool, resample,
-                         unresample, uv_resample, MappedConvolutionFunction,
+                         unresample, uv_resample, voting_resample, MappedConvolutionFunction,
                          MappedTransposedConvolutionFunction, MappedMaxPoolFunction,
                          MappedAvgPoolFunction, MappedAvgUnpoolFunction, ResampleFunction,
                          UnresampleFunction, UVResampleFunction)

@@ -12,6 +12,7 @@ import _spherical_distortion_ext._mapped_max_pooling as _mapped_max_pool
 import _spherical_distortion_ext._mapped_transposed_convolution as _mapped_transposed_conv
 import _spherical_distortion_ext._resample as _resample
 import _spherical_distortion_ext._uv_resample as _uv_resample
+import _spherical_distortion_ext._voting_resample as _voting_resample
 import _spherical_distortion_ext._weighted_mapped_avg_pooling as _weighted_mapped_avg_pool
 import _spherical_distortion_ext._weighted_mapped_convolution as _weighted_mapped_conv
 import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mapped_max_pool
@@ -312,4 +313,17 @@ def uv_resample(input, quad_idx, tex_uv, interp):
     added = input.dim() == 4
     out = UVResampleFunction.apply(input.unsqueeze(0) if added else input, quad_idx, tex_uv,
                                    interp)
+    return out.squeeze(0) if added else out
+
+
+def voting_resample(input, sample_map, interp_weights, output_shape, num_candidates):
+    """Labels scattered through the map, every output pixel keeping the label with the most
+    votes; input and map are cast to int64 as the reference does, `interp_weights` is accepted
+    and unused as there (layers/functional/resample.py:160-189)."""
+    batched, added = _with_batch_dim(input)
+    check_input_map_shape(batched, sample_map)
+    out = _voting_resample.voting_resample_to_map(batched.long().contiguous(),
+                                                  sample_map.long().contiguous(),
+                                                  output_shape[0], output_shape[1],
+                                                  num_candidates)
     return out.squeeze(0) if added else out

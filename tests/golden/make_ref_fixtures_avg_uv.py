@@ -2,7 +2,7 @@
 extensions (compiled by `make -C oracle ref` from the reference sources) for mapped average
 pooling / unpooling (unweighted and weighted, all three interpolations, float32 and float64;
 the reference's tests hold one bilinear float64 vector) and for UV resampling in both
-directions (the reference's tests hold none).
+directions and for voting resample (the reference's tests hold none for either).
 
 Run in the build container only (it needs the compiled reference):
     python tests/golden/make_ref_fixtures_avg_uv.py
@@ -65,6 +65,16 @@ def main():
             U = R._uv_resample
             data[pre + "from_uv"] = U.resample_from_uv_maps(tex, quad, uv, it).numpy()
             data[pre + "to_uv"] = U.resample_to_uv_maps(x, quad, uv, NT, TH, TW, it).numpy()
+    # voting resample: integer labels through an integer map, targets partly outside the output,
+    # several sources per target so that ties and clear majorities both occur
+    gen = torch.Generator().manual_seed(77300)
+    NC, VH, VW = 5, 9, 11
+    labels = torch.randint(0, NC, (B, C, VH, VW), generator=gen, dtype=torch.int64)
+    vmap = torch.stack([torch.randint(-1, W + 1, (VH, VW), generator=gen, dtype=torch.int64),
+                        torch.randint(-1, H + 1, (VH, VW), generator=gen, dtype=torch.int64)], -1)
+    data["vote/in/labels"], data["vote/in/map"] = labels.numpy(), vmap.contiguous().numpy()
+    data["vote/out"] = R._voting_resample.voting_resample_to_map(
+        labels, vmap.contiguous(), H, W, NC).numpy()
     np.savez_compressed(OUT, **data)
     print("wrote", OUT, len(data), "arrays", os.path.getsize(OUT), "bytes")
 

@@ -201,3 +201,56 @@ def test_uv_errors(ops):
     # empty batch: nothing to do, nothing launched
     out = ops.resample_from_uv_maps(tex[:0], quad, uv, 1)
     assert out.shape == (0, 2, 6, 7)
+
+
+# ----------------------------------------------------------------------------- voting resample
+def test_voting_resample_is_bit_exact(ops, oracle):
+    """Integer work: bit-exact against the compiled reference's fixture (three channels, whose
+    histograms overlap in the reference; reproduced) and against the oracle on larger seeded
+    cases with targets outside the output and labels outside the range."""
+    fx = np.load(os.path.join(GOLDEN_DIR, "ref_fixtures_avg_uv.npz"))
+    labels, vmap, want = fx["vote/in/labels"], fx["vote/in/map"], fx["vote/out"]
+    got = ops.voting_resample_to_map(_t(labels), _t(vmap), want.shape[2], want.shape[3], 5)
+    assert got.dtype == torch.int64 and np.array_equal(_n(got), want)
+    for seed, (b, c, ih, iw, oh, ow, nc) in enumerate(((3, 1, 64, 96, 20, 30, 13),
+                                                       (2, 4, 33, 47, 31, 45, 3),
+                                                       (1, 1, 5, 700, 2, 3, 40),
+                                                       (2, 2, 17, 19, 40, 50, 1))):
+        rng = np.random.default_rng(60 + seed)
+        labels = rng.integers(-1, nc + 1, (b, c, ih, iw))
+        vmap = np.stack([rng.integers(-1, ow + 1, (ih, iw)),
+                         rng.integers(-1, oh + 1, (ih, iw))], -1)
+        got = _n(ops.voting_resample_to_map(_t(labels), _t(vmap), oh, ow, nc))
+        assert np.array_equal(got, oracle.voting_resample_to_map(labels, vmap, oh, ow, nc))
+
+
+def test_voting_resample_functional_and_errors(ops, oracle):
+    import spherical_distortion.functional as F
+    from _spherical_distortion_ext import _capi
+    rng = np.random.default_rng(77)
+    labels = rng.integers(0, 6, (1, 12, 20))                 # one image without batch axis
+    vmap = np.stack([rng.integers(0, 10, (12, 20)), rng.integers(0, 6, (12, 20))], -1)
+    got = F.voting_resample(_t(labels.astype(np.float32)), _t(vmap.astype(np.float32)), None,
+                            (6, 10), 6)
+    assert got.shape == (1, 6, 10)
+    assert np.array_equal(_n(got), oracle.voting_resample_to_map(labels[None], vmap, 6, 10, 6)[0])
+    with pytest.raises(RuntimeError, match="int64"):
+        ops.voting_resample_to_map(_t(labels[None]).int(), _t(vmap), 6, 10, 6)
+    with pytest.raises(RuntimeError, match="sample_map"):
+        ops.voting_resample_to_map(_t(labels[None]), _t(vmap[:5]), 6, 10, 6)
+    # a workspace of one histogram serves a batch in passes: same result as all at once
+    lab4 = rng.integers(0, 6, (4, 2, 12, 20))
+    t4 = _t(lab4)
+    nws = _capi.load().sdk_voting_resample_workspace_bytes(2, 6, 10, 6)
+    ws = torch.empty(nws, dtype=torch.uint8, device=DEV)
+    out4 = torch.empty((4, 2, 6, 10), dtype=torch.int64, device=DEV)
+    _capi.call("sdk_voting_resample_to_map", ops._ptr(t4), ops._ptr(_t(vmap)), ops._ptr(out4),
+               ops._ptr(ws), nws, 4, 2, 12, 20, 6, 10, 6, ops._stream(t4))
+    assert np.array_equal(_n(out4), oracle.voting_resample_to_map(lab4, vmap, 6, 10, 6))
+    assert torch.equal(out4, ops.voting_resample_to_map(t4, _t(vmap), 6, 10, 6))
+    # the histogram workspace is required
+    tl, tm = _t(labels[None]), _t(vmap)
+    out = torch.empty((1, 1, 6, 10), dtype=torch.int64, device=DEV)
+    with pytest.raises(RuntimeError, match="workspace"):
+        _capi.call("sdk_voting_resample_to_map", ops._ptr(tl), ops._ptr(tm), ops._ptr(out), None,
+                   0, 1, 1, 12, 20, 6, 10, 6, ops._stream(tl))

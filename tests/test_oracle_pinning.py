@@ -329,3 +329,28 @@ def test_uv_resampling_is_the_plain_gather_per_texture(oracle, interp):
     ok = ((bad >= 0) & (bad < nt)).astype(np.float64)
     assert relerr(oracle.resample_to_uv_maps(y, bad, uv, nt, th, tw, interp),
                   oracle.resample_to_uv_maps(y * ok, quad, uv, nt, th, tw, interp)) <= 1e-13
+
+
+# ----------------------------------------------------------------------------- voting resample
+def test_voting_resample_against_compiled_reference_and_brute_force(oracle, fx2):
+    labels, vmap, want = fx2["vote/in/labels"], fx2["vote/in/map"], fx2["vote/out"]
+    oh, ow = want.shape[2:]
+    assert np.array_equal(oracle.voting_resample_to_map(labels, vmap, oh, ow, 5), want)
+    # brute force with bincount on another seeded case: most frequent label, smallest on a tie,
+    # 0 where no source lands; targets outside the output and labels outside the range ignored.
+    # One channel: with more the reference's histograms overlap (fixture above: 3 channels).
+    rng = np.random.default_rng(8)
+    b, c, ih, iw, oh, ow, nc = 4, 1, 13, 17, 5, 6, 4
+    labels = rng.integers(-1, nc + 1, (b, c, ih, iw))
+    vmap = np.stack([rng.integers(-1, ow + 1, (ih, iw)), rng.integers(-1, oh + 1, (ih, iw))], -1)
+    got = oracle.voting_resample_to_map(labels, vmap, oh, ow, nc)
+    want = np.zeros((b, c, oh, ow), np.int64)
+    for bi in range(b):
+        for ci in range(c):
+            for y in range(oh):
+                for x in range(ow):
+                    src = labels[bi, ci][(vmap[..., 0] == x) & (vmap[..., 1] == y)]
+                    src = src[(src >= 0) & (src < nc)]
+                    if src.size:
+                        want[bi, ci, y, x] = np.bincount(src, minlength=nc).argmax()
+    assert np.array_equal(got, want)
