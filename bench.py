@@ -200,8 +200,10 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     vote_bytes = _nbytes(labels, vmap) + B * (H // 2) * (W // 2) * 8.0
     return {"voting_resample": dict(ms=ms_v, **_roof("hbm", vote_bytes, ms_v)),
             "map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
-            "uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf)),
-            "uv_scatter": dict(ms=ms_ub, **_roof("hbm", uv_bytes, ms_ub)),
+            "uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf,
+                                                traffic=_measured_traffic("resample_from_uv_maps"))),
+            "uv_scatter": dict(ms=ms_ub, **_roof("hbm", uv_bytes, ms_ub,
+                                                 traffic=_measured_traffic("resample_to_uv_maps"))),
             "gather": dict(ms=ms_g, **_roof("hbm", gather_bytes, ms_g,
                                             traffic=_measured_traffic("resample_from_map"))),
             "scatter_normalise": dict(ms=ms_s, **_roof("hbm", scatter_bytes, ms_s,
@@ -230,8 +232,10 @@ def bench_pool3(torch, ops, timer, steps, warmup):
                                                   traffic=_measured_traffic("mapped_max_pool"))),
             "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b,
                                                    traffic=_measured_traffic("mapped_max_unpool"))),
-            "avg_pool_forward": dict(ms=ms_af, **_roof("hbm", avg_bytes, ms_af)),
-            "avg_pool_backward": dict(ms=ms_ab, **_roof("hbm", avg_bytes, ms_ab)),
+            "avg_pool_forward": dict(ms=ms_af, **_roof("hbm", avg_bytes, ms_af,
+                                                       traffic=_measured_traffic("mapped_avg_pool"))),
+            "avg_pool_backward": dict(ms=ms_ab, **_roof("hbm", avg_bytes, ms_ab,
+                                                        traffic=_measured_traffic("mapped_avg_unpool"))),
             "no_winner_outputs": int((idx < 0).sum().item())}
 
 

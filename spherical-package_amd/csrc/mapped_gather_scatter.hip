@@ -170,11 +170,15 @@ constexpr int kInvSlots = 16;
 template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void resample_inverse_fill_kernel(
     const T* __restrict__ map, const T* __restrict__ wts, int H, int W, int MP, int P,
-    int* __restrict__ cnt, int* __restrict__ src, T* __restrict__ co, int* __restrict__ gate) {
+    int* __restrict__ cnt, int* __restrict__ src, T* __restrict__ co, int* __restrict__ gate,
+    int group) {
   const int pix = blockIdx.x * kBlock + threadIdx.x;
   if (pix >= MP) return;
   const int q = WEIGHTED ? P : 1;
   const size_t HW = (size_t)H * W;
+  // group > 1 (average unpooling): `group` consecutive map entries are the samples of one
+  // source pixel; the lists name that pixel
+  const int source = group > 1 ? pix / group : pix;
   PointTaps<T, INTERP> t;
   for (int p = 0; p < q; ++p) {
     const size_t s = (size_t)pix * q + p;
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_fill_kernel(
         const int u = t.off[i];
         const int slot = atomicAdd(&cnt[u], 1);
         if (slot < kInvSlots) {
-          src[(size_t)slot * HW + u] = pix;
+          src[(size_t)slot * HW + u] = source;
           co[(size_t)slot * HW + u] = INTERP == 0 ? wt : t.w[i] * wt;
         } else {
           atomicAdd(gate, 1);
@@ -213,16 +217,17 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
   for (int j = 0; j < PC; ++j) acc[j] = T(0);
   T wtot = T(0);
   for (int s = 0; s < n; ++s) {
-    int m = src[(size_t)s * HW + u];
-    if (group > 1) m /= group;   // map entry -> source pixel (average unpooling)
+    const int m = src[(size_t)s * HW + u];
     const T c = co[(size_t)s * HW + u];
     wtot += c;
 #pragma unroll
-    for (int j = 0; j < PC; ++j) {
-      T v = in[(size_t)(plane0 + (j < np ? j : 0)) * in_plane + m];
-      if (group > 1) v = v / T(group);
-      acc[j] += c * v;
-    }
+    for (int j = 0; j < PC; ++j)
+      acc[j] += c * in[(size_t)(plane0 + (j < np ? j : 0)) * in_plane + m];
+  }
+  // average unpooling hands every sample value / group: divided once here, after the sum
+  if (group > 1) {
+#pragma unroll
+    for (int j = 0; j < PC; ++j) acc[j] = acc[j] / T(group);
   }
   // normalised: the weight sum of the pixel is the sum of its list, no second pass needed
   const T den = wtot + eps;
@@ -911,7 +916,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
     SDK_DISPATCH_INTERP(interp, P,
                         (launch((resample_inverse_fill_kernel<T, INTERP, WEIGHTED>),
                                 dim3((unsigned)ceil_div(MP, kBlock)), dim3(kBlock), stream, map,
-                                wts, H, W, MP, P, cnt, src, co, g)));
+                                wts, H, W, MP, P, cnt, src, co, g, group)));
     SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
     if (planes > 0 || wsum) {
       const int pc = planes_per_thread(planes);
