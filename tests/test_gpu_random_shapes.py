@@ -161,3 +161,48 @@ def test_pooling_and_resampling(ops, oracle, seed):
     y = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
     back = _n(ops.resample_to_map(_t(y), _t(mr), _t(iwr), H, W, interp))
     assert relerr(back, oracle.resample_to_map(y, mr, H, W, interp, iwr)) <= BWD
+
+
+@pytest.mark.parametrize("seed", range(200, 224))
+def test_uv_resampling_voting_and_generated_maps(ops, oracle, seed):
+    """The entry points either side of the mapped operators on random geometries: UV gather
+    (nearest bit-exact) and its adjoint, the label vote (bit-exact), and a device-generated
+    kernel map used by a pooling call against the oracle's map and pooling."""
+    rng = np.random.default_rng(9000 + seed)
+    interp = int(rng.integers(0, 3))
+    B, C = int(rng.integers(1, 4)), int(rng.choice([1, 3, 8, 17, 40]))
+    NT = int(rng.choice([1, 2, 5, 20, 80, 300]))
+    TH, TW = int(rng.integers(1, 20)), int(rng.integers(2, 24))
+    H, W = int(rng.integers(1, 40)), int(rng.integers(2, 120))
+    tex = rng.standard_normal((B, C, NT, TH, TW)).astype(np.float32)
+    if rng.uniform() < 0.5:                          # coherent: runs of pixels on one texture
+        quad = np.repeat((np.arange(H) * 7 % NT)[:, None], W, 1).astype(np.int64)
+        uv = np.stack(np.broadcast_arrays(np.linspace(-1, TW, W)[None, :] * rng.uniform(0.2, 1),
+                                          (np.arange(H)[:, None] * 0.61) % (TH + 1) - 0.5), -1)
+    else:
+        quad = rng.integers(-1, NT + 1, (H, W)).astype(np.int64)
+        uv = np.stack([rng.uniform(-1.5, TW + 0.5, (H, W)), rng.uniform(-1.5, TH + 0.5, (H, W))], -1)
+    uv = np.ascontiguousarray(uv.astype(np.float32))
+    got = _n(ops.resample_from_uv_maps(_t(tex), _t(quad), _t(uv), interp))
+    want = oracle.resample_from_uv_maps(tex, quad, uv, interp)
+    assert np.array_equal(got, want) if interp == 0 else relerr(got, want) <= FWD
+    y = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    back = _n(ops.resample_to_uv_maps(_t(y), _t(quad), _t(uv), NT, TH, TW, interp))
+    assert relerr(back, oracle.resample_to_uv_maps(y, quad, uv, NT, TH, TW, interp)) <= BWD
+    # label vote through a random integer map
+    nc = int(rng.integers(1, 9))
+    oh, ow = int(rng.integers(1, 20)), int(rng.integers(1, 30))
+    labels = rng.integers(-1, nc + 1, (B, 1, H, W))
+    vmap = np.stack([rng.integers(-1, ow + 1, (H, W)), rng.integers(-1, oh + 1, (H, W))], -1)
+    assert np.array_equal(_n(ops.voting_resample_to_map(_t(labels), _t(vmap), oh, ow, nc)),
+                          oracle.voting_resample_to_map(labels, vmap, oh, ow, nc))
+    # a generated kernel map feeding average pooling (float64: both maps agree to rounding)
+    ih, iw_ = int(rng.integers(4, 30)), int(rng.integers(4, 50))
+    kh, kw = int(rng.choice([1, 3])), int(rng.choice([1, 3, 5]))
+    stride, proj = int(rng.integers(1, 4)), int(rng.integers(0, 3))
+    m = ops.equirect_kernel_map(ih, iw_, kh, kw, stride, 1, proj, torch.float64, DEV)
+    mo = oracle.equirect_kernel_map((ih, iw_), (kh, kw), stride, 1, proj, np.float64)
+    x = rng.standard_normal((B, 2, ih, iw_))
+    got = _n(ops.mapped_avg_pool(_t(x), m, None, kh * kw, 2))
+    want = oracle.mapped_avg_pool(x, mo, kh * kw, 2)
+    assert relerr(got, want) <= 1e-9
