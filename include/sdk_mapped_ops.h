@@ -127,6 +127,20 @@ int sdk_resample_to_map_normalized(const void* input, const void* sample_map,
 int sdk_normalize_by_weight_sum(void* data, const void* weight_sum, double eps, int64_t planes,
                                 int64_t plane_size, int32_t dtype, sdk_stream_t stream);
 
+/* The adjoint of sdk_mapped_max_unpool: out[b,c,oy,ox] = the image interpolated at the sample
+ * indices[b,c,oy,ox] names (0 for an index outside the map).  image [B,C,H,W]; indices, out
+ * [B,C,OH,OW].  This is the gradient of unpooling with respect to the pooled values, which a
+ * working `MappedMaxUnpool` layer needs; the reference's version of that layer
+ * (layers/functional/mapped_pooling.py:156-199, :235-242) refers to undefined names and cannot
+ * run, so this entry point has no reference kernel: it is the transpose of
+ * common/mapped_max_pool.h:60-78, :136-171. */
+int sdk_mapped_gather_at_index(const void* image, const int64_t* indices, const void* sample_map,
+                               const void* interp_weights, void* out, int64_t batch,
+                               int64_t channels, int64_t height, int64_t width,
+                               int64_t out_height, int64_t out_width, int64_t kernel_size,
+                               int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                               sdk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * UV resampling (tangent images back to one image).
  * textures [B,C,NT,TH,TW]; quad_idx [H,W] int64 names, per image pixel, one of the NT textures;

@@ -313,3 +313,17 @@ def voting_resample_to_map(labels, sample_map, out_h, out_w, num_candidates):
     _check(lib().sdk_oracle_voting_resample(_p(x), _p(m), _p(out),
                                             *_i64(B, C, IH, IW, out_h, out_w, num_candidates)))
     return out
+
+
+def mapped_gather_at_index(image, idx_mask, sample_map, interp, interp_weights=None):
+    """image [B,C,H,W], idx_mask [B,C,OH,OW] int64 -> [B,C,OH,OW]: the image interpolated at the
+    sample every index names; the transpose of mapped_max_unpool."""
+    x = _c(image); m = _c(sample_map, x.dtype); w = _c(interp_weights, x.dtype)
+    idx = _c(idx_mask, np.int64)
+    B, C, H, W = x.shape
+    OH, OW = idx.shape[2:]
+    out = np.empty((B, C, OH, OW), x.dtype)
+    _check(lib().sdk_oracle_mapped_gather_at_index(
+        _p(x), _p(idx), _p(m), _p(w), _p(out), *_i64(B, C, H, W, OH, OW),
+        *_i32(_num_pts(m, w), int(interp), _dt(x))))
+    return out

@@ -29,6 +29,8 @@
 //   sample-map generation: closed forms in pixel units (grid, inverse equirectangular), the
 //       forward gnomonic projection of every sample giving back its tangent-plane offset,
 //       centre sample = the pixel, stride = sub-sampling, float32 against float64.
+//   gather at index (gradient of unpooling): adjoint identity with the pinned unpool, and
+//       "pooling's value is the gather at pooling's own index".
 //   voting resample: compiled-reference fixtures + brute force with numpy's bincount.
 //   UV resampling: compiled-reference fixtures + "per texture it is the pinned gather" +
 //       adjoint identity (the reference's test-suite holds no vector for it).
@@ -478,6 +480,23 @@ void max_unpool(const T* gout, const int64_t* idx, const T* map, const T* wts, T
   }
 }
 
+// The transpose of max_unpool: every pooled element reads the image at the sample its index
+// names (0 for a negative index).  No reference counterpart: the reference's unpooling layer
+// (layers/functional/mapped_pooling.py:156-199) cannot run; this is what its backward has to be.
+template <typename T>
+void gather_at_index(const T* image, const int64_t* idx, const T* map, const T* wts, T* out,
+                     int64_t B, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int P,
+                     int interp) {
+  const int64_t M = OH * OW;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < B * C * M; ++i) {
+    const int64_t plane = i / M, s = idx[i];
+    out[i] = s < 0 ? T(0)
+                   : gather_sample(image + plane * H * W, map + s, wts ? wts + s / 2 : nullptr, P,
+                                   H, W, interp);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Mapped average pool and its adjoint.  common/mapped_avg_pool.h:13-40 (:70-105
 // weighted): the K samples are summed in ascending order and the sum is divided
@@ -703,6 +722,14 @@ int sdk_oracle_mapped_max_unpool(const void* gout, const int64_t* idx, const voi
                                  int interp, int dtype) {
   DISPATCH(dtype, max_unpool<T>((const T*)gout, idx, (const T*)map, (const T*)wts, (T*)gin, B,
                                  C, H, W, OH, OW, K, P, interp));
+}
+
+int sdk_oracle_mapped_gather_at_index(const void* image, const int64_t* idx, const void* map,
+                                      const void* wts, void* out, int64_t B, int64_t C, int64_t H,
+                                      int64_t W, int64_t OH, int64_t OW, int P, int interp,
+                                      int dtype) {
+  DISPATCH(dtype, gather_at_index<T>((const T*)image, idx, (const T*)map, (const T*)wts, (T*)out,
+                                      B, C, H, W, OH, OW, P, interp));
 }
 
 int sdk_oracle_mapped_avg_pool(const void* x, const void* map, const void* wts, void* out,

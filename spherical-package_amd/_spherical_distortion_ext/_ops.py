@@ -226,6 +226,26 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, i
     return gin
 
 
+def mapped_gather_at_index(x, idx_mask, sample_map, interp_weights, kernel_size, interp):
+    """The transpose of mapped_max_unpool: x [B,C,H,W] read at the sample every index names."""
+    _check(x, x=x, idx_mask=idx_mask, sample_map=sample_map, interp_weights=interp_weights)
+    if idx_mask.dtype != torch.int64 or idx_mask.dim() != 4 or \
+            tuple(idx_mask.shape[:2]) != tuple(x.shape[:2]):
+        raise RuntimeError("idx_mask must be an int64 [B, C, OH, OW] tensor with x's B and C")
+    P = _npts(sample_map, interp_weights, 4)
+    B, C, H, W = x.shape
+    OH, OW = idx_mask.shape[2:]
+    if tuple(sample_map.shape[:3]) != (OH, OW, int(kernel_size)):
+        raise RuntimeError("sample_map %s does not match idx_mask %s / kernel_size %d"
+                           % (tuple(sample_map.shape), tuple(idx_mask.shape), int(kernel_size)))
+    out = torch.empty((B, C, OH, OW), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.call("sdk_mapped_gather_at_index", _ptr(x), _ptr(idx_mask), _ptr(sample_map),
+                   _ptr(interp_weights), _ptr(out), B, C, H, W, OH, OW, int(kernel_size), P,
+                   int(interp), _DTYPES[x.dtype], _stream(x))
+    return out
+
+
 def mapped_avg_pool(x, sample_map, interp_weights, kernel_size, interp):
     _check(x, x=x, sample_map=sample_map, interp_weights=interp_weights)
     P = _npts(sample_map, interp_weights, 4)
@@ -499,6 +519,9 @@ _SCHEMAS = (
     ("mapped_max_unpool",
      "(Tensor grad_output, Tensor idx_mask, Tensor sample_map, Tensor? interp_weights, int in_h,"
      " int in_w, int kernel_size, int interp) -> Tensor", mapped_max_unpool),
+    ("mapped_gather_at_index",
+     "(Tensor x, Tensor idx_mask, Tensor sample_map, Tensor? interp_weights, int kernel_size,"
+     " int interp) -> Tensor", mapped_gather_at_index),
     ("mapped_avg_pool",
      "(Tensor x, Tensor sample_map, Tensor? interp_weights, int kernel_size, int interp)"
      " -> Tensor", mapped_avg_pool),

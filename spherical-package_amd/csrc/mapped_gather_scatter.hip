@@ -620,6 +620,30 @@ __global__ __launch_bounds__(kBlock) void mapped_max_unpool_kernel(
   }
 }
 
+// The adjoint of the unpool: every pooled element reads the image at the sample its index
+// names (same index convention, same range rule: an index outside the map reads nothing).
+// This is the gradient of unpooling with respect to the pooled values; the reference's own
+// attempt at it (layers/functional/mapped_pooling.py:156-199) refers to undefined names and
+// pools the gradient again instead, so there is no reference kernel to follow, only the
+// transpose of common/mapped_max_pool.h:60-78, :136-171.
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_gather_at_index_kernel(
+    const T* __restrict__ image, const int64_t* __restrict__ idx, const T* __restrict__ map,
+    const T* __restrict__ wts, T* __restrict__ out, size_t total, int H, int W, int M, int P,
+    int64_t map_elems) {
+  const int q = WEIGHTED ? P : 1;
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / (size_t)M;
+    const int64_t s = idx[i];
+    T v[1] = {T(0)};
+    if (s >= 0 && s + 2 * q <= map_elems)
+      gather_sample<T, INTERP, WEIGHTED, 1>(image + plane * (size_t)H * W, 0, 1, map + s,
+                                            WEIGHTED ? wts + s / 2 : nullptr, P, H, W, v);
+    out[i] = v[0];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Unpool by image tile.  A workgroup owns a tile of kUpTile image pixels and a group of
 // planes, accumulates the tile in LDS and writes every pixel of it exactly once with a
@@ -1503,6 +1527,34 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
                                 workspace_bytes, planes, (int)height, (int)width, (int)out_height,
                                 (int)out_width, (int)kernel_size, num_interp_pts, interp,
                                 (hipStream_t)stream));
+}
+
+int sdk_mapped_gather_at_index(const void* image, const int64_t* indices, const void* sample_map,
+                               const void* interp_weights, void* out, int64_t batch,
+                               int64_t channels, int64_t height, int64_t width,
+                               int64_t out_height, int64_t out_width, int64_t kernel_size,
+                               int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                               sdk_stream_t stream) {
+  SDK_REQUIRE(indices, "mapped_gather_at_index: NULL indices");
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_gather_at_index: bad pooled size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(image, sample_map, interp_weights, out, batch, channels, height, width, M,
+                        kernel_size, num_interp_pts, "mapped_gather_at_index");
+  if (rc) return rc;
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  const size_t total = (size_t)planes * M;
+  const int64_t map_elems = M * kernel_size * pts(num_interp_pts) * 2;
+  const int blocks = (int)std::min<int64_t>(ceil_div((int64_t)total, kBlock), 256 * 32);
+  SDK_DISPATCH_DTYPE(
+      dtype, SDK_DISPATCH_INTERP(
+                 interp, num_interp_pts,
+                 (launch((mapped_gather_at_index_kernel<T, INTERP, WEIGHTED>), dim3(blocks),
+                         dim3(kBlock), (hipStream_t)stream, (const T*)image, indices,
+                         (const T*)sample_map, (const T*)interp_weights, (T*)out, total,
+                         (int)height, (int)width, (int)M, num_interp_pts, map_elems))));
+  SDK_LAUNCH_CHECK("mapped_gather_at_index");
+  return SDK_OK;
 }
 
 }  // extern "C"

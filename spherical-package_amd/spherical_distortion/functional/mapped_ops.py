@@ -19,6 +19,8 @@ import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mappe
 import _spherical_distortion_ext._weighted_mapped_transposed_convolution as _weighted_mapped_transposed_conv
 import _spherical_distortion_ext._weighted_resample as _weighted_resample
 
+from _spherical_distortion_ext._ops import ops as _sdk_ops
+
 from ..layer_utils import InterpolationType, check_args, check_input_map_shape
 
 
@@ -114,6 +116,35 @@ class MappedMaxPoolFunction(torch.autograd.Function):
                 grad_output, idx_mask, sample_map, interp_weights, ctx.in_hw[0], ctx.in_hw[1],
                 ctx.kernel_size, ctx.interp)
         return grad_input, None, None, None, None
+
+
+class MappedMaxUnpoolFunction(torch.autograd.Function):
+    """Unpooling as a layer of its own: the pooled values go back to the samples `idx_mask`
+    names, on an output of the given size; the gradient reads `grad_output` at those samples.
+    The reference's class of this name (layers/functional/mapped_pooling.py:156-199) refers to
+    undefined variables and pools the gradient again; this is the working form of it, with the
+    output size as an explicit argument."""
+
+    @staticmethod
+    def forward(ctx, input, idx_mask, sample_map, output_height, output_width, kernel_size,
+                interp, interp_weights=None):
+        interp = InterpolationType(interp)
+        ctx.save_for_backward(idx_mask, sample_map, interp_weights)
+        ctx.kernel_size = int(kernel_size)
+        ctx.interp = interp
+        if interp_weights is None:
+            return _mapped_max_pool.mapped_max_unpool(input, idx_mask, sample_map, output_height,
+                                                      output_width, kernel_size, interp)
+        return _weighted_mapped_max_pool.weighted_mapped_max_unpool(
+            input, idx_mask, sample_map, interp_weights, output_height, output_width, kernel_size,
+            interp)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        idx_mask, sample_map, interp_weights = ctx.saved_tensors
+        grad = _sdk_ops.mapped_gather_at_index(grad_output.contiguous(), idx_mask, sample_map,
+                                               interp_weights, ctx.kernel_size, int(ctx.interp))
+        return grad, None, None, None, None, None, None, None
 
 
 def _avg_pool(input, sample_map, interp_weights, kernel_size, interp):
@@ -265,6 +296,17 @@ def mapped_max_pool(input, sample_map, kernel_size, interp, interp_weights=None)
     """-> (pooled, idx_mask); layers/functional/mapped_pooling.py:225-232."""
     check_args(input, sample_map, interp_weights, None, kernel_size)
     return MappedMaxPoolFunction.apply(input, sample_map, kernel_size, interp, interp_weights)
+
+
+def mapped_max_unpool(input, idx_mask, sample_map, output_shape, kernel_size, interp,
+                      interp_weights=None):
+    """Pooled values back onto an `output_shape` = (H, W) image at the samples `idx_mask` names
+    (the reference's function of this name, layers/functional/mapped_pooling.py:235-242, calls
+    the pooling function with these arguments and cannot run)."""
+    check_args(input, sample_map, interp_weights, None, kernel_size)
+    check_input_map_shape(input, sample_map)
+    return MappedMaxUnpoolFunction.apply(input, idx_mask, sample_map, output_shape[0],
+                                         output_shape[1], kernel_size, interp, interp_weights)
 
 
 def mapped_avg_pool(input, sample_map, kernel_size, interp, interp_weights=None):

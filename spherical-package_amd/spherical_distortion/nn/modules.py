@@ -92,6 +92,21 @@ class MappedMaxPool(nn.Module):
         return (pooled, idx_mask) if self.return_indices else pooled
 
 
+class MappedMaxUnpool(nn.Module):
+    """Pooled values back to the samples that won (mapped_max_pooling_layer.py:35-47, whose
+    functional backend cannot run in the reference; `output_shape` = (H, W) of the unpooled
+    image is an added argument)."""
+
+    def __init__(self, kernel_size, interpolation=InterpolationType.BILINEAR):
+        super().__init__()
+        self.kernel_size = kernel_size
+        self.interp = interpolation
+
+    def forward(self, x, idx_mask, sample_map, output_shape, interp_weights=None):
+        return F.mapped_max_unpool(x, idx_mask, sample_map, output_shape, self.kernel_size,
+                                   self.interp, interp_weights)
+
+
 class MappedAvgPool(nn.Module):
     """(mapped_avg_pooling_layer.py:7-19)."""
 

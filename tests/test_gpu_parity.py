@@ -606,3 +606,47 @@ def test_errors_are_raised_not_fatal(ops):
     # unknown interpolation values fall back to nearest like the reference's switch default
     a = ops.resample_from_map(x + 1, m, None, 7)
     assert torch.equal(a, ops.resample_from_map(x + 1, m, None, 0))
+
+
+# ------------------------------------------------------------------------------------------
+# Unpooling as a layer: forward = the unpool entry point, backward = the gather at the index.
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("case", CASES, ids=_ids)
+def test_gather_at_index_and_unpool_layer(ops, oracle, case):
+    import spherical_distortion.functional as F
+    from spherical_distortion.nn import MappedMaxUnpool
+    interp, weighted, dt = case
+    rng = np.random.default_rng(800 + interp)
+    B, C, H, W, OH, OW, K, P = 2, 5, 23, 31, 11, 13, 5, 2
+    x = rng.standard_normal((B, C, H, W)).astype(dt)
+    m = _coords(rng, (OH, OW, K, P) if weighted else (OH, OW, K), H, W, dt, margin=0.0)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if weighted else None
+    val, idx = ops.mapped_max_pool(_t(x), _t(m), _t(iw), K, interp)
+    # the pooled value is the image read at the winning sample (same arithmetic: bit-exact)
+    got = ops.mapped_gather_at_index(_t(x), idx, _t(m), _t(iw), K, interp)
+    ok = _n(idx) >= 0
+    assert np.array_equal(_n(got)[ok], _n(val)[ok])
+    assert (_n(got)[~ok] == 0).all()
+    # arbitrary indices, some of them outside the map, against the oracle
+    q = P if weighted else 1
+    any_idx = (rng.integers(0, K, (B, C, OH, OW)) + np.arange(OH * OW).reshape(OH, OW) * K) * q * 2
+    any_idx[0, 0, 0, :3] = -1
+    got = _n(ops.mapped_gather_at_index(_t(x), _t(any_idx), _t(m), _t(iw), K, interp))
+    want = oracle.mapped_gather_at_index(x, any_idx, m, interp, iw)
+    assert np.array_equal(got, want) or relerr(got, want) <= FWD_TOL[dt]
+    # the layer: forward is the unpool, backward the gather
+    pooled = torch.from_numpy(rng.standard_normal((B, C, OH, OW)).astype(dt)).to(DEV)
+    pooled.requires_grad_(True)
+    safe = np.where(any_idx < 0, 0, any_idx)
+    layer = MappedMaxUnpool(K, interp)
+    up = layer(pooled, _t(safe), _t(m), (H, W), _t(iw))
+    want_up = oracle.mapped_max_unpool(_n(pooled), safe, m, H, W, K, interp, iw)
+    assert relerr(_n(up), want_up) <= BWD_TOL[dt]
+    up.backward(_t(x))
+    want_grad = oracle.mapped_gather_at_index(x, safe, m, interp, iw)
+    assert relerr(_n(pooled.grad), want_grad) <= FWD_TOL[dt]
+    if dt == np.float64 and interp == 1 and not weighted:
+        probe = torch.from_numpy(rng.standard_normal((1, 2, OH, OW))).to(DEV).requires_grad_(True)
+        assert torch.autograd.gradcheck(
+            lambda t: F.mapped_max_unpool(t, _t(safe[:1, :2]), _t(m), (H, W), K, interp), (probe,),
+            eps=1e-6, atol=1e-7, nondet_tol=1e-9)

@@ -354,3 +354,32 @@ def test_voting_resample_against_compiled_reference_and_brute_force(oracle, fx2)
                     if src.size:
                         want[bi, ci, y, x] = np.bincount(src, minlength=nc).argmax()
     assert np.array_equal(got, want)
+
+
+# ----------------------------------------------------------------------------- gather at index
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_gather_at_index_is_the_transpose_of_the_pinned_unpool(oracle, interp, weighted):
+    """<unpool(g), x> = <g, gather_at_index(x)> for any index tensor, and the gather at
+    pooling's own indices returns pooling's values (bit-exact): the pooled value IS the image
+    read at the winning sample."""
+    rng = np.random.default_rng(90 + interp)
+    b, c, h, w, oh, ow, k, p = 2, 3, 9, 11, 5, 7, 4, 2
+    x = rng.standard_normal((b, c, h, w))
+    shape = (oh, ow, k, p) if weighted else (oh, ow, k)
+    m = np.stack([rng.uniform(0, w - 1, shape), rng.uniform(0, h - 1, shape)], -1)
+    iw = rng.uniform(0.1, 1, shape) if weighted else None
+    val, idx = oracle.mapped_max_pool(x, m, k, interp, iw)
+    assert (idx >= 0).all()
+    assert np.array_equal(oracle.mapped_gather_at_index(x, idx, m, interp, iw), val)
+    q = p if weighted else 1
+    any_idx = (rng.integers(0, k, (b, c, oh, ow)) +
+               np.arange(oh * ow).reshape(oh, ow) * k) * q * 2
+    any_idx[0, 0, 0, :3] = -1
+    g = rng.standard_normal((b, c, oh, ow))
+    g_masked = np.where(any_idx < 0, 0.0, g)
+    lhs = oracle.mapped_max_unpool(g_masked, np.where(any_idx < 0, 0, any_idx), m, h, w, k,
+                                   interp, iw)
+    rhs = oracle.mapped_gather_at_index(x, any_idx, m, interp, iw)
+    assert (rhs[0, 0, 0, :3] == 0).all()
+    assert abs((lhs * x).sum() - (g * rhs).sum()) <= 1e-10 * np.abs(g * rhs).sum()
