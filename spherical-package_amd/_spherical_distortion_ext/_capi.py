@@ -10,7 +10,7 @@ _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG_ROOT, "libsdk_mapped_ops.so")
 
 SDK_F32, SDK_F64 = 0, 1
-SDK_COMPUTE_NATIVE, SDK_COMPUTE_BF16, SDK_COMPUTE_UNFUSED = 0, 1, 2
+SDK_COMPUTE_NATIVE, SDK_COMPUTE_BF16, SDK_COMPUTE_UNFUSED, SDK_COMPUTE_SPLIT = 0, 1, 2, 3
 
 _vp, _i64, _i32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
 

@@ -17,7 +17,8 @@ _NS = "sdk_mapped_ops"
 _DTYPES = {torch.float32: _capi.SDK_F32, torch.float64: _capi.SDK_F64}
 
 # Arithmetic of the dense contraction inside the convolution operators: "native"
-# (the tensors' type), "bf16" (bf16 operands, fp32 accumulate) or "unfused"
+# (the tensors' type), "bf16" (bf16 operands, fp32 accumulate), "split" (fp32 operands as
+# three bf16 pieces each: fp32 accuracy from the bf16 matrix unit) or "unfused"
 # (separate im2col/col2im + GEMM kernels, the cross-check path).
 _compute_mode = _capi.SDK_COMPUTE_NATIVE
 
@@ -26,15 +27,16 @@ def set_conv_compute(mode):
     """Selects the GEMM arithmetic of the mapped (transposed) convolutions."""
     global _compute_mode
     modes = {"native": _capi.SDK_COMPUTE_NATIVE, "fp32": _capi.SDK_COMPUTE_NATIVE,
-             "bf16": _capi.SDK_COMPUTE_BF16, "unfused": _capi.SDK_COMPUTE_UNFUSED}
+             "bf16": _capi.SDK_COMPUTE_BF16, "unfused": _capi.SDK_COMPUTE_UNFUSED,
+             "split": _capi.SDK_COMPUTE_SPLIT}
     if mode not in modes:
         raise ValueError("compute mode must be one of %s" % sorted(modes))
     _compute_mode = modes[mode]
 
 
 def get_conv_compute():
-    return {_capi.SDK_COMPUTE_BF16: "bf16", _capi.SDK_COMPUTE_UNFUSED: "unfused"}.get(
-        _compute_mode, "native")
+    return {_capi.SDK_COMPUTE_BF16: "bf16", _capi.SDK_COMPUTE_UNFUSED: "unfused",
+            _capi.SDK_COMPUTE_SPLIT: "split"}.get(_compute_mode, "native")
 
 
 # --------------------------------------------------------------------------- checks

@@ -29,7 +29,7 @@ int check_common(const char* what, int64_t B, int64_t Cg, int64_t H, int64_t W, 
   SDK_REQUIRE(P >= 0 && (P == 0 || wts), "%s: weighted map needs interp_weights", what);
   SDK_REQUIRE(dtype == SDK_F32 || dtype == SDK_F64, "%s: unknown dtype %d", what, dtype);
   SDK_REQUIRE(compute == SDK_COMPUTE_NATIVE || compute == SDK_COMPUTE_BF16 ||
-                  compute == SDK_COMPUTE_UNFUSED,
+                  compute == SDK_COMPUTE_UNFUSED || compute == SDK_COMPUTE_SPLIT,
               "%s: unknown compute mode %d", what, compute);
   if (compute == SDK_COMPUTE_BF16 && dtype != SDK_F32)
     return fail(SDK_ERR_UNSUPPORTED, "%s: bf16 compute needs float32 tensors", what);

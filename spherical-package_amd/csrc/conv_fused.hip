@@ -166,7 +166,7 @@ __device__ __forceinline__ void mfma_chunk_any(const float* __restrict__ As, int
 // instructions of mfma_chunk().
 constexpr int kLdK = kKC + 4;
 
-template <bool BF16>
+template <int MM>
 __device__ __forceinline__ void mfma_chunk_kc(const float* __restrict__ At, int a_base,
                                               const float* __restrict__ Bt, int b_base,
                                               floatx16 (&acc)[2][2]) {
@@ -176,21 +176,36 @@ __device__ __forceinline__ void mfma_chunk_kc(const float* __restrict__ At, int 
   const float* a1p = a0p + 32 * kLdK;
   const float* b0p = Bt + (b_base + lj) * kLdK;
   const float* b1p = b0p + 32 * kLdK;
-  if constexpr (BF16) {
+  if constexpr (MM != kMmF32) {
 #pragma unroll
     for (int t = 0; t < kKC / 16; ++t) {
       const int o = 16 * t + 8 * lk;
-      auto frag = [&](const float* p) {
+      auto read8 = [&](const float* p, float (&f)[8]) {
         const float4 lo = *reinterpret_cast<const float4*>(p + o);
         const float4 hi = *reinterpret_cast<const float4*>(p + o + 4);
-        const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        return pack_bf16x8(f);
+        f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+        f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
       };
-      const Bf16Frag a0 = frag(a0p), a1 = frag(a1p), b0 = frag(b0p), b1 = frag(b1p);
-      acc[0][0] = mfma_bf16(a0, b0, acc[0][0]);
-      acc[0][1] = mfma_bf16(a0, b1, acc[0][1]);
-      acc[1][0] = mfma_bf16(a1, b0, acc[1][0]);
-      acc[1][1] = mfma_bf16(a1, b1, acc[1][1]);
+      float fa0[8], fa1[8], fb0[8], fb1[8];
+      read8(a0p, fa0);
+      read8(a1p, fa1);
+      read8(b0p, fb0);
+      read8(b1p, fb1);
+      if constexpr (MM == kMmBf16) {
+        const Bf16Frag a0 = pack_bf16x8(fa0), a1 = pack_bf16x8(fa1);
+        const Bf16Frag b0 = pack_bf16x8(fb0), b1 = pack_bf16x8(fb1);
+        acc[0][0] = mfma_bf16(a0, b0, acc[0][0]);
+        acc[0][1] = mfma_bf16(a0, b1, acc[0][1]);
+        acc[1][0] = mfma_bf16(a1, b0, acc[1][0]);
+        acc[1][1] = mfma_bf16(a1, b1, acc[1][1]);
+      } else {
+        const Bf16Split a0 = split_bf16x8(fa0), a1 = split_bf16x8(fa1);
+        const Bf16Split b0 = split_bf16x8(fb0), b1 = split_bf16x8(fb1);
+        acc[0][0] = mfma_split(a0, b0, acc[0][0]);
+        acc[0][1] = mfma_split(a0, b1, acc[0][1]);
+        acc[1][0] = mfma_split(a1, b0, acc[1][0]);
+        acc[1][1] = mfma_split(a1, b1, acc[1][1]);
+      }
     }
   } else {
 #pragma unroll
@@ -273,7 +288,7 @@ __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
 // (conv_inverse.hip): rows inv_off / inv_co [(pixel tile * K + k) * slots + s][TM] and
 // their count inv_ns[pixel tile * K + k].  The kernel does nothing unless *gate == 0.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int TN, int TM, bool BF16, bool INV = false>
+template <int INTERP, bool WEIGHTED, int TN, int TM, int MM, bool INV = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wg, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
@@ -363,7 +378,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
         *reinterpret_cast<float4*>(As + n * kLdK + 4 * r4) = src[e];
       }
       __syncthreads();
-      mfma_chunk_kc<BF16>(As, a_base, Bs, b_base, acc);
+      mfma_chunk_kc<MM>(As, a_base, Bs, b_base, acc);
       __syncthreads();
     }
   }
@@ -632,7 +647,7 @@ static int launch_smem(const char* what, Kern kern, dim3 grid, size_t smem, hipS
 int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
                       const float* wts, const float* Wm, const float* bias, float* pix,
                       float* workspace, hipStream_t stream) {
-  const bool bf16 = compute == SDK_COMPUTE_BF16;
+  const int mm = matrix_mode(compute);
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -651,8 +666,9 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                                         CpP, slots, m_tiles, (const int*)nullptr,             \
                                         (const float*)nullptr, (const int*)nullptr,           \
                                         (const int*)nullptr)))
-  if (bf16) { if (narrow) GG(64, 256, true); else GG(128, 128, true); }
-  else { if (narrow) GG(64, 256, false); else GG(128, 128, false); }
+  if (mm == kMmBf16) { if (narrow) GG(64, 256, kMmBf16); else GG(128, 128, kMmBf16); }
+  else if (mm == kMmSplit) { if (narrow) GG(64, 256, kMmSplit); else GG(128, 128, kMmSplit); }
+  else { if (narrow) GG(64, 256, kMmF32); else GG(128, 128, kMmF32); }
 #undef GG
   return rc;
 }
@@ -789,7 +805,7 @@ static int build_inverse(const ConvGeom& g, const float* map, const float* wts, 
 }
 
 // img[b] = Ws^T x gather(pix[b]) + bias over the inverse map; does nothing if *inv.gate != 0.
-static int inverse_gather_gemm(const ConvGeom& g, bool bf16, const InverseMap& inv,
+static int inverse_gather_gemm(const ConvGeom& g, int mm, const InverseMap& inv,
                                const float* pix, const float* Wm, const float* bias, float* img,
                                hipStream_t stream) {
   // roles in the gather kernel: gathered tensor = pix (Cp channels, planes of M elements),
@@ -809,8 +825,9 @@ static int inverse_gather_gemm(const ConvGeom& g, bool bf16, const InverseMap& i
                    (const float*)inv.weights, bias, img, g.Cp, 1, g.M, g.Cg, HW, g.K, 0, CinP,   \
                    CoutP, kInvSlots, m_tiles, (const int*)inv.off, (const float*)inv.co,         \
                    (const int*)inv.ns, (const int*)inv.gate)
-  if (bf16) { if (narrow) IG(64, 256, true); else IG(128, 128, true); }
-  else { if (narrow) IG(64, 256, false); else IG(128, 128, false); }
+  if (mm == kMmBf16) { if (narrow) IG(64, 256, kMmBf16); else IG(128, 128, kMmBf16); }
+  else if (mm == kMmSplit) { if (narrow) IG(64, 256, kMmSplit); else IG(128, 128, kMmSplit); }
+  else { if (narrow) IG(64, 256, kMmF32); else IG(128, 128, kMmF32); }
 #undef IG
   return rc;
 }
@@ -831,7 +848,7 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
       InverseMap inv;
       rc = build_inverse(g, map, wts, inv_ws, stream, &inv);
       if (rc) return rc;
-      rc = inverse_gather_gemm(g, bf16, inv, pix, Wm, bias, img, stream);
+      rc = inverse_gather_gemm(g, matrix_mode(compute), inv, pix, Wm, bias, img, stream);
       if (rc) return rc;
       gate = inv.gate;
     }
@@ -872,11 +889,11 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   if (g.B == 0) return SDK_OK;
   if (planned_wgrad_supported(g)) {
     if (shared != nullptr && shared->valid)
-      return planned_wgrad(g, bf16, shared->plan, pix, img, gW, stream);
+      return planned_wgrad(g, matrix_mode(compute), shared->plan, pix, img, gW, stream);
     Plan plan;
     rc = build_plan(g, map, wts, workspace, stream, &plan);
     if (rc) return rc;
-    return planned_wgrad(g, bf16, plan, pix, img, gW, stream);
+    return planned_wgrad(g, matrix_mode(compute), plan, pix, img, gW, stream);
   }
   constexpr int KM = 64;
   const int slots = slots_for(g);

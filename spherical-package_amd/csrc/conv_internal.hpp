@@ -5,7 +5,15 @@
 
 #include <cstdint>
 
+#include "sdk_mapped_ops.h"
+#include "sdk_mfma.hpp"
+
 namespace sdk {
+
+// sdk_compute -> matrix arithmetic of the fused kernels that know all three kinds.
+inline int matrix_mode(int compute) {
+  return compute == SDK_COMPUTE_BF16 ? kMmBf16 : (compute == SDK_COMPUTE_SPLIT ? kMmSplit : kMmF32);
+}
 
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream);
 // gate: optional device flag; with one, the fill runs only if *gate != 0.

@@ -198,12 +198,14 @@ __device__ __forceinline__ void lds_only_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int KB, bool BF16, int NW>
+template <int KB, int MM, int NW>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW, int Cg,
     int H, int W, int Cp, int K, int S, PixelTiling pt, int tiles,
     int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
+  constexpr bool BF16 = MM != kMmF32;     // operands enter the matrix unit as bf16 fragments
+  constexpr bool SPLIT = MM == kMmSplit;  // ... three per operand, whose sum is the float
   __shared__ __align__(16) float region[kRegionCap * kRegE];
   __shared__ __align__(16) float colT[2][kCC * kColLd];
   __shared__ __align__(16) int2 prow[kRowCap * 64];
@@ -307,7 +309,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     for (int half = 0; half < 2; ++half) {
       // ---- A fragments of this lane's row n for the 64 pixels of the half
       float afrag[BF16 ? 1 : PXW / 2];
-      Bf16Frag afrag16[BF16 ? PXW / 16 : 1];
+      Bf16Frag afrag16[(BF16 && !SPLIT) ? PXW / 16 : 1];
+      Bf16Split afrag3[SPLIT ? PXW / 16 : 1];
       {
         constexpr int GROUPS = BF16 ? PXW / 16 : PXW / 8;   // groups of pixels per lane half ...
         constexpr int RUN = BF16 ? 8 : 4;                   // ... of which this lane holds RUN
@@ -333,7 +336,9 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
               f[u] = (n_ok && mi >= 0) ? pix_row[mi] : 0.0f;
             }
           }
-          if constexpr (BF16) {
+          if constexpr (SPLIT) {
+            afrag3[g] = split_bf16x8(reinterpret_cast<const float(&)[8]>(f));
+          } else if constexpr (BF16) {
             afrag16[g] = pack_bf16x8(reinterpret_cast<const float(&)[8]>(f));
           } else {
 #pragma unroll
@@ -364,8 +369,9 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
         // Image values of the next sample's first row, for lanes whose tap lies outside the
         // window: requested one sample ahead so that they arrive during the MFMAs (maps without
         // locality, e.g. mesh neighbourhoods, have all their taps there).
-        // (The variant with nine fp32 accumulators of 128 rows has no registers left for it.)
-        constexpr bool PRE = !(KB == 9 && NW == 4 && !BF16);
+        // (The variants with nine accumulators of 128 rows and fp32 or split A fragments have no
+        // registers left for it.)
+        constexpr bool PRE = !(KB == 9 && NW == 4 && MM != kMmBf16);
         float pre[8];
         bool pre_valid = false;
 #pragma unroll
@@ -469,7 +475,10 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
                 const float4 lo = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h) ^ sw));
                 const float4 hi = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h + 4) ^ sw));
                 const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-                d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
+                if constexpr (SPLIT)
+                  d = mfma_split(afrag3[t], split_bf16x8(f), d);
+                else
+                  d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
               }
             } else {
               float4 b = *reinterpret_cast<const float4*>(bt + ((poff + 4 * h) ^ sw));
@@ -576,7 +585,7 @@ bool planned_wgrad_supported(const ConvGeom& g) {
   return plan_supported(g) && plan_slots(g) <= kRowCap && g.B <= 65535;
 }
 
-int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* pix,
+int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                   const float* img, float* gW, hipStream_t stream) {
   const int kblocks = (int)ceil_div(g.K, 9);
   const int per = (int)ceil_div(g.K, kblocks);
@@ -593,7 +602,7 @@ int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* p
   const int64_t slots = ceil_div(groups, 8) * 8 * kinds;
   if (slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "planned_wgrad: grid too large");
   const int TX = plan.pt.TX();
-  const int vec4 = (g.OW % 4 == 0 && TX >= (bf16 ? 8 : 4) &&
+  const int vec4 = (g.OW % 4 == 0 && TX >= (mm != kMmF32 ? 8 : 4) &&
                     reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)slots);
 #define PW3(KBv, BFv, NWv)                                                                      \
@@ -604,10 +613,12 @@ int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* p
   do {                                                                                          \
     if (NW == 4) PW3(KBv, BFv, 4); else if (NW == 2) PW3(KBv, BFv, 2); else PW3(KBv, BFv, 1);   \
   } while (0)
-  if (bf16) {
-    if (KB == 1) PW(1, true); else if (KB == 4) PW(4, true); else if (KB == 7) PW(7, true); else PW(9, true);
+  if (mm == kMmBf16) {
+    if (KB == 1) PW(1, kMmBf16); else if (KB == 4) PW(4, kMmBf16); else if (KB == 7) PW(7, kMmBf16); else PW(9, kMmBf16);
+  } else if (mm == kMmSplit) {
+    if (KB == 1) PW(1, kMmSplit); else if (KB == 4) PW(4, kMmSplit); else if (KB == 7) PW(7, kMmSplit); else PW(9, kMmSplit);
   } else {
-    if (KB == 1) PW(1, false); else if (KB == 4) PW(4, false); else if (KB == 7) PW(7, false); else PW(9, false);
+    if (KB == 1) PW(1, kMmF32); else if (KB == 4) PW(4, kMmF32); else if (KB == 7) PW(7, kMmF32); else PW(9, kMmF32);
   }
 #undef PW
 #undef PW3

@@ -43,7 +43,7 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
 
 // gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
 bool planned_wgrad_supported(const ConvGeom& g);
-int planned_wgrad(const ConvGeom& g, bool bf16, const Plan& plan, const float* pix,
+int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                   const float* img, float* gW, hipStream_t stream);
 
 }  // namespace sdk

@@ -33,8 +33,51 @@ __device__ __forceinline__ Bf16Frag pack_bf16x8(const float (&f)[8]) {
   return r;
 }
 
+// Eight floats as three bf16 fragments whose sum is the float exactly: hi = the top 8 mantissa
+// bits (truncated), mid = the top 8 bits of the remainder, lo = the rest.  Each remainder is
+// exact in fp32 (it has at most 16, then 8, significant bits), so a product of two floats is
+// the sum of nine piece products, each exact in the matrix unit's fp32 accumulator.
+struct Bf16Split {
+  Bf16Frag hi, mid, lo;
+};
+
+__device__ __forceinline__ Bf16Split split_bf16x8(const float (&f)[8]) {
+  unsigned h[8], m[8], l[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    h[i] = __float_as_uint(f[i]) & 0xffff0000u;
+    const float r = f[i] - __uint_as_float(h[i]);
+    m[i] = __float_as_uint(r) & 0xffff0000u;
+    const float r2 = r - __uint_as_float(m[i]);
+    l[i] = __float_as_uint(r2) & 0xffff0000u;
+  }
+  Bf16Split s;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    s.hi.u[i] = (h[2 * i] >> 16) | h[2 * i + 1];
+    s.mid.u[i] = (m[2 * i] >> 16) | m[2 * i + 1];
+    s.lo.u[i] = (l[2 * i] >> 16) | l[2 * i + 1];
+  }
+  return s;
+}
+
 __device__ __forceinline__ floatx16 mfma_bf16(const Bf16Frag& a, const Bf16Frag& b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
 }
+
+// c += a * b from the six largest of the nine piece products (smallest first); the three left
+// out (mid*lo, lo*mid, lo*lo) are below 2^-23 of the product.
+__device__ __forceinline__ floatx16 mfma_split(const Bf16Split& a, const Bf16Split& b, floatx16 c) {
+  c = mfma_bf16(a.lo, b.hi, c);
+  c = mfma_bf16(a.hi, b.lo, c);
+  c = mfma_bf16(a.mid, b.mid, c);
+  c = mfma_bf16(a.mid, b.hi, c);
+  c = mfma_bf16(a.hi, b.mid, c);
+  return mfma_bf16(a.hi, b.hi, c);
+}
+
+// Matrix arithmetic of a fused kernel: fp32 MFMA, operands rounded to bf16, or fp32 operands
+// split into bf16 pieces (fp32 accuracy on the bf16 matrix unit).
+constexpr int kMmF32 = 0, kMmBf16 = 1, kMmSplit = 2;
 
 }  // namespace sdk

@@ -540,6 +540,76 @@ def test_bf16_compute_within_1e_2(ops, oracle, bf16_compute, tc):
                                                              iw)) <= 1e-2
 
 
+@pytest.fixture
+def split_compute(ops):
+    ops.set_conv_compute("split")
+    yield
+    ops.set_conv_compute("native")
+
+
+@pytest.mark.parametrize("tc", TILE_CASES + PLAN_CASES[:8], ids=lambda t: "x".join(map(str, t)))
+def test_split_compute_keeps_float32_accuracy(ops, oracle, split_compute, tc):
+    """float32 operands split into three bf16 pieces each (six piece products, fp32
+    accumulation): the float32 tolerances of the native mode, 1e-5 forward and 1e-4 backward,
+    on random maps (tile edges) and on coherent maps (plan-driven kernels)."""
+    Cin, Cout, H, W, OH, OW, K, P, interp = tc[:9]
+    dt = np.float32
+    rng = np.random.default_rng(17 + sum(tc[:9]))
+    B = 2
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    if len(tc) > 9:
+        m = _coherent_map(rng, OH, OW, K, P, H, W, dt, tc[9])
+    else:
+        m = _coords(rng, (OH, OW, K, P) if P else (OH, OW, K), H, W, dt)
+    iw = rng.uniform(0.1, 1, (OH, OW, K, P)).astype(dt) if P else None
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(wt), _t(b), K, interp))
+    assert relerr(got, oracle.mapped_conv_forward(x, m, wt, b, K, interp, iw)) <= 1e-5
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(wt), _t(b), K, interp)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, interp, iw)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    assert relerr(_n(gb), wb) <= 1e-4
+    xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+    wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+    bt = rng.standard_normal(Cin).astype(dt)
+    got = _n(ops.mapped_transposed_conv_forward(_t(xt), _t(m), _t(iw), _t(wtt), _t(bt), H, W, K,
+                                                interp))
+    want = oracle.mapped_transposed_conv_forward(xt, m, wtt, bt, H, W, K, interp, iw)
+    assert relerr(got, want) <= 1e-4
+
+
+def test_split_compute_on_values_that_stress_the_pieces(ops, oracle, split_compute):
+    """Operands whose low mantissa bits matter: large offsets plus small signals, powers of two,
+    denormal-range and huge magnitudes; and float64 tensors, which run as in the native mode."""
+    dt = np.float32
+    rng = np.random.default_rng(4242)
+    B, Cin, Cout, H, W, K = 2, 32, 32, 16, 32, 9
+    m = _coords(rng, (H, W, K), H, W, dt)
+    x = (1000.0 + rng.standard_normal((B, Cin, H, W)) * 1e-3).astype(dt)
+    x[0, 0] = 2.0 ** rng.integers(-20, 20, (H, W))
+    x[0, 1] *= 1e30
+    x[0, 2] *= 1e-30
+    wt = (1.0 + rng.standard_normal((Cout, Cin, K)) * 1e-4).astype(dt)
+    wt[0] = 2.0 ** -10
+    b = np.zeros(Cout, dt)
+    got = _n(ops.mapped_conv_forward(_t(x), _t(m), None, _t(wt), _t(b), K, 1))
+    want = oracle.mapped_conv_forward(x.astype(np.float64), m.astype(np.float64),
+                                      wt.astype(np.float64), b.astype(np.float64), K, 1)
+    ops.set_conv_compute("native")
+    native = _n(ops.mapped_conv_forward(_t(x), _t(m), None, _t(wt), _t(b), K, 1))
+    ops.set_conv_compute("split")
+    # no worse than twice the native mode's distance from the float64 result
+    assert relerr(got, want) <= max(2 * relerr(native, want), 1e-6)
+    x64 = rng.standard_normal((1, 3, 8, 9))
+    m64 = _coords(rng, (5, 6, 4), 8, 9, np.float64)
+    w64, b64 = rng.standard_normal((2, 3, 4)), rng.standard_normal(2)
+    got = _n(ops.mapped_conv_forward(_t(x64), _t(m64), None, _t(w64), _t(b64), 4, 1))
+    assert relerr(got, oracle.mapped_conv_forward(x64, m64, w64, b64, 4, 1)) <= 1e-12
+
+
 # ------------------------------------------------------------------------------------------
 # Against the compiled reference's fixtures directly (no oracle in between).
 # ------------------------------------------------------------------------------------------

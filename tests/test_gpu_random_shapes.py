@@ -108,6 +108,23 @@ def test_convolution_bf16_operands(ops, oracle, seed):
     assert relerr(gi, wi) <= 1e-2 and relerr(gw, ww) <= 1e-2 and _bias_grad_ok(gb, wb, g)
 
 
+@pytest.mark.parametrize("seed", range(300, 324))
+def test_convolution_split_operands(ops, oracle, seed):
+    """The split compute mode (float32 operands as three bf16 pieces, fp32 accumulation) on the
+    same sweep, at the float32 tolerances."""
+    rng, interp, K, H, W, OH, OW, B, Cin, Cout, m, iw, x, w, b, g = _conv_case(seed)
+    ops.set_conv_compute("split")
+    try:
+        y = _n(ops.mapped_conv_forward(_t(x), _t(m), _t(iw), _t(w), _t(b), K, interp))
+        gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), _t(iw), _t(x), _t(w), _t(b), K, interp)
+        gi, gw, gb = _n(gi), _n(gw), _n(gb)
+    finally:
+        ops.set_conv_compute("native")
+    assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= FWD
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
+    assert relerr(gi, wi) <= BWD and relerr(gw, ww) <= BWD and _bias_grad_ok(gb, wb, g)
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_convolution_and_transposed(ops, oracle, seed):
     rng, interp, K, H, W, OH, OW, B, Cin, Cout, m, iw, x, w, b, g = _conv_case(seed)
