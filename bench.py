@@ -385,6 +385,14 @@ def main():
                     roofline=roof)
     else:
         line.update(value=None, ms_per_step=None, roofline=None)
+    if "conv4_split" in kernels:
+        # the same step with float32 results formed on the bf16 matrix unit (operands split
+        # exactly into three bf16 pieces, fp32 accumulation, accuracy of the native mode);
+        # `value` above stays on the native fp32 arithmetic
+        line["split_compute"] = {"value": round(kernels["conv4_split"]["images_per_s"], 3),
+                                 "unit": "images/s",
+                                 "ms_per_step": round(kernels["conv4_split"]["ms_per_step"], 4),
+                                 "dtype": "f32 operands as 3 bf16 pieces, 6 products, f32 accumulate"}
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     line["kernels"] = kernels
     print(json.dumps(line))
