@@ -93,9 +93,10 @@ def _to_uv_capi(ops, y, quad, uv, NT, TH, TW, interp, with_workspace):
 
 # B, C, NT, TH, TW, H, W: ragged sizes; many textures and planes (several planes per workgroup);
 # one row of pixels and wide textures; two textures only (several workgroups share a texture);
-# textures that do not fit in on-chip memory (the workspace query answers 0)
+# textures that do not fit in on-chip memory (the workspace query answers 0); textures that just fit
 UV_SHAPES = ((2, 3, 7, 9, 13, 31, 45), (1, 12, 20, 16, 16, 64, 96), (3, 35, 4, 5, 300, 17, 260),
-             (2, 40, 300, 6, 5, 40, 70), (1, 3, 2, 12, 10, 50, 130), (1, 2, 3, 130, 140, 33, 47))
+             (2, 40, 300, 6, 5, 40, 70), (1, 3, 2, 12, 10, 50, 130), (1, 2, 3, 130, 140, 33, 47),
+             (1, 2, 3, 128, 128, 45, 100))      # float32 textures of exactly 64 KiB
 UV_CASES = [(interp, dt, shape) for interp in (0, 1, 2) for dt in (np.float32, np.float64)
             for shape in UV_SHAPES]
 
