@@ -268,6 +268,17 @@ def bench_ico5(torch, ops, timer, steps, warmup):
                                                              peak=MFMA_FP32_TFLOPS))}
 
 
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.lower().startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(budget_s=12.0):
     """Times the CPU checker on a bounded sample of configuration 4 and reports images per
     second: whole batch-1 images (forward + backward) repeated for about `budget_s` seconds
@@ -299,7 +310,7 @@ def cpu_baseline(budget_s=12.0):
             reps += 1
         dt = time.time() - t0
         return {"value": round(reps / dt, 4), "unit": "images/s",
-                "cores": int(torch.get_num_threads()), "kind": "reference",
+                "cores": int(torch.get_num_threads()), "cpu": _cpu_model(), "kind": "reference",
                 "sample": "configuration 4 at batch 1 (one 128x256x512 image, fwd+bwd), %d "
                           "repetitions in %.1f s after one warm-up" % (reps, dt)}
     rows = 64
@@ -311,7 +322,7 @@ def cpu_baseline(budget_s=12.0):
     orc.mapped_conv_backward(g, m, cfg["x"], cfg["weight"], cfg["bias"], K, 2, iw)
     dt = time.time() - t0
     return {"value": round(rows / float(H) / dt, 4), "unit": "images/s",
-            "cores": int(orc.num_threads()), "kind": "port",
+            "cores": int(orc.num_threads()), "cpu": _cpu_model(), "kind": "port",
             "sample": "configuration 4, batch 1, output rows 0..%d of %d (%.1f s of CPU work), "
                       "fwd+bwd, scaled by the pixel share" % (rows - 1, H, dt)}
 
