@@ -547,7 +547,7 @@ def split_compute(ops):
     ops.set_conv_compute("native")
 
 
-@pytest.mark.parametrize("tc", TILE_CASES + PLAN_CASES[:8], ids=lambda t: "x".join(map(str, t)))
+@pytest.mark.parametrize("tc", TILE_CASES + PLAN_CASES, ids=lambda t: "x".join(map(str, t)))
 def test_split_compute_keeps_float32_accuracy(ops, oracle, split_compute, tc):
     """float32 operands split into three bf16 pieces each (six piece products, fp32
     accumulation): the float32 tolerances of the native mode, 1e-5 forward and 1e-4 backward,
