@@ -184,6 +184,7 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
 constexpr int kColLd = 68;            // column tile row stride (floats): 16-byte rows, 4-bank skew
 constexpr int kRegE = 36;             // window element stride (floats): 32 channels + 4 of skew
 constexpr int kRowCap = 36;           // plan rows of one half held in LDS at a time
+constexpr int kSplitLd = 72;          // row stride (bf16 elements) of the split column tiles: 16-byte rows
 
 // Window layout: region[e * kRegE + c], channels fastest.  A lane reads or writes the 8
 // channels of its group for one element as two 16-byte accesses; 8 lanes on consecutive
@@ -460,8 +461,29 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
             }
           }
           float* ct = colT[buf];
+          if constexpr (SPLIT) {
+            // The column tile is split where it is written, once, instead of by each of the four
+            // waves that read it: three bf16 tiles piece[c][m] (rows of kSplitLd elements, pixel
+            // bits 4-5 flipped by the channel group to spread the groups over the banks), in
+            // the space of one fp32 tile, so the tile is single-buffered here.
+            unsigned short* pt = reinterpret_cast<unsigned short*>(&colT[0][0]);
+            const int ms = m_local ^ (cg << 4);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) ct[(8 * cg + j) * kColLd + (m_local ^ ((cg & 1) << 4))] = col[j];
+            for (int j = 0; j < 8; ++j) {
+              const unsigned hb = __float_as_uint(col[j]) & 0xffff0000u;
+              const float r = col[j] - __uint_as_float(hb);
+              const unsigned mb = __float_as_uint(r) & 0xffff0000u;
+              const float r2 = r - __uint_as_float(mb);
+              const unsigned lb = __float_as_uint(r2) & 0xffff0000u;
+              const int at = (8 * cg + j) * kSplitLd + ms;
+              pt[at] = (unsigned short)(hb >> 16);
+              pt[kCC * kSplitLd + at] = (unsigned short)(mb >> 16);
+              pt[2 * kCC * kSplitLd + at] = (unsigned short)(lb >> 16);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ct[(8 * cg + j) * kColLd + (m_local ^ ((cg & 1) << 4))] = col[j];
+          }
           lds_only_barrier();   // the requests above stay in flight
 
           // ---- D[n][c] += A[n][m] * col[c][m]; one copy of this block per accumulator
@@ -469,16 +491,25 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
           const float* bt = ct + nl * kColLd;
           const int sw = ((nl >> 3) & 1) << 4;
           auto mma = [&](floatx16& d) {
-            if constexpr (BF16) {
+            if constexpr (SPLIT) {
+              const unsigned short* pt = reinterpret_cast<const unsigned short*>(&colT[0][0]);
+              const int sws = ((nl >> 3) & 3) << 4;
+#pragma unroll
+              for (int t = 0; t < PXW / 16; ++t) {
+                const int at = nl * kSplitLd + ((poff + 16 * t + 8 * h) ^ sws);
+                Bf16Split b;
+                b.hi.v = *reinterpret_cast<const bf16x8*>(pt + at);
+                b.mid.v = *reinterpret_cast<const bf16x8*>(pt + kCC * kSplitLd + at);
+                b.lo.v = *reinterpret_cast<const bf16x8*>(pt + 2 * kCC * kSplitLd + at);
+                d = mfma_split(afrag3[t], b, d);
+              }
+            } else if constexpr (BF16) {
 #pragma unroll
               for (int t = 0; t < PXW / 16; ++t) {
                 const float4 lo = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h) ^ sw));
                 const float4 hi = *reinterpret_cast<const float4*>(bt + ((poff + 16 * t + 8 * h + 4) ^ sw));
                 const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-                if constexpr (SPLIT)
-                  d = mfma_split(afrag3[t], split_bf16x8(f), d);
-                else
-                  d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
+                d = mfma_bf16(afrag16[t], pack_bf16x8(f), d);
               }
             } else {
               float4 b = *reinterpret_cast<const float4*>(bt + ((poff + 4 * h) ^ sw));
@@ -498,7 +529,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 #pragma unroll
           for (int u = 0; u < KB; ++u)
             if (u == kk) mma(acc[u]);
-          buf ^= 1;
+          if constexpr (SPLIT) lds_only_barrier();   // single tile: all reads before the next writes
+          else buf ^= 1;
         }
         kk_beg = kk_end;
       }
