@@ -261,7 +261,21 @@ def bench_ico5(torch, ops, timer, steps, warmup):
         t["x_coarse"], t["up_map"], None, t["up_weight"], t["up_bias"], oh, ow, K, 0), steps,
         warmup)
     tflops = 2.0 * C * C * K * Vc * B
-    return {"icosphere_conv_fwd_bwd": dict(ms=ms_c, images_per_s=B / (ms_c * 1e-3),
+    # the same two workloads in the split compute mode (float32 results, bf16 matrix unit)
+    ops.set_conv_compute("split")
+    try:
+        ms_cs, _ = timer.run(conv_step, steps, warmup)
+        ms_ts, _ = timer.run(lambda: ops.mapped_transposed_conv_forward(
+            t["x_coarse"], t["up_map"], None, t["up_weight"], t["up_bias"], oh, ow, K, 0), steps,
+            warmup)
+    finally:
+        ops.set_conv_compute("native")
+    return {"icosphere_conv_fwd_bwd_split": dict(ms=ms_cs, images_per_s=B / (ms_cs * 1e-3),
+                                                 **_roof("mfma", 3 * flops, ms_cs,
+                                                         peak=MFMA_FP32_TFLOPS)),
+            "transposed_conv_forward_split": dict(ms=ms_ts, **_roof("mfma", tflops, ms_ts,
+                                                                    peak=MFMA_FP32_TFLOPS)),
+            "icosphere_conv_fwd_bwd": dict(ms=ms_c, images_per_s=B / (ms_c * 1e-3),
                                            **_roof("mfma", 3 * flops, ms_c,
                                                    peak=MFMA_FP32_TFLOPS)),
             "transposed_conv_forward": dict(ms=ms_t, **_roof("mfma", tflops, ms_t,
