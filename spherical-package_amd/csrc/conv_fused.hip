@@ -362,7 +362,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const float d = *reinterpret_cast<const float*>(base + ((unsigned)off[u] * 4u + cj));
-            col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
+            col[j] = __builtin_fmaf(co[u], co[u] != 0.0f ? d : 0.0f, col[j]);
           }
         }
       }
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const float d = *reinterpret_cast<const float*>(base + ((unsigned)off[u] * 4u + cj));
-          col[j] += co[u] * (co[u] != 0.0f ? d : 0.0f);
+          col[j] = __builtin_fmaf(co[u], co[u] != 0.0f ? d : 0.0f, col[j]);
         }
       }
     }

@@ -400,7 +400,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
               const bool g_ok = out && c0 + 8 * cg + j < Cg;
               const float dg =
                   *reinterpret_cast<const float*>(gbase + (g_ok ? o0 + (unsigned)j * plane : 0u));
-              col[j] += co * (e >= 0 ? dl[j] : (g_ok ? dg : 0.0f));
+              col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? dg : 0.0f), col[j]);
             }
           };
           int r_first = 0;
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const bool g_ok = out && c0 + 8 * cg + j < Cg;
-              col[j] += co * (e >= 0 ? dl[j] : (g_ok ? pre[j] : 0.0f));
+              col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? pre[j] : 0.0f), col[j]);
             }
             r_first = 1;
           }
@@ -434,8 +434,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
               const float d1[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
               for (int j = 0; j < 8; ++j) {
-                col[j] += co0 * d0[j];
-                col[j] += co1 * d1[j];
+                col[j] = __builtin_fmaf(co0, d0[j], col[j]);
+                col[j] = __builtin_fmaf(co1, d1[j], col[j]);
               }
             } else {
               tap_any(ec0.x, co0);
