@@ -128,3 +128,61 @@ def test_workload_generators_shapes():
     nb = ring[0, :, 1:, 0].astype(int)
     assert all(v_ in nb[n] for v_ in range(40) for n in nb[v_])  # neighbourhood is symmetric
     assert wl.tangent_patch_map(64, 128, 1, 8).shape == (80, 64, 2)
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_device():
+    """Argument checks come first in every entry point: status and message, no launch, so they
+    can be exercised without a GPU."""
+    from _spherical_distortion_ext import _capi
+    lib = _capi.load()
+    lib.sdk_last_error.restype = ctypes.c_char_p
+    one = ctypes.c_void_p(16)   # a non-NULL pointer that is never dereferenced
+
+    def rc(name, *args):
+        return getattr(lib, name)(*args)
+
+    def err():
+        return lib.sdk_last_error().decode()
+
+    # UV resampling: NULL pointers, no textures, empty planes
+    assert rc("sdk_resample_from_uv_maps", None, one, one, one, 1, 1, 3, 4, 5, 6, 7, 1, 0, None) == -1
+    assert "NULL" in err()
+    assert rc("sdk_resample_from_uv_maps", one, one, one, one, 1, 1, 0, 4, 5, 6, 7, 1, 0, None) == -1
+    assert "num_textures" in err()
+    assert rc("sdk_resample_to_uv_maps", one, one, one, one, None, 0, 1, 1, 3, 0, 5, 6, 7, 1, 0,
+              None) == -1
+    assert rc("sdk_resample_to_uv_maps", one, one, one, one, None, 0, -1, 1, 3, 4, 5, 6, 7, 1, 0,
+              None) == -1
+    # an empty batch is a valid no-op, pointers or not
+    assert rc("sdk_resample_from_uv_maps", None, None, None, None, 0, 4, 3, 4, 5, 6, 7, 1, 0,
+              None) == 0
+    assert lib.sdk_resample_to_uv_maps_workspace_bytes(80, 64, 64, 512, 1024, 0) > 512 * 1024 * 4
+    assert lib.sdk_resample_to_uv_maps_workspace_bytes(3, 130, 140, 33, 47, 0) == 0   # too large for LDS
+    assert lib.sdk_resample_to_uv_maps_workspace_bytes(0, 4, 4, 8, 8, 0) == 0
+    # voting resample: the workspace is required
+    assert rc("sdk_voting_resample_to_map", one, one, one, None, 0, 1, 1, 4, 5, 2, 3, 6, None) == -3
+    assert "workspace" in err()
+    assert rc("sdk_voting_resample_to_map", one, one, one, one, 1 << 20, 1, 1, 4, 5, 2, 3, 0,
+              None) == -1
+    assert lib.sdk_voting_resample_workspace_bytes(1, 2, 3, 6) >= 1 * 2 * 3 * 6 * 4
+    # map generation
+    assert rc("sdk_equirect_kernel_map", one, 1, 64, 3, 3, 1, 1, 1, 0, None) == -1
+    assert "height" in err()
+    assert rc("sdk_equirect_kernel_map", one, 32, 64, 3, 3, 0, 1, 1, 0, None) == -1
+    assert rc("sdk_equirect_kernel_map", one, 32, 64, 3, 3, 1, 1, 7, 0, None) == -1
+    assert "projection" in err()
+    assert rc("sdk_equirect_kernel_map", None, 32, 64, 3, 3, 1, 1, 1, 0, None) == -1
+    assert rc("sdk_gnomonic_kernel_at", None, None, 0, 3, 3, 0.1, 0.1, 0, 0, 0, None) == 0
+    assert rc("sdk_gnomonic_kernel_at", one, one, 5, 0, 3, 0.1, 0.1, 0, 0, 0, None) == -1
+    assert rc("sdk_gnomonic_kernel_at", one, one, 5, 3, 3, 0.1, 0.1, 1, 8, 0, None) == -1
+    # gather at index and average pooling share the mapped-operator checks
+    assert rc("sdk_mapped_gather_at_index", one, None, one, None, one, 1, 1, 4, 5, 2, 3, 9, 0, 1, 0,
+              None) == -1
+    assert rc("sdk_mapped_avg_pool", one, one, None, one, 1, 1, 4, 5, 2, 3, 9, 2, 1, 0, None) == -1
+    assert "interp_weights" in err()
+    # unknown compute mode of a convolution call
+    assert rc("sdk_mapped_conv_forward", one, one, None, one, one, one, None, 0, 1, 3, 8, 8, 4, 8, 8,
+              9, 0, 1, 0, 9, None) == -1
+    assert "compute" in err()
+    assert lib.sdk_mapped_conv_workspace_bytes(1, 3, 4, 8, 8, 8, 8, 9, 0, 1, 0, 3) == \
+        lib.sdk_mapped_conv_workspace_bytes(1, 3, 4, 8, 8, 8, 8, 9, 0, 1, 0, 0)
