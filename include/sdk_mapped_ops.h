@@ -241,6 +241,16 @@ int sdk_gnomonic_kernel_at(const void* lonlat, void* out, int64_t num_points, in
                            int64_t kernel_w, double res_lat, double res_lon, int64_t image_height,
                            int64_t image_width, int32_t dtype, sdk_stream_t stream);
 
+/* From a map of single points to the weighted (P = 4) form: out_map [num_samples, 4, 2] = the four
+ * pixel centres around each sample of sample_map [num_samples, 2] (integer coordinates, column
+ * wrapped, row clamped to the image), out_weights [num_samples, 4] proportional to
+ * 1 / (great-circle distance + eps), normalised to sum to one.  The benchmark's large weighted
+ * convolution is defined on such a map; the reference has no builder for it (its weighted maps
+ * come from mesh code), so the kernel follows the definition, not a reference routine. */
+int sdk_four_nearest_weighted_map(const void* sample_map, void* out_map, void* out_weights,
+                                  int64_t num_samples, int64_t height, int64_t width, double eps,
+                                  int32_t dtype, sdk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mapped im2col / col2im (batched).
  * col[b, c*K + k, pix] with pix = y_out*OW + x_out, out_pixels = OH*OW.

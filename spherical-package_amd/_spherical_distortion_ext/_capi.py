@@ -28,6 +28,7 @@ SIGNATURES = {
     "sdk_gnomonic_kernel_at": [_vp, _vp] + [_i64] * 3 + [ctypes.c_double] * 2 + [_i64] * 2
                               + [_i32, _vp],
     "sdk_voting_resample_to_map": [_vp] * 4 + [_sz] + [_i64] * 7 + [_vp],
+    "sdk_four_nearest_weighted_map": [_vp] * 3 + [_i64] * 3 + [ctypes.c_double, _i32, _vp],
     "sdk_mapped_im2col": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_pool": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],

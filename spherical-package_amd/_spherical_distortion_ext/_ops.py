@@ -489,6 +489,26 @@ def gnomonic_kernel_at(lonlat, kernel_h, kernel_w, res_lat, res_lon, image_h=0, 
     return out
 
 
+def four_nearest_weighted_map(sample_map, height, width, eps=1e-6):
+    """sample_map [..., 2] -> (map [..., 4, 2], weights [..., 4]): the four pixel centres around
+    every sample (column wrapped, row clamped) with normalised inverse great-circle distance
+    weights, the weighted form a bispherical P = 4 convolution takes."""
+    _check(sample_map, sample_map=sample_map)
+    if sample_map.shape[-1] != 2:
+        raise RuntimeError("sample_map must end in 2, got %s" % (tuple(sample_map.shape),))
+    lead = tuple(sample_map.shape[:-1])
+    n = 1
+    for v in lead:
+        n *= int(v)
+    out_map = torch.empty(lead + (4, 2), dtype=sample_map.dtype, device=sample_map.device)
+    out_w = torch.empty(lead + (4,), dtype=sample_map.dtype, device=sample_map.device)
+    with torch.cuda.device(sample_map.device):
+        _capi.call("sdk_four_nearest_weighted_map", _ptr(sample_map), _ptr(out_map), _ptr(out_w),
+                   n, int(height), int(width), float(eps), _DTYPES[sample_map.dtype],
+                   _stream(sample_map))
+    return out_map, out_w
+
+
 # --------------------------------------------------------------------------- registration
 _SCHEMAS = (
     ("resample_from_map",

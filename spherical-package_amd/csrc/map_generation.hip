@@ -137,6 +137,48 @@ __global__ __launch_bounds__(kMapBlock) void gnomonic_kernel_at_kernel(
   out[idx * 2 + 1] = img_h > 0 ? lat_to_y(olat, img_h) : olat;
 }
 
+// The four pixel centres around every sample and weights proportional to the inverse
+// great-circle distance to them, normalised to sum to one: the weighted (P = 4) form of a map
+// for an equirectangular image (columns wrap, rows clamp).  The distance comes from the
+// haversine form, 2 asin sqrt(sin^2(dlat / 2) + cos lat0 cos lat1 sin^2(dlon / 2)), with the
+// angle differences taken from the coordinate differences and cos(lat) as sin(pi y / (H - 1)):
+// exactly 0 for a sample on a pixel centre and for any two points of a pole row, and relative
+// accuracy for neighbours a pixel apart, where the arccosine of a dot product would keep half
+// its digits in float32 (the weights 1 / (d + eps) are sensitive to d at the scale of eps).
+__device__ __forceinline__ float m_sinpi(float v) { return sinpif(v); }
+__device__ __forceinline__ double m_sinpi(double v) { return sinpi(v); }
+
+template <typename T>
+__global__ __launch_bounds__(kMapBlock) void four_nearest_weighted_kernel(
+    const T* __restrict__ map, T* __restrict__ out_map, T* __restrict__ out_w, size_t count, int H,
+    int W, T eps) {
+  const size_t i = (size_t)blockIdx.x * kMapBlock + threadIdx.x;
+  if (i >= count) return;
+  const T x = map[i * 2], y = map[i * 2 + 1];
+  const T x1 = floor(x);
+  T y1 = floor(y);
+  y1 = y1 < T(0) ? T(0) : (y1 > T(H - 1) ? T(H - 1) : y1);
+  const T y2 = y1 + T(1) > T(H - 1) ? T(H - 1) : y1 + T(1);
+  const T xs[4] = {x1, x1 + T(1), x1, x1 + T(1)};
+  const T ys[4] = {y1, y1, y2, y2};
+  const T c0 = m_sinpi(y / T(H - 1));
+  T w[4], total = T(0);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const T sa = m_sinpi(T(0.5) * (y - ys[k]) / T(H - 1));
+    const T so = m_sinpi((x - xs[k]) / T(W));
+    T hav = sa * sa + c0 * m_sinpi(ys[k] / T(H - 1)) * so * so;
+    hav = hav < T(0) ? T(0) : (hav > T(1) ? T(1) : hav);
+    const T d = T(2) * m_asin(m_sqrt(hav));
+    w[k] = T(1) / (d + eps);
+    total += w[k];
+    out_map[(i * 4 + k) * 2] = floor_mod(xs[k], T(W));
+    out_map[(i * 4 + k) * 2 + 1] = ys[k];
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) out_w[i * 4 + k] = w[k] / total;
+}
+
 }  // namespace sdk
 
 using namespace sdk;
@@ -199,6 +241,27 @@ int sdk_gnomonic_kernel_at(const void* lonlat, void* out, int64_t num_points, in
                                     (int)kernel_h, (int)kernel_w, res_lat, res_lon,
                                     (int)image_height, (int)image_width)));
   SDK_LAUNCH_CHECK("gnomonic_kernel_at");
+  return SDK_OK;
+}
+
+int sdk_four_nearest_weighted_map(const void* sample_map, void* out_map, void* out_weights,
+                                  int64_t num_samples, int64_t height, int64_t width, double eps,
+                                  int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(num_samples >= 0, "four_nearest_weighted_map: negative size");
+  SDK_REQUIRE(height >= 2 && width >= 1 && height < ((int64_t)1 << 24) &&
+                  width < ((int64_t)1 << 24),
+              "four_nearest_weighted_map: image %lld x %lld", (long long)height, (long long)width);
+  SDK_REQUIRE(eps > 0.0, "four_nearest_weighted_map: eps must be positive");
+  if (num_samples == 0) return SDK_OK;
+  SDK_REQUIRE(sample_map && out_map && out_weights, "four_nearest_weighted_map: NULL pointer");
+  SDK_REQUIRE(ceil_div(num_samples, kMapBlock) < ((int64_t)1 << 31),
+              "four_nearest_weighted_map: too many samples");
+  const dim3 grid((unsigned)ceil_div(num_samples, kMapBlock));
+  SDK_DISPATCH_DTYPE(dtype, (launch(four_nearest_weighted_kernel<T>, grid, dim3(kMapBlock),
+                                    (hipStream_t)stream, (const T*)sample_map, (T*)out_map,
+                                    (T*)out_weights, (size_t)num_samples, (int)height, (int)width,
+                                    (T)eps)));
+  SDK_LAUNCH_CHECK("four_nearest_weighted_map");
   return SDK_OK;
 }
 

@@ -62,3 +62,12 @@ def gnomonic_kernel_pixels(spherical_coords, kh, kw, res_lat, res_lon, image_sha
     (layers/util/tangent_images.py:59-109)."""
     pts = spherical_coords.reshape(-1, 2).contiguous()
     return _ops.gnomonic_kernel_at(pts, kh, kw, res_lat, res_lon, image_shape[0], image_shape[1])
+
+
+def four_nearest_weighted(sample_map, image_shape, eps=1e-6):
+    """(map [..., 4, 2], weights [..., 4]) from a map of single points [..., 2]: the four pixel
+    centres around every sample of an equirectangular image (columns wrap, rows clamp) and
+    weights proportional to 1 / (great-circle distance + eps), normalised to one.  No
+    counterpart in the reference, whose weighted maps come from its mesh code."""
+    return _ops.four_nearest_weighted_map(sample_map.contiguous(), image_shape[0], image_shape[1],
+                                          eps)

@@ -132,3 +132,47 @@ def test_python_builders_and_errors(ops):
         ops.equirect_kernel_map(32, 64, 3, 3, projection=5)
     with pytest.raises(RuntimeError, match="lonlat"):
         ops.gnomonic_kernel_at(torch.zeros(4, 3, device=DEV), 3, 3, 0.1, 0.1)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_four_nearest_weighted_map_against_its_definition(ops, dtype):
+    """The weighted (P = 4) form of a map: integer neighbours bit for bit, weights against the
+    float64 arccosine form of the same definition.  A sample that coincides with a pixel centre
+    has distance 0 there, where arccos(1 - 1e-16) = 1.5e-8 against eps = 1e-6 moves the other
+    three weights (~1e-4 each) in the sixth digit: hence 5e-6 for float64; float32 coordinates
+    carry ~1e-7 rad of their own, 5e-5."""
+    import workloads as wl
+    H, W = 24, 48
+    base = wl.gnomonic_kernel_map(H, W, dtype=np.float64)
+    rng = np.random.default_rng(5)
+    extra = np.stack([rng.uniform(-3, W + 3, (H, W, 9)), rng.uniform(-2, H + 1, (H, W, 9))], -1)
+    for m in (base, extra):
+        m = m.astype(dtype)
+        want_m, want_w = wl.four_nearest_weighted(m, H, W, dtype=np.float64)
+        got_m, got_w = ops.four_nearest_weighted_map(torch.from_numpy(m).to(DEV), H, W)
+        assert got_m.shape == m.shape[:-1] + (4, 2) and got_w.shape == m.shape[:-1] + (4,)
+        assert np.array_equal(got_m.cpu().numpy().astype(np.float64), want_m)
+        tol = 5e-6 if dtype == np.float64 else 5e-5
+        assert np.abs(got_w.cpu().numpy() - want_w).max() < tol
+        assert np.abs(got_w.sum(-1).cpu().numpy() - 1).max() < 1e-6
+    empty = torch.empty(0, 2, device=DEV, dtype=TORCH[dtype])
+    assert ops.four_nearest_weighted_map(empty, H, W)[1].shape == (0, 4)
+
+
+def test_four_nearest_weighted_map_feeds_the_weighted_convolution(ops):
+    """The util front-end end to end: map built on the device, then the weighted convolution on
+    it equals the one on the host-built map."""
+    import workloads as wl
+    from spherical_distortion.util import four_nearest_weighted
+    H, W, C = 16, 32, 4
+    base = wl.gnomonic_kernel_map(H, W, dtype=np.float32)
+    hm, hw = wl.four_nearest_weighted(base, H, W)
+    dm, dw = four_nearest_weighted(torch.from_numpy(base).to(DEV), (H, W))
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, C, H, W, generator=g).to(DEV)
+    wt = torch.randn(C, C, 9, generator=g).to(DEV)
+    b = torch.zeros(C, device=DEV)
+    a = ops.mapped_conv_forward(x, dm, dw, wt, b, 9, 2)
+    r = ops.mapped_conv_forward(x, torch.from_numpy(hm).to(DEV), torch.from_numpy(hw).to(DEV),
+                                wt, b, 9, 2)
+    assert (a - r).abs().max().item() < 1e-3 * r.abs().max().item()

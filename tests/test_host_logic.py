@@ -173,6 +173,10 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert "projection" in err()
     assert rc("sdk_equirect_kernel_map", None, 32, 64, 3, 3, 1, 1, 1, 0, None) == -1
     assert rc("sdk_gnomonic_kernel_at", None, None, 0, 3, 3, 0.1, 0.1, 0, 0, 0, None) == 0
+    assert rc("sdk_four_nearest_weighted_map", None, None, None, 0, 8, 8, 1e-6, 0, None) == 0
+    assert rc("sdk_four_nearest_weighted_map", one, one, one, 4, 1, 8, 1e-6, 0, None) == -1
+    assert rc("sdk_four_nearest_weighted_map", one, one, one, 4, 8, 8, 0.0, 0, None) == -1
+    assert rc("sdk_four_nearest_weighted_map", None, one, one, 4, 8, 8, 1e-6, 0, None) == -1
     assert rc("sdk_gnomonic_kernel_at", one, one, 5, 0, 3, 0.1, 0.1, 0, 0, 0, None) == -1
     assert rc("sdk_gnomonic_kernel_at", one, one, 5, 3, 3, 0.1, 0.1, 1, 8, 0, None) == -1
     # gather at index and average pooling share the mapped-operator checks
