@@ -826,19 +826,25 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
         live[pl] = s64 >= 0 && s64 + twoq <= map_elems;   // others contribute nothing
         sv[pl] = (int)s64;                                  // map_elems < 2^31
       }
+      __builtin_amdgcn_sched_barrier(0);   // indices and gradients are requested together
       T cx[PLMAX], cy[PLMAX];
+      bool stray = false;
 #pragma unroll
       for (int pl = 0; pl < PLMAX; ++pl) {
-        if (live[pl]) {
-          const int d = sv[pl] - first;
-          if (d < 0 || d >= per_pixel || d % twoq != 0) {   // not a sample of this pixel
-            atomicAdd(gate, 1);
-            live[pl] = false;
-          }
-        }
-        cx[pl] = live[pl] ? map[sv[pl]] : T(0);
-        cy[pl] = live[pl] ? map[sv[pl] + 1] : T(0);
+        const int d = sv[pl] - first;
+        const bool mine = d >= 0 && d < per_pixel && d % twoq == 0;   // a sample of this pixel
+        stray |= live[pl] && !mine;
+        live[pl] = live[pl] && mine;
+        sv[pl] = live[pl] ? sv[pl] : 0;
       }
+      // unconditional reads (element 0 for planes that contribute nothing), so that the
+      // coordinates of all planes are fetched in one round trip
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        cx[pl] = map[sv[pl]];
+        cy[pl] = map[sv[pl] + 1];
+      }
+      if (stray) atomicAdd(gate, 1);
 #pragma unroll
       for (int pl = 0; pl < PLMAX; ++pl) {
         if (!live[pl]) continue;

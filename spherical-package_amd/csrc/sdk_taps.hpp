@@ -212,6 +212,24 @@ struct PointTaps {
     }
   }
 
+  // gather() in two steps, for callers that want the reads of several planes issued before
+  // the first of them is used: load() fetches the taps, blend() combines them as gather() does.
+  __device__ __forceinline__ void load(const T* __restrict__ plane, T (&raw)[N]) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) raw[i] = plane[off[i] < 0 ? 0 : off[i]];
+  }
+  __device__ __forceinline__ T blend(const T (&raw)[N]) const {
+    if constexpr (INTERP == 0) {
+      return off[0] < 0 ? T(0) : raw[0];
+    } else {
+      const T t0 = w[0] * (off[0] < 0 ? T(0) : raw[0]);
+      const T t1 = w[1] * (off[1] < 0 ? T(0) : raw[1]);
+      const T t2 = w[2] * (off[2] < 0 ? T(0) : raw[2]);
+      const T t3 = w[3] * (off[3] < 0 ? T(0) : raw[3]);
+      return t0 + t1 + t2 + t3;
+    }
+  }
+
   __device__ __forceinline__ void scatter(T* __restrict__ plane, T v) const {
     if constexpr (INTERP == 0) {
       if (off[0] >= 0) atomic_add_noret(plane + off[0], v);
@@ -226,29 +244,35 @@ struct PointTaps {
 // Applies one map sample (1 point, or P weighted points accumulated in
 // ascending order: core/resample.h:144-161) to PC planes that are `stride`
 // elements apart.  Planes j >= np are not touched (acc[j] = 0).
+// The reads of all PC planes are issued before the first of them is used (load, then blend).
+// Left to itself the compiler, where the results feed a chain of compares (the running
+// maximum of a pooling window) or a weighted sum, sinks every read next to its use and waits
+// for each in turn: up to 32 round trips to memory per sample instead of one.
 template <typename T, int INTERP, bool WEIGHTED, int PC>
 __device__ __forceinline__ void gather_sample(const T* __restrict__ base, size_t stride, int np,
                                               const T* __restrict__ coords,
                                               const T* __restrict__ wts, int P, int H, int W,
                                               T (&acc)[PC]) {
   PointTaps<T, INTERP> t;
-  if constexpr (!WEIGHTED) {
-    t.set(coords[0], coords[1], H, W);
+  constexpr int N = PointTaps<T, INTERP>::N;
+  const int q = WEIGHTED ? P : 1;
+#pragma unroll
+  for (int j = 0; j < PC; ++j) acc[j] = T(0);
+  for (int p = 0; p < q; ++p) {
+    t.set(coords[2 * p], coords[2 * p + 1], H, W);
+    T wt = T(1);
+    if constexpr (WEIGHTED) wt = wts[p];
+    T raw[PC][N];
+#pragma unroll
+    for (int j = 0; j < PC; ++j) t.load(base + (size_t)(j < np ? j : 0) * stride, raw[j]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < PC; ++j) {
-      const T v = t.gather(base + (size_t)(j < np ? j : 0) * stride);
-      acc[j] = j < np ? v : T(0);
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < PC; ++j) acc[j] = T(0);
-    for (int p = 0; p < P; ++p) {
-      t.set(coords[2 * p], coords[2 * p + 1], H, W);
-      const T wt = wts[p];
-#pragma unroll
-      for (int j = 0; j < PC; ++j) {
-        const T v = t.gather(base + (size_t)(j < np ? j : 0) * stride);
+      const T v = t.blend(raw[j]);
+      if constexpr (WEIGHTED) {
         if (j < np) acc[j] += wt * v;
+      } else {
+        acc[j] = j < np ? v : T(0);
       }
     }
   }
