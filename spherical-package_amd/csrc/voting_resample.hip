@@ -23,44 +23,53 @@ __global__ __launch_bounds__(kVoteBlock) void vote_clear_kernel(uint4* __restric
     p[i] = make_uint4(0, 0, 0, 0);
 }
 
-// One thread per (batch element of this pass, channel, input pixel).  A label outside
-// [0, candidates) casts no vote (the reference would write outside its histogram).
+// One thread per input pixel, grid.y over (batch element of this pass, channel): the plane
+// arithmetic is per workgroup, and the pixel's target (16 bytes of the map) and its label are
+// requested together.  A label outside [0, candidates) casts no vote (the reference would
+// write outside its histogram).
 __global__ __launch_bounds__(kVoteBlock) void vote_kernel(
     const int64_t* __restrict__ labels, const int64_t* __restrict__ map,
-    unsigned* __restrict__ votes, size_t total, int in_pixels, int channels, int OH, int OW,
-    int candidates, size_t element_stride) {
-  const size_t idx = (size_t)blockIdx.x * kVoteBlock + threadIdx.x;
-  if (idx >= total) return;
-  const int pix = (int)(idx % in_pixels);
-  const size_t plane = idx / in_pixels;
-  const size_t c = plane % channels, e = plane / channels;
+    unsigned* __restrict__ votes, int in_pixels, int channels, int OH, int OW, int candidates,
+    size_t element_stride) {
+  const int pix = blockIdx.x * kVoteBlock + threadIdx.x;
+  if (pix >= in_pixels) return;
+  const unsigned plane = blockIdx.y;
+  const unsigned e = plane / (unsigned)channels, c = plane - e * (unsigned)channels;
   const long long x = map[(size_t)pix * 2], y = map[(size_t)pix * 2 + 1];
-  const long long label = labels[idx];
+  const long long label = labels[(size_t)plane * in_pixels + pix];
   if (x < 0 || x > OW - 1 || y < 0 || y > OH - 1 || label < 0 || label >= candidates) return;
   // channel offset in histogram elements as the reference has it (common/resample.h:127-129):
   // c * OH * OW, not c whole histograms, so the histograms of several channels overlap
-  atomicAdd(&votes[e * element_stride + c * OH * OW +
+  atomicAdd(&votes[e * element_stride + (size_t)c * OH * OW +
                    ((size_t)y * OW + (size_t)x) * candidates + (size_t)label], 1u);
 }
 
-// One thread per (batch element of this pass, channel, output pixel): index of the first
-// largest count.
+// One thread per output pixel, grid.y over (batch element of this pass, channel): index of
+// the first largest count.  The counts are read eight at a time, all eight requested before
+// the first is compared.
 __global__ __launch_bounds__(kVoteBlock) void vote_argmax_kernel(
-    const unsigned* __restrict__ votes, int64_t* __restrict__ out, size_t total,
-    size_t per_element, int candidates, size_t element_stride) {
-  const size_t idx = (size_t)blockIdx.x * kVoteBlock + threadIdx.x;
-  if (idx >= total) return;
-  const unsigned* v = votes + (idx / per_element) * element_stride + (idx % per_element) * candidates;
-  unsigned best = v[0];
+    const unsigned* __restrict__ votes, int64_t* __restrict__ out, int out_pixels, int channels,
+    int candidates, size_t element_stride) {
+  const int pix = blockIdx.x * kVoteBlock + threadIdx.x;
+  if (pix >= out_pixels) return;
+  const unsigned plane = blockIdx.y;
+  const unsigned e = plane / (unsigned)channels, c = plane - e * (unsigned)channels;
+  const unsigned* v =
+      votes + e * element_stride + ((size_t)c * out_pixels + pix) * (size_t)candidates;
+  unsigned best = 0;
   int arg = 0;
-  for (int k = 1; k < candidates; ++k) {
-    const unsigned n = v[k];
-    if (n > best) {
-      best = n;
-      arg = k;
-    }
+  for (int k0 = 0; k0 < candidates; k0 += 8) {
+    unsigned n[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) n[i] = v[min(k0 + i, candidates - 1)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (k0 + i < candidates && n[i] > best) {   // strict: the first of equal counts stays
+        best = n[i];
+        arg = k0 + i;
+      }
   }
-  out[idx] = arg;
+  out[(size_t)plane * out_pixels + pix] = arg;
 }
 
 static size_t vote_bytes(int64_t channels, int64_t oh, int64_t ow, int64_t candidates) {
@@ -102,27 +111,25 @@ int sdk_voting_resample_to_map(const int64_t* input, const int64_t* sample_map, 
   hipStream_t s = (hipStream_t)stream;
   unsigned* votes = static_cast<unsigned*>(workspace);
   const int in_pixels = (int)(in_height * in_width);
+  const int out_pixels = (int)(out_height * out_width);
   const size_t n_in = (size_t)channels * in_pixels;
   const size_t n_out = (size_t)channels * out_height * out_width;
-  SDK_REQUIRE(ceil_div((int64_t)n_in, kVoteBlock) < ((int64_t)1 << 31) &&
-                  ceil_div((int64_t)n_out, kVoteBlock) < ((int64_t)1 << 31),
-              "voting_resample_to_map: too many channels");
-  // as many batch elements per pass as the workspace holds histograms
-  const int64_t per_pass = std::min<int64_t>(batch, (int64_t)(workspace_bytes / need));
-  SDK_REQUIRE(ceil_div(per_pass * (int64_t)std::max(n_in, n_out), kVoteBlock) < ((int64_t)1 << 31),
-              "voting_resample_to_map: too much work for one pass");
+  SDK_REQUIRE(channels <= 65535, "voting_resample_to_map: more than 65535 channels");
+  // as many batch elements per pass as the workspace holds histograms (and grid.y planes)
+  const int64_t per_pass = std::min<int64_t>(
+      std::min<int64_t>(batch, (int64_t)(workspace_bytes / need)), 65535 / channels);
   for (int64_t b = 0; b < batch; b += per_pass) {
     const int64_t nb = std::min<int64_t>(per_pass, batch - b);
     const size_t n16 = need / 16 * (size_t)nb;
     const int clear_blocks = (int)std::min<int64_t>(ceil_div((int64_t)n16, kVoteBlock), 4096);
     launch(vote_clear_kernel, dim3(clear_blocks), dim3(kVoteBlock), s, (uint4*)workspace, n16);
-    launch(vote_kernel, dim3((unsigned)ceil_div((int64_t)(n_in * nb), kVoteBlock)),
-           dim3(kVoteBlock), s, input + (size_t)b * n_in, sample_map, votes, n_in * (size_t)nb,
-           in_pixels, (int)channels, (int)out_height, (int)out_width, (int)num_candidates,
-           need / sizeof(unsigned));
-    launch(vote_argmax_kernel, dim3((unsigned)ceil_div((int64_t)(n_out * nb), kVoteBlock)),
-           dim3(kVoteBlock), s, (const unsigned*)votes, out + (size_t)b * n_out,
-           n_out * (size_t)nb, n_out, (int)num_candidates, need / sizeof(unsigned));
+    const unsigned planes = (unsigned)(nb * channels);
+    launch(vote_kernel, dim3((unsigned)ceil_div(in_pixels, kVoteBlock), planes), dim3(kVoteBlock),
+           s, input + (size_t)b * n_in, sample_map, votes, in_pixels, (int)channels,
+           (int)out_height, (int)out_width, (int)num_candidates, need / sizeof(unsigned));
+    launch(vote_argmax_kernel, dim3((unsigned)ceil_div(out_pixels, kVoteBlock), planes),
+           dim3(kVoteBlock), s, (const unsigned*)votes, out + (size_t)b * n_out, out_pixels,
+           (int)channels, (int)num_candidates, need / sizeof(unsigned));
   }
   SDK_LAUNCH_CHECK("voting_resample_to_map");
   return SDK_OK;
