@@ -665,16 +665,18 @@ __global__ __launch_bounds__(kBlock) void mapped_gather_at_index_kernel(
 // another pooled pixel than its own (mapped_max_pool never writes one, but the scatter
 // accepts it): such a sample may reach tiles whose windows do not hold the pixel.
 // ---------------------------------------------------------------------------
-constexpr int kUpTile = 1024;     // image pixels per workgroup (4 per thread); 2^10, see tile_of
+constexpr int kUpTileLog2 = 11;
+constexpr int kUpTile = 1 << kUpTileLog2;   // image pixels per workgroup
+constexpr int kUpPer = kUpTile / kBlock;    // ... and per thread
 constexpr int kUpWindow = 8192;   // pooled pixels a tile may have to look at
-constexpr int kUpBytes = 16384;   // LDS of the tile accumulators: kUpTile x planes per pass
+constexpr int kUpBytes = 32768;   // LDS of the tile accumulators: kUpTile x planes per pass
 
 struct UnpoolTiling {
   int H, W, tw_shift, tiles_x, tiles_y;
   __host__ __device__ int TW() const { return 1 << tw_shift; }
   __host__ __device__ int TH() const { return kUpTile >> tw_shift; }
   __device__ int tile_of(int y, int x) const {
-    return (y >> (10 - tw_shift)) * tiles_x + (x >> tw_shift);   // TH = kUpTile >> tw_shift
+    return (y >> (kUpTileLog2 - tw_shift)) * tiles_x + (x >> tw_shift);   // TH = kUpTile >> tw_shift
   }
 };
 
@@ -790,18 +792,18 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
   const float rcp_ww = WW > 0 ? 1.0f / (float)WW : 0.0f;
   const int per_pixel = K * twoq;   // map elements of one pooled pixel
   // the thread's 4 image pixels: waves own 4 consecutive 64-pixel runs of the tile
-  int u[4];
+  int u[kUpPer];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int L = (((tid >> 6) * 4 + j) << 6) + (tid & 63);
+  for (int j = 0; j < kUpPer; ++j) {
+    const int L = (((tid >> 6) * kUpPer + j) << 6) + (tid & 63);
     const int y = ty0 + (L >> ut.tw_shift), x = tx0 + (L & (ut.TW() - 1));
     u[j] = (y < ut.H && x < ut.W) ? y * ut.W + x : -1;
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < kUpPer; ++j)
 #pragma unroll
     for (int pl = 0; pl < PLMAX; ++pl)
-      acc[pl * kUpTile + (((tid >> 6) * 4 + j) << 6) + (tid & 63)] = T(0);
+      acc[pl * kUpTile + (((tid >> 6) * kUpPer + j) << 6) + (tid & 63)] = T(0);
   __syncthreads();
   for (int p0 = p_begin; p0 < p_end; p0 += PLMAX) {
     const int np = min(PLMAX, p_end - p0);
@@ -871,10 +873,10 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
     __syncthreads();
     // store the tile and clear it for the next pass
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kUpPer; ++j) {
 #pragma unroll
       for (int pl = 0; pl < PLMAX; ++pl) {
-        T* cell = acc + pl * kUpTile + (((tid >> 6) * 4 + j) << 6) + (tid & 63);
+        T* cell = acc + pl * kUpTile + (((tid >> 6) * kUpPer + j) << 6) + (tid & 63);
         const T v = *cell;
         *cell = T(0);
         if (u[j] >= 0 && pl < np) gin[(size_t)(p0 + pl) * HW + u[j]] = v;
@@ -1109,8 +1111,8 @@ static UnpoolTiling unpool_tiling(int H, int W) {
   UnpoolTiling ut;
   ut.H = H;
   ut.W = W;
-  ut.tw_shift = 6;
-  while ((kUpTile >> ut.tw_shift) > H && ut.tw_shift < 10) ++ut.tw_shift;   // flat images: wider tiles
+  ut.tw_shift = 7;
+  while ((kUpTile >> ut.tw_shift) > H && ut.tw_shift < kUpTileLog2) ++ut.tw_shift;   // flat images: wider tiles
   while (ut.tw_shift > 0 && (1 << (ut.tw_shift - 1)) >= W) --ut.tw_shift;   // narrow ones: taller
   ut.tiles_x = (int)ceil_div(W, ut.TW());
   ut.tiles_y = (int)ceil_div(H, ut.TH());
