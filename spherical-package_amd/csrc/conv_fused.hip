@@ -616,7 +616,18 @@ size_t fused_workspace_bytes(const ConvGeom& g) {
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
   if (planned_scatter_supported(g) && inverse_candidate(g))
     need = ((need + 255) & ~(size_t)255) + inverse_bytes(g);
+  // last: the weight gradient's partial sums (the plan and, in a combined backward call,
+  // everything before it are still in use when they are written)
+  if (planned_wgrad_partial_bytes(g) != 0)
+    need = ((need + 255) & ~(size_t)255) + planned_wgrad_partial_bytes(g);
   return need;
+}
+
+static float* wgrad_partial(const ConvGeom& g, float* workspace) {
+  const size_t bytes = planned_wgrad_partial_bytes(g);
+  if (bytes == 0) return nullptr;
+  return reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
+                                  (fused_workspace_bytes(g) - bytes));
 }
 
 static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
@@ -889,11 +900,13 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   if (g.B == 0) return SDK_OK;
   if (planned_wgrad_supported(g)) {
     if (shared != nullptr && shared->valid)
-      return planned_wgrad(g, matrix_mode(compute), shared->plan, pix, img, gW, stream);
+      return planned_wgrad(g, matrix_mode(compute), shared->plan, pix, img, gW,
+                           wgrad_partial(g, workspace), stream);
     Plan plan;
     rc = build_plan(g, map, wts, workspace, stream, &plan);
     if (rc) return rc;
-    return planned_wgrad(g, matrix_mode(compute), plan, pix, img, gW, stream);
+    return planned_wgrad(g, matrix_mode(compute), plan, pix, img, gW, wgrad_partial(g, workspace),
+                         stream);
   }
   constexpr int KM = 64;
   const int slots = slots_for(g);

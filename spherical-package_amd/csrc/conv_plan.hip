@@ -202,9 +202,9 @@ __device__ __forceinline__ void lds_only_barrier() {
 template <int KB, int MM, int NW>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
-    const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW, int Cg,
-    int H, int W, int Cp, int K, int S, PixelTiling pt, int tiles,
-    int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
+    const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW,
+    float* __restrict__ partial, int Cg, int H, int W, int Cp, int K, int S, PixelTiling pt,
+    int tiles, int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
   constexpr bool BF16 = MM != kMmF32;     // operands enter the matrix unit as bf16 fragments
   constexpr bool SPLIT = MM == kMmSplit;  // ... three per operand, whose sum is the float
   __shared__ __align__(16) float region[kRegionCap * kRegE];
@@ -537,6 +537,18 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     }
   }
 
+  // ---- with a partial-sum buffer: every accumulator register is stored as it lies
+  // (register-major, thread fastest: full 256-byte rows per wave) and wgrad_reduce_kernel sums the
+  // workgroups' copies.  All workgroups finish together, so adding 147 KB each to the same
+  // addresses of gW here would queue their device-scope atomics behind one another.
+  if (partial != nullptr) {
+    float* dst = partial + (size_t)blockIdx.x * (KB * 16 * kPlThreads) + tid;
+#pragma unroll
+    for (int kk = 0; kk < KB; ++kk)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dst[(kk * 16 + v) * kPlThreads] = acc[kk][v];
+    return;
+  }
   // ---- gW[n][c*K + k] += D[n][c]; accumulator register v: row 8*(v/4) + 4*h + v%4, column nl
   const int c = c0 + nl;
   if (c < Cg) {
@@ -552,6 +564,33 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
       }
     }
   }
+}
+
+// Sums the accumulator copies planned_wgrad_kernel left in `partial` and adds them to gW.
+// Block (x, y, z): accumulator register x = kk * 16 + v of thread threadIdx.x, for the
+// workgroup kind y (channel chunk, row-block tile, sample block), over every z-th of the
+// batches * groups workgroups of that kind.  The index arithmetic mirrors the kernel's.
+__global__ __launch_bounds__(kPlThreads) void wgrad_reduce_kernel(
+    const float* __restrict__ partial, float* __restrict__ gW, int Cg, int Cp, int K, int KB,
+    int NW, int groups, int batches, int c_chunks, int n_tiles, int kblocks) {
+  const int tid = threadIdx.x, kkv = blockIdx.x, kk = kkv >> 4, v = kkv & 15;
+  const int kb = blockIdx.y % kblocks, nt = (blockIdx.y / kblocks) % n_tiles;
+  const int cc = blockIdx.y / (kblocks * n_tiles);
+  const int kinds = c_chunks * n_tiles * kblocks * batches;
+  const int total = batches * groups;
+  const size_t per_wg = (size_t)KB * 16 * kPlThreads;
+  float s = 0.0f;
+  for (int i = blockIdx.z; i < total; i += gridDim.z) {
+    const int b = i / groups, grp = i % groups;
+    const int kind = ((b * c_chunks + cc) * n_tiles + nt) * kblocks + kb;
+    const size_t wg = ((size_t)(grp >> 3) * kinds + kind) * 8 + (grp & 7);
+    s += partial[wg * per_wg + (size_t)kkv * kPlThreads + tid];
+  }
+  const int wave = tid >> 6, lane = tid & 63, nl = lane & 31, h = lane >> 5;
+  const int c = cc * kCC + nl;
+  const int n = nt * (32 * NW) + 32 * (wave % NW) + 8 * (v >> 2) + 4 * h + (v & 3);
+  const int k = kb * KB + kk;
+  if (c < Cg && n < Cp && k < K) atomic_add_noret(gW + (size_t)n * Cg * K + (size_t)c * K + k, s);
 }
 
 // ---------------------------------------------------------------------------
@@ -617,21 +656,52 @@ bool planned_wgrad_supported(const ConvGeom& g) {
   return plan_supported(g) && plan_slots(g) <= kRowCap && g.B <= 65535;
 }
 
-int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
-                  const float* img, float* gW, hipStream_t stream) {
+namespace {
+// Launch shape of planned_wgrad_kernel: KB samples per workgroup, NW row blocks, and how many
+// tile runs (`groups`) each kind of workgroup is split into.
+struct WgradGrid {
+  int KB, kb_count, NW, c_chunks, n_tiles, groups;
+  int64_t kinds, slots;
+};
+
+WgradGrid wgrad_grid(const ConvGeom& g, int tiles) {
+  WgradGrid w;
   const int kblocks = (int)ceil_div(g.K, 9);
   const int per = (int)ceil_div(g.K, kblocks);
-  const int KB = per <= 1 ? 1 : (per <= 4 ? 4 : (per <= 7 ? 7 : 9));
-  const int kb_count = (int)ceil_div(g.K, KB);
-  const int NW = g.Cp > 64 ? 4 : (g.Cp > 32 ? 2 : 1);
-  const int c_chunks = (int)ceil_div(g.Cg, kCC), n_tiles = (int)ceil_div(g.Cp, 32 * NW);
-  const int64_t kinds = (int64_t)c_chunks * n_tiles * kb_count * g.B;
+  w.KB = per <= 1 ? 1 : (per <= 4 ? 4 : (per <= 7 ? 7 : 9));
+  w.kb_count = (int)ceil_div(g.K, w.KB);
+  w.NW = g.Cp > 64 ? 4 : (g.Cp > 32 ? 2 : 1);
+  w.c_chunks = (int)ceil_div(g.Cg, kCC);
+  w.n_tiles = (int)ceil_div(g.Cp, 32 * w.NW);
+  w.kinds = (int64_t)w.c_chunks * w.n_tiles * w.kb_count * g.B;
   // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall
-  int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, kinds), 8) * 8);
-  int groups = (int)std::min<int64_t>(plan.tiles, want);
-  const int tpg = (int)ceil_div(plan.tiles, groups);
-  groups = (int)ceil_div(plan.tiles, tpg);
-  const int64_t slots = ceil_div(groups, 8) * 8 * kinds;
+  const int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, w.kinds), 8) * 8);
+  w.groups = (int)std::min<int64_t>(tiles, want);
+  const int tpg = (int)ceil_div(tiles, w.groups);
+  w.groups = (int)ceil_div(tiles, tpg);
+  w.slots = ceil_div(w.groups, 8) * 8 * w.kinds;
+  return w;
+}
+
+// Largest partial-sum buffer worth reserving; calls that would need more add to gW directly.
+constexpr size_t kWgradPartialCap = (size_t)160 << 20;
+}  // namespace
+
+size_t planned_wgrad_partial_bytes(const ConvGeom& g) {
+  if (g.B == 0 || !planned_wgrad_supported(g)) return 0;
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  const WgradGrid w = wgrad_grid(g, pt.tiles_x * pt.tiles_y);
+  if (w.slots >= ((int64_t)1 << 31)) return 0;
+  const size_t bytes = (size_t)w.slots * w.KB * 16 * kPlThreads * sizeof(float);
+  return bytes <= kWgradPartialCap ? bytes : 0;
+}
+
+int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
+                  const float* img, float* gW, float* partial, hipStream_t stream) {
+  const WgradGrid wg = wgrad_grid(g, plan.tiles);
+  const int KB = wg.KB, kb_count = wg.kb_count, NW = wg.NW;
+  const int c_chunks = wg.c_chunks, n_tiles = wg.n_tiles, groups = wg.groups;
+  const int64_t slots = wg.slots;
   if (slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "planned_wgrad: grid too large");
   const int TX = plan.pt.TX();
   const int vec4 = (g.OW % 4 == 0 && TX >= (mm != kMmF32 ? 8 : 4) &&
@@ -639,7 +709,7 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
   const dim3 grid((unsigned)slots);
 #define PW3(KBv, BFv, NWv)                                                                      \
   launch(planned_wgrad_kernel<KBv, BFv, NWv>, grid, dim3(kPlThreads), stream, pix, img,         \
-         plan.hdr, plan.ns, plan.taps, gW, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt,          \
+         plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
          plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4)
 #define PW(KBv, BFv)                                                                            \
   do {                                                                                          \
@@ -655,6 +725,15 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 #undef PW
 #undef PW3
   SDK_LAUNCH_CHECK("planned_wgrad");
+  if (partial != nullptr) {
+    const int kinds0 = c_chunks * n_tiles * kb_count, total = (int)g.B * groups;
+    // enough blocks to fill the GPU: the workgroups of a kind are summed in up to 16 parts
+    const int parts = (int)std::min<int64_t>(std::min(total, 16), ceil_div(2048, (int64_t)KB * 16 * kinds0));
+    launch(wgrad_reduce_kernel, dim3((unsigned)(KB * 16), (unsigned)kinds0, (unsigned)std::max(parts, 1)),
+           dim3(kPlThreads), stream, (const float*)partial, gW, g.Cg, g.Cp, g.K, KB, NW, groups,
+           (int)g.B, c_chunks, n_tiles, kb_count);
+    SDK_LAUNCH_CHECK("wgrad_reduce");
+  }
   return SDK_OK;
 }
 

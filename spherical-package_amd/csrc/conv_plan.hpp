@@ -42,8 +42,11 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
                hipStream_t stream, Plan* plan, const int* gate = nullptr);
 
 // gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
+// partial: planned_wgrad_partial_bytes(g) bytes (when that is not 0) in which the workgroups
+// leave their sums for a second, summing kernel; nullptr: they add to gW themselves.
 bool planned_wgrad_supported(const ConvGeom& g);
+size_t planned_wgrad_partial_bytes(const ConvGeom& g);
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
-                  const float* img, float* gW, hipStream_t stream);
+                  const float* img, float* gW, float* partial, hipStream_t stream);
 
 }  // namespace sdk
