@@ -354,7 +354,9 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
  * least that many bytes, 256-byte aligned.  Besides the
  * weights the scratch holds the call's tap plan (the sample map resolved into
  * window indices and coefficients), up to
- * 8 * map pixels * kernel_size * points * taps-per-point bytes.
+ * 8 * map pixels * kernel_size * points * taps-per-point bytes, and the weight
+ * gradient's per-workgroup partial sums (at most 160 MB; larger ones are not
+ * reserved and that call adds to grad_weight directly).
  * ------------------------------------------------------------------------- */
 size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64_t out_channels,
                                        int64_t image_height, int64_t image_width,
