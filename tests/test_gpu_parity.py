@@ -406,6 +406,26 @@ def test_fused_conv_tile_edges(ops, oracle, tc):
     assert relerr(_n(gb), wb) <= 1e-4
 
 
+def test_weight_gradient_without_partial_sums(ops, oracle):
+    """The weight gradient normally leaves per-workgroup sums in the workspace and a second
+    kernel adds them up; a call whose sums would need more than 160 MB adds to grad_weight
+    directly.  192 -> 256 channels at batch 12 on 8 tiles is such a call: 6 channel chunks x 2
+    row-block tiles x 12 batch elements x 8 tile runs = 1152 workgroups of 147 456 bytes."""
+    dt = np.float32
+    rng = np.random.default_rng(77)
+    B, Cin, Cout, H, W, K = 12, 192, 256, 16, 64, 9
+    x = rng.standard_normal((B, Cin, H, W)).astype(dt)
+    m = _coherent_map(rng, H, W, K, 0, H, W, dt)
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, H, W)).astype(dt)
+    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), None, _t(x), _t(wt), _t(b), K, 1)
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, wt, b, K, 1, None)
+    assert relerr(_n(gi), wi) <= 1e-4
+    assert relerr(_n(gw), ww) <= 1e-4
+    assert relerr(_n(gb), wb) <= 1e-4
+
+
 def _coherent_map(rng, OH, OW, K, P, H, W, dtype, scale=1.0, jitter=0.45):
     """Locally coherent map: pixel (y, x) samples around (x, y) * scale * (W/OW, H/OH) with a
     ring of K offsets, as a convolution-style map does; a few samples fall outside the image."""
