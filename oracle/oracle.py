@@ -237,6 +237,21 @@ def mapped_conv_backward(grad_output, sample_map, x, weight, bias, kernel_size, 
     return gi, gw, gb
 
 
+def mapped_conv_backward_input(grad_output, sample_map, x_shape, weight, kernel_size, interp,
+                               interp_weights=None):
+    """grad_input [B,Cin,H,W] alone (x_shape = the input's shape)."""
+    g = _c(grad_output); m = _c(sample_map, g.dtype); w = _c(interp_weights, g.dtype)
+    weight = _c(weight, g.dtype)
+    B, Cin, H, W = (int(v) for v in x_shape)
+    Cout = weight.shape[0]
+    OH, OW = m.shape[:2]
+    gi = np.empty((B, Cin, H, W), g.dtype)
+    _check(lib().sdk_oracle_mapped_conv_backward_input(
+        _p(g), _p(m), _p(w), _p(weight), _p(gi), *_i64(B, Cin, H, W, Cout, OH, OW, kernel_size),
+        *_i32(_num_pts(m, w), int(interp), _dt(g))))
+    return gi
+
+
 def mapped_transposed_conv_forward(x, sample_map, weight, bias, out_h, out_w,
                                    kernel_size, interp, interp_weights=None):
     x = _c(x); m = _c(sample_map, x.dtype); w = _c(interp_weights, x.dtype)

@@ -704,7 +704,10 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
   const int64_t slots = wg.slots;
   if (slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "planned_wgrad: grid too large");
   const int TX = plan.pt.TX();
-  const int vec4 = (g.OW % 4 == 0 && TX >= (mm != kMmF32 ? 8 : 4) &&
+  // a lane loads one run of 4 (fp32) or 8 (bf16, split) consecutive pixels of a tile row with
+  // 16-byte loads and checks the run's first pixel only: runs must not straddle the row end
+  const int run = mm != kMmF32 ? 8 : 4;
+  const int vec4 = (g.OW % run == 0 && TX >= run &&
                     reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)slots);
 #define PW3(KBv, BFv, NWv)                                                                      \

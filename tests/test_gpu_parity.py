@@ -740,3 +740,50 @@ def test_gather_at_index_and_unpool_layer(ops, oracle, case):
         assert torch.autograd.gradcheck(
             lambda t: F.mapped_max_unpool(t, _t(safe[:1, :2]), _t(m), (H, W), K, interp), (probe,),
             eps=1e-6, atol=1e-7, nondet_tol=1e-9)
+
+
+@pytest.mark.parametrize("mode", ["native", "bf16", "split"])
+@pytest.mark.parametrize("shape", [(9, 12), (16, 20), (8, 28), (20, 36)],
+                         ids=lambda s: "%dx%d" % s)
+def test_weight_gradient_reads_nothing_behind_its_rows(ops, oracle, mode, shape):
+    """Grids whose width is a multiple of 4 but not of 8: the weight gradient loads runs of 4
+    (float32) or 8 (bf16, split) pixels per lane.  The pixel-side tensor is the tail of a buffer
+    whose remaining bytes are NaN, so a run that leaves its row, or the tensor, poisons
+    grad_weight."""
+    OH, OW = shape
+    dt = np.float32
+    rng = np.random.default_rng(5 + OH * OW)
+    B, Cin, Cout, K = 2, 16, 32, 9
+    x = rng.standard_normal((B, Cin, OH, OW)).astype(dt)
+    m = _coherent_map(rng, OH, OW, K, 0, OH, OW, dt)
+    wt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(dt)
+    b = rng.standard_normal(Cout).astype(dt)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+
+    def guarded(a):
+        """a on the device, followed directly by 64 NaNs of the same allocation."""
+        buf = torch.full((a.size + 64,), float("nan"), dtype=torch.float32, device=DEV)
+        buf[:a.size] = _t(a).reshape(-1)
+        return buf[:a.size].view(*a.shape), buf
+
+    tol = 1e-2 if mode == "bf16" else 1e-4
+    ops.set_conv_compute(mode)
+    try:
+        gg, keep_g = guarded(g)
+        _, gw, _ = ops.mapped_conv_backward(gg, _t(m), None, _t(x), _t(wt), _t(b), K, 1)
+        ww = oracle.mapped_conv_backward(g, m, x, wt, b, K, 1, None)[1]
+        assert bool(torch.isfinite(gw).all())
+        assert relerr(_n(gw), ww) <= tol
+        # transposed layer: its input is the pixel-side tensor of the weight gradient
+        xt = rng.standard_normal((B, Cout, OH, OW)).astype(dt)
+        wtt = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cout * K)).astype(dt)
+        bt = rng.standard_normal(Cin).astype(dt)
+        gt = rng.standard_normal((B, Cin, OH, OW)).astype(dt)
+        xg, keep_x = guarded(xt)
+        _, gw, _ = ops.mapped_transposed_conv_backward(_t(gt), _t(m), None, xg, _t(wtt), _t(bt),
+                                                       K, 1)
+        ww = oracle.mapped_transposed_conv_backward(gt, m, xt, wtt, bt, K, 1, None)[1]
+        assert bool(torch.isfinite(gw).all())
+        assert relerr(_n(gw), ww) <= tol
+    finally:
+        ops.set_conv_compute("native")
