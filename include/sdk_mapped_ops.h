@@ -340,6 +340,27 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
                           int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
                           int32_t dtype, sdk_stream_t stream);
 
+/* sdk_mapped_max_unpool for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and results as sdk_mapped_max_unpool without the workspace pair:
+ * the tile-window scratch (256 + 32 bytes per 2048-pixel tile of the input plane) is a
+ * 262 400-byte array inside the library, one copy per GPU, held until the process ends.  The
+ * call allocates and frees nothing.  Limit: the input plane may have at most
+ * SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES tiles, ceil(width / TW) * ceil(height / (2048 / TW))
+ * with TW = 128 (wider for planes lower than 16 rows, narrower for planes under 65 columns),
+ * i.e. any plane up to 4096 x 4096; a larger one returns SDK_ERR_WORKSPACE with a message.
+ * Every call on one GPU uses that GPU's array (the part it needs is cleared by a fill kernel at
+ * the start of the call): calls that overlap on one GPU, on different streams or from different
+ * threads, race; calls on one stream are ordered and safe.  The first call on a device looks up
+ * the array's address (hipGetSymbolAddress) and should happen outside a graph capture. */
+#define SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES 8192
+int sdk_mapped_max_unpool_static(const void* grad_output, const int64_t* indices,
+                                 const void* sample_map, const void* interp_weights,
+                                 void* grad_input, int64_t batch, int64_t channels,
+                                 int64_t height, int64_t width, int64_t out_height,
+                                 int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
+                                 int32_t interp, int32_t dtype, sdk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mapped convolution.  weight [Cout, Cin, K]; bias [Cout];
  * input [B,Cin,H,W]; sample_map [OH,OW,K,(P,)2]; output [B,Cout,OH,OW].

@@ -33,6 +33,7 @@ SIGNATURES = {
     "sdk_mapped_col2im": [_vp] * 4 + [_i64] * 6 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_pool": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_unpool": [_vp] * 6 + [_sz] + [_i64] * 7 + [_i32] * 3 + [_vp],
+    "sdk_mapped_max_unpool_static": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],
     "sdk_mapped_gather_at_index": [_vp] * 5 + [_i64] * 7 + [_i32] * 3 + [_vp],
     "sdk_mapped_avg_pool": [_vp] * 4 + [_i64] * 7 + [_i32] * 3 + [_vp],
     "sdk_mapped_avg_unpool": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 3 + [_vp],

@@ -10,6 +10,8 @@
 // flight per lane.  grid.x walks pixels, grid.y walks plane chunks.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include <cfloat>
 #include <climits>
 
@@ -1221,6 +1223,43 @@ template int launch_mapped_col2im<double>(const double*, const double*, const do
 using namespace sdk;
 
 // ---------------------------------------------------------------------------
+// The unpool for callers that cannot allocate: the tile-window scratch of
+// sdk_mapped_max_unpool lives in a file-scope device array.  The array's name is
+// only a host-side handle: its device address is asked for once per device and
+// that pointer is what the fill kernel and the unpool kernels receive.
+// ---------------------------------------------------------------------------
+static constexpr int kStaticUnpoolTiles = SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES;   // of 2048 pixels
+static constexpr size_t kStaticUnpoolBytes = 256 + (size_t)kStaticUnpoolTiles * 8 * sizeof(int);
+static __device__ __align__(256) unsigned char scratch[kStaticUnpoolBytes];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static void* scratch_ptr[kMaxDevices] = {};   // per device: every GPU holds its own copy of the array
+
+// The current device's address of `scratch` (resolved on the first call on that device).
+static int static_unpool_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "mapped_max_unpool_static: hipGetDevice: %s",
+                hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(SDK_ERR_UNSUPPORTED, "mapped_max_unpool_static: device %d (at most %d devices)",
+                dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(SDK_ERR_DEVICE, "mapped_max_unpool_static: hipGetSymbolAddress: %s",
+                  hipGetErrorString(e));
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return SDK_OK;
+}
+
+// ---------------------------------------------------------------------------
 // C entry points.
 // ---------------------------------------------------------------------------
 extern "C" {
@@ -1535,6 +1574,30 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
                                 workspace_bytes, planes, (int)height, (int)width, (int)out_height,
                                 (int)out_width, (int)kernel_size, num_interp_pts, interp,
                                 (hipStream_t)stream));
+}
+
+int sdk_mapped_max_unpool_static(const void* grad_output, const int64_t* indices,
+                                 const void* sample_map, const void* interp_weights,
+                                 void* grad_input, int64_t batch, int64_t channels,
+                                 int64_t height, int64_t width, int64_t out_height,
+                                 int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
+                                 int32_t interp, int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(height >= 1 && width >= 1 && height * width < ((int64_t)1 << 31),
+              "mapped_max_unpool_static: bad plane size");
+  const size_t need = unpool_layout(unpool_tiling((int)height, (int)width));
+  if (need > kStaticUnpoolBytes)
+    return fail(SDK_ERR_WORKSPACE,
+                "mapped_max_unpool_static: a %lld x %lld plane needs %zu bytes of tile windows, "
+                "the built-in scratch holds %zu (%d tiles of %d pixels); use sdk_mapped_max_unpool "
+                "with a workspace",
+                (long long)height, (long long)width, need, kStaticUnpoolBytes, kStaticUnpoolTiles,
+                kUpTile);
+  void* ws = nullptr;
+  int rc = static_unpool_scratch(&ws);
+  if (rc) return rc;
+  return sdk_mapped_max_unpool(grad_output, indices, sample_map, interp_weights, grad_input, ws,
+                               kStaticUnpoolBytes, batch, channels, height, width, out_height,
+                               out_width, kernel_size, num_interp_pts, interp, dtype, stream);
 }
 
 int sdk_mapped_gather_at_index(const void* image, const int64_t* indices, const void* sample_map,
