@@ -114,7 +114,41 @@ def _conv_entry_points(torch, ops, x, m, iw, w, b, g, K, interp, compute):
     }, (ws, out, gi, gw, gb)
 
 
-def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
+def verify_conv4(torch, ops, cfg, t, compute):
+    """Outside the timed loop: the very tensors and launch shapes that were timed, compared
+    element-wise with the CPU oracle on sampled pixels (tests/sampled_parity.py: the oracle
+    evaluates the full image through the map sliced to those pixels).  Forward on both polar
+    row pairs, the seam columns and random pixels; grad_input, grad_weight and grad_bias for a
+    grad_output that is zero elsewhere; grad_input of the dense grad_output on sampled image
+    pixels.  Tolerances (max|a-b| / max|b|): forward 1e-5, backward 1e-4; 1e-2 with bf16
+    operands."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import sampled_parity as sp
+    from oracle import oracle
+    chk = sp.ConvOracle(oracle, cfg, n_random=512, n_targets=256, seed=4)
+    K, interp = cfg["kernel_size"], cfg["interp"]
+    x, m, iw, w, b, g = t
+    ops.set_conv_compute(compute)
+    try:
+        y = ops.mapped_conv_forward(x, m, iw, w, b, K, interp)
+        gs = torch.from_numpy(chk.g_sparse).to(x.device)
+        gi, gw, gb = ops.mapped_conv_backward(gs, m, iw, x, w, b, K, interp)
+        err = {"forward": chk.check_forward(y)}
+        err["grad_input"], err["grad_weight"], err["grad_bias"] = \
+            chk.check_backward_sparse(gi, gw, gb)
+        del gs, gi, gw, gb, y
+        gi, _, _ = ops.mapped_conv_backward(g, m, iw, x, w, b, K, interp)
+        err["grad_input_dense"] = chk.check_backward_dense(gi)
+    finally:
+        ops.set_conv_compute("native")
+    fwd, bwd = (1e-2, 1e-2) if compute == "bf16" else (1e-5, 1e-4)
+    ok = err["forward"] <= fwd and all(v <= bwd for k, v in err.items() if k != "forward")
+    return {"verified": bool(ok), "pixels": int(len(chk.pix)), "targets": int(len(chk.targets)),
+            "max_rel_err": {k: float("%.3g" % v) for k, v in err.items()},
+            "tolerance": {"forward": fwd, "backward": bwd}}
+
+
+def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8, verify=False):
     import workloads
     cfg = workloads.config4(batch=batch)
     dev = "cuda:0"
@@ -123,7 +157,8 @@ def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
     K, interp = cfg["kernel_size"], cfg["interp"]
     B, Cin, H, W = x.shape
     Cout = w.shape[0]
-    flops = 2.0 * Cout * Cin * K * H * W * B
+    OH, OW = m.shape[:2]
+    flops = 2.0 * Cout * Cin * K * OH * OW * B
     # the split mode delivers fp32 results, so it is priced against the fp32 peak like native
     peak = MFMA_BF16_TFLOPS if compute == "bf16" else MFMA_FP32_TFLOPS
     ops.set_conv_compute(compute)
@@ -143,8 +178,10 @@ def bench_conv4(torch, ops, timer, steps, warmup, compute="native", batch=8):
                                     if name != "bias_grad" else _roof("hbm", _nbytes(g), t)))
     del keep
     dominant = max(("forward", "backward_input", "backward_weight"), key=lambda n: parts[n]["ms"])
+    check = verify_conv4(torch, ops, cfg, (x, m, iw, w, b, g), compute) if verify else None
     return {"ms_per_step": ms, "ms_min": ms_min, "images_per_s": B / (ms * 1e-3),
-            "flops_per_contraction": flops, "parts": parts, "dominant": dominant}
+            "flops_per_contraction": flops, "parts": parts, "dominant": dominant,
+            "verification": check}
 
 
 def bench_conv1(torch, ops, timer, steps, warmup):
@@ -348,6 +385,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of: conv4,conv4_bf16,conv4_split,conv1,resample2,pool3,ico5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-verify", action="store_true",
+                    help="skip the oracle check of the timed configuration after the timed loop")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); "
@@ -365,7 +404,8 @@ def main():
     kernels = {}
     head = None
     if want("conv4"):
-        head = bench_conv4(torch, ops, timer, args.steps, args.warmup)
+        head = bench_conv4(torch, ops, timer, args.steps, args.warmup,
+                           verify=not args.no_verify)
         kernels["conv4_fp32"] = dict(ms_per_step=head["ms_per_step"],
                                      images_per_s=head["images_per_s"], **head["parts"])
         torch.cuda.empty_cache()
@@ -408,6 +448,9 @@ def main():
         roof["traffic"] = _measured_traffic(roof["kernel"])
         line.update(value=round(head["images_per_s"], 3), ms_per_step=round(head["ms_per_step"], 4),
                     roofline=roof)
+        if head["verification"] is not None:
+            line.update(verified=head["verification"]["verified"],
+                        verification=head["verification"])
     else:
         line.update(value=None, ms_per_step=None, roofline=None)
     if "conv4_split" in kernels:

@@ -53,7 +53,8 @@ __device__ __forceinline__ int xcd_band_tile(int bid, int ntiles) {
 }
 
 // ---------------------------------------------------------------------------
-// Tap table of one kernel sample k for TP consecutive pixels starting at pix0.
+// Tap table of one kernel sample k for the TP pixels of a tile; thread tid < TP owns pixel
+// `pix` (-1: no pixel).
 // Layout tap_off[slot][TP], tap_co[slot][TP] (slot-major, so lanes that own
 // consecutive pixels hit consecutive LDS banks).  Every pixel's active taps are
 // packed to the front; slots up to the tile-wide maximum *smax are padded with
@@ -61,7 +62,7 @@ __device__ __forceinline__ int xcd_band_tile(int bid, int ntiles) {
 // ---------------------------------------------------------------------------
 template <int INTERP, bool WEIGHTED, int TP>
 __device__ __forceinline__ void build_taps(const float* __restrict__ map,
-                                           const float* __restrict__ wts, int pix0, int M, int K,
+                                           const float* __restrict__ wts, int pix, int K,
                                            int k, int P, int H, int W, int* __restrict__ tap_off,
                                            float* __restrict__ tap_co, int* __restrict__ smax) {
   const int tid = threadIdx.x;
@@ -69,8 +70,7 @@ __device__ __forceinline__ void build_taps(const float* __restrict__ map,
   __syncthreads();
   int cnt = 0;
   if (tid < TP) {
-    const int pix = pix0 + tid;
-    if (pix < M) {
+    if (pix >= 0) {
       const int q = WEIGHTED ? P : 1;
       const size_t s = ((size_t)pix * K + k) * q;
       PointTaps<float, INTERP> t;
@@ -287,14 +287,21 @@ __global__ __launch_bounds__(kThreads) void relayout_weight_kernel(
 // INV: the tap lists do not come from the sample map but from an inverse map
 // (conv_inverse.hip): rows inv_off / inv_co [(pixel tile * K + k) * slots + s][TM] and
 // their count inv_ns[pixel tile * K + k].  The kernel does nothing unless *gate == 0.
+//
+// TILED (TM = 128): the workgroup's pixels are not TM consecutive ones but a 2-D tile of the
+// tiling pt, taken from a device-side list (tile_list[i], i < *tile_count): the tiles a
+// plan-driven kernel leaves to this one.
 // ---------------------------------------------------------------------------
-template <int INTERP, bool WEIGHTED, int TN, int TM, int MM, bool INV = false>
+template <int INTERP, bool WEIGHTED, int TN, int TM, int MM, bool INV = false, bool TILED = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const float* __restrict__ img, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wg, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
     int H, int W, int Cp, int M, int K, int P, int CgP, int CpP, int slots, int m_tiles,
     const int* __restrict__ inv_off = nullptr, const float* __restrict__ inv_co = nullptr,
-    const int* __restrict__ inv_ns = nullptr, const int* __restrict__ gate = nullptr) {
+    const int* __restrict__ inv_ns = nullptr, const int* __restrict__ gate = nullptr,
+    PixelTiling pt = PixelTiling(), const int* __restrict__ tile_list = nullptr,
+    const int* __restrict__ tile_count = nullptr) {
+  static_assert(!TILED || (TM == 128 && !INV), "tiled pixel order: 128-pixel tiles of a sample map");
   if constexpr (INV) {
     if (*gate != 0) return;
   }
@@ -310,8 +317,29 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   constexpr int RPT = kKC / SPLIT;           // column rows per thread and chunk
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n_tiles = CpP / TN;
-  const int tile = xcd_band_tile(blockIdx.x, m_tiles * n_tiles);
+  int tile = TILED ? 0 : xcd_band_tile(blockIdx.x, m_tiles * n_tiles);
+  // pixel (index into the pixel grid, -1: none) of tile-local pixel p
+  int ty0 = 0, tx0 = 0;
+  if constexpr (TILED) {
+    // XCD x (workgroup ids go round-robin over the 8 XCDs) takes an eighth of the list,
+    // however long the list is
+    const int cnt = *tile_count, per = (cnt + 7) >> 3;
+    const int wg = blockIdx.x / n_tiles, slot = (wg & 7) * per + (wg >> 3);
+    if ((wg >> 3) >= per || slot >= cnt) return;
+    tile = blockIdx.x % n_tiles;   // (only the n tile is taken from `tile` below)
+    const int t2 = tile_list[slot];
+    ty0 = (t2 / pt.tiles_x) * pt.TY();
+    tx0 = (t2 % pt.tiles_x) << pt.tx_shift;
+  }
   const int m0 = (tile / n_tiles) * TM, n0 = (tile % n_tiles) * TN;
+  auto pixel_of = [&](int p) -> int {
+    if constexpr (TILED) {
+      const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
+      return (oy < pt.OH && ox < pt.OW) ? oy * pt.OW + ox : -1;
+    } else {
+      return m0 + p < M ? m0 + p : -1;
+    }
+  };
   const int a_base = (wave % WAVES_N) * 64, b_base = (wave / WAVES_N) * 64;
   const size_t HW = (size_t)H * W;
   const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
@@ -332,7 +360,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
       }
       __syncthreads();
     } else {
-      build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+      build_taps<INTERP, WEIGHTED, TM>(map, wts, tid < TM ? pixel_of(tid) : -1, K, k, P, H, W,
+                                       tap_off, tap_co, smax);
     }
     const int ns = *smax;
     for (int c0 = 0; c0 < CgP; c0 += kKC) {
@@ -389,11 +418,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const int m = m0 + b_base + 32 * b + (lane & 31);
+      const int m = pixel_of(b_base + 32 * b + (lane & 31));
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int n = n0 + a_base + 32 * a + mfma_row(v, lane);
-        if (n < Cp && m < M) pix_b[(size_t)n * M + m] = acc[a][b][v] + (bias ? bias[n] : 0.0f);
+        if (n < Cp && m >= 0) pix_b[(size_t)n * M + m] = acc[a][b][v] + (bias ? bias[n] : 0.0f);
       }
     }
 }
@@ -429,7 +458,8 @@ __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
   const bool vec_ok = (M % 4 == 0);
 
   for (int k = 0; k < K; ++k) {
-    build_taps<INTERP, WEIGHTED, TM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    build_taps<INTERP, WEIGHTED, TM>(map, wts, m0 + tid < M ? m0 + tid : -1, K, k, P, H, W,
+                                     tap_off, tap_co, smax);
     const int ns = *smax;
     for (int c0 = 0; c0 < CgP; c0 += TC) {
       floatx16 acc[2][2];
@@ -531,7 +561,8 @@ __global__ __launch_bounds__(kThreads) void gather_wgrad_kernel(
   const int chunk_end = min(chunk_beg + chunks_per_range, (M + KM - 1) / KM);
   for (int ch = chunk_beg; ch < chunk_end; ++ch) {
     const int m0 = ch * KM;
-    build_taps<INTERP, WEIGHTED, KM>(map, wts, m0, M, K, k, P, H, W, tap_off, tap_co, smax);
+    build_taps<INTERP, WEIGHTED, KM>(map, wts, m0 + tid < M ? m0 + tid : -1, K, k, P, H, W,
+                                     tap_off, tap_co, smax);
     const int ns = *smax;
     // ---- gather columns for KM pixels x TC channels -> Bs[m][c]
     float col[CPT];
@@ -610,9 +641,26 @@ bool fused_supported(const ConvGeom& g) {
 static bool inverse_candidate(const ConvGeom& g);
 static size_t inverse_bytes(const ConvGeom& g);
 
+// Scratch of the forward-style contraction when it runs from the plan: the weight copy of the
+// global-gather kernel, the plan, the tile lists and the weight copy of the window kernel.
+struct GatherLayout {
+  size_t plan, lists, window_weights, total;
+};
+static GatherLayout gather_layout(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  GatherLayout l;
+  l.plan = up((size_t)g.K * round_up(g.Cp, 128) * round_up(g.Cg, 128) * sizeof(float));
+  l.lists = l.plan + up(plan_bytes(g));
+  l.window_weights = l.lists + up(tile_lists_bytes(g));
+  l.total = l.window_weights + up(window_gemm_weight_bytes(g));
+  return l;
+}
+static bool gather_from_window(const ConvGeom& g) { return window_gemm_supported(g) && g.Cp > 64; }
+
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
   size_t need = std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
+  if (gather_from_window(g)) need = std::max(need, gather_layout(g).total);
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
   if (planned_scatter_supported(g) && inverse_candidate(g))
     need = ((need + 255) & ~(size_t)255) + inverse_bytes(g);
@@ -665,9 +713,39 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
   const int CpP = round_up(g.Cp, TN), CgP = round_up(g.Cg, kKC);
   int rc = relayout(g, Wm, workspace, CpP, CgP, 2, stream);
   if (rc) return rc;
+  const size_t smem = sizeof(float) * kLdK * (TM + TN) + (size_t)slots * TM * 8 + 16;
+  if (gather_from_window(g)) {
+    // Tiles whose taps stay inside an LDS-sized window of the image are gathered from that
+    // window (window_gemm), the others (polar rows of a spherical map, incoherent maps) from
+    // global memory by the kernel below, which takes their list.
+    const GatherLayout l = gather_layout(g);
+    char* ws = reinterpret_cast<char*>(workspace);
+    Plan plan;
+    rc = build_plan(g, map, wts, ws + l.plan, stream, &plan);
+    if (rc) return rc;
+    TileLists tl;
+    rc = build_tile_lists(plan, ws + l.lists, stream, &tl);
+    if (rc) return rc;
+    rc = window_gemm(g, mm, plan, tl, img, Wm, bias, pix,
+                     reinterpret_cast<float*>(ws + l.window_weights), stream);
+    if (rc) return rc;
+    const dim3 grid_t((unsigned)(plan.tiles * (CpP / TN)), (unsigned)g.B);
+#define GT(BFv)                                                                                   \
+  SDK_DISPATCH_INTERP(g.interp, g.P,                                                              \
+                      (rc = launch_smem("gather_gemm(tiles)",                                     \
+                                        gather_gemm_kernel<INTERP, WEIGHTED, 128, 128, BFv, false, true>, \
+                                        grid_t, smem, stream, img, map, wts,                      \
+                                        (const float*)workspace, bias, pix, g.Cg, g.H, g.W, g.Cp, \
+                                        g.M, g.K, g.P, CgP, CpP, slots, plan.tiles,               \
+                                        (const int*)nullptr, (const float*)nullptr,               \
+                                        (const int*)nullptr, (const int*)nullptr, plan.pt,        \
+                                        tl.rest, tl.count + 1)))
+    if (mm == kMmBf16) GT(kMmBf16); else if (mm == kMmSplit) GT(kMmSplit); else GT(kMmF32);
+#undef GT
+    return rc;
+  }
   const int m_tiles = (int)ceil_div(g.M, TM), n_tiles = CpP / TN;
   const dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)g.B);
-  const size_t smem = sizeof(float) * kLdK * (TM + TN) + (size_t)slots * TM * 8 + 16;
 #define GG(TNv, TMv, BFv)                                                                          \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                          \
                       (rc = launch_smem("gather_gemm",                                        \
@@ -676,6 +754,7 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                                         bias, pix, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP,  \
                                         CpP, slots, m_tiles, (const int*)nullptr,             \
                                         (const float*)nullptr, (const int*)nullptr,           \
+                                        (const int*)nullptr, PixelTiling(), (const int*)nullptr, \
                                         (const int*)nullptr)))
   if (mm == kMmBf16) { if (narrow) GG(64, 256, kMmBf16); else GG(128, 128, kMmBf16); }
   else if (mm == kMmSplit) { if (narrow) GG(64, 256, kMmSplit); else GG(128, 128, kMmSplit); }
@@ -835,7 +914,8 @@ static int inverse_gather_gemm(const ConvGeom& g, int mm, const InverseMap& inv,
                    smem, stream, pix, (const float*)nullptr, (const float*)nullptr,              \
                    (const float*)inv.weights, bias, img, g.Cp, 1, g.M, g.Cg, HW, g.K, 0, CinP,   \
                    CoutP, kInvSlots, m_tiles, (const int*)inv.off, (const float*)inv.co,         \
-                   (const int*)inv.ns, (const int*)inv.gate)
+                   (const int*)inv.ns, (const int*)inv.gate, PixelTiling(), (const int*)nullptr, \
+                   (const int*)nullptr)
   if (mm == kMmBf16) { if (narrow) IG(64, 256, kMmBf16); else IG(128, 128, kMmBf16); }
   else if (mm == kMmSplit) { if (narrow) IG(64, 256, kMmSplit); else IG(128, 128, kMmSplit); }
   else { if (narrow) IG(64, 256, kMmF32); else IG(128, 128, kMmF32); }

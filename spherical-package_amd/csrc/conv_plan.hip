@@ -133,6 +133,10 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     hdr[tile * 8 + 1] = rg.rx0;
     hdr[tile * 8 + 2] = rg.RH;
     hdr[tile * 8 + 3] = rg.RW;
+    // the window is the whole bounding box of the taps unless that exceeded the capacity
+    const bool whole = bb[0] > bb[1] ||
+                       (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, W) <= kRegionCap;
+    hdr[tile * 8 + 4] = whole ? 1 : 0;
   }
   for (int k = tid; k < K; k += kPlThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
 

@@ -5,6 +5,7 @@
 // The pixel grid is cut into 2-D tiles of 128 pixels (PixelTiling).  For tile t:
 //   hdr[8*t + 0..3]  window of the image the tile's taps fall into: first row,
 //                    first column, rows, columns (columns wrap modulo W)
+//   hdr[8*t + 4]     1 when every active tap of the tile lies inside that window
 //   ns[t*K + k]      rows of kernel sample k: the largest number of active taps
 //                    any pixel of the tile has for that sample
 //   taps[((t*K + k)*S + r)*128 + p]   row r < ns of pixel p (tile-local index):
@@ -44,6 +45,24 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
 // gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
 // partial: planned_wgrad_partial_bytes(g) bytes (when that is not 0) in which the workgroups
 // leave their sums for a second, summing kernel; nullptr: they add to gW themselves.
+// The plan's tiles by class, on the device (conv_window_gemm.hip): those whose taps all lie
+// inside their window, in ascending order, and the others; count[0], count[1] entries.
+struct TileLists {
+  const int* inside;
+  const int* rest;
+  const int* count;
+};
+size_t tile_lists_bytes(const ConvGeom& g);
+int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out);
+
+// pix[b] = Wm x im2col(img[b]) + bias on the tiles of tl.inside, gathered from an LDS window.
+// weights: window_gemm_weight_bytes(g) bytes of scratch for the re-laid-out weight matrix.
+bool window_gemm_supported(const ConvGeom& g);
+size_t window_gemm_weight_bytes(const ConvGeom& g);
+int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
+                const float* img, const float* Wm, const float* bias, float* pix,
+                float* weights, hipStream_t stream);
+
 bool planned_wgrad_supported(const ConvGeom& g);
 size_t planned_wgrad_partial_bytes(const ConvGeom& g);
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,

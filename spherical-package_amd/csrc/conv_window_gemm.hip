@@ -1,0 +1,425 @@
+// Gather -> MFMA contraction from an LDS window, driven by a tap plan (gfx950, float32 tensors):
+//
+//   pix[b][n, m] = sum_{c, k} Wm[n, (c, k)] * col[b][(c, k), m] + bias[n]
+//   col[b][(c, k), m] = sum_r coefficient(m, k, r) * img[b][c][tap(m, k, r)]
+//
+// for the tiles of a plan (conv_plan.hpp) whose taps all fall into the tile's image window.
+// Those tiles never gather from global memory: per chunk of 32 image channels the window
+// (at most kRegionCap elements) is staged in LDS with the channels of one element side by
+// side, and the column values are produced straight into MFMA B fragments:
+//
+//   workgroup  = one 2-D tile of 128 pixels x TN = 32 * NB pixel-side channels x one batch element
+//   wave w     = pixels 32w .. 32w+31 of the tile x all TN channels (NB accumulators of 32 x 32)
+//   lane l     = pixel j = l % 32, reduction half h = l / 32
+//
+// v_mfma_f32_32x32x2_f32 step s contracts channels 2s + h, so a lane needs the 16 channels
+// {h, h+2, ...} of its pixel; v_mfma_f32_32x32x16_bf16 instruction t contracts channels
+// 16t + 8h + 0..7.  The window and the weight tile keep the 32 channels of a chunk in that
+// order (position 16h + s, or 16h + 8t + j), so a lane reads its 16 values of one tap, and its
+// 16 weights of one row n, as four 16-byte LDS reads.  Per kernel sample and chunk a wave issues
+// 16 NB MFMAs, 64 fused multiply-adds, about 16 + 4 NB LDS reads and no global gather; plan rows
+// (window index, coefficient) are read from global memory one sample ahead, weights are staged
+// through a double-buffered LDS tile, and there is one barrier per sample.
+//
+// Rows padded by the plan (coefficient 0) are pointed at a zero element behind the window, so
+// a non-finite image value never meets a zero coefficient.
+#include <hip/hip_runtime.h>
+
+#include "conv_fused.hpp"
+#include "conv_plan.hpp"
+#include "conv_window.hpp"
+#include "sdk_host.hpp"
+#include "sdk_mfma.hpp"
+
+namespace sdk {
+
+namespace {
+
+constexpr int kWgThreads = 256;
+constexpr int kWE = 36;   // floats per window element / weight row: 32 channels + 4 of skew
+
+// Position of channel c (0..31 inside its chunk) in a window element or weight row.
+__host__ __device__ constexpr int chunk_pos(int c, bool bf16) {
+  return bf16 ? 16 * ((c >> 3) & 1) + 8 * (c >> 4) + (c & 7) : 16 * (c & 1) + (c >> 1);
+}
+
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Wp[k][chunk][n][pos] (n padded to CpP, channels to whole chunks, zeros in the padding):
+// one (k, chunk, 128-row block) is 16 KB of consecutive memory.
+__global__ __launch_bounds__(kWgThreads) void window_weight_kernel(
+    const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int CpP,
+    int chunks, int bf16) {
+  const size_t total = (size_t)K * chunks * CpP * kCC;
+  for (size_t e = (size_t)blockIdx.x * kWgThreads + threadIdx.x; e < total;
+       e += (size_t)gridDim.x * kWgThreads) {
+    const int pos = (int)(e % kCC);
+    const int n = (int)((e / kCC) % CpP);
+    const size_t rest = e / ((size_t)kCC * CpP);
+    const int chunk = (int)(rest % chunks), k = (int)(rest / chunks);
+    // inverse of chunk_pos
+    const int hh = pos >> 4, lo = pos & 15;
+    const int cl = bf16 ? 16 * (lo >> 3) + 8 * hh + (lo & 7) : 2 * lo + hh;
+    const int c = chunk * kCC + cl;
+    out[e] = (n < Cp && c < Cg) ? Wm[(size_t)n * Cg * K + (size_t)c * K + k] : 0.0f;
+  }
+}
+
+// Splits the plan's tiles into those whose taps all lie inside their window (hdr[8t+4] != 0)
+// and the rest, both in ascending tile order.  One workgroup.
+//   lists[0 .. tiles)         tiles inside their window, count[0] of them
+//   lists[tiles .. 2*tiles)   the others, count[1] of them
+__global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict__ hdr, int tiles,
+                                                          int* __restrict__ lists,
+                                                          int* __restrict__ count) {
+  __shared__ int wave_fit[16], wave_rest[16];
+  __shared__ int base[2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) base[0] = base[1] = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < tiles; t0 += 1024) {
+    const int t = t0 + tid;
+    const bool live = t < tiles;
+    const bool fit = live && hdr[t * 8 + 4] != 0;
+    const unsigned long long mf = __ballot(fit), mr = __ballot(live && !fit);
+    if (lane == 0) {
+      wave_fit[wave] = __popcll(mf);
+      wave_rest[wave] = __popcll(mr);
+    }
+    __syncthreads();
+    int of = base[0], orr = base[1];
+    for (int w = 0; w < wave; ++w) {
+      of += wave_fit[w];
+      orr += wave_rest[w];
+    }
+    const unsigned long long below = (1ull << lane) - 1ull;
+    if (fit) lists[of + __popcll(mf & below)] = t;
+    else if (live) lists[tiles + orr + __popcll(mr & below)] = t;
+    __syncthreads();
+    if (tid == 0) {
+      int a = 0, b = 0;
+      for (int w = 0; w < 16; ++w) {
+        a += wave_fit[w];
+        b += wave_rest[w];
+      }
+      base[0] += a;
+      base[1] += b;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    count[0] = base[0];
+    count[1] = base[1];
+  }
+}
+
+
+template <int MM, int NB>
+__global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
+    const float* __restrict__ img, const int* __restrict__ hdr, const int* __restrict__ ns,
+    const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
+    const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
+    int H, int W, int Cp, int K, int S, int CpP, int chunks, PixelTiling pt, int tiles,
+    int n_tiles) {
+  constexpr bool BF16 = MM != kMmF32;
+  constexpr int TN = 32 * NB;
+  __shared__ __align__(16) float region[(kRegionCap + 1) * kWE];
+  __shared__ __align__(16) float As[2][TN * kWE];
+  __shared__ int src[kRegionCap];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int j = lane & 31, h = lane >> 5;
+  // Workgroup ids go round-robin over the 8 XCDs (each with its own L2): XCD x takes the
+  // list entries [x * per, (x + 1) * per), so neighbouring tiles meet in one L2 and every XCD
+  // gets the same share of the list however long it is.
+  const int cnt = *count;
+  const int per = (cnt + 7) >> 3;
+  const int wg = blockIdx.x / n_tiles;
+  const int slot = (wg & 7) * per + (wg >> 3);
+  if ((wg >> 3) >= per || slot >= cnt) return;
+  const int tile = list[slot];
+  const int n0 = (blockIdx.x % n_tiles) * TN;
+  const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
+  const int M = pt.OH * pt.OW;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
+
+  Region rg;
+  rg.ry0 = hdr[tile * 8 + 0];
+  rg.rx0 = hdr[tile * 8 + 1];
+  rg.RH = hdr[tile * 8 + 2];
+  rg.RW = hdr[tile * 8 + 3];
+  rg.RS = rg.RH * rg.RW;
+  rg.RSp = rg.RS;
+  const int RS = rg.RS;
+  build_region_lut(rg, H, W, src);
+  if (tid < kWE) region[RS * kWE + tid] = 0.0f;   // the zero element padded rows point at
+
+  // this lane's pixel and its plan rows: row r of sample k at rows_p[(k * S + r) * 128]
+  const int p_local = 32 * wave + j;
+  const int2* rows_p = taps + (size_t)tile * K * S * 128 + p_local;
+  const int* ns_t = ns + (size_t)tile * K;
+
+  floatx16 acc[NB];
+#pragma unroll
+  for (int a = 0; a < NB; ++a)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[a][v] = 0.0f;
+
+  // weight tile of (k, chunk): TN rows of 32 values, 16-byte pieces e = tid + 256 i
+  constexpr int WPT = TN * kCC / 4 / kWgThreads;   // float4 per thread: 4 (TN = 128) or 2
+  static_assert(WPT == 4 || WPT == 2, "weight tile of 128 or 64 rows");
+  float4 w0, w1, w2, w3;   // (named registers: an array here ends up in scratch memory)
+  w0 = w1 = w2 = w3 = make_float4(0.f, 0.f, 0.f, 0.f);
+#define SDK_LOAD_WEIGHTS(kv, chunkv)                                              \
+  do {                                                                            \
+    const float4* srcw = reinterpret_cast<const float4*>(                         \
+        Wp + (((size_t)(kv) * chunks + (chunkv)) * CpP + n0) * kCC) + tid;        \
+    w0 = srcw[0];                                                                 \
+    w1 = srcw[kWgThreads];                                                        \
+    if constexpr (WPT == 4) {                                                     \
+      w2 = srcw[2 * kWgThreads];                                                  \
+      w3 = srcw[3 * kWgThreads];                                                  \
+    }                                                                             \
+  } while (0)
+#define SDK_STORE_WEIGHTS(bufv)                                                   \
+  do {                                                                            \
+    float* dstw = &As[bufv][(tid >> 3) * kWE + 4 * (tid & 7)];                    \
+    *reinterpret_cast<float4*>(dstw) = w0;                                        \
+    *reinterpret_cast<float4*>(dstw + 32 * kWE) = w1;                             \
+    if constexpr (WPT == 4) {                                                     \
+      *reinterpret_cast<float4*>(dstw + 64 * kWE) = w2;                           \
+      *reinterpret_cast<float4*>(dstw + 96 * kWE) = w3;                           \
+    }                                                                             \
+  } while (0)
+
+  // Plan rows of one sample: the first four are requested a whole sample ahead, without
+  // conditions (rows past the sample's count re-read its last slot and are masked when they
+  // are used), so that no branch and no wait sits between a request and the MFMAs that cover
+  // its latency.  Samples with more than four rows fetch the others when they need them.
+  constexpr int RB = 4;
+  int2 rows[RB], rows_next[RB];
+#define SDK_LOAD_ROWS(dst, kv, r0v)                                               \
+  do {                                                                            \
+    _Pragma("unroll") for (int u = 0; u < RB; ++u)                                \
+      dst[u] = rows_p[((size_t)(kv) * S + min((r0v) + u, S - 1)) * 128];          \
+  } while (0)
+  // col[] += the taps of up to four rows
+#define SDK_GATHER_ROWS(src, r0v)                                                 \
+  do {                                                                            \
+    int e[RB];                                                                    \
+    float co[RB];                                                                 \
+    _Pragma("unroll") for (int u = 0; u < RB; ++u) {                              \
+      co[u] = (r0v) + u < n_rows ? __int_as_float(src[u].y) : 0.0f;               \
+      e[u] = co[u] != 0.0f ? src[u].x : RS;                                       \
+    }                                                                             \
+    _Pragma("unroll") for (int u = 0; u < RB; ++u) {                              \
+      const float4* rp = reinterpret_cast<const float4*>(region + e[u] * kWE + 16 * h); \
+      const float4 d0 = rp[0], d1 = rp[1], d2 = rp[2], d3 = rp[3];                \
+      const float d[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w,        \
+                           d2.x, d2.y, d2.z, d2.w, d3.x, d3.y, d3.z, d3.w};       \
+      _Pragma("unroll") for (int i = 0; i < 16; ++i)                              \
+        colv[i] = __builtin_fmaf(co[u], d[i], colv[i]);                           \
+    }                                                                             \
+  } while (0)
+
+  int buf = 0;
+  SDK_LOAD_WEIGHTS(0, 0);
+  int n_rows = ns_t[0];
+  SDK_LOAD_ROWS(rows, 0, 0);
+  for (int chunk = 0; chunk < chunks; ++chunk) {
+    const int c0 = chunk * kCC;
+    __syncthreads();   // every wave is done with the previous chunk's window (and src is built)
+    {
+      // wave w stages channels 8w .. 8w+7 of every window element; a lane owns elements
+      // lane, lane + 64, ... and has all its loads in flight before the first LDS write
+      constexpr int ITER = (kRegionCap + 63) / 64;
+      const int cw = c0 + 8 * wave;
+      const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
+      const unsigned plane = (unsigned)HW * 4u;
+      float v[ITER][8];
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        const int o = e < RS ? src[e] : -1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const bool ok = o >= 0 && cw + i < Cg;
+          const float d = *reinterpret_cast<const float*>(
+              cbase + (ok ? (unsigned)i * plane + (unsigned)o * 4u : 0u));
+          v[it][i] = ok ? d : 0.0f;
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        if (e < RS) {
+          float* dst = region + e * kWE;
+          if constexpr (BF16) {
+            float4* d4 = reinterpret_cast<float4*>(dst + 16 * (wave & 1) + 8 * (wave >> 1));
+            d4[0] = make_float4(v[it][0], v[it][1], v[it][2], v[it][3]);
+            d4[1] = make_float4(v[it][4], v[it][5], v[it][6], v[it][7]);
+          } else {
+            *reinterpret_cast<float4*>(dst + 4 * wave) =
+                make_float4(v[it][0], v[it][2], v[it][4], v[it][6]);
+            *reinterpret_cast<float4*>(dst + 16 + 4 * wave) =
+                make_float4(v[it][1], v[it][3], v[it][5], v[it][7]);
+          }
+        }
+      }
+    }
+    if (chunk == 0) SDK_STORE_WEIGHTS(buf);   // (later chunks: stored behind the previous chunk's last sample)
+    __syncthreads();
+
+    for (int k = 0; k < K; ++k) {
+      // ---- request the next sample's weights and first rows (after the last sample of the
+      // last chunk: the first ones again, unused)
+      const bool last_k = k + 1 == K;
+      const int kn = last_k ? 0 : k + 1;
+      const int chunk_n = last_k ? (chunk + 1 < chunks ? chunk + 1 : 0) : chunk;
+      SDK_LOAD_WEIGHTS(kn, chunk_n);
+      SDK_LOAD_ROWS(rows_next, kn, 0);
+      const int n_rows_next = ns_t[kn];
+      asm volatile("" ::: "memory");   // the requests stay here, ahead of the gather and the MFMAs
+
+      // ---- gather: col[c][pixel j] for this lane's 16 channels of the chunk
+      float colv[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) colv[i] = 0.0f;
+      SDK_GATHER_ROWS(rows, 0);
+      if (n_rows > RB) {
+        for (int r0 = RB; r0 < n_rows; r0 += RB) {
+          int2 more[RB];
+          SDK_LOAD_ROWS(more, k, r0);
+          SDK_GATHER_ROWS(more, r0);
+        }
+      }
+      // ---- contraction
+      const float* at = &As[buf][j * kWE + 16 * h];
+      if constexpr (MM == kMmF32) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float4 aq[NB];
+#pragma unroll
+          for (int a = 0; a < NB; ++a)
+            aq[a] = *reinterpret_cast<const float4*>(at + a * 32 * kWE + 4 * q);
+#pragma unroll
+          for (int a = 0; a < NB; ++a) {
+            acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[a].x, colv[4 * q + 0], acc[a], 0, 0, 0);
+            acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[a].y, colv[4 * q + 1], acc[a], 0, 0, 0);
+            acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[a].z, colv[4 * q + 2], acc[a], 0, 0, 0);
+            acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[a].w, colv[4 * q + 3], acc[a], 0, 0, 0);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const float fb[8] = {colv[8 * t + 0], colv[8 * t + 1], colv[8 * t + 2], colv[8 * t + 3],
+                               colv[8 * t + 4], colv[8 * t + 5], colv[8 * t + 6], colv[8 * t + 7]};
+          Bf16Frag b16;
+          Bf16Split b3;
+          if constexpr (MM == kMmSplit) b3 = split_bf16x8(fb);
+          else b16 = pack_bf16x8(fb);
+#pragma unroll
+          for (int a = 0; a < NB; ++a) {
+            const float4 lo = *reinterpret_cast<const float4*>(at + a * 32 * kWE + 8 * t);
+            const float4 hi = *reinterpret_cast<const float4*>(at + a * 32 * kWE + 8 * t + 4);
+            const float fa[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            if constexpr (MM == kMmSplit) acc[a] = mfma_split(split_bf16x8(fa), b3, acc[a]);
+            else acc[a] = mfma_bf16(pack_bf16x8(fa), b16, acc[a]);
+          }
+        }
+      }
+      SDK_STORE_WEIGHTS(buf ^ 1);
+      lds_barrier();
+      buf ^= 1;
+      n_rows = n_rows_next;
+#pragma unroll
+      for (int u = 0; u < RB; ++u) rows[u] = rows_next[u];
+    }
+  }
+  // ---- epilogue: + bias, store.  Accumulator register v of lane l: row 8*(v/4) + 4*h + v%4
+  // (pixel-side channel), column j (pixel).
+  const int oy = ty0 + (p_local >> pt.tx_shift), ox = tx0 + (p_local & (pt.TX() - 1));
+  if (oy < pt.OH && ox < pt.OW) {
+    float* out = pix + (size_t)blockIdx.y * Cp * M + (size_t)oy * pt.OW + ox;
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (n < Cp) out[(size_t)n * M] = acc[a][v] + (bias ? bias[n] : 0.0f);
+      }
+  }
+#undef SDK_LOAD_WEIGHTS
+#undef SDK_STORE_WEIGHTS
+#undef SDK_LOAD_ROWS
+#undef SDK_GATHER_ROWS
+}
+
+}  // namespace
+
+
+bool window_gemm_supported(const ConvGeom& g) {
+  return plan_supported(g) && g.Cp > 32 && g.B <= 65535 &&
+         (int64_t)g.H * g.W <= ((int64_t)1 << 24);
+}
+
+size_t window_gemm_weight_bytes(const ConvGeom& g) {
+  const size_t CpP = (size_t)(g.Cp + 127) / 128 * 128;
+  const size_t chunks = (size_t)(g.Cg + kCC - 1) / kCC;
+  return (size_t)g.K * chunks * CpP * kCC * sizeof(float);
+}
+
+size_t tile_lists_bytes(const ConvGeom& g) {
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  return ((size_t)2 * pt.tiles_x * pt.tiles_y + 2) * sizeof(int);
+}
+
+int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out) {
+  int* lists = static_cast<int*>(workspace);
+  int* count = lists + (size_t)2 * plan.tiles;
+  launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles, lists, count);
+  SDK_LAUNCH_CHECK("tile_lists");
+  out->inside = lists;
+  out->rest = lists + plan.tiles;
+  out->count = count;
+  return SDK_OK;
+}
+
+int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
+                const float* img, const float* Wm, const float* bias, float* pix,
+                float* weights, hipStream_t stream) {
+  const int CpP = (g.Cp + 127) / 128 * 128;
+  const int chunks = (g.Cg + kCC - 1) / kCC;
+  {
+    const size_t total = (size_t)g.K * chunks * CpP * kCC;
+    const int blocks = (int)std::min<size_t>((total + kWgThreads - 1) / kWgThreads, 2048);
+    launch(window_weight_kernel, dim3(blocks), dim3(kWgThreads), stream, Wm, weights, g.Cp, g.Cg,
+           g.K, CpP, chunks, mm != kMmF32 ? 1 : 0);
+    SDK_LAUNCH_CHECK("window_weight");
+  }
+  const bool wide = g.Cp > 64;
+  const int TN = wide ? 128 : 64;
+  const int n_tiles = (int)ceil_div(g.Cp, TN);
+  const dim3 grid((unsigned)(plan.tiles * n_tiles), (unsigned)g.B);
+#define WG2(MMv, NBv)                                                                          \
+  launch(window_gemm_kernel<MMv, NBv>, grid, dim3(kWgThreads), stream, img, plan.hdr, plan.ns, \
+         plan.taps, (const int*)tl.inside, (const int*)tl.count, (const float*)weights, bias,  \
+         pix, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles)
+#define WG1(MMv)                              \
+  do {                                        \
+    if (wide) WG2(MMv, 4); else WG2(MMv, 2);  \
+  } while (0)
+  if (mm == kMmBf16) WG1(kMmBf16);
+  else if (mm == kMmSplit) WG1(kMmSplit);
+  else WG1(kMmF32);
+#undef WG1
+#undef WG2
+  SDK_LAUNCH_CHECK("window_gemm");
+  return SDK_OK;
+}
+
+}  // namespace sdk
