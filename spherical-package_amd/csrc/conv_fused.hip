@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const int* __restrict__ inv_ns = nullptr, const int* __restrict__ gate = nullptr,
     PixelTiling pt = PixelTiling(), const int* __restrict__ tile_list = nullptr,
     const int* __restrict__ tile_count = nullptr) {
-  static_assert(!TILED || (TM == 128 && !INV), "tiled pixel order: 128-pixel tiles of a sample map");
+  static_assert(!TILED || TM == 128, "tiled pixel order: 128-pixel tiles");
   if constexpr (INV) {
     if (*gate != 0) return;
   }
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   const int n_tiles = CpP / TN;
   int tile = TILED ? 0 : xcd_band_tile(blockIdx.x, m_tiles * n_tiles);
   // pixel (index into the pixel grid, -1: none) of tile-local pixel p
-  int ty0 = 0, tx0 = 0;
+  int ty0 = 0, tx0 = 0, ptile = 0;   // ptile: the pixel tile whose inverse rows are read
   if constexpr (TILED) {
     // XCD x (workgroup ids go round-robin over the 8 XCDs) takes an eighth of the list,
     // however long the list is
@@ -330,6 +330,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const int t2 = tile_list[slot];
     ty0 = (t2 / pt.tiles_x) * pt.TY();
     tx0 = (t2 % pt.tiles_x) << pt.tx_shift;
+    ptile = t2;
+  } else {
+    ptile = tile / n_tiles;
   }
   const int m0 = (tile / n_tiles) * TM, n0 = (tile % n_tiles) * TN;
   auto pixel_of = [&](int p) -> int {
@@ -350,8 +353,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
 
   for (int k = 0; k < K; ++k) {
     if constexpr (INV) {
-      const size_t rows = ((size_t)(tile / n_tiles) * K + k) * slots * TM;
-      if (tid == 0) *smax = min(inv_ns[(size_t)(tile / n_tiles) * K + k], slots);
+      const size_t rows = ((size_t)ptile * K + k) * slots * TM;
+      if (tid == 0) *smax = min(inv_ns[(size_t)ptile * K + k], slots);
       __syncthreads();
       for (int e = tid; e < *smax * TM; e += kThreads) {
         const float co = inv_co[rows + e];
@@ -726,10 +729,10 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
     TileLists tl;
     rc = build_tile_lists(plan, ws + l.lists, stream, &tl);
     if (rc) return rc;
-    rc = window_gemm(g, mm, plan, tl, img, Wm, bias, pix,
-                     reinterpret_cast<float*>(ws + l.window_weights), stream);
+    rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
+                     reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream);
     if (rc) return rc;
-    const dim3 grid_t((unsigned)(plan.tiles * (CpP / TN)), (unsigned)g.B);
+    const dim3 grid_t((unsigned)((plan.tiles + 7) / 8 * 8 * (CpP / TN)), (unsigned)g.B);
 #define GT(BFv)                                                                                   \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                              \
                       (rc = launch_smem("gather_gemm(tiles)",                                     \
@@ -858,7 +861,43 @@ static void inverse_layout(const ConvGeom& g, size_t (&off)[7]) {
   off[6] = off[5] + up((size_t)g.K * round_up(g.Cp, kKC) * round_up(g.Cg, TN) * 4);
 }
 
+// The scatter's geometry seen as the gather it becomes over the inverse plan: the pixel-side
+// tensor is gathered (planes of OH x OW), the image side is produced.
+static ConvGeom inverse_geom(const ConvGeom& g) {
+  ConvGeom r = g;
+  r.Cg = g.Cp;
+  r.H = g.M / g.OW;
+  r.W = g.OW;
+  r.Cp = g.Cg;
+  r.M = g.H * g.W;
+  r.OW = g.W;
+  r.P = kInversePlanRows / 4;   // plan rows per sample: kInversePlanRows (bilinear slots x P)
+  r.interp = 1;
+  return r;
+}
+static bool scatter_from_window(const ConvGeom& g) {
+  return g.Cg > 64 && g.M % g.OW == 0 && window_gemm_supported(inverse_geom(g)) &&
+         (int64_t)g.H * g.W * g.K < ((int64_t)1 << 31);
+}
+// Scratch of the scatter run from the inverse plan (behind the forward plan's region).
+struct ScatterLayout {
+  size_t inverse, lists, window_weights, gather_weights, total;
+};
+static ScatterLayout scatter_layout(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  const ConvGeom r = inverse_geom(g);
+  ScatterLayout l;
+  l.inverse = 0;
+  l.lists = up(inverse_plan_bytes(g));
+  l.window_weights = l.lists + up(tile_lists_bytes(r));
+  l.gather_weights = l.window_weights + up(window_gemm_weight_bytes(r));
+  l.total = l.gather_weights +
+            up((size_t)g.K * round_up(g.Cp, kKC) * round_up(g.Cg, 128) * sizeof(float));
+  return l;
+}
+
 static size_t inverse_bytes(const ConvGeom& g) {
+  if (scatter_from_window(g)) return scatter_layout(g).total;
   size_t off[7];
   inverse_layout(g, off);
   return off[6];
@@ -936,12 +975,46 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
       // and the fill and the scatter kernel below run instead (and vice versa).
       const size_t base = ((staged_workspace_bytes(g) + 255) & ~(size_t)255) + plan_bytes(g);
       char* inv_ws = reinterpret_cast<char*>(workspace) + ((base + 255) & ~(size_t)255);
-      InverseMap inv;
-      rc = build_inverse(g, map, wts, inv_ws, stream, &inv);
-      if (rc) return rc;
-      rc = inverse_gather_gemm(g, matrix_mode(compute), inv, pix, Wm, bias, img, stream);
-      if (rc) return rc;
-      gate = inv.gate;
+      if (scatter_from_window(g)) {
+        // the inverse lists as a plan: image tiles whose sources stay inside a window of the
+        // pixel grid gather from LDS, the others from global memory
+        const int mm = matrix_mode(compute);
+        const ScatterLayout l = scatter_layout(g);
+        const ConvGeom r = inverse_geom(g);
+        InversePlan ip;
+        rc = build_inverse_plan(g, map, wts, inv_ws + l.inverse, stream, &ip);
+        if (rc) return rc;
+        TileLists tl;
+        rc = build_tile_lists(ip.plan, inv_ws + l.lists, stream, &tl);
+        if (rc) return rc;
+        rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
+                         reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream);
+        if (rc) return rc;
+        float* gw = reinterpret_cast<float*>(inv_ws + l.gather_weights);
+        const int CoutP = round_up(g.Cg, 128), CinP = round_up(g.Cp, kKC);
+        rc = relayout(g, Wm, gw, CoutP, CinP, 3, stream);
+        if (rc) return rc;
+        const dim3 grid_t((unsigned)((ip.plan.tiles + 7) / 8 * 8 * (CoutP / 128)), (unsigned)g.B);
+        const size_t smem = sizeof(float) * kLdK * (128 + 128) + (size_t)kInversePlanRows * 128 * 8 + 16;
+#define IT(BFv)                                                                                  \
+  rc = launch_smem("inverse_gather_gemm(tiles)",                                                 \
+                   gather_gemm_kernel<0, false, 128, 128, BFv, true, true>, grid_t, smem, stream, \
+                   pix, (const float*)nullptr, (const float*)nullptr, (const float*)gw, bias,    \
+                   img, g.Cp, 1, g.M, g.Cg, g.H * g.W, g.K, 0, CinP, CoutP, kInversePlanRows,    \
+                   ip.plan.tiles, (const int*)ip.raw_off, (const float*)ip.raw_co,               \
+                   (const int*)ip.plan.ns, (const int*)ip.gate, ip.plan.pt, tl.rest, tl.count + 1)
+        if (mm == kMmBf16) IT(kMmBf16); else if (mm == kMmSplit) IT(kMmSplit); else IT(kMmF32);
+#undef IT
+        if (rc) return rc;
+        gate = ip.gate;
+      } else {
+        InverseMap inv;
+        rc = build_inverse(g, map, wts, inv_ws, stream, &inv);
+        if (rc) return rc;
+        rc = inverse_gather_gemm(g, matrix_mode(compute), inv, pix, Wm, bias, img, stream);
+        if (rc) return rc;
+        gate = inv.gate;
+      }
     }
     rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream, gate);
     if (rc) return rc;

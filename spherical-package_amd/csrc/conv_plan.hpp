@@ -56,12 +56,29 @@ size_t tile_lists_bytes(const ConvGeom& g);
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out);
 
 // pix[b] = Wm x im2col(img[b]) + bias on the tiles of tl.inside, gathered from an LDS window.
-// weights: window_gemm_weight_bytes(g) bytes of scratch for the re-laid-out weight matrix.
+// g: the contraction's geometry (gather side = img).  swapped: Wm is [Cg, Cp * K] instead of
+// [Cp, Cg * K].  weights: window_gemm_weight_bytes(g) bytes of scratch for the re-laid-out
+// weight matrix.  gate (optional): the kernel runs only if *gate == 0.
 bool window_gemm_supported(const ConvGeom& g);
 size_t window_gemm_weight_bytes(const ConvGeom& g);
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
-                const float* img, const float* Wm, const float* bias, float* pix,
-                float* weights, hipStream_t stream);
+                const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
+                float* weights, const int* gate, hipStream_t stream);
+
+// The scatter of geometry g regrouped by target as a plan over tiles of the image grid, whose
+// windows lie in the pixel grid; valid only if *gate == 0 after it was built (a target with
+// more than kInversePlanRows sources per sample raises it).  The raw lists (source pixel,
+// coefficient; rows of 128 tile pixels like the plan's) serve the global-gather kernel.
+constexpr int kInversePlanRows = 16;
+struct InversePlan {
+  Plan plan;
+  int* gate;
+  const int* raw_off;
+  const float* raw_co;
+};
+size_t inverse_plan_bytes(const ConvGeom& g);
+int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+                       hipStream_t stream, InversePlan* out);
 
 bool planned_wgrad_supported(const ConvGeom& g);
 size_t planned_wgrad_partial_bytes(const ConvGeom& g);

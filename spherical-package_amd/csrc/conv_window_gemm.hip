@@ -49,9 +49,11 @@ __device__ __forceinline__ void lds_barrier() {
 
 // Wp[k][chunk][n][pos] (n padded to CpP, channels to whole chunks, zeros in the padding):
 // one (k, chunk, 128-row block) is 16 KB of consecutive memory.
+// swapped: the roles of the two channel indices of Wm are exchanged (Wm is [Cg, Cp * K]): the
+// contraction over the inverse plan gathers the pixel side and produces the image side.
 __global__ __launch_bounds__(kWgThreads) void window_weight_kernel(
     const float* __restrict__ Wm, float* __restrict__ out, int Cp, int Cg, int K, int CpP,
-    int chunks, int bf16) {
+    int chunks, int bf16, int swapped) {
   const size_t total = (size_t)K * chunks * CpP * kCC;
   for (size_t e = (size_t)blockIdx.x * kWgThreads + threadIdx.x; e < total;
        e += (size_t)gridDim.x * kWgThreads) {
@@ -63,7 +65,172 @@ __global__ __launch_bounds__(kWgThreads) void window_weight_kernel(
     const int hh = pos >> 4, lo = pos & 15;
     const int cl = bf16 ? 16 * (lo >> 3) + 8 * hh + (lo & 7) : 2 * lo + hh;
     const int c = chunk * kCC + cl;
-    out[e] = (n < Cp && c < Cg) ? Wm[(size_t)n * Cg * K + (size_t)c * K + k] : 0.0f;
+    float v = 0.0f;
+    if (n < Cp && c < Cg)
+      v = swapped ? Wm[(size_t)c * Cp * K + (size_t)n * K + k]
+                  : Wm[(size_t)n * Cg * K + (size_t)c * K + k];
+    out[e] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Inverse plan.  The scatter  img[u] += co * v[m, k]  over all taps (m, k) -> u, regrouped by
+// target u, is a gather over the pixel-side tensor: per image pixel u and sample k a list of
+// (source pixel m, coefficient) pairs.  The lists are collected with integer atomics
+// (inverse_fill_tiled_kernel: at most kInvRows entries per list, *gate counts the taps that
+// found theirs full) in tiles of the image grid, then turned into a plan whose windows lie
+// in the pixel grid (inverse_plan_kernel), so the same window kernel runs the contraction.
+// Lists are sorted by source pixel: the summation order does not depend on the order in
+// which the atomics were served.
+//   raw_off / raw_co [((tile * K + k) * kInvRows + slot) * 128 + p]   p: tile-local image pixel
+//   cnt[u * K + k]                                                    entries of (u, k)
+// ---------------------------------------------------------------------------
+constexpr int kInvRows = kInversePlanRows;
+
+template <int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kWgThreads) void inverse_fill_tiled_kernel(
+    const float* __restrict__ map, const float* __restrict__ wts, int M, int K, int P, int H, int W,
+    PixelTiling it, int* __restrict__ cnt, int* __restrict__ raw_off, float* __restrict__ raw_co,
+    int* __restrict__ gate) {
+  const size_t i = (size_t)blockIdx.x * kWgThreads + threadIdx.x;
+  if (i >= (size_t)M * K) return;
+  const int m = (int)(i / K), k = (int)(i % K);
+  const int q = WEIGHTED ? P : 1;
+  PointTaps<float, INTERP> t;
+  for (int p = 0; p < q; ++p) {
+    const size_t s = i * q + p;
+    t.set(map[s * 2], map[s * 2 + 1], H, W);
+    const float wt = WEIGHTED ? wts[s] : 1.0f;
+#pragma unroll
+    for (int jj = 0; jj < PointTaps<float, INTERP>::N; ++jj) {
+      const float co = WEIGHTED ? wt * t.w[jj] : t.w[jj];
+      if (t.off[jj] >= 0 && co != 0.0f) {
+        const int u = t.off[jj], uy = t.ty[jj], ux = t.tx[jj];
+        const int slot = atomicAdd(&cnt[(size_t)u * K + k], 1);
+        if (slot < kInvRows) {
+          const int tile = (uy / it.TY()) * it.tiles_x + (ux >> it.tx_shift);
+          const int pl = (uy % it.TY()) * it.TX() + (ux & (it.TX() - 1));
+          const size_t e = (((size_t)tile * K + k) * kInvRows + slot) * 128 + pl;
+          raw_off[e] = m;
+          raw_co[e] = co;
+        } else {
+          atomicAdd(gate, 1);
+        }
+      }
+    }
+  }
+}
+
+// One workgroup per image tile; thread = (tile pixel p, parity of the sample).  Writes the
+// plan of the tile (conv_plan.hpp; windows in the OH x OW pixel grid, columns modulo OW) and
+// sorts the tile's raw lists by source pixel in place.
+__global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
+    const int* __restrict__ cnt, int* __restrict__ raw_off, float* __restrict__ raw_co,
+    PixelTiling it, int K, int OH, int OW, int* __restrict__ hdr, int* __restrict__ ns_out,
+    int2* __restrict__ taps, const int* __restrict__ gate) {
+  if (*gate != 0) return;
+  __shared__ int bb[4];
+  __shared__ int ns_l[kPlanKMax];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int tile = blockIdx.x;
+  const int ty0 = (tile / it.tiles_x) * it.TY(), tx0 = (tile % it.tiles_x) << it.tx_shift;
+  const int p = tid & 127, kpar = tid >> 7;
+  const int uy = ty0 + (p >> it.tx_shift), ux = tx0 + (p & (it.TX() - 1));
+  const bool pix_ok = uy < it.OH && ux < it.OW;
+  const int u = uy * it.OW + ux;
+  // anchor: the tile's first pixel, scaled to the pixel grid
+  const int ay = min((int)((long long)ty0 * OH / it.OH), OH - 1);
+  const int ax = min((int)((long long)tx0 * OW / it.OW), OW - 1);
+  for (int k = tid; k < K; k += kWgThreads) ns_l[k] = 0;
+  if (tid == 0) {
+    bb[0] = INT_MAX;
+    bb[1] = INT_MIN;
+    bb[2] = INT_MAX;
+    bb[3] = INT_MIN;
+  }
+  __syncthreads();
+
+  int dy0 = INT_MAX, dy1 = INT_MIN, dx0 = INT_MAX, dx1 = INT_MIN;
+  for (int k = kpar; k < K; k += 2) {
+    const int n = pix_ok ? min(cnt[(size_t)u * K + k], kInvRows) : 0;
+    int* ro = raw_off + ((size_t)tile * K + k) * kInvRows * 128 + p;
+    float* rc = raw_co + ((size_t)tile * K + k) * kInvRows * 128 + p;
+    // insertion sort by source pixel (n <= 16)
+    int so[kInvRows];
+    float sc[kInvRows];
+#pragma unroll
+    for (int a = 0; a < kInvRows; ++a) {
+      so[a] = a < n ? ro[a * 128] : INT_MAX;
+      sc[a] = a < n ? rc[a * 128] : 0.0f;
+    }
+#pragma unroll
+    for (int a = 1; a < kInvRows; ++a) {
+#pragma unroll
+      for (int b = a; b > 0; --b) {
+        const bool sw = so[b] < so[b - 1];
+        const int o1 = sw ? so[b] : so[b - 1], o2 = sw ? so[b - 1] : so[b];
+        const float c1 = sw ? sc[b] : sc[b - 1], c2 = sw ? sc[b - 1] : sc[b];
+        so[b - 1] = o1;
+        so[b] = o2;
+        sc[b - 1] = c1;
+        sc[b] = c2;
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < kInvRows; ++a) {
+      if (a < n) {
+        ro[a * 128] = so[a];
+        rc[a * 128] = sc[a];
+        const int my = so[a] / OW, mx = so[a] - my * OW;
+        const int dy = my - ay;
+        int dx = mx - ax;
+        dx += (dx > OW / 2) ? -OW : ((dx < -(OW / 2)) ? OW : 0);
+        dy0 = min(dy0, dy);
+        dy1 = max(dy1, dy);
+        dx0 = min(dx0, dx);
+        dx1 = max(dx1, dx);
+      }
+    }
+    const int nmax = wave_max(n);
+    if (lane == 0) atomicMax(&ns_l[k], nmax);
+  }
+  dy0 = wave_min(dy0);
+  dy1 = wave_max(dy1);
+  dx0 = wave_min(dx0);
+  dx1 = wave_max(dx1);
+  if (lane == 0) {
+    atomicMin(&bb[0], dy0);
+    atomicMax(&bb[1], dy1);
+    atomicMin(&bb[2], dx0);
+    atomicMax(&bb[3], dx1);
+  }
+  __syncthreads();   // (also orders the sorted lists written above before they are re-read)
+  const Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, it.TY(), it.TX(), OW);
+  if (tid == 0) {
+    hdr[tile * 8 + 0] = rg.ry0;
+    hdr[tile * 8 + 1] = rg.rx0;
+    hdr[tile * 8 + 2] = rg.RH;
+    hdr[tile * 8 + 3] = rg.RW;
+    const bool whole = bb[0] > bb[1] ||
+                       (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, OW) <= kRegionCap;
+    hdr[tile * 8 + 4] = whole ? 1 : 0;
+  }
+  for (int k = tid; k < K; k += kWgThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
+  for (int k = kpar; k < K; k += 2) {
+    const int n = pix_ok ? min(cnt[(size_t)u * K + k], kInvRows) : 0;
+    const int top = ns_l[k];
+    const int* ro = raw_off + ((size_t)tile * K + k) * kInvRows * 128 + p;
+    const float* rc = raw_co + ((size_t)tile * K + k) * kInvRows * 128 + p;
+    int2* row = taps + ((size_t)tile * K + k) * kInvRows * 128 + p;
+    for (int a = 0; a < top; ++a) {
+      int2 v = make_int2(0, 0);
+      if (a < n) {
+        const int mm = ro[a * 128];
+        const int my = mm / OW, mx = mm - my * OW;
+        v = make_int2(rg.encode(my, mx, OW), __float_as_int(rc[a * 128]));
+      }
+      row[(size_t)a * 128] = v;
+    }
   }
 }
 
@@ -122,7 +289,8 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
     const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
     const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
     int H, int W, int Cp, int K, int S, int CpP, int chunks, PixelTiling pt, int tiles,
-    int n_tiles) {
+    int n_tiles, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate != 0) return;   // the plan is not valid: another kernel does the work
   constexpr bool BF16 = MM != kMmF32;
   constexpr int TN = 32 * NB;
   __shared__ __align__(16) float region[(kRegionCap + 1) * kWE];
@@ -390,25 +558,27 @@ int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, Tile
 }
 
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
-                const float* img, const float* Wm, const float* bias, float* pix,
-                float* weights, hipStream_t stream) {
+                const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
+                float* weights, const int* gate, hipStream_t stream) {
   const int CpP = (g.Cp + 127) / 128 * 128;
   const int chunks = (g.Cg + kCC - 1) / kCC;
   {
     const size_t total = (size_t)g.K * chunks * CpP * kCC;
     const int blocks = (int)std::min<size_t>((total + kWgThreads - 1) / kWgThreads, 2048);
     launch(window_weight_kernel, dim3(blocks), dim3(kWgThreads), stream, Wm, weights, g.Cp, g.Cg,
-           g.K, CpP, chunks, mm != kMmF32 ? 1 : 0);
+           g.K, CpP, chunks, mm != kMmF32 ? 1 : 0, swapped ? 1 : 0);
     SDK_LAUNCH_CHECK("window_weight");
   }
   const bool wide = g.Cp > 64;
   const int TN = wide ? 128 : 64;
   const int n_tiles = (int)ceil_div(g.Cp, TN);
-  const dim3 grid((unsigned)(plan.tiles * n_tiles), (unsigned)g.B);
+  // list entries are dealt to the XCDs in eighths: whole multiples of 8 workgroups
+  const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
 #define WG2(MMv, NBv)                                                                          \
   launch(window_gemm_kernel<MMv, NBv>, grid, dim3(kWgThreads), stream, img, plan.hdr, plan.ns, \
          plan.taps, (const int*)tl.inside, (const int*)tl.count, (const float*)weights, bias,  \
-         pix, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles)
+         pix, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles,    \
+         gate)
 #define WG1(MMv)                              \
   do {                                        \
     if (wide) WG2(MMv, 4); else WG2(MMv, 2);  \
@@ -419,6 +589,68 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
 #undef WG1
 #undef WG2
   SDK_LAUNCH_CHECK("window_gemm");
+  return SDK_OK;
+}
+
+namespace {
+struct InverseOffsets {
+  size_t gate, cnt, raw_co, raw_off, hdr, ns, taps, total;
+};
+InverseOffsets inverse_offsets(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  const PixelTiling it = plan_tiling(g.H, g.W);
+  const size_t tiles = (size_t)it.tiles_x * it.tiles_y;
+  const size_t rows = tiles * g.K * kInvRows * 128;
+  InverseOffsets o;
+  o.gate = 0;
+  o.cnt = 256;
+  o.raw_co = o.cnt + up((size_t)g.H * g.W * g.K * sizeof(int));   // gate, cnt, raw_co: cleared together
+  o.raw_off = o.raw_co + up(rows * sizeof(float));
+  o.hdr = o.raw_off + up(rows * sizeof(int));
+  o.ns = o.hdr + up(tiles * 8 * sizeof(int));
+  o.taps = o.ns + up(tiles * g.K * sizeof(int));
+  o.total = o.taps + up(rows * sizeof(int2));
+  return o;
+}
+}  // namespace
+
+size_t inverse_plan_bytes(const ConvGeom& g) { return inverse_offsets(g).total; }
+
+int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+                       hipStream_t stream, InversePlan* out) {
+  const InverseOffsets o = inverse_offsets(g);
+  const PixelTiling it = plan_tiling(g.H, g.W);
+  const int tiles = it.tiles_x * it.tiles_y;
+  char* ws = static_cast<char*>(workspace);
+  int* gate = reinterpret_cast<int*>(ws + o.gate);
+  int* cnt = reinterpret_cast<int*>(ws + o.cnt);
+  float* raw_co = reinterpret_cast<float*>(ws + o.raw_co);
+  int* raw_off = reinterpret_cast<int*>(ws + o.raw_off);
+  int* hdr = reinterpret_cast<int*>(ws + o.hdr);
+  int* ns = reinterpret_cast<int*>(ws + o.ns);
+  int2* taps = reinterpret_cast<int2*>(ws + o.taps);
+  int rc = zero_fill(ws, o.raw_off, stream);
+  if (rc) return rc;
+  const int64_t total = (int64_t)g.M * g.K;
+  if (ceil_div(total, kWgThreads) >= ((int64_t)1 << 31))
+    return fail(SDK_ERR_UNSUPPORTED, "inverse plan: too many samples");
+  SDK_DISPATCH_INTERP(g.interp, g.P,
+                      (launch(inverse_fill_tiled_kernel<INTERP, WEIGHTED>,
+                              dim3((unsigned)ceil_div(total, kWgThreads)), dim3(kWgThreads), stream,
+                              map, wts, g.M, g.K, g.P, g.H, g.W, it, cnt, raw_off, raw_co, gate)));
+  SDK_LAUNCH_CHECK("inverse_fill");
+  launch(inverse_plan_kernel, dim3((unsigned)tiles), dim3(kWgThreads), stream, (const int*)cnt,
+         raw_off, raw_co, it, g.K, g.M / g.OW, g.OW, hdr, ns, taps, (const int*)gate);
+  SDK_LAUNCH_CHECK("inverse_plan");
+  out->plan.pt = it;
+  out->plan.tiles = tiles;
+  out->plan.S = kInvRows;
+  out->plan.hdr = hdr;
+  out->plan.ns = ns;
+  out->plan.taps = taps;
+  out->gate = gate;
+  out->raw_off = raw_off;
+  out->raw_co = raw_co;
   return SDK_OK;
 }
 
