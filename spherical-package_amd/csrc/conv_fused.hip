@@ -643,6 +643,20 @@ bool fused_supported(const ConvGeom& g) {
 
 static bool inverse_candidate(const ConvGeom& g);
 static size_t inverse_bytes(const ConvGeom& g);
+// Tail of the workspace used by the weight gradient: partial sums of the plan-driven kernel,
+// those of the window kernel, the tile lists.
+struct WgradTail {
+  size_t partial, window_partial, lists, total;
+};
+static WgradTail wgrad_tail(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  WgradTail t;
+  t.partial = 0;
+  t.window_partial = up(planned_wgrad_partial_bytes(g));
+  t.lists = t.window_partial + up(window_wgrad_partial_bytes(g));
+  t.total = t.lists + (window_wgrad_partial_bytes(g) != 0 ? up(tile_lists_bytes(g)) : 0);
+  return t;
+}
 
 // Scratch of the forward-style contraction when it runs from the plan: the weight copy of the
 // global-gather kernel, the plan, the tile lists and the weight copy of the window kernel.
@@ -667,18 +681,36 @@ size_t fused_workspace_bytes(const ConvGeom& g) {
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
   if (planned_scatter_supported(g) && inverse_candidate(g))
     need = ((need + 255) & ~(size_t)255) + inverse_bytes(g);
-  // last: the weight gradient's partial sums (the plan and, in a combined backward call,
-  // everything before it are still in use when they are written)
-  if (planned_wgrad_partial_bytes(g) != 0)
-    need = ((need + 255) & ~(size_t)255) + planned_wgrad_partial_bytes(g);
-  return need;
+  // last: the weight gradient's tile lists and partial sums (the plan and, in a combined
+  // backward call, everything before it are still in use when they are written)
+  return ((need + 255) & ~(size_t)255) + wgrad_tail(g).total;
 }
 
+static char* wgrad_tail_base(const ConvGeom& g, float* workspace) {
+  return reinterpret_cast<char*>(workspace) + (fused_workspace_bytes(g) - wgrad_tail(g).total);
+}
 static float* wgrad_partial(const ConvGeom& g, float* workspace) {
-  const size_t bytes = planned_wgrad_partial_bytes(g);
-  if (bytes == 0) return nullptr;
-  return reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
-                                  (fused_workspace_bytes(g) - bytes));
+  if (planned_wgrad_partial_bytes(g) == 0) return nullptr;
+  return reinterpret_cast<float*>(wgrad_tail_base(g, workspace) + wgrad_tail(g).partial);
+}
+
+// gW += the sums of a plan: tiles that fit the window kernel there, the others (and every
+// tile when that kernel does not cover the call) in the plan-driven kernel.
+static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
+                           const float* img, float* gW, float* workspace, hipStream_t stream) {
+  if (window_wgrad_supported(g, mm) && window_wgrad_partial_bytes(g) != 0) {
+    const WgradTail t = wgrad_tail(g);
+    char* base = wgrad_tail_base(g, workspace);
+    TileLists tl;
+    int rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
+    if (rc) return rc;
+    rc = window_wgrad(g, plan, tl, pix, img, gW, reinterpret_cast<float*>(base + t.window_partial),
+                      stream);
+    if (rc) return rc;
+    return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream, tl.rest,
+                         tl.count + 1);
+  }
+  return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream);
 }
 
 static int relayout(const ConvGeom& g, const float* Wm, float* out, int CpP, int CgP,
@@ -1053,13 +1085,12 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   if (g.B == 0) return SDK_OK;
   if (planned_wgrad_supported(g)) {
     if (shared != nullptr && shared->valid)
-      return planned_wgrad(g, matrix_mode(compute), shared->plan, pix, img, gW,
-                           wgrad_partial(g, workspace), stream);
+      return wgrad_from_plan(g, matrix_mode(compute), shared->plan, pix, img, gW, workspace,
+                             stream);
     Plan plan;
     rc = build_plan(g, map, wts, workspace, stream, &plan);
     if (rc) return rc;
-    return planned_wgrad(g, matrix_mode(compute), plan, pix, img, gW, wgrad_partial(g, workspace),
-                         stream);
+    return wgrad_from_plan(g, matrix_mode(compute), plan, pix, img, gW, workspace, stream);
   }
   constexpr int KM = 64;
   const int slots = slots_for(g);

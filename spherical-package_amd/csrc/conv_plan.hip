@@ -137,6 +137,9 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     const bool whole = bb[0] > bb[1] ||
                        (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, W) <= kRegionCap;
     hdr[tile * 8 + 4] = whole ? 1 : 0;
+    int most = 0;
+    for (int k = 0; k < K; ++k) most = max(most, ns_l[k]);
+    hdr[tile * 8 + 5] = most;   // the longest row list of the tile's samples
   }
   for (int k = tid; k < K; k += kPlThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
 
@@ -208,7 +211,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW,
     float* __restrict__ partial, int Cg, int H, int W, int Cp, int K, int S, PixelTiling pt,
-    int tiles, int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4) {
+    int tiles, int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4,
+    const int* __restrict__ tile_list, const int* __restrict__ tile_count) {
   constexpr bool BF16 = MM != kMmF32;     // operands enter the matrix unit as bf16 fragments
   constexpr bool SPLIT = MM == kMmSplit;  // ... three per operand, whose sum is the float
   __shared__ __align__(16) float region[kRegionCap * kRegE];
@@ -257,7 +261,10 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
   // Tiles are dealt round-robin to the tile runs: costly tiles (taps outside the window,
   // e.g. polar rows of a spherical map) are spread over all workgroups.
   int buf = 0;
-  for (int tile = group; tile < tiles; tile += groups) {
+  // all tiles, or the listed ones (tile_list[i], i < *tile_count)
+  const int n_listed = tile_list != nullptr ? *tile_count : tiles;
+  for (int ti = group; ti < n_listed; ti += groups) {
+    const int tile = tile_list != nullptr ? tile_list[ti] : ti;
     const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
     // pixel index (inside the image of the pixel side) of tile-local pixel p, or -1
     auto pixel_index = [&](int p) -> int {
@@ -701,7 +708,8 @@ size_t planned_wgrad_partial_bytes(const ConvGeom& g) {
 }
 
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
-                  const float* img, float* gW, float* partial, hipStream_t stream) {
+                  const float* img, float* gW, float* partial, hipStream_t stream,
+                  const int* tile_list, const int* tile_count) {
   const WgradGrid wg = wgrad_grid(g, plan.tiles);
   const int KB = wg.KB, kb_count = wg.kb_count, NW = wg.NW;
   const int c_chunks = wg.c_chunks, n_tiles = wg.n_tiles, groups = wg.groups;
@@ -717,7 +725,7 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 #define PW3(KBv, BFv, NWv)                                                                      \
   launch(planned_wgrad_kernel<KBv, BFv, NWv>, grid, dim3(kPlThreads), stream, pix, img,         \
          plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
-         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4)
+         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
 #define PW(KBv, BFv)                                                                            \
   do {                                                                                          \
     if (NW == 4) PW3(KBv, BFv, 4); else if (NW == 2) PW3(KBv, BFv, 2); else PW3(KBv, BFv, 1);   \

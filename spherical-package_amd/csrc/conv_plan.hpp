@@ -6,6 +6,7 @@
 //   hdr[8*t + 0..3]  window of the image the tile's taps fall into: first row,
 //                    first column, rows, columns (columns wrap modulo W)
 //   hdr[8*t + 4]     1 when every active tap of the tile lies inside that window
+//   hdr[8*t + 5]     the largest ns of the tile's samples (plan_kernel only)
 //   ns[t*K + k]      rows of kernel sample k: the largest number of active taps
 //                    any pixel of the tile has for that sample
 //   taps[((t*K + k)*S + r)*128 + p]   row r < ns of pixel p (tile-local index):
@@ -52,8 +53,10 @@ struct TileLists {
   const int* rest;
   const int* count;
 };
+// max_rows > 0: tiles with a sample of more than max_rows plan rows (hdr[8t+5]) go to `rest`.
 size_t tile_lists_bytes(const ConvGeom& g);
-int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out);
+int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
+                     int max_rows = 0);
 
 // pix[b] = Wm x im2col(img[b]) + bias on the tiles of tl.inside, gathered from an LDS window.
 // g: the contraction's geometry (gather side = img).  swapped: Wm is [Cg, Cp * K] instead of
@@ -82,7 +85,17 @@ int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, vo
 
 bool planned_wgrad_supported(const ConvGeom& g);
 size_t planned_wgrad_partial_bytes(const ConvGeom& g);
+// tile_list / tile_count (optional, device): only the listed tiles are summed.
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
-                  const float* img, float* gW, float* partial, hipStream_t stream);
+                  const float* img, float* gW, float* partial, hipStream_t stream,
+                  const int* tile_list = nullptr, const int* tile_count = nullptr);
+
+// The same sums over the tiles of tl.inside, from an LDS window with the column values built
+// straight into MFMA operands (conv_window_wgrad.hip; fp32 MFMA, K <= 10, at most four plan
+// rows per sample: build the lists with max_rows = 4).  partial: window_wgrad_partial_bytes(g).
+bool window_wgrad_supported(const ConvGeom& g, int mm);
+size_t window_wgrad_partial_bytes(const ConvGeom& g);
+int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
+                 const float* img, float* gW, float* partial, hipStream_t stream);
 
 }  // namespace sdk

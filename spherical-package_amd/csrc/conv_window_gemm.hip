@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
 //   lists[tiles .. 2*tiles)   the others, count[1] of them
 __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict__ hdr, int tiles,
                                                           int* __restrict__ lists,
-                                                          int* __restrict__ count) {
+                                                          int* __restrict__ count, int max_rows) {
   __shared__ int wave_fit[16], wave_rest[16];
   __shared__ int base[2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
   for (int t0 = 0; t0 < tiles; t0 += 1024) {
     const int t = t0 + tid;
     const bool live = t < tiles;
-    const bool fit = live && hdr[t * 8 + 4] != 0;
+    const bool fit = live && hdr[t * 8 + 4] != 0 && (max_rows <= 0 || hdr[t * 8 + 5] <= max_rows);
     const unsigned long long mf = __ballot(fit), mr = __ballot(live && !fit);
     if (lane == 0) {
       wave_fit[wave] = __popcll(mf);
@@ -546,10 +546,12 @@ size_t tile_lists_bytes(const ConvGeom& g) {
   return ((size_t)2 * pt.tiles_x * pt.tiles_y + 2) * sizeof(int);
 }
 
-int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out) {
+int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
+                     int max_rows) {
   int* lists = static_cast<int*>(workspace);
   int* count = lists + (size_t)2 * plan.tiles;
-  launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles, lists, count);
+  launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles, lists, count,
+         max_rows);
   SDK_LAUNCH_CHECK("tile_lists");
   out->inside = lists;
   out->rest = lists + plan.tiles;

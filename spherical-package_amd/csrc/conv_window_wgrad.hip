@@ -1,0 +1,359 @@
+// Weight gradient of mapped convolution from an LDS window, driven by a tap plan (gfx950,
+// float32 tensors, fp32 MFMA):
+//
+//   gW[n][c][k] += sum_{b, m} pix[b][n][m] * col[b][(c, k)][m]
+//   col[b][(c, k)][m] = sum_r coefficient(m, k, r) * img[b][c][tap(m, k, r)]
+//
+// for the tiles of a plan (conv_plan.hpp) whose taps all lie inside the tile's image window
+// and whose samples have at most four plan rows.  The reduction index of the MFMA is the
+// pixel: v_mfma_f32_32x32x2_f32 step s contracts the two pixels m = s and m = 16 + s of a
+// quarter tile (32 pixels), lane l supplying row n = l % 32 of the pixel-side tile as A and
+// channel c = l % 32 of the column tile as B, each for pixel 16 (l / 32) + s.
+//
+//   workgroup = 32 image channels (one chunk) x 128 pixel-side channels x all K samples x one
+//               batch element x every groups-th tile of the list
+//   wave w    = samples w KP .. w KP + KP - 1 for all four 32-row blocks of n ("full" samples,
+//               K = 4 KP + R), and row block w for each of the R remaining samples
+//
+// so a wave builds the column values of its own samples itself, straight into B operands:
+// per step and sample two LDS reads fetch the four plan rows of the lane's pixel (window byte
+// offset, coefficient; the same address across a half wave), four LDS reads the window values
+// of the lane's channel, four multiply-adds blend them.  Nothing is exchanged between waves
+// and there is no barrier inside a quarter tile.  The pixel-side tile (128 x 32 values) and the
+// quarter's plan rows are staged in LDS once per quarter, the window once per tile.  The
+// accumulators ((4 KP + R) x 16 registers) stay in registers over all tiles and leave the
+// workgroup once, into a partial-sum buffer that window_wgrad_reduce_kernel adds up.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "conv_fused.hpp"
+#include "conv_plan.hpp"
+#include "conv_window.hpp"
+#include "sdk_host.hpp"
+#include "sdk_mfma.hpp"
+
+namespace sdk {
+
+namespace {
+
+constexpr int kWwThreads = 256;
+constexpr int kWwE = 36;   // floats per window element: 32 channels + 4 of skew
+constexpr int kWwG = 36;   // floats per row of the pixel-side tile: 32 pixels + 4 of skew
+constexpr int kWwQ = 32;   // pixels per quarter tile
+constexpr int kWwRows = 4; // plan rows per sample this kernel applies
+
+template <int KP, int R>
+__global__ __launch_bounds__(kWwThreads, 2) void window_wgrad_kernel(
+    const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
+    const int* __restrict__ ns, const int2* __restrict__ taps, const int* __restrict__ list,
+    const int* __restrict__ count, float* __restrict__ partial, int Cg, int H, int W, int Cp,
+    int S, PixelTiling pt, int groups, int batches, int c_chunks, int n_tiles, int vec4) {
+  constexpr int K = 4 * KP + R;
+  __shared__ __align__(16) float region[(kRegionCap + 1) * kWwE];
+  __shared__ __align__(16) float gt[128 * kWwG];
+  __shared__ __align__(16) int2 rowsL[K * kWwQ * kWwRows];
+  __shared__ int src[kRegionCap];
+  __shared__ int ns_l[K];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int j = lane & 31, h = lane >> 5;
+  // Workgroup ids go round-robin over the 8 XCDs.  All workgroups of one tile run (every
+  // batch element and channel chunk) read the same plan rows, those of one batch element the
+  // same pixel-side tiles: they take consecutive slots of one XCD and meet in its L2.
+  const int kinds = c_chunks * n_tiles * batches;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int kind = slot % kinds, group = (slot / kinds) * 8 + xcd;
+  if (group >= groups) return;
+  const int nt = kind % n_tiles, cc = (kind / n_tiles) % c_chunks;
+  const int batch = kind / (n_tiles * c_chunks);
+  const int c0 = cc * kCC, n0 = nt * 128;
+  const int M = pt.OH * pt.OW;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + ((size_t)batch * Cg) * HW;
+  const float* pix_b = pix + ((size_t)batch * Cp) * M;
+
+  floatx16 accF[KP > 0 ? KP : 1][4];
+  floatx16 accR[R > 0 ? R : 1];
+#pragma unroll
+  for (int i = 0; i < (KP > 0 ? KP : 1); ++i)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) accF[i][a][v] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < (R > 0 ? R : 1); ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) accR[i][v] = 0.0f;
+
+  // B values: window element at byte offset o -> channel j at regb + o
+  const char* regb = reinterpret_cast<const char*>(region) + 4 * j;
+  // pixel-side tile staging role: row n_s, pixels 16 hr_s .. 16 hr_s + 15 of the quarter
+  const int n_s = tid >> 1, hr_s = tid & 1;
+  const bool n_ok = n0 + n_s < Cp;
+  const float* pix_row = pix_b + (size_t)(n_ok ? n0 + n_s : 0) * M;
+
+  const int cnt = *count;
+  for (int ti = group; ti < cnt; ti += groups) {
+    const int tile = list[ti];
+    const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
+    Region rg;
+    rg.ry0 = hdr[tile * 8 + 0];
+    rg.rx0 = hdr[tile * 8 + 1];
+    rg.RH = hdr[tile * 8 + 2];
+    rg.RW = hdr[tile * 8 + 3];
+    rg.RS = rg.RH * rg.RW;
+    rg.RSp = rg.RS;
+    const int RS = rg.RS;
+    const int2* tile_taps = taps + (size_t)tile * K * S * 128;
+
+    __syncthreads();   // every wave is done with the previous tile
+    build_region_lut(rg, H, W, src);
+    if (tid < K) ns_l[tid] = min(ns[(size_t)tile * K + tid], min(S, kWwRows));
+    if (tid < kWwE) region[RS * kWwE + tid] = 0.0f;   // the zero element inactive rows point at
+    __syncthreads();
+    {
+      // window: wave w stages channels 8w .. 8w+7 of every element; a lane owns elements
+      // lane, lane + 64, ... and has all its loads in flight before the first LDS write
+      constexpr int ITER = (kRegionCap + 63) / 64;
+      const int cw = c0 + 8 * wave;
+      const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
+      const unsigned plane = (unsigned)HW * 4u;
+      float v[ITER][8];
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        const int o = e < RS ? src[e] : -1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const bool ok = o >= 0 && cw + i < Cg;
+          const float d = *reinterpret_cast<const float*>(
+              cbase + (ok ? (unsigned)i * plane + (unsigned)o * 4u : 0u));
+          v[it][i] = ok ? d : 0.0f;
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int e = lane + 64 * it;
+        if (e < RS) {
+          float4* d4 = reinterpret_cast<float4*>(region + e * kWwE + 8 * wave);
+          d4[0] = make_float4(v[it][0], v[it][1], v[it][2], v[it][3]);
+          d4[1] = make_float4(v[it][4], v[it][5], v[it][6], v[it][7]);
+        }
+      }
+    }
+
+#pragma unroll 1
+    for (int q = 0; q < 4; ++q) {
+      if (q > 0) __syncthreads();   // the previous quarter's reads of gt / rowsL are done
+      // ---- pixel-side tile of the quarter: gt[n][m], m = 16 hr + i
+      {
+        const int p0 = kWwQ * q + 16 * hr_s;
+        float4 gq[4];
+        if (vec4) {
+          const int oy = ty0 + (p0 >> pt.tx_shift), ox = tx0 + (p0 & (pt.TX() - 1));
+          const float* rowp = pix_row + (size_t)oy * pt.OW + ox;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            gq[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (n_ok && oy < pt.OH && ox + 4 * i < pt.OW)
+              gq[i] = *reinterpret_cast<const float4*>(rowp + 4 * i);
+          }
+        } else {
+          float f[16];
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int p = p0 + i;
+            const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
+            const bool ok = n_ok && oy < pt.OH && ox < pt.OW;
+            const float d = pix_row[ok ? (size_t)oy * pt.OW + ox : 0];
+            f[i] = ok ? d : 0.0f;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) gq[i] = make_float4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+        }
+        float4* dst = reinterpret_cast<float4*>(gt + n_s * kWwG + 16 * hr_s);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[i] = gq[i];
+      }
+      // ---- plan rows of the quarter: rowsL[(k * 32 + m) * 4 + r] = (window byte offset, coefficient)
+      {
+        constexpr int TOTAL = K * kWwRows * kWwQ;
+#pragma unroll
+        for (int i0 = 0; i0 < TOTAL; i0 += kWwThreads) {
+          const int idx = i0 + tid;
+          if (idx < TOTAL) {
+            const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
+            int2 ec = make_int2(0, 0);
+            if (r < ns_l[k]) ec = tile_taps[((size_t)k * S + r) * 128 + kWwQ * q + m];
+            const bool on = __int_as_float(ec.y) != 0.0f;
+            rowsL[(k * kWwQ + m) * kWwRows + r] =
+                make_int2((on ? ec.x : RS) * (kWwE * 4), on ? ec.y : 0);
+          }
+        }
+      }
+      __syncthreads();   // (for q == 0 this also publishes the window)
+
+      // ---- 16 MFMA steps over the quarter's pixels m = 16 h + s
+#pragma unroll 1
+      for (int s4 = 0; s4 < 4; ++s4) {
+        float4 A[4], Aw;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          A[a] = *reinterpret_cast<const float4*>(gt + (32 * a + j) * kWwG + 16 * h + 4 * s4);
+        Aw = *reinterpret_cast<const float4*>(gt + (32 * wave + j) * kWwG + 16 * h + 4 * s4);
+#pragma unroll
+        for (int ss = 0; ss < 4; ++ss) {
+          const int m = 16 * h + 4 * s4 + ss;
+          // column value of channel j, pixel m, sample k
+          auto column = [&](int k) -> float {
+            const int4* rp = reinterpret_cast<const int4*>(&rowsL[(k * kWwQ + m) * kWwRows]);
+            const int4 r01 = rp[0], r23 = rp[1];
+            const float v0 = *reinterpret_cast<const float*>(regb + r01.x);
+            const float v1 = *reinterpret_cast<const float*>(regb + r01.z);
+            const float v2 = *reinterpret_cast<const float*>(regb + r23.x);
+            const float v3 = *reinterpret_cast<const float*>(regb + r23.z);
+            float b = __int_as_float(r01.y) * v0;
+            b = __builtin_fmaf(__int_as_float(r01.w), v1, b);
+            b = __builtin_fmaf(__int_as_float(r23.y), v2, b);
+            b = __builtin_fmaf(__int_as_float(r23.w), v3, b);
+            return b;
+          };
+          const float a0 = ss == 0 ? A[0].x : (ss == 1 ? A[0].y : (ss == 2 ? A[0].z : A[0].w));
+          const float a1 = ss == 0 ? A[1].x : (ss == 1 ? A[1].y : (ss == 2 ? A[1].z : A[1].w));
+          const float a2 = ss == 0 ? A[2].x : (ss == 1 ? A[2].y : (ss == 2 ? A[2].z : A[2].w));
+          const float a3 = ss == 0 ? A[3].x : (ss == 1 ? A[3].y : (ss == 2 ? A[3].z : A[3].w));
+          const float aw = ss == 0 ? Aw.x : (ss == 1 ? Aw.y : (ss == 2 ? Aw.z : Aw.w));
+#pragma unroll
+          for (int kk = 0; kk < KP; ++kk) {
+            const float b = column(wave * KP + kk);
+            accF[kk][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b, accF[kk][0], 0, 0, 0);
+            accF[kk][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b, accF[kk][1], 0, 0, 0);
+            accF[kk][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2, b, accF[kk][2], 0, 0, 0);
+            accF[kk][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a3, b, accF[kk][3], 0, 0, 0);
+          }
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            const float b = column(4 * KP + r);
+            accR[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(aw, b, accR[r], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- every accumulator register is stored as it lies (register-major, thread fastest)
+  constexpr int NREG = (4 * KP + R) * 16;
+  float* dst = partial + (size_t)blockIdx.x * (NREG * kWwThreads) + tid;
+#pragma unroll
+  for (int kk = 0; kk < KP; ++kk)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dst[((kk * 4 + a) * 16 + v) * kWwThreads] = accF[kk][a][v];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dst[((KP * 4 + r) * 16 + v) * kWwThreads] = accR[r][v];
+}
+
+// Sums the accumulator copies of window_wgrad_kernel and adds them to gW.  Block (x, y, z):
+// accumulator register x of thread threadIdx.x, for the workgroup kind y = (channel chunk,
+// row tile), over every z-th of the batches * groups workgroups of that kind.
+__global__ __launch_bounds__(kWwThreads) void window_wgrad_reduce_kernel(
+    const float* __restrict__ partial, float* __restrict__ gW, int Cg, int Cp, int K, int KP,
+    int R, int groups, int batches, int c_chunks, int n_tiles) {
+  const int tid = threadIdx.x, reg = blockIdx.x;
+  const int nt = blockIdx.y % n_tiles, cc = blockIdx.y / n_tiles;
+  const int kinds = c_chunks * n_tiles * batches;
+  const int total = batches * groups;
+  const size_t per_wg = (size_t)(4 * KP + R) * 16 * kWwThreads;
+  float s = 0.0f;
+  for (int i = blockIdx.z; i < total; i += gridDim.z) {
+    const int b = i / groups, grp = i % groups;
+    const int kind = (b * c_chunks + cc) * n_tiles + nt;
+    const size_t wg = ((size_t)(grp >> 3) * kinds + kind) * 8 + (grp & 7);
+    s += partial[wg * per_wg + (size_t)reg * kWwThreads + tid];
+  }
+  const int wave = tid >> 6, lane = tid & 63, j = lane & 31, h = lane >> 5;
+  const int v = reg & 15, blk = reg >> 4;
+  int k, a;
+  if (blk < 4 * KP) {
+    k = wave * KP + blk / 4;
+    a = blk & 3;
+  } else {
+    k = 4 * KP + (blk - 4 * KP);
+    a = wave;
+  }
+  const int n = nt * 128 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
+  const int c = cc * kCC + j;
+  if (c < Cg && n < Cp && k < K) atomic_add_noret(gW + (size_t)n * Cg * K + (size_t)c * K + k, s);
+}
+
+struct WwGrid {
+  int c_chunks, n_tiles, groups, nreg;
+  int64_t kinds, slots;
+};
+WwGrid ww_grid(const ConvGeom& g, int tiles) {
+  WwGrid w;
+  w.c_chunks = (int)ceil_div(g.Cg, kCC);
+  w.n_tiles = (int)ceil_div(g.Cp, 128);
+  w.kinds = (int64_t)w.c_chunks * w.n_tiles * g.B;
+  // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall
+  const int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, w.kinds), 8) * 8);
+  w.groups = (int)std::min<int64_t>(ceil_div(tiles, 8) * 8, want);
+  w.slots = (int64_t)w.groups * w.kinds;
+  w.nreg = g.K * 16;
+  return w;
+}
+}  // namespace
+
+bool window_wgrad_supported(const ConvGeom& g, int mm) {
+  return mm == kMmF32 && planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 32 &&
+         (int64_t)g.H * g.W <= ((int64_t)1 << 24);
+}
+
+size_t window_wgrad_partial_bytes(const ConvGeom& g) {
+  if (g.B == 0 || !window_wgrad_supported(g, kMmF32)) return 0;
+  const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
+  const WwGrid w = ww_grid(g, pt.tiles_x * pt.tiles_y);
+  return (size_t)w.slots * w.nreg * kWwThreads * sizeof(float);
+}
+
+int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
+                 const float* img, float* gW, float* partial, hipStream_t stream) {
+  const WwGrid w = ww_grid(g, plan.tiles);
+  if (w.slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "window_wgrad: grid too large");
+  const int TX = plan.pt.TX();
+  const int vec4 = (g.OW % 4 == 0 && TX >= 16 && reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
+  const dim3 grid((unsigned)w.slots);
+  const int KP = g.K / 4, R = g.K % 4;
+#define WW(KPv, Rv)                                                                              \
+  launch(window_wgrad_kernel<KPv, Rv>, grid, dim3(kWwThreads), stream, pix, img, plan.hdr,       \
+         plan.ns, plan.taps, (const int*)tl.inside, (const int*)tl.count, partial, g.Cg, g.H,    \
+         g.W, g.Cp, plan.S, plan.pt, w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4)
+  switch (g.K) {
+    case 1: WW(0, 1); break;
+    case 2: WW(0, 2); break;
+    case 3: WW(0, 3); break;
+    case 4: WW(1, 0); break;
+    case 5: WW(1, 1); break;
+    case 6: WW(1, 2); break;
+    case 7: WW(1, 3); break;
+    case 8: WW(2, 0); break;
+    case 9: WW(2, 1); break;
+    default: WW(2, 2); break;
+  }
+#undef WW
+  SDK_LAUNCH_CHECK("window_wgrad");
+  const int kinds0 = w.c_chunks * w.n_tiles, total = (int)g.B * w.groups;
+  const int parts = (int)std::min<int64_t>(std::min(total, 16),
+                                           ceil_div(2048, (int64_t)w.nreg * kinds0));
+  launch(window_wgrad_reduce_kernel, dim3((unsigned)w.nreg, (unsigned)kinds0, (unsigned)std::max(parts, 1)),
+         dim3(kWwThreads), stream, (const float*)partial, gW, g.Cg, g.Cp, g.K, KP, R, w.groups,
+         (int)g.B, w.c_chunks, w.n_tiles);
+  SDK_LAUNCH_CHECK("window_wgrad_reduce");
+  return SDK_OK;
+}
+
+}  // namespace sdk
