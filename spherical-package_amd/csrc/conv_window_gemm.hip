@@ -296,6 +296,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
   __shared__ __align__(16) float region[(kRegionCap + 1) * kWE];
   __shared__ __align__(16) float As[2][TN * kWE];
   __shared__ int src[kRegionCap];
+  __shared__ int ns_l[kPlanKMax];   // rows per sample (a scalar load here would sit in the LDS waits)
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int j = lane & 31, h = lane >> 5;
@@ -324,11 +325,11 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
   const int RS = rg.RS;
   build_region_lut(rg, H, W, src);
   if (tid < kWE) region[RS * kWE + tid] = 0.0f;   // the zero element padded rows point at
+  for (int k = tid; k < K; k += kWgThreads) ns_l[k] = ns[(size_t)tile * K + k];
 
   // this lane's pixel and its plan rows: row r of sample k at rows_p[(k * S + r) * 128]
   const int p_local = 32 * wave + j;
   const int2* rows_p = taps + (size_t)tile * K * S * 128 + p_local;
-  const int* ns_t = ns + (size_t)tile * K;
 
   floatx16 acc[NB];
 #pragma unroll
@@ -395,7 +396,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
 
   int buf = 0;
   SDK_LOAD_WEIGHTS(0, 0);
-  int n_rows = ns_t[0];
+  int n_rows = ns[(size_t)tile * K];
   SDK_LOAD_ROWS(rows, 0, 0);
   for (int chunk = 0; chunk < chunks; ++chunk) {
     const int c0 = chunk * kCC;
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
       const int chunk_n = last_k ? (chunk + 1 < chunks ? chunk + 1 : 0) : chunk;
       SDK_LOAD_WEIGHTS(kn, chunk_n);
       SDK_LOAD_ROWS(rows_next, kn, 0);
-      const int n_rows_next = ns_t[kn];
+      const int n_rows_next = __builtin_amdgcn_readfirstlane(ns_l[kn]);
       asm volatile("" ::: "memory");   // the requests stay here, ahead of the gather and the MFMAs
 
       // ---- gather: col[c][pixel j] for this lane's 16 channels of the chunk

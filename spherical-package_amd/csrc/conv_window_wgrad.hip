@@ -194,51 +194,88 @@ __global__ __launch_bounds__(kWwThreads, 2) void window_wgrad_kernel(
       }
       __syncthreads();   // (for q == 0 this also publishes the window)
 
-      // ---- 16 MFMA steps over the quarter's pixels m = 16 h + s
-#pragma unroll 1
-      for (int s4 = 0; s4 < 4; ++s4) {
-        float4 A[4], Aw;
+      // ---- 16 MFMA steps over the quarter's pixels m = 16 h + s, as a three-stage pipeline:
+      // while the MFMAs of step s issue, the window values of step s + 1 and the plan rows of
+      // step s + 2 are in flight, so no LDS round trip stands between two steps' MFMAs.
+      constexpr int KW = KP + R;   // columns (samples) this wave builds per step
+      int4 R01[KW], R23[KW];       // plan rows, two steps ahead
+      float co[KW][4], val[KW][4]; // coefficients and window values, one step ahead
+      float bcur[KW];
+      const int2* rows_h = rowsL + (16 * h) * kWwRows;
+#define SDK_ROWS_ISSUE(stepv)                                                        \
+  do {                                                                               \
+    const int st = (stepv) < 16 ? (stepv) : 15;                                      \
+    _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
+      const int k = c < KP ? wave * KP + c : 4 * KP + (c - KP);                      \
+      const int4* rp = reinterpret_cast<const int4*>(rows_h + (k * kWwQ + st) * kWwRows); \
+      R01[c] = rp[0];                                                                \
+      R23[c] = rp[1];                                                                \
+    }                                                                                \
+  } while (0)
+#define SDK_VALS_ISSUE()                                                             \
+  do {                                                                               \
+    _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
+      val[c][0] = *reinterpret_cast<const float*>(regb + R01[c].x);                  \
+      val[c][1] = *reinterpret_cast<const float*>(regb + R01[c].z);                  \
+      val[c][2] = *reinterpret_cast<const float*>(regb + R23[c].x);                  \
+      val[c][3] = *reinterpret_cast<const float*>(regb + R23[c].z);                  \
+      co[c][0] = __int_as_float(R01[c].y);                                           \
+      co[c][1] = __int_as_float(R01[c].w);                                           \
+      co[c][2] = __int_as_float(R23[c].y);                                           \
+      co[c][3] = __int_as_float(R23[c].w);                                           \
+    }                                                                                \
+  } while (0)
+#define SDK_BLEND(dst)                                                               \
+  do {                                                                               \
+    _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
+      float bv = co[c][0] * val[c][0];                                               \
+      bv = __builtin_fmaf(co[c][1], val[c][1], bv);                                  \
+      bv = __builtin_fmaf(co[c][2], val[c][2], bv);                                  \
+      dst[c] = __builtin_fmaf(co[c][3], val[c][3], bv);                              \
+    }                                                                                \
+  } while (0)
+      SDK_ROWS_ISSUE(0);
+      SDK_VALS_ISSUE();    // step 0
+      SDK_ROWS_ISSUE(1);
+      SDK_BLEND(bcur);     // step 0
+      SDK_VALS_ISSUE();    // step 1
+      SDK_ROWS_ISSUE(2);
+      float4 A[4], Aw;
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
-          A[a] = *reinterpret_cast<const float4*>(gt + (32 * a + j) * kWwG + 16 * h + 4 * s4);
-        Aw = *reinterpret_cast<const float4*>(gt + (32 * wave + j) * kWwG + 16 * h + 4 * s4);
+      for (int step = 0; step < 16; ++step) {
+        if ((step & 3) == 0) {
 #pragma unroll
-        for (int ss = 0; ss < 4; ++ss) {
-          const int m = 16 * h + 4 * s4 + ss;
-          // column value of channel j, pixel m, sample k
-          auto column = [&](int k) -> float {
-            const int4* rp = reinterpret_cast<const int4*>(&rowsL[(k * kWwQ + m) * kWwRows]);
-            const int4 r01 = rp[0], r23 = rp[1];
-            const float v0 = *reinterpret_cast<const float*>(regb + r01.x);
-            const float v1 = *reinterpret_cast<const float*>(regb + r01.z);
-            const float v2 = *reinterpret_cast<const float*>(regb + r23.x);
-            const float v3 = *reinterpret_cast<const float*>(regb + r23.z);
-            float b = __int_as_float(r01.y) * v0;
-            b = __builtin_fmaf(__int_as_float(r01.w), v1, b);
-            b = __builtin_fmaf(__int_as_float(r23.y), v2, b);
-            b = __builtin_fmaf(__int_as_float(r23.w), v3, b);
-            return b;
-          };
-          const float a0 = ss == 0 ? A[0].x : (ss == 1 ? A[0].y : (ss == 2 ? A[0].z : A[0].w));
-          const float a1 = ss == 0 ? A[1].x : (ss == 1 ? A[1].y : (ss == 2 ? A[1].z : A[1].w));
-          const float a2 = ss == 0 ? A[2].x : (ss == 1 ? A[2].y : (ss == 2 ? A[2].z : A[2].w));
-          const float a3 = ss == 0 ? A[3].x : (ss == 1 ? A[3].y : (ss == 2 ? A[3].z : A[3].w));
-          const float aw = ss == 0 ? Aw.x : (ss == 1 ? Aw.y : (ss == 2 ? Aw.z : Aw.w));
+          for (int a = 0; a < 4; ++a)
+            A[a] = *reinterpret_cast<const float4*>(gt + (32 * a + j) * kWwG + 16 * h + step);
+          Aw = *reinterpret_cast<const float4*>(gt + (32 * wave + j) * kWwG + 16 * h + step);
+        }
+        const int ss = step & 3;
+        const float a0 = ss == 0 ? A[0].x : (ss == 1 ? A[0].y : (ss == 2 ? A[0].z : A[0].w));
+        const float a1 = ss == 0 ? A[1].x : (ss == 1 ? A[1].y : (ss == 2 ? A[1].z : A[1].w));
+        const float a2 = ss == 0 ? A[2].x : (ss == 1 ? A[2].y : (ss == 2 ? A[2].z : A[2].w));
+        const float a3 = ss == 0 ? A[3].x : (ss == 1 ? A[3].y : (ss == 2 ? A[3].z : A[3].w));
+        const float aw = ss == 0 ? Aw.x : (ss == 1 ? Aw.y : (ss == 2 ? Aw.z : Aw.w));
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int kk = 0; kk < KP; ++kk) {
-            const float b = column(wave * KP + kk);
-            accF[kk][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b, accF[kk][0], 0, 0, 0);
-            accF[kk][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b, accF[kk][1], 0, 0, 0);
-            accF[kk][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2, b, accF[kk][2], 0, 0, 0);
-            accF[kk][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a3, b, accF[kk][3], 0, 0, 0);
-          }
+        for (int kk = 0; kk < KP; ++kk) {
+          accF[kk][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, bcur[kk], accF[kk][0], 0, 0, 0);
+          accF[kk][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, bcur[kk], accF[kk][1], 0, 0, 0);
+          accF[kk][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2, bcur[kk], accF[kk][2], 0, 0, 0);
+          accF[kk][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a3, bcur[kk], accF[kk][3], 0, 0, 0);
+        }
 #pragma unroll
-          for (int r = 0; r < R; ++r) {
-            const float b = column(4 * KP + r);
-            accR[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(aw, b, accR[r], 0, 0, 0);
-          }
+        for (int r = 0; r < R; ++r)
+          accR[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(aw, bcur[KP + r], accR[r], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (step < 15) {
+          SDK_BLEND(bcur);                      // step + 1
+          if (step < 14) SDK_VALS_ISSUE();      // step + 2
+          if (step < 13) SDK_ROWS_ISSUE(step + 3);
         }
       }
+#undef SDK_ROWS_ISSUE
+#undef SDK_VALS_ISSUE
+#undef SDK_BLEND
     }
   }
 
