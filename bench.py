@@ -103,15 +103,28 @@ def _conv_entry_points(torch, ops, x, m, iw, w, b, g, K, interp, compute):
     gb = torch.empty(Cout, device=x.device)
     p, s = ops._ptr, ops._stream(x)
     dims = (B, Cin, H, W, Cout, OH, OW, K, P, interp, 0, mode, s)
+    # the layer's plan, built once per map as the operators do (steady state of a training run)
+    plan, nplan = ops._conv_plan(x, m, iw, H, W, K, P, interp)
+    if plan is None:
+        return {
+            "forward": lambda: _capi.call("sdk_mapped_conv_forward", p(x), p(m), p(iw), p(w),
+                                          p(b), p(out), p(ws), nws, *dims),
+            "backward_input": lambda: _capi.call("sdk_mapped_conv_backward_input", p(g), p(m),
+                                                 p(iw), p(w), p(gi), p(ws), nws, *dims),
+            "backward_weight": lambda: _capi.call("sdk_mapped_conv_backward_weight", p(g), p(m),
+                                                  p(iw), p(x), p(gw), p(ws), nws, *dims),
+            "bias_grad": lambda: _capi.call("sdk_bias_grad", p(g), p(gb), B, Cout, OH * OW, 0, s),
+        }, (ws, out, gi, gw, gb)
+    pl = (p(plan), nplan)
     return {
-        "forward": lambda: _capi.call("sdk_mapped_conv_forward", p(x), p(m), p(iw), p(w), p(b),
-                                      p(out), p(ws), nws, *dims),
-        "backward_input": lambda: _capi.call("sdk_mapped_conv_backward_input", p(g), p(m), p(iw),
-                                             p(w), p(gi), p(ws), nws, *dims),
-        "backward_weight": lambda: _capi.call("sdk_mapped_conv_backward_weight", p(g), p(m),
-                                              p(iw), p(x), p(gw), p(ws), nws, *dims),
+        "forward": lambda: _capi.call("sdk_mapped_conv_forward_planned", p(x), p(m), p(iw), p(w),
+                                      p(b), p(out), p(ws), nws, *pl, *dims),
+        "backward_input": lambda: _capi.call("sdk_mapped_conv_backward_input_planned", p(g), p(m),
+                                             p(iw), p(w), p(gi), p(ws), nws, *pl, *dims),
+        "backward_weight": lambda: _capi.call("sdk_mapped_conv_backward_weight_planned", p(g),
+                                              p(m), p(iw), p(x), p(gw), p(ws), nws, *pl, *dims),
         "bias_grad": lambda: _capi.call("sdk_bias_grad", p(g), p(gb), B, Cout, OH * OW, 0, s),
-    }, (ws, out, gi, gw, gb)
+    }, (ws, out, gi, gw, gb, plan)
 
 
 def verify_conv4(torch, ops, cfg, t, compute):

@@ -500,6 +500,87 @@ int sdk_mapped_transposed_conv_backward(const void* grad_output, const void* sam
                                         int32_t interp, int32_t dtype, int32_t compute,
                                         sdk_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Plans: what the convolution kernels derive from the sample map alone, kept
+ * between calls.  The reference is stateless (every call of
+ * ext_modules/src/cuda/mapped_convolution_layer.cu:16-194 re-reads the map); a
+ * layer's map is constant over a training run, so the tap plan (the map
+ * resolved into window indices and coefficients per pixel tile, with the lists
+ * of tiles by kind) and its inverse (per image pixel the pixels that sample
+ * it) can be built once into caller-owned device memory:
+ *
+ *   sdk_mapped_conv_plan_bytes(...)   size of the buffer, 0 when this geometry
+ *                                     has no plan (then use the plain entry points)
+ *   sdk_mapped_conv_plan_build(...)   fills it from sample_map / interp_weights
+ *   sdk_..._planned(...)              the entry point of the same name with
+ *                                     (plan, plan_bytes) after the workspace
+ *                                     pair; identical results
+ *
+ * A plan depends on the map, on the size of the image it points into
+ * (image_height x image_width), on the map's grid (map_height x map_width),
+ * kernel_size, num_interp_pts and interp; not on batch size, channel counts,
+ * weights or the compute mode, and one plan serves a mapped convolution and a
+ * mapped transposed convolution over the same map.  The buffer must be
+ * 256-byte aligned, is only read by the planned calls, and must be rebuilt
+ * when the map's contents change.  float32 tensors only (dtype = SDK_F32).
+ * ------------------------------------------------------------------------- */
+size_t sdk_mapped_conv_plan_bytes(int64_t image_height, int64_t image_width, int64_t map_height,
+                                  int64_t map_width, int64_t kernel_size, int32_t num_interp_pts,
+                                  int32_t interp, int32_t dtype);
+int sdk_mapped_conv_plan_build(const void* sample_map, const void* interp_weights, void* plan,
+                               size_t plan_bytes, int64_t image_height, int64_t image_width,
+                               int64_t map_height, int64_t map_width, int64_t kernel_size,
+                               int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                               sdk_stream_t stream);
+int sdk_mapped_conv_forward_planned(const void* input, const void* sample_map, const void*
+    interp_weights, const void* weight, const void* bias, void* output, void* workspace, size_t
+    workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels, int64_t
+    height, int64_t width, int64_t out_channels, int64_t out_height, int64_t out_width, int64_t
+    kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t compute,
+    sdk_stream_t stream);
+int sdk_mapped_conv_backward_input_planned(const void* grad_output, const void* sample_map, const
+    void* interp_weights, const void* weight, void* grad_input, void* workspace, size_t
+    workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels, int64_t
+    height, int64_t width, int64_t out_channels, int64_t out_height, int64_t out_width, int64_t
+    kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t compute,
+    sdk_stream_t stream);
+int sdk_mapped_conv_backward_weight_planned(const void* grad_output, const void* sample_map, const
+    void* interp_weights, const void* input, void* grad_weight, void* workspace, size_t
+    workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels, int64_t
+    height, int64_t width, int64_t out_channels, int64_t out_height, int64_t out_width, int64_t
+    kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t compute,
+    sdk_stream_t stream);
+int sdk_mapped_conv_backward_planned(const void* grad_output, const void* sample_map, const void*
+    interp_weights, const void* input, const void* weight, void* grad_input, void* grad_weight,
+    void* grad_bias, void* workspace, size_t workspace_bytes, void* plan, size_t plan_bytes,
+    int64_t batch, int64_t in_channels, int64_t height, int64_t width, int64_t out_channels,
+    int64_t out_height, int64_t out_width, int64_t kernel_size, int32_t num_interp_pts, int32_t
+    interp, int32_t dtype, int32_t compute, sdk_stream_t stream);
+int sdk_mapped_transposed_conv_forward_planned(const void* input, const void* sample_map, const
+    void* interp_weights, const void* weight, const void* bias, void* output, void* workspace,
+    size_t workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels,
+    int64_t in_height, int64_t in_width, int64_t out_channels, int64_t out_height, int64_t
+    out_width, int64_t kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t
+    compute, sdk_stream_t stream);
+int sdk_mapped_transposed_conv_backward_input_planned(const void* grad_output, const void*
+    sample_map, const void* interp_weights, const void* weight, void* grad_input, void* workspace,
+    size_t workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels,
+    int64_t in_height, int64_t in_width, int64_t out_channels, int64_t out_height, int64_t
+    out_width, int64_t kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t
+    compute, sdk_stream_t stream);
+int sdk_mapped_transposed_conv_backward_weight_planned(const void* grad_output, const void*
+    sample_map, const void* interp_weights, const void* input, void* grad_weight, void* workspace,
+    size_t workspace_bytes, void* plan, size_t plan_bytes, int64_t batch, int64_t in_channels,
+    int64_t in_height, int64_t in_width, int64_t out_channels, int64_t out_height, int64_t
+    out_width, int64_t kernel_size, int32_t num_interp_pts, int32_t interp, int32_t dtype, int32_t
+    compute, sdk_stream_t stream);
+int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const void* sample_map,
+    const void* interp_weights, const void* input, const void* weight, void* grad_input, void*
+    grad_weight, void* grad_bias, void* workspace, size_t workspace_bytes, void* plan, size_t
+    plan_bytes, int64_t batch, int64_t in_channels, int64_t in_height, int64_t in_width, int64_t
+    out_channels, int64_t out_height, int64_t out_width, int64_t kernel_size, int32_t
+    num_interp_pts, int32_t interp, int32_t dtype, int32_t compute, sdk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

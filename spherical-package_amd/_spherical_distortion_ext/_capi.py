@@ -46,10 +46,21 @@ SIGNATURES = {
     "sdk_mapped_transposed_conv_forward": [_vp] * 7 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_input": [_vp] * 6 + [_sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_weight": [_vp] * 6 + [_sz] + _CONV_DIMS,
+    # the same entry points taking a plan (pointer, bytes) after the workspace pair
+    "sdk_mapped_conv_forward_planned": [_vp] * 7 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_conv_backward_input_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_conv_backward_weight_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_conv_backward_planned": [_vp] * 9 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_transposed_conv_backward_planned": [_vp] * 9 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_transposed_conv_forward_planned": [_vp] * 7 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_transposed_conv_backward_input_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_transposed_conv_backward_weight_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
+    "sdk_mapped_conv_plan_build": [_vp] * 3 + [_sz] + [_i64] * 5 + [_i32] * 3 + [_vp],
 }
 OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes",
                  "sdk_resample_to_map_workspace_bytes", "sdk_mapped_max_unpool_workspace_bytes",
-                 "sdk_resample_to_uv_maps_workspace_bytes", "sdk_voting_resample_workspace_bytes")
+                 "sdk_resample_to_uv_maps_workspace_bytes", "sdk_voting_resample_workspace_bytes",
+                 "sdk_mapped_conv_plan_bytes")
 
 _lib = None
 
@@ -82,6 +93,8 @@ def load():
     lib.sdk_resample_to_uv_maps_workspace_bytes.restype = _sz
     lib.sdk_voting_resample_workspace_bytes.argtypes = [_i64] * 4
     lib.sdk_voting_resample_workspace_bytes.restype = _sz
+    lib.sdk_mapped_conv_plan_bytes.argtypes = [_i64] * 5 + [_i32] * 3
+    lib.sdk_mapped_conv_plan_bytes.restype = _sz
     _lib = lib
     return lib
 

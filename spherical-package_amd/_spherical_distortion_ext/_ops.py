@@ -90,6 +90,61 @@ def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
 
 
+# --------------------------------------------------------------------------- conv plans
+# What the convolution kernels derive from a sample map alone (include/sdk_mapped_ops.h, "Plans")
+# is built once per map and reused by every later call on it.  An entry is keyed on the map's
+# (and the point weights') storage address, offset, version counter, shape and the geometry, and
+# holds the storages, so an address cannot be handed to another tensor while its entry lives;
+# in-place changes of a map bump its version and miss.
+_PLAN_CACHE = {}
+_PLAN_CACHE_MAX = 16
+_plan_cache_enabled = True
+
+
+def set_conv_plan_cache(enabled):
+    """Keeps (default) or rebuilds per call the plans of the mapped (transposed) convolutions."""
+    global _plan_cache_enabled
+    _plan_cache_enabled = bool(enabled)
+    if not enabled:
+        _PLAN_CACHE.clear()
+
+
+def _tensor_key(t):
+    if t is None:
+        return None
+    return (t.untyped_storage().data_ptr(), t.storage_offset(), t._version, tuple(t.shape))
+
+
+def _conv_plan(ref, sample_map, interp_weights, img_h, img_w, K, P, interp):
+    """(plan tensor, bytes) for this map and geometry, built on first use; (None, 0) when the
+    library has no plan for it or the cache is off."""
+    if not _plan_cache_enabled or ref.dtype != torch.float32:
+        return None, 0
+    MH, MW = int(sample_map.shape[0]), int(sample_map.shape[1])
+    key = (ref.device, _tensor_key(sample_map), _tensor_key(interp_weights), int(img_h),
+           int(img_w), int(K), int(P), int(interp))
+    ent = _PLAN_CACHE.get(key)
+    cur = torch.cuda.current_stream(ref.device)
+    if ent is not None:
+        if ent[3] != cur:
+            cur.wait_stream(ent[3])   # built on another stream: order this call behind the build
+        return ent[0], ent[1]
+    n = _capi.load().sdk_mapped_conv_plan_bytes(int(img_h), int(img_w), MH, MW, int(K), int(P),
+                                                int(interp), _capi.SDK_F32)
+    if n == 0:
+        return None, 0
+    plan = torch.empty(n, dtype=torch.uint8, device=ref.device)
+    _capi.call("sdk_mapped_conv_plan_build", _ptr(sample_map), _ptr(interp_weights), _ptr(plan), n,
+               int(img_h), int(img_w), MH, MW, int(K), int(P), int(interp), _capi.SDK_F32,
+               _stream(ref))
+    while len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
+        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
+    keep = (sample_map.untyped_storage(),
+            None if interp_weights is None else interp_weights.untyped_storage())
+    _PLAN_CACHE[key] = (plan, n, keep, cur)
+    return plan, n
+
+
 def _scatter_workspace(ref, out_h, out_w, query="sdk_resample_to_map_workspace_bytes"):
     n = getattr(_capi.load(), query)(int(out_h), int(out_w), _DTYPES[ref.dtype])
     if n == 0:
@@ -306,9 +361,16 @@ def mapped_conv_forward(x, sample_map, interp_weights, weight, bias, kernel_size
     out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
-        _capi.call("sdk_mapped_conv_forward", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
-                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B, Cin, H, W, Cout, OH,
-                   OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode, _stream(x))
+        plan, nplan = _conv_plan(x, sample_map, interp_weights, H, W, K, P, int(interp))
+        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode,
+                _stream(x))
+        if plan is None:
+            _capi.call("sdk_mapped_conv_forward", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
+                       _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, *dims)
+        else:
+            _capi.call("sdk_mapped_conv_forward_planned", _ptr(x), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws,
+                       _ptr(plan), nplan, *dims)
     return out
 
 
@@ -331,9 +393,15 @@ def mapped_conv_backward(grad_output, sample_map, interp_weights, x, weight, bia
         ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
-        _capi.call("sdk_mapped_conv_backward", _ptr(grad_output), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
-                   _ptr(ws), nws, *dims)
+        plan, nplan = _conv_plan(x, sample_map, interp_weights, H, W, K, P, int(interp))
+        if plan is None:
+            _capi.call("sdk_mapped_conv_backward", _ptr(grad_output), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
+                       _ptr(ws), nws, *dims)
+        else:
+            _capi.call("sdk_mapped_conv_backward_planned", _ptr(grad_output), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
+                       _ptr(ws), nws, _ptr(plan), nplan, *dims)
     return gi, gw, gb
 
 
@@ -351,10 +419,17 @@ def mapped_transposed_conv_forward(x, sample_map, interp_weights, weight, bias, 
     out = torch.empty((B, Cout, OH, OW), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
-        _capi.call("sdk_mapped_transposed_conv_forward", _ptr(x), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws, B,
-                   Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype],
-                   _compute_mode, _stream(x))
+        plan, nplan = _conv_plan(x, sample_map, interp_weights, OH, OW, K, P, int(interp))
+        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode,
+                _stream(x))
+        if plan is None:
+            _capi.call("sdk_mapped_transposed_conv_forward", _ptr(x), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws,
+                       *dims)
+        else:
+            _capi.call("sdk_mapped_transposed_conv_forward_planned", _ptr(x), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nws,
+                       _ptr(plan), nplan, *dims)
     return out
 
 
@@ -375,9 +450,15 @@ def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, 
         ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         s = _stream(x)
         dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
-        _capi.call("sdk_mapped_transposed_conv_backward", _ptr(grad_output), _ptr(sample_map),
-                   _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
-                   _ptr(ws), nws, *dims)
+        plan, nplan = _conv_plan(x, sample_map, interp_weights, OH, OW, K, P, int(interp))
+        if plan is None:
+            _capi.call("sdk_mapped_transposed_conv_backward", _ptr(grad_output), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi), _ptr(gw), _ptr(gb),
+                       _ptr(ws), nws, *dims)
+        else:
+            _capi.call("sdk_mapped_transposed_conv_backward_planned", _ptr(grad_output),
+                       _ptr(sample_map), _ptr(interp_weights), _ptr(x), _ptr(weight), _ptr(gi),
+                       _ptr(gw), _ptr(gb), _ptr(ws), nws, _ptr(plan), nplan, *dims)
     return gi, gw, gb
 
 

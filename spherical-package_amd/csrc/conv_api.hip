@@ -46,25 +46,42 @@ int check_workspace(const char* what, size_t need, void* ws, size_t ws_bytes) {
 enum Op { GATHER_GEMM, GEMM_SCATTER, GATHER_WGRAD };
 
 // a: pixel-side tensor for GEMM_SCATTER / GATHER_WGRAD inputs, image otherwise (see call sites).
+// A plan buffer handed in by the caller (sdk_mapped_conv_plan_build), or none.
+struct PlanArg {
+  void* buffer = nullptr;
+  size_t bytes = 0;
+};
+
 int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, const void* in0,
         const void* map, const void* wts, const void* in1, const void* bias, void* out, void* ws,
-        size_t ws_bytes, hipStream_t stream, SharedPlan* shared = nullptr) {
+        size_t ws_bytes, hipStream_t stream, SharedPlan* shared = nullptr,
+        PlanArg plan = PlanArg()) {
   if (g.B == 0 && op != GATHER_WGRAD) return SDK_OK;
   if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(g)) {
     int rc = check_workspace(what, fused_workspace_bytes(g), ws, ws_bytes);
     if (rc) return rc;
+    CachedPlan cached;
+    const CachedPlan* cp = nullptr;
+    if (plan.buffer != nullptr) {
+      const size_t need = cached_plan_bytes(g);
+      if (need == 0 || plan.bytes < need)
+        return fail(SDK_ERR_WORKSPACE, "%s: the plan buffer has %zu bytes, this geometry's plan %zu",
+                    what, plan.bytes, need);
+      load_cached_plan(g, plan.buffer, &cached);
+      cp = &cached;
+    }
     const float* m = (const float*)map;
     const float* w = (const float*)wts;
     switch (op) {
       case GATHER_GEMM:
         return fused_gather_gemm(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                 (const float*)bias, (float*)out, (float*)ws, stream);
+                                 (const float*)bias, (float*)out, (float*)ws, stream, cp);
       case GEMM_SCATTER:
         return fused_gemm_scatter(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                  (const float*)bias, (float*)out, (float*)ws, stream, shared);
+                                  (const float*)bias, (float*)out, (float*)ws, stream, shared, cp);
       case GATHER_WGRAD:
         return fused_gather_wgrad(g, compute, (const float*)in0, m, w, (const float*)in1,
-                                  (float*)out, (float*)ws, stream, shared);
+                                  (float*)out, (float*)ws, stream, shared, cp);
     }
   }
   if (compute == SDK_COMPUTE_BF16)
@@ -113,13 +130,13 @@ size_t sdk_mapped_conv_workspace_bytes(int64_t batch, int64_t in_channels, int64
                                  dtype);
 }
 
-int sdk_mapped_conv_forward(const void* input, const void* sample_map, const void* interp_weights,
+static int impl_mapped_conv_forward(const void* input, const void* sample_map, const void* interp_weights,
                             const void* weight, const void* bias, void* output, void* workspace,
                             size_t workspace_bytes, int64_t batch, int64_t in_channels,
                             int64_t height, int64_t width, int64_t out_channels,
                             int64_t out_height, int64_t out_width, int64_t kernel_size,
                             int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                            int32_t compute, sdk_stream_t stream) {
+                            int32_t compute, sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_conv_forward";
   SDK_REQUIRE(input && sample_map && weight && bias && output, "%s: NULL pointer", what);
   SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
@@ -130,17 +147,17 @@ int sdk_mapped_conv_forward(const void* input, const void* sample_map, const voi
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GATHER_GEMM, g, dtype, compute, input, sample_map, interp_weights, weight, bias,
-             output, workspace, workspace_bytes, (hipStream_t)stream);
+             output, workspace, workspace_bytes, (hipStream_t)stream, nullptr, plan);
 }
 
-int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_map,
+static int impl_mapped_conv_backward_input(const void* grad_output, const void* sample_map,
                                    const void* interp_weights, const void* weight,
                                    void* grad_input, void* workspace, size_t workspace_bytes,
                                    int64_t batch, int64_t in_channels, int64_t height,
                                    int64_t width, int64_t out_channels, int64_t out_height,
                                    int64_t out_width, int64_t kernel_size,
                                    int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                                   int32_t compute, sdk_stream_t stream) {
+                                   int32_t compute, sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_conv_backward_input";
   SDK_REQUIRE(grad_output && sample_map && weight && grad_input, "%s: NULL pointer", what);
   SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
@@ -151,17 +168,18 @@ int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_m
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights,
-             weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
+             weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, nullptr,
+             plan);
 }
 
-int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_map,
+static int impl_mapped_conv_backward_weight(const void* grad_output, const void* sample_map,
                                     const void* interp_weights, const void* input,
                                     void* grad_weight, void* workspace, size_t workspace_bytes,
                                     int64_t batch, int64_t in_channels, int64_t height,
                                     int64_t width, int64_t out_channels, int64_t out_height,
                                     int64_t out_width, int64_t kernel_size,
                                     int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                                    int32_t compute, sdk_stream_t stream) {
+                                    int32_t compute, sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_conv_backward_weight";
   SDK_REQUIRE(grad_output && sample_map && input && grad_weight, "%s: NULL pointer", what);
   SDK_REQUIRE(out_height >= 1 && out_width >= 1, "%s: bad output size", what);
@@ -172,10 +190,10 @@ int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
   return run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
-             nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
+             nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, nullptr, plan);
 }
 
-int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map,
+static int impl_mapped_transposed_conv_forward(const void* input, const void* sample_map,
                                        const void* interp_weights, const void* weight,
                                        const void* bias, void* output, void* workspace,
                                        size_t workspace_bytes, int64_t batch,
@@ -183,7 +201,7 @@ int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map
                                        int64_t out_channels, int64_t out_height,
                                        int64_t out_width, int64_t kernel_size,
                                        int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                                       int32_t compute, sdk_stream_t stream) {
+                                       int32_t compute, sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_transposed_conv_forward";
   SDK_REQUIRE(input && sample_map && weight && bias && output, "%s: NULL pointer", what);
   SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
@@ -194,10 +212,10 @@ int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GEMM_SCATTER, g, dtype, compute, input, sample_map, interp_weights, weight,
-             bias, output, workspace, workspace_bytes, (hipStream_t)stream);
+             bias, output, workspace, workspace_bytes, (hipStream_t)stream, nullptr, plan);
 }
 
-int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const void* sample_map,
+static int impl_mapped_transposed_conv_backward_input(const void* grad_output, const void* sample_map,
                                               const void* interp_weights, const void* weight,
                                               void* grad_input, void* workspace,
                                               size_t workspace_bytes, int64_t batch,
@@ -206,7 +224,7 @@ int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const voi
                                               int64_t out_height, int64_t out_width,
                                               int64_t kernel_size, int32_t num_interp_pts,
                                               int32_t interp, int32_t dtype, int32_t compute,
-                                              sdk_stream_t stream) {
+                                              sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_transposed_conv_backward_input";
   SDK_REQUIRE(grad_output && sample_map && weight && grad_input, "%s: NULL pointer", what);
   SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
@@ -220,7 +238,7 @@ int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const voi
              nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
-int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
+static int impl_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
                                                const void* interp_weights, const void* input,
                                                void* grad_weight, void* workspace,
                                                size_t workspace_bytes, int64_t batch,
@@ -229,7 +247,7 @@ int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const vo
                                                int64_t out_height, int64_t out_width,
                                                int64_t kernel_size, int32_t num_interp_pts,
                                                int32_t interp, int32_t dtype, int32_t compute,
-                                               sdk_stream_t stream) {
+                                               sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_transposed_conv_backward_weight";
   SDK_REQUIRE(grad_output && sample_map && input && grad_weight, "%s: NULL pointer", what);
   SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
@@ -240,17 +258,18 @@ int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const vo
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GATHER_WGRAD, g, dtype, compute, input, sample_map, interp_weights,
-             grad_output, nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream);
+             grad_output, nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream,
+             nullptr, plan);
 }
 
-int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
+static int impl_mapped_conv_backward(const void* grad_output, const void* sample_map,
                              const void* interp_weights, const void* input, const void* weight,
                              void* grad_input, void* grad_weight, void* grad_bias,
                              void* workspace, size_t workspace_bytes, int64_t batch,
                              int64_t in_channels, int64_t height, int64_t width,
                              int64_t out_channels, int64_t out_height, int64_t out_width,
                              int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
-                             int32_t dtype, int32_t compute, sdk_stream_t stream) {
+                             int32_t dtype, int32_t compute, sdk_stream_t stream, PlanArg plan) {
   const char* what = "mapped_conv_backward";
   SDK_REQUIRE(grad_output && sample_map && input && weight && grad_input && grad_weight &&
                   grad_bias,
@@ -264,12 +283,263 @@ int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
   SharedPlan shared;   // the tap plan of the map is built once for both contractions
   rc = run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
-           nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared);
+           nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared, plan);
   if (rc) return rc;
   rc = run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
-           nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, &shared);
+           nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, &shared, plan);
   if (rc) return rc;
   return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, stream);
+}
+
+static int impl_mapped_transposed_conv_backward(const void* grad_output, const void* sample_map,
+                                        const void* interp_weights, const void* input,
+                                        const void* weight, void* grad_input, void* grad_weight,
+                                        void* grad_bias, void* workspace, size_t workspace_bytes,
+                                        int64_t batch, int64_t in_channels, int64_t in_height,
+                                        int64_t in_width, int64_t out_channels,
+                                        int64_t out_height, int64_t out_width,
+                                        int64_t kernel_size, int32_t num_interp_pts,
+                                        int32_t interp, int32_t dtype, int32_t compute,
+                                        sdk_stream_t stream, PlanArg plan) {
+  int rc = impl_mapped_transposed_conv_backward_input(
+      grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes,
+      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
+      num_interp_pts, interp, dtype, compute, stream, plan);
+  if (rc) return rc;
+  rc = impl_mapped_transposed_conv_backward_weight(
+      grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes,
+      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
+      num_interp_pts, interp, dtype, compute, stream, plan);
+  if (rc) return rc;
+  SDK_REQUIRE(grad_bias, "mapped_transposed_conv_backward: NULL pointer");
+  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype,
+                       stream);
+}
+
+
+size_t sdk_mapped_conv_plan_bytes(int64_t image_height, int64_t image_width, int64_t map_height,
+                                  int64_t map_width, int64_t kernel_size, int32_t num_interp_pts,
+                                  int32_t interp, int32_t dtype) {
+  if (dtype != SDK_F32 || map_height < 1 || map_width < 1 || image_height < 1 || image_width < 1 ||
+      kernel_size < 1 || num_interp_pts < 0 ||
+      map_height * map_width >= ((int64_t)1 << 31) || image_height * image_width >= ((int64_t)1 << 31))
+    return 0;
+  ConvGeom g{1, 1, (int)image_height, (int)image_width, 1, (int)(map_height * map_width),
+             (int)kernel_size, num_interp_pts, interp, (int)map_width};
+  if (!fused_supported(g)) return 0;
+  return cached_plan_bytes(g);
+}
+
+int sdk_mapped_conv_plan_build(const void* sample_map, const void* interp_weights, void* plan,
+                               size_t plan_bytes, int64_t image_height, int64_t image_width,
+                               int64_t map_height, int64_t map_width, int64_t kernel_size,
+                               int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                               sdk_stream_t stream) {
+  const char* what = "mapped_conv_plan_build";
+  SDK_REQUIRE(sample_map && plan, "%s: NULL pointer", what);
+  SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
+              "%s: weighted map needs interp_weights", what);
+  const size_t need = sdk_mapped_conv_plan_bytes(image_height, image_width, map_height, map_width,
+                                                 kernel_size, num_interp_pts, interp, dtype);
+  if (need == 0)
+    return fail(SDK_ERR_UNSUPPORTED, "%s: no plan for this geometry (ask sdk_mapped_conv_plan_bytes)",
+                what);
+  if (plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "%s: needs %zu bytes, got %zu", what, need, plan_bytes);
+  ConvGeom g{1, 1, (int)image_height, (int)image_width, 1, (int)(map_height * map_width),
+             (int)kernel_size, num_interp_pts, interp, (int)map_width};
+  return build_cached_plan(g, (const float*)sample_map, (const float*)interp_weights, plan,
+                           (hipStream_t)stream);
+}
+
+int sdk_mapped_conv_forward(const void* input, const void* sample_map, const void* interp_weights,
+                            const void* weight, const void* bias, void* output, void* workspace,
+                            size_t workspace_bytes, int64_t batch, int64_t in_channels,
+                            int64_t height, int64_t width, int64_t out_channels,
+                            int64_t out_height, int64_t out_width, int64_t kernel_size,
+                            int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                            int32_t compute, sdk_stream_t stream) {
+  return impl_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, output, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_conv_forward_planned(const void* input, const void* sample_map, const void* interp_weights,
+                            const void* weight, const void* bias, void* output, void* workspace,
+                            size_t workspace_bytes, void* plan,
+    size_t plan_bytes, int64_t batch, int64_t in_channels,
+                            int64_t height, int64_t width, int64_t out_channels,
+                            int64_t out_height, int64_t out_width, int64_t kernel_size,
+                            int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                            int32_t compute, sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, output, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_conv_backward_input(const void* grad_output, const void* sample_map,
+                                   const void* interp_weights, const void* weight,
+                                   void* grad_input, void* workspace, size_t workspace_bytes,
+                                   int64_t batch, int64_t in_channels, int64_t height,
+                                   int64_t width, int64_t out_channels, int64_t out_height,
+                                   int64_t out_width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   int32_t compute, sdk_stream_t stream) {
+  return impl_mapped_conv_backward_input(grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_conv_backward_input_planned(const void* grad_output, const void* sample_map,
+                                   const void* interp_weights, const void* weight,
+                                   void* grad_input, void* workspace, size_t workspace_bytes, void* plan,
+    size_t plan_bytes,
+                                   int64_t batch, int64_t in_channels, int64_t height,
+                                   int64_t width, int64_t out_channels, int64_t out_height,
+                                   int64_t out_width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   int32_t compute, sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_conv_backward_input(grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                    const void* interp_weights, const void* input,
+                                    void* grad_weight, void* workspace, size_t workspace_bytes,
+                                    int64_t batch, int64_t in_channels, int64_t height,
+                                    int64_t width, int64_t out_channels, int64_t out_height,
+                                    int64_t out_width, int64_t kernel_size,
+                                    int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                    int32_t compute, sdk_stream_t stream) {
+  return impl_mapped_conv_backward_weight(grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_conv_backward_weight_planned(const void* grad_output, const void* sample_map,
+                                    const void* interp_weights, const void* input,
+                                    void* grad_weight, void* workspace, size_t workspace_bytes, void* plan,
+    size_t plan_bytes,
+                                    int64_t batch, int64_t in_channels, int64_t height,
+                                    int64_t width, int64_t out_channels, int64_t out_height,
+                                    int64_t out_width, int64_t kernel_size,
+                                    int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                    int32_t compute, sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_conv_backward_weight(grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_transposed_conv_forward(const void* input, const void* sample_map,
+                                       const void* interp_weights, const void* weight,
+                                       const void* bias, void* output, void* workspace,
+                                       size_t workspace_bytes, int64_t batch,
+                                       int64_t in_channels, int64_t in_height, int64_t in_width,
+                                       int64_t out_channels, int64_t out_height,
+                                       int64_t out_width, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute, sdk_stream_t stream) {
+  return impl_mapped_transposed_conv_forward(input, sample_map, interp_weights, weight, bias, output, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_transposed_conv_forward_planned(const void* input, const void* sample_map,
+                                       const void* interp_weights, const void* weight,
+                                       const void* bias, void* output, void* workspace,
+                                       size_t workspace_bytes, void* plan,
+    size_t plan_bytes, int64_t batch,
+                                       int64_t in_channels, int64_t in_height, int64_t in_width,
+                                       int64_t out_channels, int64_t out_height,
+                                       int64_t out_width, int64_t kernel_size,
+                                       int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                       int32_t compute, sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_transposed_conv_forward(input, sample_map, interp_weights, weight, bias, output, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_transposed_conv_backward_input(const void* grad_output, const void* sample_map,
+                                              const void* interp_weights, const void* weight,
+                                              void* grad_input, void* workspace,
+                                              size_t workspace_bytes, int64_t batch,
+                                              int64_t in_channels, int64_t in_height,
+                                              int64_t in_width, int64_t out_channels,
+                                              int64_t out_height, int64_t out_width,
+                                              int64_t kernel_size, int32_t num_interp_pts,
+                                              int32_t interp, int32_t dtype, int32_t compute,
+                                              sdk_stream_t stream) {
+  return impl_mapped_transposed_conv_backward_input(grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_transposed_conv_backward_input_planned(const void* grad_output, const void* sample_map,
+                                              const void* interp_weights, const void* weight,
+                                              void* grad_input, void* workspace,
+                                              size_t workspace_bytes, void* plan,
+    size_t plan_bytes, int64_t batch,
+                                              int64_t in_channels, int64_t in_height,
+                                              int64_t in_width, int64_t out_channels,
+                                              int64_t out_height, int64_t out_width,
+                                              int64_t kernel_size, int32_t num_interp_pts,
+                                              int32_t interp, int32_t dtype, int32_t compute,
+                                              sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_transposed_conv_backward_input(grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
+                                               const void* interp_weights, const void* input,
+                                               void* grad_weight, void* workspace,
+                                               size_t workspace_bytes, int64_t batch,
+                                               int64_t in_channels, int64_t in_height,
+                                               int64_t in_width, int64_t out_channels,
+                                               int64_t out_height, int64_t out_width,
+                                               int64_t kernel_size, int32_t num_interp_pts,
+                                               int32_t interp, int32_t dtype, int32_t compute,
+                                               sdk_stream_t stream) {
+  return impl_mapped_transposed_conv_backward_weight(grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_transposed_conv_backward_weight_planned(const void* grad_output, const void* sample_map,
+                                               const void* interp_weights, const void* input,
+                                               void* grad_weight, void* workspace,
+                                               size_t workspace_bytes, void* plan,
+    size_t plan_bytes, int64_t batch,
+                                               int64_t in_channels, int64_t in_height,
+                                               int64_t in_width, int64_t out_channels,
+                                               int64_t out_height, int64_t out_width,
+                                               int64_t kernel_size, int32_t num_interp_pts,
+                                               int32_t interp, int32_t dtype, int32_t compute,
+                                               sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_transposed_conv_backward_weight(grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
+}
+
+int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
+                             const void* interp_weights, const void* input, const void* weight,
+                             void* grad_input, void* grad_weight, void* grad_bias,
+                             void* workspace, size_t workspace_bytes, int64_t batch,
+                             int64_t in_channels, int64_t height, int64_t width,
+                             int64_t out_channels, int64_t out_height, int64_t out_width,
+                             int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                             int32_t dtype, int32_t compute, sdk_stream_t stream) {
+  return impl_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_conv_backward_planned(const void* grad_output, const void* sample_map,
+                             const void* interp_weights, const void* input, const void* weight,
+                             void* grad_input, void* grad_weight, void* grad_bias,
+                             void* workspace, size_t workspace_bytes, void* plan,
+    size_t plan_bytes, int64_t batch,
+                             int64_t in_channels, int64_t height, int64_t width,
+                             int64_t out_channels, int64_t out_height, int64_t out_width,
+                             int64_t kernel_size, int32_t num_interp_pts, int32_t interp,
+                             int32_t dtype, int32_t compute, sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, batch, in_channels, height, width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
 }
 
 int sdk_mapped_transposed_conv_backward(const void* grad_output, const void* sample_map,
@@ -282,19 +552,24 @@ int sdk_mapped_transposed_conv_backward(const void* grad_output, const void* sam
                                         int64_t kernel_size, int32_t num_interp_pts,
                                         int32_t interp, int32_t dtype, int32_t compute,
                                         sdk_stream_t stream) {
-  int rc = sdk_mapped_transposed_conv_backward_input(
-      grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes,
-      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
-      num_interp_pts, interp, dtype, compute, stream);
-  if (rc) return rc;
-  rc = sdk_mapped_transposed_conv_backward_weight(
-      grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes,
-      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
-      num_interp_pts, interp, dtype, compute, stream);
-  if (rc) return rc;
-  SDK_REQUIRE(grad_bias, "mapped_transposed_conv_backward: NULL pointer");
-  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype,
-                       stream);
+  return impl_mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, input, weight, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, PlanArg());
+}
+
+int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const void* sample_map,
+                                        const void* interp_weights, const void* input,
+                                        const void* weight, void* grad_input, void* grad_weight,
+                                        void* grad_bias, void* workspace, size_t workspace_bytes, void* plan,
+    size_t plan_bytes,
+                                        int64_t batch, int64_t in_channels, int64_t in_height,
+                                        int64_t in_width, int64_t out_channels,
+                                        int64_t out_height, int64_t out_width,
+                                        int64_t kernel_size, int32_t num_interp_pts,
+                                        int32_t interp, int32_t dtype, int32_t compute,
+                                        sdk_stream_t stream) {
+  PlanArg pa;
+  pa.buffer = plan;
+  pa.bytes = plan_bytes;
+  return impl_mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, input, weight, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size, num_interp_pts, interp, dtype, compute, stream, pa);
 }
 
 }  // extern "C"

@@ -697,12 +697,15 @@ static float* wgrad_partial(const ConvGeom& g, float* workspace) {
 // gW += the sums of a plan: tiles that fit the window kernel there, the others (and every
 // tile when that kernel does not cover the call) in the plan-driven kernel.
 static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
-                           const float* img, float* gW, float* workspace, hipStream_t stream) {
+                           const float* img, float* gW, float* workspace, hipStream_t stream,
+                           const TileLists* lists4 = nullptr) {
   if (window_wgrad_supported(g, mm) && window_wgrad_partial_bytes(g) != 0) {
     const WgradTail t = wgrad_tail(g);
     char* base = wgrad_tail_base(g, workspace);
     TileLists tl;
-    int rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
+    int rc = SDK_OK;
+    if (lists4 != nullptr) tl = *lists4;
+    else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
     if (rc) return rc;
     rc = window_wgrad(g, plan, tl, pix, img, gW, reinterpret_cast<float*>(base + t.window_partial),
                       stream);
@@ -740,7 +743,7 @@ static int launch_smem(const char* what, Kern kern, dim3 grid, size_t smem, hipS
 
 int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
                       const float* wts, const float* Wm, const float* bias, float* pix,
-                      float* workspace, hipStream_t stream) {
+                      float* workspace, hipStream_t stream, const CachedPlan* cached) {
   const int mm = matrix_mode(compute);
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
@@ -756,11 +759,16 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
     const GatherLayout l = gather_layout(g);
     char* ws = reinterpret_cast<char*>(workspace);
     Plan plan;
-    rc = build_plan(g, map, wts, ws + l.plan, stream, &plan);
-    if (rc) return rc;
     TileLists tl;
-    rc = build_tile_lists(plan, ws + l.lists, stream, &tl);
-    if (rc) return rc;
+    if (cached != nullptr) {
+      plan = cached->plan;
+      tl = cached->lists;
+    } else {
+      rc = build_plan(g, map, wts, ws + l.plan, stream, &plan);
+      if (rc) return rc;
+      rc = build_tile_lists(plan, ws + l.lists, stream, &tl);
+      if (rc) return rc;
+    }
     rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
                      reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream);
     if (rc) return rc;
@@ -996,7 +1004,8 @@ static int inverse_gather_gemm(const ConvGeom& g, int mm, const InverseMap& inv,
 
 int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* Wm, const float* bias, float* img,
-                       float* workspace, hipStream_t stream, SharedPlan* shared) {
+                       float* workspace, hipStream_t stream, SharedPlan* shared,
+                       const CachedPlan* cached) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = SDK_OK;
   if (planned_scatter_supported(g)) {
@@ -1014,11 +1023,16 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
         const ScatterLayout l = scatter_layout(g);
         const ConvGeom r = inverse_geom(g);
         InversePlan ip;
-        rc = build_inverse_plan(g, map, wts, inv_ws + l.inverse, stream, &ip);
-        if (rc) return rc;
         TileLists tl;
-        rc = build_tile_lists(ip.plan, inv_ws + l.lists, stream, &tl);
-        if (rc) return rc;
+        if (cached != nullptr && cached->has_inverse) {
+          ip = cached->inverse;
+          tl = cached->inverse_lists;
+        } else {
+          rc = build_inverse_plan(g, map, wts, inv_ws + l.inverse, stream, &ip);
+          if (rc) return rc;
+          rc = build_tile_lists(ip.plan, inv_ws + l.lists, stream, &tl);
+          if (rc) return rc;
+        }
         rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
                          reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream);
         if (rc) return rc;
@@ -1050,6 +1064,14 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     }
     rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream, gate);
     if (rc) return rc;
+    if (cached != nullptr && shared != nullptr) {
+      // the weight gradient of this call takes the cached plan; the scatter kernel (which runs
+      // only if the gate is raised) builds its own
+      shared->plan = cached->plan;
+      shared->valid = true;
+      return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream,
+                                  nullptr);
+    }
     return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream, shared);
   }
   rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
@@ -1078,12 +1100,15 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
 
 int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const float* map,
                        const float* wts, const float* img, float* gW, float* workspace,
-                       hipStream_t stream, const SharedPlan* shared) {
+                       hipStream_t stream, const SharedPlan* shared, const CachedPlan* cached) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
   if (planned_wgrad_supported(g)) {
+    if (cached != nullptr)
+      return wgrad_from_plan(g, matrix_mode(compute), cached->plan, pix, img, gW, workspace,
+                             stream, &cached->lists4);
     if (shared != nullptr && shared->valid)
       return wgrad_from_plan(g, matrix_mode(compute), shared->plan, pix, img, gW, workspace,
                              stream);
@@ -1117,6 +1142,69 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   if (bf16) GW(true); else GW(false);
 #undef GW
   return rc;
+}
+
+// ---------------------------------------------------------------------------
+// Cached plan: [tap plan][tile lists][tile lists, at most four rows][inverse plan][its lists]
+// ---------------------------------------------------------------------------
+namespace {
+struct CachedLayout {
+  size_t plan, lists, lists4, inverse, inverse_lists, total;
+  bool has_inverse;
+};
+CachedLayout cached_layout(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  CachedLayout l;
+  l.plan = 0;
+  l.lists = up(plan_bytes(g));
+  l.lists4 = l.lists + up(tile_lists_bytes(g));
+  l.inverse = l.lists4 + up(tile_lists_bytes(g));
+  // the inverse plan as scatter_from_window() needs it, whatever the channel counts
+  l.has_inverse = g.K <= 256 && g.M <= (1 << 24) && g.M % g.OW == 0 &&
+                  plan_supported(inverse_geom(g)) &&
+                  (int64_t)g.H * g.W * g.K < ((int64_t)1 << 31);
+  l.inverse_lists = l.inverse + (l.has_inverse ? up(inverse_plan_bytes(g)) : 0);
+  l.total = l.inverse_lists + (l.has_inverse ? up(tile_lists_bytes(inverse_geom(g))) : 0);
+  return l;
+}
+}  // namespace
+
+size_t cached_plan_bytes(const ConvGeom& g) {
+  if (!plan_supported(g) || (int64_t)g.H * g.W > ((int64_t)1 << 24)) return 0;
+  return cached_layout(g).total;
+}
+
+void load_cached_plan(const ConvGeom& g, void* buffer, CachedPlan* out) {
+  const CachedLayout l = cached_layout(g);
+  char* b = static_cast<char*>(buffer);
+  load_plan(g, b + l.plan, &out->plan);
+  load_tile_lists(out->plan, b + l.lists, &out->lists);
+  load_tile_lists(out->plan, b + l.lists4, &out->lists4);
+  out->has_inverse = l.has_inverse;
+  if (l.has_inverse) {
+    load_inverse_plan(g, b + l.inverse, &out->inverse);
+    load_tile_lists(out->inverse.plan, b + l.inverse_lists, &out->inverse_lists);
+  }
+}
+
+int build_cached_plan(const ConvGeom& g, const float* map, const float* wts, void* buffer,
+                      hipStream_t stream) {
+  const CachedLayout l = cached_layout(g);
+  char* b = static_cast<char*>(buffer);
+  CachedPlan cp;
+  int rc = build_plan(g, map, wts, b + l.plan, stream, &cp.plan);
+  if (rc) return rc;
+  rc = build_tile_lists(cp.plan, b + l.lists, stream, &cp.lists, 0);
+  if (rc) return rc;
+  rc = build_tile_lists(cp.plan, b + l.lists4, stream, &cp.lists4, 4);
+  if (rc) return rc;
+  if (l.has_inverse) {
+    rc = build_inverse_plan(g, map, wts, b + l.inverse, stream, &cp.inverse);
+    if (rc) return rc;
+    rc = build_tile_lists(cp.inverse.plan, b + l.inverse_lists, stream, &cp.inverse_lists, 0);
+    if (rc) return rc;
+  }
+  return SDK_OK;
 }
 
 }  // namespace sdk

@@ -639,27 +639,28 @@ size_t plan_bytes(const ConvGeom& g) {
          tiles * g.K * plan_slots(g) * 128 * sizeof(int2);
 }
 
-int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-               hipStream_t stream, Plan* plan, const int* gate) {
+void load_plan(const ConvGeom& g, void* workspace, Plan* plan) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
-  const int S = plan_slots(g);
   char* base = static_cast<char*>(workspace);
-  int* hdr = reinterpret_cast<int*>(base);
-  int* ns = reinterpret_cast<int*>(base + align16(tiles * 8 * sizeof(int)));
-  int2* taps = reinterpret_cast<int2*>(base + align16(tiles * 8 * sizeof(int)) +
-                                       align16(tiles * g.K * sizeof(int)));
-  SDK_DISPATCH_INTERP(g.interp, g.P,
-                      (launch(plan_kernel<INTERP, WEIGHTED>, dim3((unsigned)tiles),
-                              dim3(kPlThreads), stream, map, wts, pt, g.K, g.P, g.H, g.W, S, hdr,
-                              ns, taps, gate)));
-  SDK_LAUNCH_CHECK("plan");
   plan->pt = pt;
   plan->tiles = (int)tiles;
-  plan->S = S;
-  plan->hdr = hdr;
-  plan->ns = ns;
-  plan->taps = taps;
+  plan->S = plan_slots(g);
+  plan->hdr = reinterpret_cast<int*>(base);
+  plan->ns = reinterpret_cast<int*>(base + align16(tiles * 8 * sizeof(int)));
+  plan->taps = reinterpret_cast<int2*>(base + align16(tiles * 8 * sizeof(int)) +
+                                       align16(tiles * g.K * sizeof(int)));
+}
+
+int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+               hipStream_t stream, Plan* plan, const int* gate) {
+  load_plan(g, workspace, plan);
+  SDK_DISPATCH_INTERP(g.interp, g.P,
+                      (launch(plan_kernel<INTERP, WEIGHTED>, dim3((unsigned)plan->tiles),
+                              dim3(kPlThreads), stream, map, wts, plan->pt, g.K, g.P, g.H, g.W,
+                              plan->S, const_cast<int*>(plan->hdr), const_cast<int*>(plan->ns),
+                              const_cast<int2*>(plan->taps), gate)));
+  SDK_LAUNCH_CHECK("plan");
   return SDK_OK;
 }
 

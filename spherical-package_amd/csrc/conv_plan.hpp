@@ -82,6 +82,11 @@ struct InversePlan {
 size_t inverse_plan_bytes(const ConvGeom& g);
 int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
                        hipStream_t stream, InversePlan* out);
+// Pointers into a workspace build_inverse_plan filled for the same geometry.
+void load_inverse_plan(const ConvGeom& g, void* workspace, InversePlan* out);
+// Likewise for build_plan and build_tile_lists.
+void load_plan(const ConvGeom& g, void* workspace, Plan* out);
+void load_tile_lists(const Plan& plan, void* workspace, TileLists* out);
 
 bool planned_wgrad_supported(const ConvGeom& g);
 size_t planned_wgrad_partial_bytes(const ConvGeom& g);

@@ -547,16 +547,19 @@ size_t tile_lists_bytes(const ConvGeom& g) {
   return ((size_t)2 * pt.tiles_x * pt.tiles_y + 2) * sizeof(int);
 }
 
-int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
-                     int max_rows) {
+void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
   int* lists = static_cast<int*>(workspace);
-  int* count = lists + (size_t)2 * plan.tiles;
-  launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles, lists, count,
-         max_rows);
-  SDK_LAUNCH_CHECK("tile_lists");
   out->inside = lists;
   out->rest = lists + plan.tiles;
-  out->count = count;
+  out->count = lists + (size_t)2 * plan.tiles;
+}
+
+int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
+                     int max_rows) {
+  load_tile_lists(plan, workspace, out);
+  launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles,
+         const_cast<int*>(out->inside), const_cast<int*>(out->count), max_rows);
+  SDK_LAUNCH_CHECK("tile_lists");
   return SDK_OK;
 }
 
@@ -619,19 +622,29 @@ InverseOffsets inverse_offsets(const ConvGeom& g) {
 
 size_t inverse_plan_bytes(const ConvGeom& g) { return inverse_offsets(g).total; }
 
-int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-                       hipStream_t stream, InversePlan* out) {
+void load_inverse_plan(const ConvGeom& g, void* workspace, InversePlan* out) {
   const InverseOffsets o = inverse_offsets(g);
   const PixelTiling it = plan_tiling(g.H, g.W);
-  const int tiles = it.tiles_x * it.tiles_y;
   char* ws = static_cast<char*>(workspace);
-  int* gate = reinterpret_cast<int*>(ws + o.gate);
+  out->plan.pt = it;
+  out->plan.tiles = it.tiles_x * it.tiles_y;
+  out->plan.S = kInvRows;
+  out->plan.hdr = reinterpret_cast<int*>(ws + o.hdr);
+  out->plan.ns = reinterpret_cast<int*>(ws + o.ns);
+  out->plan.taps = reinterpret_cast<int2*>(ws + o.taps);
+  out->gate = reinterpret_cast<int*>(ws + o.gate);
+  out->raw_off = reinterpret_cast<int*>(ws + o.raw_off);
+  out->raw_co = reinterpret_cast<float*>(ws + o.raw_co);
+}
+
+int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
+                       hipStream_t stream, InversePlan* out) {
+  load_inverse_plan(g, workspace, out);
+  const InverseOffsets o = inverse_offsets(g);
+  char* ws = static_cast<char*>(workspace);
   int* cnt = reinterpret_cast<int*>(ws + o.cnt);
-  float* raw_co = reinterpret_cast<float*>(ws + o.raw_co);
-  int* raw_off = reinterpret_cast<int*>(ws + o.raw_off);
-  int* hdr = reinterpret_cast<int*>(ws + o.hdr);
-  int* ns = reinterpret_cast<int*>(ws + o.ns);
-  int2* taps = reinterpret_cast<int2*>(ws + o.taps);
+  int* raw_off = const_cast<int*>(out->raw_off);
+  float* raw_co = const_cast<float*>(out->raw_co);
   int rc = zero_fill(ws, o.raw_off, stream);
   if (rc) return rc;
   const int64_t total = (int64_t)g.M * g.K;
@@ -640,20 +653,14 @@ int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, vo
   SDK_DISPATCH_INTERP(g.interp, g.P,
                       (launch(inverse_fill_tiled_kernel<INTERP, WEIGHTED>,
                               dim3((unsigned)ceil_div(total, kWgThreads)), dim3(kWgThreads), stream,
-                              map, wts, g.M, g.K, g.P, g.H, g.W, it, cnt, raw_off, raw_co, gate)));
+                              map, wts, g.M, g.K, g.P, g.H, g.W, out->plan.pt, cnt, raw_off, raw_co,
+                              out->gate)));
   SDK_LAUNCH_CHECK("inverse_fill");
-  launch(inverse_plan_kernel, dim3((unsigned)tiles), dim3(kWgThreads), stream, (const int*)cnt,
-         raw_off, raw_co, it, g.K, g.M / g.OW, g.OW, hdr, ns, taps, (const int*)gate);
+  launch(inverse_plan_kernel, dim3((unsigned)out->plan.tiles), dim3(kWgThreads), stream,
+         (const int*)cnt, raw_off, raw_co, out->plan.pt, g.K, g.M / g.OW, g.OW,
+         const_cast<int*>(out->plan.hdr), const_cast<int*>(out->plan.ns),
+         const_cast<int2*>(out->plan.taps), (const int*)out->gate);
   SDK_LAUNCH_CHECK("inverse_plan");
-  out->plan.pt = it;
-  out->plan.tiles = tiles;
-  out->plan.S = kInvRows;
-  out->plan.hdr = hdr;
-  out->plan.ns = ns;
-  out->plan.taps = taps;
-  out->gate = gate;
-  out->raw_off = raw_off;
-  out->raw_co = raw_co;
   return SDK_OK;
 }
 

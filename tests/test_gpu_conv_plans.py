@@ -1,0 +1,132 @@
+"""Plans kept between calls (sdk_mapped_conv_plan_build and the *_planned entry points) against
+the plain entry points, which build the same plan inside every call: identical results, for
+mapped and mapped transposed convolution, on maps whose tiles take every route (inside their
+window, outside it, more than four rows per sample, target lists too long for the inverse
+plan).  The operator-level cache must miss when a map is changed in place.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import relerr
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from _spherical_distortion_ext import _ops
+    return _ops
+
+
+def _t(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _case(seed, Cin, Cout, H, W, OH, OW, K, P, interp, kind):
+    rng = np.random.default_rng(seed)
+    ys, xs = np.meshgrid(np.arange(OH), np.arange(OW), indexing="ij")
+    ang = 2 * np.pi * np.arange(K) / K
+    cx = xs[..., None] * (W / OW) + 1.5 * np.cos(ang)
+    cy = ys[..., None] * (H / OH) + 1.5 * np.sin(ang)
+    if kind == "polar":          # rows near the top spread their samples wide, as near a pole
+        spread = 1.0 + 30.0 / (1.0 + ys[..., None])
+        cx = xs[..., None] * (W / OW) + spread * 1.5 * np.cos(ang)
+    if kind == "crowded":        # a fifth of the samples land on one spot: long target lists
+        sel = rng.uniform(size=cx.shape) < 0.2
+        cx = np.where(sel, 5.3, cx)
+        cy = np.where(sel, 4.1, cy)
+    if P:
+        cx = cx[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
+        cy = cy[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
+    m = np.stack([cx, cy], -1) + rng.uniform(-0.4, 0.4, cx.shape + (2,))
+    m = np.ascontiguousarray(m.astype(np.float32))
+    iw = rng.uniform(0.1, 1, m.shape[:-1]).astype(np.float32) if P else None
+    B = 2
+    x = rng.standard_normal((B, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    g = rng.standard_normal((B, Cout, OH, OW)).astype(np.float32)
+    bt = rng.standard_normal(Cin).astype(np.float32)   # bias of the transposed layer (Cout -> Cin)
+    return m, iw, x, w, b, g, bt
+
+
+# (Cin, Cout, H, W, OH, OW, K, P, interp, kind)
+CASES = [
+    (72, 80, 40, 64, 40, 64, 9, 0, 1, "plain"),      # every tile inside its window
+    (96, 72, 48, 96, 48, 96, 9, 0, 1, "polar"),      # top tile rows outside, the rest inside
+    (80, 96, 24, 40, 24, 40, 5, 2, 1, "plain"),      # eight rows per sample: weight gradient's rest list
+    (72, 72, 20, 36, 20, 36, 6, 0, 0, "crowded"),    # inverse lists overflow: scatter fallback
+    (130, 40, 27, 42, 24, 42, 10, 0, 2, "plain"),    # 12 tiles (not a multiple of 8), K = 10
+    (16, 24, 30, 50, 30, 50, 7, 0, 1, "plain"),      # narrow layers: kernels that ignore the plan
+]
+
+
+@pytest.mark.parametrize("mode", ["native", "split", "bf16"])
+@pytest.mark.parametrize("tc", CASES, ids=lambda t: "x".join(map(str, t)))
+def test_planned_calls_match_plain_calls_and_the_oracle(ops, oracle, tc, mode):
+    Cin, Cout, H, W, OH, OW, K, P, interp, kind = tc
+    m, iw, x, w, b, g, bt = _case(7 + sum(tc[:9]), *tc)
+    tol_f, tol_b = (1e-2, 1e-2) if mode == "bf16" else (1e-5, 1e-4)
+    res = {}
+    ops.set_conv_compute(mode)
+    try:
+        for cached in (False, True):
+            ops.set_conv_plan_cache(cached)
+            tm, tiw = _t(m), _t(iw)
+            for rep in range(2 if cached else 1):       # second pass: the plan comes from the cache
+                y = ops.mapped_conv_forward(_t(x), tm, tiw, _t(w), _t(b), K, interp)
+                gi, gw, gb = ops.mapped_conv_backward(_t(g), tm, tiw, _t(x), _t(w), _t(b), K, interp)
+                # transposed layer over the same map (Cout -> Cin channels, weight [Cout, Cin, K]):
+                # its input lives on the map's grid, its output is H x W
+                yt = ops.mapped_transposed_conv_forward(_t(g), tm, tiw, _t(w), _t(bt), H, W, K,
+                                                        interp)
+            res[cached] = [t.cpu().numpy() for t in (y, gi, gw, gb, yt)]
+    finally:
+        ops.set_conv_plan_cache(True)
+        ops.set_conv_compute("native")
+    y0, gi0, gw0, gb0, yt0 = res[False]
+    y1, gi1, gw1, gb1, yt1 = res[True]
+    assert np.array_equal(y0, y1)
+    if kind == "crowded" or Cin <= 64:
+        # scatter fallback (float atomics) / narrow layers (source lists in the order the
+        # atomics were served): the summation order varies from run to run
+        # (with bf16 operands a last-bit difference of a column value can flip its rounding)
+        loose = 1e-3 if mode == "bf16" else 1e-5
+        assert relerr(gi1, gi0) <= loose and relerr(yt1, yt0) <= loose
+    else:                        # gathers over sorted lists: the same bits
+        assert np.array_equal(gi0, gi1)
+        assert np.array_equal(yt0, yt1)
+    assert relerr(gw1, gw0) <= 1e-6
+    assert relerr(y1, oracle.mapped_conv_forward(x, m, w, b, K, interp, iw)) <= tol_f
+    wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, interp, iw)
+    assert relerr(gi1, wi) <= tol_b and relerr(gw1, ww) <= tol_b
+    assert relerr(yt1, oracle.mapped_transposed_conv_forward(g, m, w, bt, H, W, K, interp,
+                                                             iw)) <= tol_b
+
+
+def test_cache_misses_after_an_in_place_change_of_the_map(ops, oracle):
+    Cin, Cout, H, W, OH, OW, K, P, interp, kind = CASES[0]
+    m, iw, x, w, b, g, _ = _case(3, *CASES[0])
+    tm = _t(m)
+    y0 = ops.mapped_conv_forward(_t(x), tm, None, _t(w), _t(b), K, interp).cpu().numpy()
+    m2 = np.ascontiguousarray(m[:, ::-1].copy())
+    tm.copy_(_t(m2))                                    # same storage, new contents
+    y1 = ops.mapped_conv_forward(_t(x), tm, None, _t(w), _t(b), K, interp).cpu().numpy()
+    assert relerr(y0, oracle.mapped_conv_forward(x, m, w, b, K, interp, None)) <= 1e-5
+    assert relerr(y1, oracle.mapped_conv_forward(x, m2, w, b, K, interp, None)) <= 1e-5
+
+
+def test_plan_buffer_of_the_wrong_size_is_refused(ops):
+    from _spherical_distortion_ext import _capi
+    lib = _capi.load()
+    n = lib.sdk_mapped_conv_plan_bytes(40, 64, 40, 64, 9, 0, 1, _capi.SDK_F32)
+    assert n > 0
+    assert lib.sdk_mapped_conv_plan_bytes(40, 64, 40, 64, 9, 0, 1, _capi.SDK_F64) == 0
+    one = ctypes.c_void_p(256)   # never dereferenced: the size check comes first
+    rc = lib.sdk_mapped_conv_plan_build(one, None, one, n - 1, 40, 64, 40, 64, 9, 0, 1,
+                                        _capi.SDK_F32, None)
+    assert rc != 0 and b"needs" in lib.sdk_last_error()
