@@ -206,7 +206,11 @@ __device__ __forceinline__ void lds_only_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int KB, int MM, int NW>
+// REST: the launch covers a list of tiles most of whose taps lie outside their window (polar
+// rows of a spherical map).  All rows of a sample (up to four) are then requested from the
+// image together, one sample ahead, whatever the lanes' taps say, so that one memory latency
+// per run of samples is exposed instead of one per pair of rows.
+template <int KB, int MM, int NW, bool REST>
 __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW,
@@ -383,18 +387,82 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
         // locality, e.g. mesh neighbourhoods, have all their taps there).
         // (The variants with nine accumulators of 128 rows and fp32 or split A fragments have no
         // registers left for it.)
-        constexpr bool PRE = !(KB == 9 && NW == 4 && MM != kMmBf16);
+        constexpr bool PRE = !REST && !(KB == 9 && NW == 4 && MM != kMmBf16);
         float pre[8];
         bool pre_valid = false;
 #pragma unroll
         for (int j = 0; j < 8; ++j) pre[j] = 0.0f;
+        // REST: image values of rows 0..3 of the sample about to be gathered
+        float pre0[8], pre1[8], pre2[8], pre3[8];
+        const char* const rest_base = reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
+        const unsigned rest_plane = (unsigned)HW * 4u;
+        const unsigned rest_cg = (unsigned)(8 * cg) * rest_plane;
+        // requests the image values of row R of the sample whose rows start at BASE (NR rows)
+#define SDK_REQ_ROW(R, BASE, NR)                                                              \
+  if ((R) < (NR)) {                                                                           \
+    const int2 ec = prow[((BASE) + (R)) * 64 + m_local];                                      \
+    const bool out = ec.x < 0 && __int_as_float(ec.y) != 0.0f;                                \
+    const unsigned o0 = out ? rest_cg + (unsigned)(-ec.x - 1) * 4u : 0u;                      \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
+      const bool g_ok = out && c0 + 8 * cg + j < Cg;                                          \
+      pre##R[j] = *reinterpret_cast<const float*>(rest_base +                                 \
+                                                  (g_ok ? o0 + (unsigned)j * rest_plane : 0u)); \
+    }                                                                                         \
+  }
+        // adds row R (window value or requested image value, times the coefficient) to col[]
+#define SDK_USE_ROW(R, BASE, NR)                                                              \
+  if ((R) < (NR)) {                                                                           \
+    const int2 ec = prow[((BASE) + (R)) * 64 + m_local];                                      \
+    const int e = ec.x;                                                                       \
+    const float co = __int_as_float(ec.y);                                                    \
+    const bool out = e < 0 && co != 0.0f;                                                     \
+    const float4* rp =                                                                        \
+        reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);          \
+    const float4 l0 = rp[0], l1 = rp[1];                                                      \
+    const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};                     \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
+      const bool g_ok = out && c0 + 8 * cg + j < Cg;                                          \
+      col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? pre##R[j] : 0.0f), col[j]);        \
+    }                                                                                         \
+  }
+        if constexpr (REST) {
+          const int nr = min(__builtin_amdgcn_readfirstlane(ns_l[kk_beg]), 4);
+          SDK_REQ_ROW(0, 0, nr) SDK_REQ_ROW(1, 0, nr) SDK_REQ_ROW(2, 0, nr) SDK_REQ_ROW(3, 0, nr)
+        }
 #pragma unroll 1
         for (int kk = kk_beg; kk < kk_end; ++kk) {
-          const int nrows = ns_l[kk];
+          const int nrows = REST ? __builtin_amdgcn_readfirstlane(ns_l[kk]) : ns_l[kk];
           // ---- gather: column values of pixel m_local, channels 8*cg + j
           float col[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j) col[j] = 0.0f;
+          if constexpr (REST) {
+            const int nr = min(nrows, 4);
+            SDK_USE_ROW(0, row0, nr) SDK_USE_ROW(1, row0, nr) SDK_USE_ROW(2, row0, nr) SDK_USE_ROW(3, row0, nr)
+            for (int r = 4; r < nrows; ++r) {   // further rows: one at a time, not requested ahead
+              const int2 ec = prow[(row0 + r) * 64 + m_local];
+              const int e = ec.x;
+              const float co = __int_as_float(ec.y);
+              const bool out = e < 0 && co != 0.0f;
+              const float4* rp =
+                  reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);
+              const float4 l0 = rp[0], l1 = rp[1];
+              const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+              const unsigned o0 = out ? rest_cg + (unsigned)(-e - 1) * 4u : 0u;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const bool g_ok = out && c0 + 8 * cg + j < Cg;
+                const float dg = *reinterpret_cast<const float*>(
+                    rest_base + (g_ok ? o0 + (unsigned)j * rest_plane : 0u));
+                col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? dg : 0.0f), col[j]);
+              }
+            }
+            row0 += nrows;
+            if (kk + 1 < kk_end) {
+              const int nn = min(__builtin_amdgcn_readfirstlane(ns_l[kk + 1]), 4);
+              SDK_REQ_ROW(0, row0, nn) SDK_REQ_ROW(1, row0, nn) SDK_REQ_ROW(2, row0, nn) SDK_REQ_ROW(3, row0, nn)
+            }
+          } else {
           // adds one row (window index or image offset e, coefficient co) to col[]
           auto tap_any = [&](int e, float co) {
             // some lane's tap lies outside the window: that lane reads the image directly
@@ -471,6 +539,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
               pre_valid = true;
             }
           }
+          }  // !REST
           float* ct = colT[buf];
           if constexpr (SPLIT) {
             // The column tile is split where it is written, once, instead of by each of the four
@@ -543,6 +612,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
           if constexpr (SPLIT) lds_only_barrier();   // single tile: all reads before the next writes
           else buf ^= 1;
         }
+#undef SDK_REQ_ROW
+#undef SDK_USE_ROW
         kk_beg = kk_end;
       }
     }
@@ -676,11 +747,13 @@ struct WgradGrid {
   int64_t kinds, slots;
 };
 
-WgradGrid wgrad_grid(const ConvGeom& g, int tiles) {
+// rest: the launch shape of the REST variant of the kernel (at most 5 samples per workgroup,
+// which leaves registers for the values requested ahead).
+WgradGrid wgrad_grid(const ConvGeom& g, int tiles, bool rest) {
   WgradGrid w;
-  const int kblocks = (int)ceil_div(g.K, 9);
+  const int kblocks = (int)ceil_div(g.K, rest ? 5 : 9);
   const int per = (int)ceil_div(g.K, kblocks);
-  w.KB = per <= 1 ? 1 : (per <= 4 ? 4 : (per <= 7 ? 7 : 9));
+  w.KB = per <= 1 ? 1 : (per <= 4 ? 4 : (rest ? 5 : (per <= 7 ? 7 : 9)));
   w.kb_count = (int)ceil_div(g.K, w.KB);
   w.NW = g.Cp > 64 ? 4 : (g.Cp > 32 ? 2 : 1);
   w.c_chunks = (int)ceil_div(g.Cg, kCC);
@@ -702,16 +775,22 @@ constexpr size_t kWgradPartialCap = (size_t)160 << 20;
 size_t planned_wgrad_partial_bytes(const ConvGeom& g) {
   if (g.B == 0 || !planned_wgrad_supported(g)) return 0;
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  const WgradGrid w = wgrad_grid(g, pt.tiles_x * pt.tiles_y);
-  if (w.slots >= ((int64_t)1 << 31)) return 0;
-  const size_t bytes = (size_t)w.slots * w.KB * 16 * kPlThreads * sizeof(float);
+  // room for either launch shape
+  size_t bytes = 0;
+  for (int rest = 0; rest < 2; ++rest) {
+    const WgradGrid w = wgrad_grid(g, pt.tiles_x * pt.tiles_y, rest != 0);
+    if (w.slots >= ((int64_t)1 << 31)) return 0;
+    bytes = std::max(bytes, (size_t)w.slots * w.KB * 16 * kPlThreads * sizeof(float));
+  }
   return bytes <= kWgradPartialCap ? bytes : 0;
 }
 
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                   const float* img, float* gW, float* partial, hipStream_t stream,
                   const int* tile_list, const int* tile_count) {
-  const WgradGrid wg = wgrad_grid(g, plan.tiles);
+  // a listed launch in float32 covers the tiles the window kernel left: REST variant
+  const bool rest = tile_list != nullptr && mm == kMmF32;
+  const WgradGrid wg = wgrad_grid(g, plan.tiles, rest);
   const int KB = wg.KB, kb_count = wg.kb_count, NW = wg.NW;
   const int c_chunks = wg.c_chunks, n_tiles = wg.n_tiles, groups = wg.groups;
   const int64_t slots = wg.slots;
@@ -724,7 +803,7 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                     reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)slots);
 #define PW3(KBv, BFv, NWv)                                                                      \
-  launch(planned_wgrad_kernel<KBv, BFv, NWv>, grid, dim3(kPlThreads), stream, pix, img,         \
+  launch(planned_wgrad_kernel<KBv, BFv, NWv, false>, grid, dim3(kPlThreads), stream, pix, img,         \
          plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
          plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
 #define PW(KBv, BFv)                                                                            \
@@ -735,6 +814,18 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
     if (KB == 1) PW(1, kMmBf16); else if (KB == 4) PW(4, kMmBf16); else if (KB == 7) PW(7, kMmBf16); else PW(9, kMmBf16);
   } else if (mm == kMmSplit) {
     if (KB == 1) PW(1, kMmSplit); else if (KB == 4) PW(4, kMmSplit); else if (KB == 7) PW(7, kMmSplit); else PW(9, kMmSplit);
+  } else if (rest) {
+#define PR3(KBv, NWv)                                                                           \
+  launch(planned_wgrad_kernel<KBv, kMmF32, NWv, true>, grid, dim3(kPlThreads), stream, pix, img, \
+         plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
+         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
+#define PR(KBv)                                                                                 \
+  do {                                                                                          \
+    if (NW == 4) PR3(KBv, 4); else if (NW == 2) PR3(KBv, 2); else PR3(KBv, 1);                  \
+  } while (0)
+    if (KB == 1) PR(1); else if (KB == 4) PR(4); else PR(5);
+#undef PR
+#undef PR3
   } else {
     if (KB == 1) PW(1, kMmF32); else if (KB == 4) PW(4, kMmF32); else if (KB == 7) PW(7, kMmF32); else PW(9, kMmF32);
   }
