@@ -262,6 +262,13 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
 
+  // REST: byte offset of this lane's channel 8 cg + j inside the chunk's planes.  Channels past
+  // Cg repeat the last one: their columns of the product are dropped at the end.
+  unsigned ch_off[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    ch_off[j] = REST ? (unsigned)min(8 * cg + j, Cg - 1 - c0) * ((unsigned)HW * 4u) : 0u;
+
   // Tiles are dealt round-robin to the tile runs: costly tiles (taps outside the window,
   // e.g. polar rows of a spherical map) are spread over all workgroups.
   int buf = 0;
@@ -394,22 +401,21 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
         for (int j = 0; j < 8; ++j) pre[j] = 0.0f;
         // REST: image values of rows 0..3 of the sample about to be gathered
         float pre0[8], pre1[8], pre2[8], pre3[8];
-        const char* const rest_base = reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
-        const unsigned rest_plane = (unsigned)HW * 4u;
-        const unsigned rest_cg = (unsigned)(8 * cg) * rest_plane;
-        // requests the image values of row R of the sample whose rows start at BASE (NR rows)
+        const char* const rest_base =
+            reinterpret_cast<const char*>(img_b + (size_t)c0 * HW);
+        // requests the image values of row R of the sample whose rows start at BASE (NR rows);
+        // lanes whose tap lies in the window (or weighs nothing) read the image's first pixel
 #define SDK_REQ_ROW(R, BASE, NR)                                                              \
   if ((R) < (NR)) {                                                                           \
     const int2 ec = prow[((BASE) + (R)) * 64 + m_local];                                      \
     const bool out = ec.x < 0 && __int_as_float(ec.y) != 0.0f;                                \
-    const unsigned o0 = out ? rest_cg + (unsigned)(-ec.x - 1) * 4u : 0u;                      \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
-      const bool g_ok = out && c0 + 8 * cg + j < Cg;                                          \
-      pre##R[j] = *reinterpret_cast<const float*>(rest_base +                                 \
-                                                  (g_ok ? o0 + (unsigned)j * rest_plane : 0u)); \
-    }                                                                                         \
+    const unsigned o0 = out ? (unsigned)(-ec.x - 1) * 4u : 0u;                                \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)                                             \
+      pre##R[j] = *reinterpret_cast<const float*>(rest_base + (o0 + ch_off[j]));              \
   }
-        // adds row R (window value or requested image value, times the coefficient) to col[]
+        // adds row R (window value or requested image value, times the coefficient) to col[];
+        // a tap outside the window that weighs nothing takes the window's first element, as
+        // the padding rows of a plan do
 #define SDK_USE_ROW(R, BASE, NR)                                                              \
   if ((R) < (NR)) {                                                                           \
     const int2 ec = prow[((BASE) + (R)) * 64 + m_local];                                      \
@@ -420,10 +426,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
         reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);          \
     const float4 l0 = rp[0], l1 = rp[1];                                                      \
     const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};                     \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
-      const bool g_ok = out && c0 + 8 * cg + j < Cg;                                          \
-      col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? pre##R[j] : 0.0f), col[j]);        \
-    }                                                                                         \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)                                             \
+      col[j] = __builtin_fmaf(co, out ? pre##R[j] : dl[j], col[j]);                           \
   }
         if constexpr (REST) {
           const int nr = min(__builtin_amdgcn_readfirstlane(ns_l[kk_beg]), 4);
@@ -448,13 +452,11 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
                   reinterpret_cast<const float4*>(region + (e >= 0 ? e : 0) * kRegE + 8 * cg);
               const float4 l0 = rp[0], l1 = rp[1];
               const float dl[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
-              const unsigned o0 = out ? rest_cg + (unsigned)(-e - 1) * 4u : 0u;
+              const unsigned o0 = out ? (unsigned)(-e - 1) * 4u : 0u;
 #pragma unroll
               for (int j = 0; j < 8; ++j) {
-                const bool g_ok = out && c0 + 8 * cg + j < Cg;
-                const float dg = *reinterpret_cast<const float*>(
-                    rest_base + (g_ok ? o0 + (unsigned)j * rest_plane : 0u));
-                col[j] = __builtin_fmaf(co, e >= 0 ? dl[j] : (g_ok ? dg : 0.0f), col[j]);
+                const float dg = *reinterpret_cast<const float*>(rest_base + (o0 + ch_off[j]));
+                col[j] = __builtin_fmaf(co, out ? dg : dl[j], col[j]);
               }
             }
             row0 += nrows;
@@ -788,9 +790,12 @@ size_t planned_wgrad_partial_bytes(const ConvGeom& g) {
 int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                   const float* img, float* gW, float* partial, hipStream_t stream,
                   const int* tile_list, const int* tile_count) {
-  // a listed launch in float32 covers the tiles the window kernel left: REST variant
-  const bool rest = tile_list != nullptr && mm == kMmF32;
-  const WgradGrid wg = wgrad_grid(g, plan.tiles, rest);
+  // A listed launch in float32 covers the tiles the window kernel left.  Where the plain
+  // variant has no registers to request values ahead (nine samples, 128 rows), the REST
+  // variant takes its place.
+  const WgradGrid plain = wgrad_grid(g, plan.tiles, false);
+  const bool rest = tile_list != nullptr && mm == kMmF32 && plain.KB == 9 && plain.NW == 4;
+  const WgradGrid wg = rest ? wgrad_grid(g, plan.tiles, true) : plain;
   const int KB = wg.KB, kb_count = wg.kb_count, NW = wg.NW;
   const int c_chunks = wg.c_chunks, n_tiles = wg.n_tiles, groups = wg.groups;
   const int64_t slots = wg.slots;
@@ -819,12 +824,7 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
   launch(planned_wgrad_kernel<KBv, kMmF32, NWv, true>, grid, dim3(kPlThreads), stream, pix, img, \
          plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
          plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
-#define PR(KBv)                                                                                 \
-  do {                                                                                          \
-    if (NW == 4) PR3(KBv, 4); else if (NW == 2) PR3(KBv, 2); else PR3(KBv, 1);                  \
-  } while (0)
-    if (KB == 1) PR(1); else if (KB == 4) PR(4); else PR(5);
-#undef PR
+    if (KB == 4) PR3(4, 4); else PR3(5, 4);   // K = 10 .. 16 -> two or more blocks of 4 or 5
 #undef PR3
   } else {
     if (KB == 1) PW(1, kMmF32); else if (KB == 4) PW(4, kMmF32); else if (KB == 7) PW(7, kMmF32); else PW(9, kMmF32);
