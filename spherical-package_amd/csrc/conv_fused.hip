@@ -672,7 +672,7 @@ static GatherLayout gather_layout(const ConvGeom& g) {
   l.total = l.window_weights + up(window_gemm_weight_bytes(g));
   return l;
 }
-static bool gather_from_window(const ConvGeom& g) { return window_gemm_supported(g) && g.Cp > 64; }
+static bool gather_from_window(const ConvGeom& g) { return window_gemm_supported(g) && g.Cp > 32; }
 
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
@@ -746,7 +746,8 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                       float* workspace, hipStream_t stream, const CachedPlan* cached) {
   const int mm = matrix_mode(compute);
   const int slots = slots_for(g);
-  const bool narrow = g.Cp <= 64;
+  // (the listed-tile kernel behind the window kernel has 128 x 128 tiles only)
+  const bool narrow = g.Cp <= 64 && !gather_from_window(g);
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
   const int CpP = round_up(g.Cp, TN), CgP = round_up(g.Cg, kKC);
   int rc = relayout(g, Wm, workspace, CpP, CgP, 2, stream);
@@ -916,7 +917,7 @@ static ConvGeom inverse_geom(const ConvGeom& g) {
   return r;
 }
 static bool scatter_from_window(const ConvGeom& g) {
-  return g.Cg > 64 && g.M % g.OW == 0 && window_gemm_supported(inverse_geom(g)) &&
+  return g.Cg > 32 && g.M % g.OW == 0 && window_gemm_supported(inverse_geom(g)) &&
          (int64_t)g.H * g.W * g.K < ((int64_t)1 << 31);
 }
 // Scratch of the scatter run from the inverse plan (behind the forward plan's region).

@@ -31,6 +31,7 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
   __shared__ __align__(8) float stage[kPlanStage / sizeof(float)];
+  __shared__ WindowSet wset;
   const int tid = threadIdx.x, lane = tid & 63;
   const int tile = blockIdx.x;
   const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
@@ -127,19 +128,55 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     atomicMax(&bb[3], dx1);
   }
   __syncthreads();
-  const Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, pt.TY(), pt.TX(), W);
+  Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, pt.TY(), pt.TX(), W);
+  // the window is the whole bounding box of the taps unless that exceeded the capacity
+  bool whole = bb[0] > bb[1] || (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, W) <= kRegionCap;
+  int listed = -1;   // >= 0: elements of a listed window
+  if (!whole) {
+    // the distinct elements the tile touches may still fit: try a listed window
+    set_clear(wset);
+    __syncthreads();
+    if (pix_ok) {
+      for (int k = kpar; k < K; k += 2) {
+        for (int pp = 0; pp < q; ++pp) {
+          float sx, sy, sw;
+          point(k, pp, sx, sy, sw);
+          t.set(sx, sy, H, W, sw);
+#pragma unroll
+          for (int i = 0; i < NT; ++i)
+            if (t.w[i] != 0.0f) set_insert(wset, t.y[i] * W + t.x[i]);
+        }
+      }
+    }
+    __syncthreads();
+    listed = set_finish(wset);
+    if (listed >= 0) {
+      rg.ry0 = 0;
+      rg.rx0 = 0;
+      rg.RH = 1;
+      rg.RW = listed;
+      rg.RS = listed;
+      rg.RSp = listed | 1;
+      whole = true;
+    }
+  }
+  int* tile_hdr = hdr + (size_t)tile * kHdrStride;
   if (tid == 0) {
-    hdr[tile * 8 + 0] = rg.ry0;
-    hdr[tile * 8 + 1] = rg.rx0;
-    hdr[tile * 8 + 2] = rg.RH;
-    hdr[tile * 8 + 3] = rg.RW;
-    // the window is the whole bounding box of the taps unless that exceeded the capacity
-    const bool whole = bb[0] > bb[1] ||
-                       (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, W) <= kRegionCap;
-    hdr[tile * 8 + 4] = whole ? 1 : 0;
+    tile_hdr[0] = rg.ry0;
+    tile_hdr[1] = rg.rx0;
+    tile_hdr[2] = rg.RH;
+    tile_hdr[3] = rg.RW;
+    tile_hdr[4] = whole ? 1 : 0;
     int most = 0;
     for (int k = 0; k < K; ++k) most = max(most, ns_l[k]);
-    hdr[tile * 8 + 5] = most;   // the longest row list of the tile's samples
+    tile_hdr[5] = most;   // the longest row list of the tile's samples
+    tile_hdr[6] = listed >= 0 ? 1 : 0;
+    tile_hdr[7] = 0;
+  }
+  if (listed >= 0) {
+    for (int e = tid; e < listed; e += kPlThreads) tile_hdr[kHdrLut + e] = wset.list[e];
+  } else {
+    write_region_lut(rg, H, W, tile_hdr + kHdrLut);
   }
   for (int k = tid; k < K; k += kPlThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
 
@@ -155,7 +192,9 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
           if (t.w[i] != 0.0f) {
-            row[(size_t)cnt * 128] = make_int2(rg.encode(t.y[i], t.x[i], W), __float_as_int(t.w[i]));
+            const int at = listed >= 0 ? set_rank(wset, listed, t.y[i] * W + t.x[i])
+                                       : rg.encode(t.y[i], t.x[i], W);
+            row[(size_t)cnt * 128] = make_int2(at, __float_as_int(t.w[i]));
             ++cnt;
           }
         }
@@ -283,10 +322,10 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
       return (oy < pt.OH && ox < pt.OW) ? oy * pt.OW + ox : -1;
     };
     Region rg;
-    rg.ry0 = hdr[tile * 8 + 0];
-    rg.rx0 = hdr[tile * 8 + 1];
-    rg.RH = hdr[tile * 8 + 2];
-    rg.RW = hdr[tile * 8 + 3];
+    rg.ry0 = hdr[tile * kHdrStride + 0];
+    rg.rx0 = hdr[tile * kHdrStride + 1];
+    rg.RH = hdr[tile * kHdrStride + 2];
+    rg.RW = hdr[tile * kHdrStride + 3];
     rg.RS = rg.RH * rg.RW;
     rg.RSp = rg.RS;
     // plan rows of this tile and sample block: uniform base, 32-bit lane offsets
@@ -294,7 +333,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 
     __syncthreads();  // every wave is done with the previous tile's window, rows and column tiles
     if (tid < kcount) ns_l[tid] = ns[(size_t)tile * K + k0 + tid];
-    build_region_lut(rg, H, W, src);
+    load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
     __syncthreads();
     {
       // wave w stages channels 8w .. 8w+7; a lane owns window elements lane, lane+64, ...
@@ -700,7 +739,7 @@ bool plan_supported(const ConvGeom& g) {
   if (g.OW < 1 || g.M % g.OW != 0 || g.K > kPlanKMax) return false;
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const int64_t tiles = (int64_t)pt.tiles_x * pt.tiles_y;
-  return tiles * g.K * plan_slots(g) * 128 < ((int64_t)1 << 40) && tiles * 8 < ((int64_t)1 << 31);
+  return tiles * g.K * plan_slots(g) * 128 < ((int64_t)1 << 40) && tiles * kHdrStride < ((int64_t)1 << 31);
 }
 
 static size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
@@ -708,7 +747,7 @@ static size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 size_t plan_bytes(const ConvGeom& g) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
-  return align16(tiles * 8 * sizeof(int)) + align16(tiles * g.K * sizeof(int)) +
+  return align16(tiles * kHdrStride * sizeof(int)) + align16(tiles * g.K * sizeof(int)) +
          tiles * g.K * plan_slots(g) * 128 * sizeof(int2);
 }
 
@@ -720,8 +759,8 @@ void load_plan(const ConvGeom& g, void* workspace, Plan* plan) {
   plan->tiles = (int)tiles;
   plan->S = plan_slots(g);
   plan->hdr = reinterpret_cast<int*>(base);
-  plan->ns = reinterpret_cast<int*>(base + align16(tiles * 8 * sizeof(int)));
-  plan->taps = reinterpret_cast<int2*>(base + align16(tiles * 8 * sizeof(int)) +
+  plan->ns = reinterpret_cast<int*>(base + align16(tiles * kHdrStride * sizeof(int)));
+  plan->taps = reinterpret_cast<int2*>(base + align16(tiles * kHdrStride * sizeof(int)) +
                                        align16(tiles * g.K * sizeof(int)));
 }
 

@@ -2,15 +2,22 @@
 // per-tile lists of (window index, coefficient) pairs that every batch element
 // and channel chunk reuses.
 //
-// The pixel grid is cut into 2-D tiles of 128 pixels (PixelTiling).  For tile t:
-//   hdr[8*t + 0..3]  window of the image the tile's taps fall into: first row,
-//                    first column, rows, columns (columns wrap modulo W)
-//   hdr[8*t + 4]     1 when every active tap of the tile lies inside that window
-//   hdr[8*t + 5]     the largest ns of the tile's samples (plan_kernel only)
+// The pixel grid is cut into 2-D tiles of 128 pixels (PixelTiling).  For tile t, with
+// h = hdr + kHdrStride * t (conv_window.hpp):
+//   h[0..3]          window of the image the tile's taps fall into: first row,
+//                    first column, rows, columns (columns wrap modulo W).  When the
+//                    bounding box of the taps is too large for a window but the taps touch
+//                    at most kRegionCap distinct elements, the window is the sorted list of
+//                    those elements instead (a "listed" window: 0, 0, 1, count)
+//   h[4]             1 when every active tap of the tile lies inside that window
+//   h[5]             the largest ns of the tile's samples (plan_kernel only)
+//   h[6]             1 for a listed window
+//   h[8 + e]         flat image offset of window element e (-1: outside the image)
 //   ns[t*K + k]      rows of kernel sample k: the largest number of active taps
 //                    any pixel of the tile has for that sample
 //   taps[((t*K + k)*S + r)*128 + p]   row r < ns of pixel p (tile-local index):
-//                    .x >= 0: element index inside the window (row * columns + column)
+//                    .x >= 0: element index inside the window (row * columns + column,
+//                             or the rank in the list)
 //                    .x <  0: -(flat offset inside the image plane) - 1 (outside the window)
 //                    .y: float bits of the coefficient (interpolation weight times
 //                    point weight); pixels with fewer taps are padded with 0.

@@ -107,13 +107,13 @@ __global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
   const float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
 
   Region rg;
-  rg.ry0 = hdr[tile * 8 + 0];
-  rg.rx0 = hdr[tile * 8 + 1];
-  rg.RH = hdr[tile * 8 + 2];
-  rg.RW = hdr[tile * 8 + 3];
+  rg.ry0 = hdr[tile * kHdrStride + 0];
+  rg.rx0 = hdr[tile * kHdrStride + 1];
+  rg.RH = hdr[tile * kHdrStride + 2];
+  rg.RW = hdr[tile * kHdrStride + 3];
   rg.RS = rg.RH * rg.RW;
   rg.RSp = rg.RS | 1;
-  build_region_lut(rg, H, W, src);
+  load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
   for (int k = tid; k < K; k += kStThreads) ns_l[k] = ns[(size_t)tile * K + k];
   // plan rows of this tile: uniform base, 32-bit lane offsets
   const char* tile_taps = reinterpret_cast<const char*>(taps + (size_t)tile * K * S * 128);

@@ -20,6 +20,12 @@ namespace sdk {
 
 constexpr int kCC = 32;          // channels staged per region chunk
 constexpr int kRegionCap = 288;  // region elements per channel (kCC * 289 * 4 B = 36 KB)
+// A plan's header: kHdrStride ints per tile.  [0..3] window origin and size (row, column,
+// rows, columns; a listed window reads 0, 0, 1, count), [4] 1 when every tap of the tile lies
+// inside the window, [5] most rows of a sample, [6] 1 for a listed window, [8 + e] the flat
+// image offset of window element e (-1: outside the image).
+constexpr int kHdrLut = 8;
+constexpr int kHdrStride = kHdrLut + kRegionCap;
 
 // Up to four taps of one sample point as (row, column, coefficient).  A tap that
 // is out of range or has zero weight gets coefficient 0 (and row = column = 0).
@@ -140,17 +146,104 @@ __device__ __forceinline__ Region choose_region(int dy0, int dy1, int dx0, int d
   return r;
 }
 
-// src[e], e < RS: flat offset inside one image plane of region element e, or -1
-// for a row outside the image.
-__device__ __forceinline__ void build_region_lut(const Region& r, int H, int W,
-                                                 int* __restrict__ src) {
+// lut[e], e < RS: flat offset inside one image plane of element e of a box window, or -1
+// for a row outside the image.  Written into the plan's header by the kernels that build plans.
+__device__ __forceinline__ void write_region_lut(const Region& r, int H, int W,
+                                                 int* __restrict__ lut) {
   for (int e = threadIdx.x; e < r.RS; e += blockDim.x) {
     const int ry = e / r.RW, rx = e - ry * r.RW;
     const int y = r.ry0 + ry;
     int x = r.rx0 + rx;
     x -= x >= W ? W : 0;
-    src[e] = ((unsigned)y < (unsigned)H) ? y * W + x : -1;
+    lut[e] = ((unsigned)y < (unsigned)H) ? y * W + x : -1;
   }
+}
+
+// src[e] = the tile's window LUT (tile_hdr = hdr + tile * kHdrStride), e < RS.
+__device__ __forceinline__ void load_region_lut(const int* __restrict__ tile_hdr, int RS,
+                                                int* __restrict__ src) {
+  for (int e = threadIdx.x; e < RS; e += blockDim.x) src[e] = tile_hdr[kHdrLut + e];
+}
+
+// ---------------------------------------------------------------------------
+// Listed windows.  A tile whose taps have a bounding box beyond kRegionCap (neighbour lists
+// of a mesh, whose indices say little about distance) may still touch few distinct image
+// elements.  The kernels that build plans collect the tile's distinct offsets in an LDS hash
+// set; when there are at most kRegionCap, the sorted list becomes the window and a tap's
+// window index is its rank in it.
+// ---------------------------------------------------------------------------
+constexpr int kSetSlots = 1024;  // hash slots (> kRegionCap + the threads that may insert at once)
+constexpr int kSetSort = 512;    // length of the padded sorted list (power of two >= kRegionCap)
+
+struct WindowSet {
+  int table[kSetSlots];
+  int list[kSetSort];
+  int count;   // distinct offsets claimed; inserting stops once it exceeds kRegionCap
+  int filled;
+};
+
+// All threads; a barrier must follow.
+__device__ __forceinline__ void set_clear(WindowSet& ws) {
+  for (int i = threadIdx.x; i < kSetSlots; i += blockDim.x) ws.table[i] = -1;
+  for (int i = threadIdx.x; i < kSetSort; i += blockDim.x) ws.list[i] = INT_MAX;
+  if (threadIdx.x == 0) {
+    ws.count = 0;
+    ws.filled = 0;
+  }
+}
+
+__device__ __forceinline__ void set_insert(WindowSet& ws, int off) {
+  if (*reinterpret_cast<volatile int*>(&ws.count) > kRegionCap) return;
+  unsigned h = ((unsigned)off * 2654435761u) >> 22;
+  for (int probe = 0; probe < kSetSlots; ++probe) {
+    const int prev = atomicCAS(&ws.table[h], -1, off);
+    if (prev == -1) {
+      atomicAdd(&ws.count, 1);
+      return;
+    }
+    if (prev == off) return;
+    h = (h + 1) & (kSetSlots - 1);
+  }
+}
+
+// All threads, after a barrier behind the last set_insert.  Returns the number of distinct
+// offsets when they fit a window (ws.list[0 .. n) is then sorted), otherwise -1.
+__device__ __forceinline__ int set_finish(WindowSet& ws) {
+  const int n = ws.count;
+  if (n > kRegionCap) return -1;
+  for (int i = threadIdx.x; i < kSetSlots; i += blockDim.x) {
+    const int key = ws.table[i];
+    if (key != -1) ws.list[atomicAdd(&ws.filled, 1)] = key;
+  }
+  __syncthreads();
+  for (int k = 2; k <= kSetSort; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = threadIdx.x; i < kSetSort; i += blockDim.x) {
+        const int o = i ^ j;
+        if (o > i) {
+          const int a = ws.list[i], b = ws.list[o];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) {
+            ws.list[i] = b;
+            ws.list[o] = a;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  return n;
+}
+
+// Rank of `off` in the sorted list of n offsets (it is one of them).
+__device__ __forceinline__ int set_rank(const WindowSet& ws, int n, int off) {
+  int lo = 0, hi = n - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (ws.list[mid] < off) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo;
 }
 
 }  // namespace sdk

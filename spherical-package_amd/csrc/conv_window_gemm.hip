@@ -131,6 +131,7 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
   if (*gate != 0) return;
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
+  __shared__ WindowSet wset;
   const int tid = threadIdx.x, lane = tid & 63;
   const int tile = blockIdx.x;
   const int ty0 = (tile / it.tiles_x) * it.TY(), tx0 = (tile % it.tiles_x) << it.tx_shift;
@@ -205,15 +206,47 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
     atomicMax(&bb[3], dx1);
   }
   __syncthreads();   // (also orders the sorted lists written above before they are re-read)
-  const Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, it.TY(), it.TX(), OW);
+  Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, it.TY(), it.TX(), OW);
+  bool whole = bb[0] > bb[1] || (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, OW) <= kRegionCap;
+  int listed = -1;   // >= 0: elements of a listed window
+  if (!whole) {
+    // the distinct sources of the tile may still fit: try a listed window
+    set_clear(wset);
+    __syncthreads();
+    for (int k = kpar; k < K; k += 2) {
+      const int n = pix_ok ? min(cnt[(size_t)u * K + k], kInvRows) : 0;
+      const int* ro = raw_off + ((size_t)tile * K + k) * kInvRows * 128 + p;
+      for (int a = 0; a < n; ++a) set_insert(wset, ro[a * 128]);
+    }
+    __syncthreads();
+    listed = set_finish(wset);
+    if (listed >= 0) {
+      rg.ry0 = 0;
+      rg.rx0 = 0;
+      rg.RH = 1;
+      rg.RW = listed;
+      rg.RS = listed;
+      rg.RSp = listed | 1;
+      whole = true;
+    }
+  }
+  int* tile_hdr = hdr + (size_t)tile * kHdrStride;
   if (tid == 0) {
-    hdr[tile * 8 + 0] = rg.ry0;
-    hdr[tile * 8 + 1] = rg.rx0;
-    hdr[tile * 8 + 2] = rg.RH;
-    hdr[tile * 8 + 3] = rg.RW;
-    const bool whole = bb[0] > bb[1] ||
-                       (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, OW) <= kRegionCap;
-    hdr[tile * 8 + 4] = whole ? 1 : 0;
+    tile_hdr[0] = rg.ry0;
+    tile_hdr[1] = rg.rx0;
+    tile_hdr[2] = rg.RH;
+    tile_hdr[3] = rg.RW;
+    tile_hdr[4] = whole ? 1 : 0;
+    int most = 0;
+    for (int k = 0; k < K; ++k) most = max(most, ns_l[k]);
+    tile_hdr[5] = most;
+    tile_hdr[6] = listed >= 0 ? 1 : 0;
+    tile_hdr[7] = 0;
+  }
+  if (listed >= 0) {
+    for (int e = tid; e < listed; e += kWgThreads) tile_hdr[kHdrLut + e] = wset.list[e];
+  } else {
+    write_region_lut(rg, OH, OW, tile_hdr + kHdrLut);
   }
   for (int k = tid; k < K; k += kWgThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
   for (int k = kpar; k < K; k += 2) {
@@ -227,14 +260,15 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
       if (a < n) {
         const int mm = ro[a * 128];
         const int my = mm / OW, mx = mm - my * OW;
-        v = make_int2(rg.encode(my, mx, OW), __float_as_int(rc[a * 128]));
+        const int at = listed >= 0 ? set_rank(wset, listed, mm) : rg.encode(my, mx, OW);
+        v = make_int2(at, __float_as_int(rc[a * 128]));
       }
       row[(size_t)a * 128] = v;
     }
   }
 }
 
-// Splits the plan's tiles into those whose taps all lie inside their window (hdr[8t+4] != 0)
+// Splits the plan's tiles into those whose taps all lie inside their window (header value 4 != 0)
 // and the rest, both in ascending tile order.  One workgroup.
 //   lists[0 .. tiles)         tiles inside their window, count[0] of them
 //   lists[tiles .. 2*tiles)   the others, count[1] of them
@@ -249,7 +283,7 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
   for (int t0 = 0; t0 < tiles; t0 += 1024) {
     const int t = t0 + tid;
     const bool live = t < tiles;
-    const bool fit = live && hdr[t * 8 + 4] != 0 && (max_rows <= 0 || hdr[t * 8 + 5] <= max_rows);
+    const bool fit = live && hdr[t * kHdrStride + 4] != 0 && (max_rows <= 0 || hdr[t * kHdrStride + 5] <= max_rows);
     const unsigned long long mf = __ballot(fit), mr = __ballot(live && !fit);
     if (lane == 0) {
       wave_fit[wave] = __popcll(mf);
@@ -316,14 +350,14 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
   const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
 
   Region rg;
-  rg.ry0 = hdr[tile * 8 + 0];
-  rg.rx0 = hdr[tile * 8 + 1];
-  rg.RH = hdr[tile * 8 + 2];
-  rg.RW = hdr[tile * 8 + 3];
+  rg.ry0 = hdr[tile * kHdrStride + 0];
+  rg.rx0 = hdr[tile * kHdrStride + 1];
+  rg.RH = hdr[tile * kHdrStride + 2];
+  rg.RW = hdr[tile * kHdrStride + 3];
   rg.RS = rg.RH * rg.RW;
   rg.RSp = rg.RS;
   const int RS = rg.RS;
-  build_region_lut(rg, H, W, src);
+  load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
   if (tid < kWE) region[RS * kWE + tid] = 0.0f;   // the zero element padded rows point at
   for (int k = tid; k < K; k += kWgThreads) ns_l[k] = ns[(size_t)tile * K + k];
 
@@ -613,7 +647,7 @@ InverseOffsets inverse_offsets(const ConvGeom& g) {
   o.raw_co = o.cnt + up((size_t)g.H * g.W * g.K * sizeof(int));   // gate, cnt, raw_co: cleared together
   o.raw_off = o.raw_co + up(rows * sizeof(float));
   o.hdr = o.raw_off + up(rows * sizeof(int));
-  o.ns = o.hdr + up(tiles * 8 * sizeof(int));
+  o.ns = o.hdr + up(tiles * kHdrStride * sizeof(int));
   o.taps = o.ns + up(tiles * g.K * sizeof(int));
   o.total = o.taps + up(rows * sizeof(int2));
   return o;

@@ -98,17 +98,17 @@ __global__ __launch_bounds__(kWwThreads, 2) void window_wgrad_kernel(
     const int tile = list[ti];
     const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
     Region rg;
-    rg.ry0 = hdr[tile * 8 + 0];
-    rg.rx0 = hdr[tile * 8 + 1];
-    rg.RH = hdr[tile * 8 + 2];
-    rg.RW = hdr[tile * 8 + 3];
+    rg.ry0 = hdr[tile * kHdrStride + 0];
+    rg.rx0 = hdr[tile * kHdrStride + 1];
+    rg.RH = hdr[tile * kHdrStride + 2];
+    rg.RW = hdr[tile * kHdrStride + 3];
     rg.RS = rg.RH * rg.RW;
     rg.RSp = rg.RS;
     const int RS = rg.RS;
     const int2* tile_taps = taps + (size_t)tile * K * S * 128;
 
     __syncthreads();   // every wave is done with the previous tile
-    build_region_lut(rg, H, W, src);
+    load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
     if (tid < K) ns_l[tid] = min(ns[(size_t)tile * K + tid], min(S, kWwRows));
     if (tid < kWwE) region[RS * kWwE + tid] = 0.0f;   // the zero element inactive rows point at
     __syncthreads();

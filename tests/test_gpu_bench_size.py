@@ -127,9 +127,9 @@ def test_conv4_batch8_identities_with_a_structured_cotangent(ops, conv4):
 
 
 # --------------------------------------------------------------------------- configuration 5
-@pytest.fixture(scope="module")
-def conv5(oracle):
-    cfg = workloads.config5(batch=4)
+@pytest.fixture(scope="module", params=["hierarchical", "append"])
+def conv5(oracle, request):
+    cfg = workloads.config5(batch=4, order=request.param)
     # one-row vertex image: no polar rows; the 12 five-neighbour vertices, the vertices of
     # the coarsest levels and the last ones appended, plus random ones
     cols = tuple(range(0, 64)) + tuple(range(-64, 0))

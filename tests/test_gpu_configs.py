@@ -98,10 +98,11 @@ def test_configuration4_reduced(ops, oracle):
     _conv_both_ways(ops, oracle, workloads.config4(batch=2, cin=40, cout=24, H=32, W=64))
 
 
-def test_configuration5_reduced(ops, oracle):
+@pytest.mark.parametrize("order", ["hierarchical", "append"])
+def test_configuration5_reduced(ops, oracle, order):
     """Level-3 icosphere (642 vertices): vertex convolution and transposed up-sampling from
-    level 2, nearest."""
-    c = workloads.config5(batch=2, channels=16, level=3)
+    level 2, nearest; with the vertices numbered for locality and in subdivision order."""
+    c = workloads.config5(batch=2, channels=16, level=3, order=order)
     _conv_both_ways(ops, oracle, c)
     K, it = c["kernel_size"], c["interp"]
     xc, um, uw, ub = c["x_coarse"], c["up_map"], c["up_weight"], c["up_bias"]

@@ -128,6 +128,20 @@ def test_workload_generators_shapes():
     nb = ring[0, :, 1:, 0].astype(int)
     assert all(v_ in nb[n] for v_ in range(40) for n in nb[v_])  # neighbourhood is symmetric
     assert wl.tangent_patch_map(64, 128, 1, 8).shape == (80, 64, 2)
+    # the locality numbering is the same mesh: same vertex set, same neighbourhoods, and the
+    # parent -> child map names the coarse vertices' own positions
+    vh, fh = wl.icosphere(3, "hierarchical")
+    assert np.allclose(np.sort(v, 0), np.sort(vh, 0)) and fh.shape == f.shape
+    ring_h = wl.vertex_ring_map(3, order="hierarchical")[0, :, :, 0].astype(int)
+    key = lambda pts: set(map(tuple, np.round(pts, 6)))
+    for n in (0, 100, 641):
+        old = int(np.argmin(np.abs(v - vh[n]).sum(1)))
+        assert key(vh[ring_h[n]]) == key(v[ring[0, old, :, 0].astype(int)])
+    c2f = wl.coarse_to_fine(3, "hierarchical")
+    assert np.allclose(vh[c2f], wl.icosphere(2, "hierarchical")[0])
+    assert np.array_equal(wl.coarse_to_fine(3), np.arange(162))
+    spread = np.abs(ring_h[:, 1:] - ring_h[:, :1])
+    assert np.median(spread) < 16   # neighbours are close in index
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_device():

@@ -87,9 +87,11 @@ def _icosahedron():
     return v, f
 
 
-def icosphere(level):
+def _icosphere_append(level):
     """Midpoint-subdivided, re-normalised icosahedron: (vertices [V,3], faces [F,3]).
-    Vertices of level L keep their indices in level L+1; V = 10*4^L + 2."""
+    Midpoints are appended level by level, so vertices of level L keep their indices in
+    level L+1 (V = 10*4^L + 2).  The four children of a face lie next to each other in the
+    face list (corner 0, corner 1, corner 2, centre), so the list is in quadtree order."""
     v, f = _icosahedron()
     for _ in range(level):
         e = np.concatenate([f[:, [0, 1]], f[:, [1, 2]], f[:, [2, 0]]], 0)
@@ -102,15 +104,58 @@ def icosphere(level):
         v = np.concatenate([v, mid], 0)
         nf = len(f)
         a, b, c = base + inv[:nf], base + inv[nf:2 * nf], base + inv[2 * nf:]
-        f = np.concatenate([np.stack([f[:, 0], a, c], 1), np.stack([f[:, 1], b, a], 1),
-                            np.stack([f[:, 2], c, b], 1), np.stack([a, b, c], 1)], 0)
+        f = np.stack([np.stack([f[:, 0], a, c], 1), np.stack([f[:, 1], b, a], 1),
+                      np.stack([f[:, 2], c, b], 1), np.stack([a, b, c], 1)], 1).reshape(-1, 3)
     return v, f
 
 
-def vertex_ring_map(level, num_vertices=None, dtype=np.float32):
+def _hierarchical_order(f, V):
+    """Permutation old_of_new [V]: vertices in the order in which the quadtree-ordered face list
+    first names them, so that vertices close on the sphere are close in index."""
+    flat = f.reshape(-1)
+    vals, first = np.unique(flat, return_index=True)
+    assert len(vals) == V
+    return vals[np.argsort(first, kind="stable")]
+
+
+def icosphere(level, order="append"):
+    """(vertices [V,3], faces [F,3]) of the level-`level` icosphere.
+
+    order="append": the numbering of midpoint subdivision (level-L vertices keep their indices
+    at level L+1; neighbours are up to V apart in index: no locality).
+    order="hierarchical": the same mesh renumbered along its quadtree face order
+    (_hierarchical_order): a run of consecutive indices is a compact patch of the sphere."""
+    v, f = _icosphere_append(level)
+    if order == "append":
+        return v, f
+    if order != "hierarchical":
+        raise ValueError("order must be 'append' or 'hierarchical'")
+    old_of_new = _hierarchical_order(f, len(v))
+    new_of_old = np.empty_like(old_of_new)
+    new_of_old[old_of_new] = np.arange(len(v))
+    return v[old_of_new], new_of_old[f]
+
+
+def coarse_to_fine(level, order="append"):
+    """[Vc] index, at level `level`, of every vertex of level `level` - 1 (in that level's own
+    numbering of the same order): the parent -> child map of an up-sampling layer."""
+    Vc = 10 * 4 ** (level - 1) + 2
+    if order == "append":
+        return np.arange(Vc)
+    vf, ff = _icosphere_append(level)
+    vc, fc = _icosphere_append(level - 1)
+    fine_old_of_new = _hierarchical_order(ff, len(vf))
+    fine_new_of_old = np.empty_like(fine_old_of_new)
+    fine_new_of_old[fine_old_of_new] = np.arange(len(vf))
+    coarse_old_of_new = _hierarchical_order(fc, len(vc))
+    # append numbering: coarse vertex i is fine vertex i
+    return fine_new_of_old[coarse_old_of_new]
+
+
+def vertex_ring_map(level, num_vertices=None, dtype=np.float32, order="append"):
     """[1, V, 7, 2]: every vertex followed by its 1-ring neighbours as (index, 0)
     samples; the 12 five-neighbour vertices repeat their last neighbour."""
-    v, f = icosphere(level)
+    v, f = icosphere(level, order)
     V = len(v)
     e = np.concatenate([f[:, [0, 1]], f[:, [1, 2]], f[:, [2, 0]], f[:, [1, 0]], f[:, [2, 1]],
                         f[:, [0, 2]]], 0)
@@ -242,17 +287,23 @@ def config4(batch=8, cin=128, cout=128, H=256, W=512, dtype=np.float32):
                 kernel_size=9, interp=2)
 
 
-def config5(batch=4, channels=64, level=7, dtype=np.float32):
-    """Icosphere vertex convolution (level L) and transposed up-sampling (L-1 -> L)."""
+def config5(batch=4, channels=64, level=7, dtype=np.float32, order="hierarchical"):
+    """Icosphere vertex convolution (level L) and transposed up-sampling (L-1 -> L).
+
+    order: numbering of the vertices (icosphere()).  The layers only see index lists, so the
+    numbering is the data layout of the workload; "hierarchical" keeps neighbours close in
+    memory, "append" (what plain midpoint subdivision yields) is the incoherent case.  The
+    up-sampling map lists, for every coarse vertex, its own fine index and its fine 1-ring."""
     rng = _rng(5)
     V = 10 * 4 ** level + 2
     Vc = 10 * 4 ** (level - 1) + 2
-    ring = vertex_ring_map(level, dtype=dtype)
+    ring = vertex_ring_map(level, dtype=dtype, order=order)
     w, b = _conv_weights(rng, channels, channels, 7, dtype)
     wt, bt = _conv_weights(rng, channels, channels, 7, dtype)
+    up_map = np.ascontiguousarray(ring[:, coarse_to_fine(level, order)])
     return dict(x=rng.standard_normal((batch, channels, 1, V)).astype(dtype), sample_map=ring,
                 weight=w, bias=b,
                 grad_output=rng.standard_normal((batch, channels, 1, V)).astype(dtype),
                 x_coarse=rng.standard_normal((batch, channels, 1, Vc)).astype(dtype),
-                up_map=np.ascontiguousarray(ring[:, :Vc]), up_weight=wt.transpose(1, 0, 2).copy(),
+                up_map=up_map, up_weight=wt.transpose(1, 0, 2).copy(),
                 up_bias=bt, out_hw=(1, V), kernel_size=7, interp=0)
