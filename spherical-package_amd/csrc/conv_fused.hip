@@ -301,7 +301,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     const int* __restrict__ inv_ns = nullptr, const int* __restrict__ gate = nullptr,
     PixelTiling pt = PixelTiling(), const int* __restrict__ tile_list = nullptr,
     const int* __restrict__ tile_count = nullptr) {
-  static_assert(!TILED || TM == 128, "tiled pixel order: 128-pixel tiles");
+  static_assert(!TILED || TM % 128 == 0, "tiled pixel order: 128-pixel tiles");
+  constexpr int TPW = TILED ? TM / 128 : 1;   // listed tiles per workgroup
   if constexpr (INV) {
     if (*gate != 0) return;
   }
@@ -319,25 +320,31 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   const int n_tiles = CpP / TN;
   int tile = TILED ? 0 : xcd_band_tile(blockIdx.x, m_tiles * n_tiles);
   // pixel (index into the pixel grid, -1: none) of tile-local pixel p
-  int ty0 = 0, tx0 = 0, ptile = 0;   // ptile: the pixel tile whose inverse rows are read
+  int lt[TPW];       // TILED: the listed pixel tiles of this workgroup (-1: none)
+  int ptile = 0;     // otherwise: the run of TM pixels whose inverse rows are read
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) lt[i] = -1;
   if constexpr (TILED) {
     // XCD x (workgroup ids go round-robin over the 8 XCDs) takes an eighth of the list,
-    // however long the list is
-    const int cnt = *tile_count, per = (cnt + 7) >> 3;
+    // however long the list is; a workgroup takes TPW consecutive entries
+    const int cnt = *tile_count, units = (cnt + TPW - 1) / TPW, per = (units + 7) >> 3;
     const int wg = blockIdx.x / n_tiles, slot = (wg & 7) * per + (wg >> 3);
-    if ((wg >> 3) >= per || slot >= cnt) return;
+    if ((wg >> 3) >= per || slot >= units) return;
     tile = blockIdx.x % n_tiles;   // (only the n tile is taken from `tile` below)
-    const int t2 = tile_list[slot];
-    ty0 = (t2 / pt.tiles_x) * pt.TY();
-    tx0 = (t2 % pt.tiles_x) << pt.tx_shift;
-    ptile = t2;
+#pragma unroll
+    for (int i = 0; i < TPW; ++i)
+      lt[i] = slot * TPW + i < cnt ? tile_list[slot * TPW + i] : -1;
   } else {
     ptile = tile / n_tiles;
   }
   const int m0 = (tile / n_tiles) * TM, n0 = (tile % n_tiles) * TN;
   auto pixel_of = [&](int p) -> int {
     if constexpr (TILED) {
-      const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
+      const int t2 = TPW == 1 ? lt[0] : (p < 128 ? lt[0] : lt[TPW - 1]);
+      if (t2 < 0) return -1;
+      const int pl = p & 127;
+      const int oy = (t2 / pt.tiles_x) * pt.TY() + (pl >> pt.tx_shift);
+      const int ox = ((t2 % pt.tiles_x) << pt.tx_shift) + (pl & (pt.TX() - 1));
       return (oy < pt.OH && ox < pt.OW) ? oy * pt.OW + ox : -1;
     } else {
       return m0 + p < M ? m0 + p : -1;
@@ -352,7 +359,31 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   zero_acc(acc);
 
   for (int k = 0; k < K; ++k) {
-    if constexpr (INV) {
+    if constexpr (INV && TILED) {
+      // rows of the listed image tiles: ((tile * K + k) * slots + s) * 128 + pixel
+      if (tid == 0) {
+        int top = 0;
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+          if (lt[i] >= 0) top = max(top, inv_ns[(size_t)lt[i] * K + k]);
+        *smax = min(top, slots);
+      }
+      __syncthreads();
+      for (int e = tid; e < *smax * TM; e += kThreads) {
+        const int s = e / TM, p = e - s * TM;
+        const int t2 = TPW == 1 ? lt[0] : (p < 128 ? lt[0] : lt[TPW - 1]);
+        float co = 0.0f;
+        int off = 0;
+        if (t2 >= 0) {
+          const size_t at = (((size_t)t2 * K + k) * slots + s) * 128 + (p & 127);
+          co = s < inv_ns[(size_t)t2 * K + k] ? inv_co[at] : 0.0f;
+          off = co != 0.0f ? inv_off[at] : 0;
+        }
+        tap_co[e] = co;
+        tap_off[e] = off;
+      }
+      __syncthreads();
+    } else if constexpr (INV) {
       const size_t rows = ((size_t)ptile * K + k) * slots * TM;
       if (tid == 0) *smax = min(inv_ns[(size_t)ptile * K + k], slots);
       __syncthreads();
@@ -746,8 +777,7 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                       float* workspace, hipStream_t stream, const CachedPlan* cached) {
   const int mm = matrix_mode(compute);
   const int slots = slots_for(g);
-  // (the listed-tile kernel behind the window kernel has 128 x 128 tiles only)
-  const bool narrow = g.Cp <= 64 && !gather_from_window(g);
+  const bool narrow = g.Cp <= 64;
   const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
   const int CpP = round_up(g.Cp, TN), CgP = round_up(g.Cg, kKC);
   int rc = relayout(g, Wm, workspace, CpP, CgP, 2, stream);
@@ -773,18 +803,25 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
     rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
                      reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream);
     if (rc) return rc;
-    const dim3 grid_t((unsigned)((plan.tiles + 7) / 8 * 8 * (CpP / TN)), (unsigned)g.B);
-#define GT(BFv)                                                                                   \
+    // the listed rest: 128 x 128 tiles, or 64 channels x two listed tiles for narrow layers
+    const int units = (int)ceil_div(plan.tiles, TM / 128);
+    const dim3 grid_t((unsigned)((units + 7) / 8 * 8 * (CpP / TN)), (unsigned)g.B);
+#define GT2(TNv, TMv, BFv)                                                                        \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                              \
                       (rc = launch_smem("gather_gemm(tiles)",                                     \
-                                        gather_gemm_kernel<INTERP, WEIGHTED, 128, 128, BFv, false, true>, \
+                                        gather_gemm_kernel<INTERP, WEIGHTED, TNv, TMv, BFv, false, true>, \
                                         grid_t, smem, stream, img, map, wts,                      \
                                         (const float*)workspace, bias, pix, g.Cg, g.H, g.W, g.Cp, \
                                         g.M, g.K, g.P, CgP, CpP, slots, plan.tiles,               \
                                         (const int*)nullptr, (const float*)nullptr,               \
                                         (const int*)nullptr, (const int*)nullptr, plan.pt,        \
                                         tl.rest, tl.count + 1)))
+#define GT(BFv)                                                  \
+  do {                                                           \
+    if (narrow) GT2(64, 256, BFv); else GT2(128, 128, BFv);      \
+  } while (0)
     if (mm == kMmBf16) GT(kMmBf16); else if (mm == kMmSplit) GT(kMmSplit); else GT(kMmF32);
+#undef GT2
 #undef GT
     return rc;
   }
@@ -1038,19 +1075,28 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                          reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream);
         if (rc) return rc;
         float* gw = reinterpret_cast<float*>(inv_ws + l.gather_weights);
-        const int CoutP = round_up(g.Cg, 128), CinP = round_up(g.Cp, kKC);
+        // the listed rest: 128 x 128 tiles, or 64 channels x two listed tiles for narrow images
+        const bool narrow = g.Cg <= 64;
+        const int TN = narrow ? 64 : 128, TM = narrow ? 256 : 128;
+        const int CoutP = round_up(g.Cg, TN), CinP = round_up(g.Cp, kKC);
         rc = relayout(g, Wm, gw, CoutP, CinP, 3, stream);
         if (rc) return rc;
-        const dim3 grid_t((unsigned)((ip.plan.tiles + 7) / 8 * 8 * (CoutP / 128)), (unsigned)g.B);
-        const size_t smem = sizeof(float) * kLdK * (128 + 128) + (size_t)kInversePlanRows * 128 * 8 + 16;
-#define IT(BFv)                                                                                  \
+        const int units = (int)ceil_div(ip.plan.tiles, TM / 128);
+        const dim3 grid_t((unsigned)((units + 7) / 8 * 8 * (CoutP / TN)), (unsigned)g.B);
+        const size_t smem = sizeof(float) * kLdK * (TM + TN) + (size_t)kInversePlanRows * TM * 8 + 16;
+#define IT2(TNv, TMv, BFv)                                                                       \
   rc = launch_smem("inverse_gather_gemm(tiles)",                                                 \
-                   gather_gemm_kernel<0, false, 128, 128, BFv, true, true>, grid_t, smem, stream, \
+                   gather_gemm_kernel<0, false, TNv, TMv, BFv, true, true>, grid_t, smem, stream, \
                    pix, (const float*)nullptr, (const float*)nullptr, (const float*)gw, bias,    \
                    img, g.Cp, 1, g.M, g.Cg, g.H * g.W, g.K, 0, CinP, CoutP, kInversePlanRows,    \
                    ip.plan.tiles, (const int*)ip.raw_off, (const float*)ip.raw_co,               \
                    (const int*)ip.plan.ns, (const int*)ip.gate, ip.plan.pt, tl.rest, tl.count + 1)
+#define IT(BFv)                                                  \
+  do {                                                           \
+    if (narrow) IT2(64, 256, BFv); else IT2(128, 128, BFv);      \
+  } while (0)
         if (mm == kMmBf16) IT(kMmBf16); else if (mm == kMmSplit) IT(kMmSplit); else IT(kMmF32);
+#undef IT2
 #undef IT
         if (rc) return rc;
         gate = ip.gate;

@@ -346,7 +346,9 @@ WwGrid ww_grid(const ConvGeom& g, int tiles) {
 }  // namespace
 
 bool window_wgrad_supported(const ConvGeom& g, int mm) {
-  return mm == kMmF32 && planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 32 &&
+  // (every wave multiplies four 32-row blocks: with 64 rows or fewer half of that is padding,
+  // and the plan-driven kernel, which splits the pixels instead, is the faster one)
+  return mm == kMmF32 && planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 64 &&
          (int64_t)g.H * g.W <= ((int64_t)1 << 24);
 }
 
