@@ -581,6 +581,72 @@ int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const v
     out_channels, int64_t out_height, int64_t out_width, int64_t kernel_size, int32_t
     num_interp_pts, int32_t interp, int32_t dtype, int32_t compute, sdk_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Plans of the scatter direction.  The optional workspaces of
+ * sdk_resample_to_map / sdk_resample_to_map_normalized, sdk_mapped_avg_unpool
+ * and sdk_mapped_max_unpool hold what those calls derive from the map alone
+ * (the inverted map: per target pixel its sources; the pooled window of every
+ * image tile).  A caller whose map stays the same builds that once into its
+ * own device memory ("plan", as large as the workspace of the same call) and
+ * passes it to the *_planned entry point, which skips the rebuild and gives
+ * the same results.  The reference has no counterpart (its entry points,
+ * ext_modules/include/layers/resample_layer.h:40-60,
+ * mapped_avg_pooling_layer.h, mapped_max_pooling_layer.h:64-88, are stateless).
+ *
+ * sdk_resample_to_map_plan_build: plan_bytes >=
+ *   sdk_resample_to_map_workspace_bytes(height, width, dtype).  kernel_size = 1
+ *   for a resampling map [map_height, map_width, (P,) 2]; for average
+ *   unpooling pass the pooled grid as map_height x map_width and the map's K.
+ * sdk_resample_plan_complete: synchronises `stream` and sets *complete to 1
+ *   when every target's list holds all its sources (at most 16 each).  The
+ *   planned calls take that as plan_complete: with 1 they launch the gather
+ *   alone (sample_map / interp_weights are then not read by
+ *   sdk_resample_to_map_planned and may be NULL); with 0 they also launch the
+ *   gated fallback (fill, atomic scatter, division), which runs only if the
+ *   plan is incomplete.  Passing 1 for an incomplete plan drops the sources
+ *   that did not fit.
+ * sdk_resample_to_map_planned: normalize = 0 is sdk_resample_to_map (weight_sum
+ *   optional), normalize = 1 sdk_resample_to_map_normalized (weight_sum
+ *   required, eps used).
+ * sdk_mapped_max_unpool_plan_build / _planned: plan_bytes >=
+ *   sdk_mapped_max_unpool_workspace_bytes(height, width, dtype).  The first
+ *   256 bytes of this plan are the call's fallback flag and are rewritten by
+ *   every planned call: calls that share one plan must not overlap.
+ * ------------------------------------------------------------------------- */
+int sdk_resample_to_map_plan_build(const void* sample_map, const void* interp_weights, void* plan,
+                                   size_t plan_bytes, int64_t map_height, int64_t map_width,
+                                   int64_t height, int64_t width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   sdk_stream_t stream);
+int sdk_resample_plan_complete(const void* plan, size_t plan_bytes, sdk_stream_t stream,
+                               int32_t* complete);
+int sdk_resample_to_map_planned(const void* input, const void* sample_map,
+                                const void* interp_weights, void* out, void* weight_sum,
+                                void* plan, size_t plan_bytes, int32_t plan_complete,
+                                int32_t normalize, double eps, int64_t batch, int64_t channels,
+                                int64_t map_height, int64_t map_width, int64_t height,
+                                int64_t width, int32_t num_interp_pts, int32_t interp,
+                                int32_t dtype, sdk_stream_t stream);
+int sdk_mapped_avg_unpool_planned(const void* grad_output, const void* sample_map,
+                                  const void* interp_weights, void* grad_input, void* plan,
+                                  size_t plan_bytes, int32_t plan_complete, int64_t batch,
+                                  int64_t channels, int64_t height, int64_t width,
+                                  int64_t out_height, int64_t out_width, int64_t kernel_size,
+                                  int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                  sdk_stream_t stream);
+int sdk_mapped_max_unpool_plan_build(const void* sample_map, void* plan, size_t plan_bytes,
+                                     int64_t height, int64_t width, int64_t out_height,
+                                     int64_t out_width, int64_t kernel_size,
+                                     int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                     sdk_stream_t stream);
+int sdk_mapped_max_unpool_planned(const void* grad_output, const int64_t* indices,
+                                  const void* sample_map, const void* interp_weights,
+                                  void* grad_input, void* plan, size_t plan_bytes, int64_t batch,
+                                  int64_t channels, int64_t height, int64_t width,
+                                  int64_t out_height, int64_t out_width, int64_t kernel_size,
+                                  int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                  sdk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

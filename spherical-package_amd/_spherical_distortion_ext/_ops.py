@@ -102,7 +102,9 @@ _plan_cache_enabled = True
 
 
 def set_conv_plan_cache(enabled):
-    """Keeps (default) or rebuilds per call the plans of the mapped (transposed) convolutions."""
+    """Keeps (default) or rebuilds per call what the operators derive from a map alone: the
+    plans of the mapped (transposed) convolutions, the inverted maps of resample_to_map and
+    average unpooling, the tile windows of max unpooling."""
     global _plan_cache_enabled
     _plan_cache_enabled = bool(enabled)
     if not enabled:
@@ -145,6 +147,54 @@ def _conv_plan(ref, sample_map, interp_weights, img_h, img_w, K, P, interp):
     return plan, n
 
 
+def _scatter_plan(kind, ref, sample_map, interp_weights, out_h, out_w, K, P, interp):
+    """(plan tensor, bytes, complete) of a scatter-direction operator for this map, built on
+    first use and kept like the convolution plans; (None, 0, 0) when the cache is off.
+
+    kind "resample" / "avg_unpool": the inverted map (sdk_resample_to_map_plan_build; K = 1 for
+    a resampling map), complete = 1 when every target's list holds all its sources, checked
+    once after the build (not under stream capture, where the check's synchronisation is not
+    allowed).  kind "max_unpool": the tile windows (sdk_mapped_max_unpool_plan_build)."""
+    if not _plan_cache_enabled:
+        return None, 0, 0
+    dt = _DTYPES[ref.dtype]
+    key = (kind, ref.device, dt, _tensor_key(sample_map), _tensor_key(interp_weights),
+           int(out_h), int(out_w), int(K), int(P), int(interp))
+    ent = _PLAN_CACHE.get(key)
+    cur = torch.cuda.current_stream(ref.device)
+    if ent is not None:
+        if ent[3] != cur:
+            cur.wait_stream(ent[3])
+        return ent[0], ent[1], ent[4]
+    lib = _capi.load()
+    query = ("sdk_mapped_max_unpool_workspace_bytes" if kind == "max_unpool"
+             else "sdk_resample_to_map_workspace_bytes")
+    n = getattr(lib, query)(int(out_h), int(out_w), dt)
+    if n == 0:
+        return None, 0, 0
+    plan = torch.empty(n, dtype=torch.uint8, device=ref.device)
+    MH, MW = int(sample_map.shape[0]), int(sample_map.shape[1])
+    complete = 0
+    if kind == "max_unpool":
+        _capi.call("sdk_mapped_max_unpool_plan_build", _ptr(sample_map), _ptr(plan), n, int(out_h),
+                   int(out_w), MH, MW, int(K), int(P), int(interp), dt, _stream(ref))
+    else:
+        _capi.call("sdk_resample_to_map_plan_build", _ptr(sample_map), _ptr(interp_weights),
+                   _ptr(plan), n, MH, MW, int(out_h), int(out_w), int(K), int(P), int(interp), dt,
+                   _stream(ref))
+        if not torch.cuda.is_current_stream_capturing():
+            flag = ctypes.c_int32(0)
+            _capi.call("sdk_resample_plan_complete", _ptr(plan), n, _stream(ref),
+                       ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+            complete = int(flag.value)
+    while len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
+        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
+    keep = (sample_map.untyped_storage(),
+            None if interp_weights is None else interp_weights.untyped_storage())
+    _PLAN_CACHE[key] = (plan, n, keep, cur, complete)
+    return plan, n, complete
+
+
 def _scatter_workspace(ref, out_h, out_w, query="sdk_resample_to_map_workspace_bytes"):
     n = getattr(_capi.load(), query)(int(out_h), int(out_w), _DTYPES[ref.dtype])
     if n == 0:
@@ -174,6 +224,14 @@ def resample_to_map(x, sample_map, interp_weights, out_h, out_w, interp):
                            % (tuple(sample_map.shape[:2]), (MH, MW)))
     out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
+        plan, nplan, complete = _scatter_plan("resample", x, sample_map, interp_weights, out_h,
+                                              out_w, 1, P, interp)
+        if plan is not None:
+            _capi.call("sdk_resample_to_map_planned", _ptr(x), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(out), ctypes.c_void_p(0), _ptr(plan), nplan,
+                       complete, 0, 0.0, B, C, MH, MW, int(out_h), int(out_w), P, int(interp),
+                       _DTYPES[x.dtype], _stream(x))
+            return out
         ws, nws = _scatter_workspace(x, out_h, out_w)
         _capi.call("sdk_resample_to_map", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
                    _ptr(out), ctypes.c_void_p(0), _ptr(ws), nws, B, C, MH, MW, int(out_h),
@@ -191,6 +249,14 @@ def resample_to_map_normalized(x, sample_map, interp_weights, out_h, out_w, inte
     out = torch.empty((B, C, int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     wsum = torch.empty((int(out_h), int(out_w)), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
+        plan, nplan, complete = _scatter_plan("resample", x, sample_map, interp_weights, out_h,
+                                              out_w, 1, P, interp)
+        if plan is not None:
+            _capi.call("sdk_resample_to_map_planned", _ptr(x), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(out), _ptr(wsum), _ptr(plan), nplan, complete,
+                       1, float(eps), B, C, MH, MW, int(out_h), int(out_w), P, int(interp),
+                       _DTYPES[x.dtype], _stream(x))
+            return out, wsum
         ws, nws = _scatter_workspace(x, out_h, out_w)
         _capi.call("sdk_resample_to_map_normalized", _ptr(x), _ptr(sample_map),
                    _ptr(interp_weights), _ptr(out), _ptr(wsum), _ptr(ws), nws, float(eps), B, C,
@@ -271,6 +337,15 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, i
     gin = torch.empty((B, C, int(in_h), int(in_w)), dtype=grad_output.dtype,
                       device=grad_output.device)
     with torch.cuda.device(grad_output.device):
+        if _UNPOOL_WORKSPACE:
+            plan, nplan, _ = _scatter_plan("max_unpool", grad_output, sample_map, interp_weights,
+                                           in_h, in_w, kernel_size, P, interp)
+            if plan is not None:
+                _capi.call("sdk_mapped_max_unpool_planned", _ptr(grad_output), _ptr(idx_mask),
+                           _ptr(sample_map), _ptr(interp_weights), _ptr(gin), _ptr(plan), nplan,
+                           B, C, int(in_h), int(in_w), OH, OW, int(kernel_size), P, int(interp),
+                           _DTYPES[grad_output.dtype], _stream(grad_output))
+                return gin
         ws, nws = _scatter_workspace(grad_output, in_h, in_w,
                                      "sdk_mapped_max_unpool_workspace_bytes")
         if not _UNPOOL_WORKSPACE:
@@ -329,6 +404,14 @@ def mapped_avg_unpool(grad_output, sample_map, interp_weights, in_h, in_w, kerne
     gin = torch.empty((B, C, int(in_h), int(in_w)), dtype=grad_output.dtype,
                       device=grad_output.device)
     with torch.cuda.device(grad_output.device):
+        plan, nplan, complete = _scatter_plan("avg_unpool", grad_output, sample_map,
+                                              interp_weights, in_h, in_w, kernel_size, P, interp)
+        if plan is not None:
+            _capi.call("sdk_mapped_avg_unpool_planned", _ptr(grad_output), _ptr(sample_map),
+                       _ptr(interp_weights), _ptr(gin), _ptr(plan), nplan, complete, B, C,
+                       int(in_h), int(in_w), OH, OW, int(kernel_size), P, int(interp),
+                       _DTYPES[grad_output.dtype], _stream(grad_output))
+            return gin
         ws, nws = _scatter_workspace(grad_output, in_h, in_w)
         _capi.call("sdk_mapped_avg_unpool", _ptr(grad_output), _ptr(sample_map),
                    _ptr(interp_weights), _ptr(gin), _ptr(ws), nws, B, C, int(in_h), int(in_w),

@@ -931,11 +931,36 @@ static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
   return off[3] + up((size_t)HW * kInvSlots * esz);
 }
 
+// Inverts a map into `workspace` (inverse_layout bytes): per target pixel the list of its
+// (source, coefficient) pairs, and the gate word that counts sources that found their list full.
+template <typename T>
+static int build_inverse_lists(const T* map, const T* wts, void* workspace, int H, int W, int MP,
+                               int P, int interp, int group, hipStream_t stream) {
+  size_t off[4];
+  inverse_layout((int64_t)H * W, sizeof(T), off);
+  char* ws = static_cast<char*>(workspace);
+  int* g = reinterpret_cast<int*>(ws + off[0]);
+  int* cnt = reinterpret_cast<int*>(ws + off[1]);
+  int* src = reinterpret_cast<int*>(ws + off[2]);
+  T* co = reinterpret_cast<T*>(ws + off[3]);
+  int rc = zero_fill(ws, off[2], stream);
+  if (rc != SDK_OK) return rc;
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((resample_inverse_fill_kernel<T, INTERP, WEIGHTED>),
+                              dim3((unsigned)ceil_div(MP, kBlock)), dim3(kBlock), stream, map,
+                              wts, H, W, MP, P, cnt, src, co, g, group)));
+  SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
+  return SDK_OK;
+}
+
+// prebuilt: `workspace` already holds the lists of this map (build_inverse_lists);
+// complete: ... and the caller knows that its gate is 0, so the fallback launches are left out.
 template <typename T>
 static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
                                   void* workspace, size_t workspace_bytes, int64_t planes, int H,
                                   int W, int MP, int P, int interp, hipStream_t stream,
-                                  bool normalize = false, double eps = 0.0, int group = 1) {
+                                  bool normalize = false, double eps = 0.0, int group = 1,
+                                  bool prebuilt = false, bool complete = false) {
   const int HW = H * W;
   const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
   size_t off[4];
@@ -945,13 +970,10 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
     int* cnt = reinterpret_cast<int*>(ws + off[1]);
     int* src = reinterpret_cast<int*>(ws + off[2]);
     T* co = reinterpret_cast<T*>(ws + off[3]);
-    int rc = zero_fill(ws, off[2], stream);
-    if (rc != SDK_OK) return rc;
-    SDK_DISPATCH_INTERP(interp, P,
-                        (launch((resample_inverse_fill_kernel<T, INTERP, WEIGHTED>),
-                                dim3((unsigned)ceil_div(MP, kBlock)), dim3(kBlock), stream, map,
-                                wts, H, W, MP, P, cnt, src, co, g, group)));
-    SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
+    if (!prebuilt) {
+      const int rc = build_inverse_lists<T>(map, wts, workspace, H, W, MP, P, interp, group, stream);
+      if (rc != SDK_OK) return rc;
+    }
     if (planes > 0 || wsum) {
       const int pc = planes_per_thread(planes);
 #define RIG(PCv)                                                                                 \
@@ -964,6 +986,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
       SDK_LAUNCH_CHECK("resample_to_map(inverse gather)");
     }
     gate = g;
+    if (prebuilt && complete) return SDK_OK;
   }
   // the scatter: fills, then one launch for all planes and (an extra grid row) the weight sum
   const size_t out_bytes = sizeof(T) * (size_t)planes * H * W, sum_bytes = sizeof(T) * (size_t)H * W;
@@ -1126,10 +1149,34 @@ static size_t unpool_layout(const UnpoolTiling& ut) {
   return 256 + (size_t)ut.tiles_x * ut.tiles_y * 8 * sizeof(int);
 }
 
+// The tile windows of the tiled unpool (a function of the map alone) into `workspace`
+// (unpool_layout bytes), gate word cleared.
+template <typename T>
+static int build_unpool_windows(const T* map, void* workspace, int H, int W, int OH, int OW, int K,
+                                int P, int interp, hipStream_t stream) {
+  const UnpoolTiling ut = unpool_tiling(H, W);
+  char* ws = static_cast<char*>(workspace);
+  int* win = reinterpret_cast<int*>(ws + 256);
+  int rc = zero_fill(ws, unpool_layout(ut), stream);
+  if (rc != SDK_OK) return rc;
+  const int64_t samples = (int64_t)OH * OW * K;
+  const dim3 grid_s((unsigned)ceil_div(samples, kBlock));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((unpool_window_kernel<T, INTERP, WEIGHTED, false>), grid_s,
+                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+  SDK_LAUNCH_CHECK("mapped_max_unpool(anchors)");
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((unpool_window_kernel<T, INTERP, WEIGHTED, true>), grid_s,
+                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+  SDK_LAUNCH_CHECK("mapped_max_unpool(windows)");
+  return SDK_OK;
+}
+
 template <typename T>
 static int launch_unpool(const T* gout, const int64_t* indices, const T* map, const T* wts, T* gin,
                          void* workspace, size_t workspace_bytes, int64_t planes, int H, int W,
-                         int OH, int OW, int K, int P, int interp, hipStream_t stream) {
+                         int OH, int OW, int K, int P, int interp, hipStream_t stream,
+                         bool prebuilt = false) {
   const int64_t HW = (int64_t)H * W, M = (int64_t)OH * OW;
   const int q = pts(P);
   const size_t total = (size_t)planes * M;
@@ -1150,18 +1197,14 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
     char* ws = static_cast<char*>(workspace);
     int* g = reinterpret_cast<int*>(ws);
     int* win = reinterpret_cast<int*>(ws + 256);
-    int rc = zero_fill(ws, unpool_layout(ut), stream);
+    int rc;
+    if (prebuilt) {
+      // the windows are there; the gate word is this call's own (the tile kernel raises it)
+      rc = zero_fill(ws, 256, stream);
+    } else {
+      rc = build_unpool_windows<T>(map, workspace, H, W, OH, OW, K, P, interp, stream);
+    }
     if (rc != SDK_OK) return rc;
-    const int64_t samples = M * K;
-    const dim3 grid_s((unsigned)ceil_div(samples, kBlock));
-    SDK_DISPATCH_INTERP(interp, P,
-                        (launch((unpool_window_kernel<T, INTERP, WEIGHTED, false>), grid_s,
-                                dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
-    SDK_LAUNCH_CHECK("mapped_max_unpool(anchors)");
-    SDK_DISPATCH_INTERP(interp, P,
-                        (launch((unpool_window_kernel<T, INTERP, WEIGHTED, true>), grid_s,
-                                dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
-    SDK_LAUNCH_CHECK("mapped_max_unpool(windows)");
     const dim3 grid_t((unsigned)tiles, (unsigned)groups);
     SDK_DISPATCH_INTERP(interp, P,
                         (launch((unpool_tiles_kernel<T, INTERP, WEIGHTED>), grid_t, dim3(kBlock),
@@ -1626,6 +1669,169 @@ int sdk_mapped_gather_at_index(const void* image, const int64_t* indices, const 
                          (int)height, (int)width, (int)M, num_interp_pts, map_elems))));
   SDK_LAUNCH_CHECK("mapped_gather_at_index");
   return SDK_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Plans of the scatter direction: the map-dependent scratch of sdk_resample_to_map,
+// sdk_mapped_avg_unpool and sdk_mapped_max_unpool, built once and kept by the caller.
+// ---------------------------------------------------------------------------
+int sdk_resample_to_map_plan_build(const void* sample_map, const void* interp_weights, void* plan,
+                                   size_t plan_bytes, int64_t map_height, int64_t map_width,
+                                   int64_t height, int64_t width, int64_t kernel_size,
+                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                   sdk_stream_t stream) {
+  SDK_REQUIRE(sample_map && plan, "resample_to_map_plan_build: NULL pointer");
+  SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights),
+              "resample_to_map_plan_build: weighted map needs interp_weights");
+  SDK_REQUIRE(kernel_size >= 1, "resample_to_map_plan_build: bad kernel_size");
+  int rc = check_plane(height, width, "resample_to_map_plan_build(out)");
+  if (rc) return rc;
+  SDK_REQUIRE(map_height > 0 && map_width > 0 &&
+                  map_height * map_width * kernel_size < ((int64_t)1 << 31),
+              "resample_to_map_plan_build: bad map size");
+  const size_t need = sdk_resample_to_map_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "resample_to_map_plan_build: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  SDK_DISPATCH_DTYPE(dtype, return build_inverse_lists<T>(
+                                (const T*)sample_map, (const T*)interp_weights, plan, (int)height,
+                                (int)width, (int)(map_height * map_width * kernel_size),
+                                num_interp_pts, interp, (int)kernel_size, (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_resample_plan_complete(const void* plan, size_t plan_bytes, sdk_stream_t stream,
+                               int32_t* complete) {
+  SDK_REQUIRE(plan && complete && plan_bytes >= 256, "resample_plan_complete: bad argument");
+  int gate = 1;
+  hipError_t e = hipMemcpyAsync(&gate, plan, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream);
+  if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+  if (e != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "resample_plan_complete: %s", hipGetErrorString(e));
+  *complete = gate == 0 ? 1 : 0;
+  return SDK_OK;
+}
+
+int sdk_resample_to_map_planned(const void* input, const void* sample_map,
+                                const void* interp_weights, void* out, void* weight_sum,
+                                void* plan, size_t plan_bytes, int32_t plan_complete,
+                                int32_t normalize, double eps, int64_t batch, int64_t channels,
+                                int64_t map_height, int64_t map_width, int64_t height,
+                                int64_t width, int32_t num_interp_pts, int32_t interp,
+                                int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(input && out && plan, "resample_to_map_planned: NULL pointer");
+  SDK_REQUIRE(plan_complete || sample_map,
+              "resample_to_map_planned: the map is needed unless the plan is known complete");
+  SDK_REQUIRE(!normalize || weight_sum, "resample_to_map_planned: NULL weight_sum");
+  SDK_REQUIRE(num_interp_pts >= 0 && (num_interp_pts == 0 || interp_weights || plan_complete),
+              "resample_to_map_planned: weighted map needs interp_weights");
+  SDK_REQUIRE(batch >= 0 && channels >= 0, "resample_to_map_planned: negative size");
+  int rc = check_plane(height, width, "resample_to_map_planned(out)");
+  if (rc) return rc;
+  rc = check_plane(map_height, map_width, "resample_to_map_planned(map)");
+  if (rc) return rc;
+  const size_t need = sdk_resample_to_map_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "resample_to_map_planned: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  const int64_t planes = batch * channels;
+  rc = check_grid_y(planes, "resample_to_map_planned");
+  if (rc) return rc;
+  if (planes == 0 && !weight_sum) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_resample_to_map<T>(
+                                (const T*)input, (const T*)sample_map, (const T*)interp_weights,
+                                (T*)out, (T*)weight_sum, plan, plan_bytes, planes, (int)height,
+                                (int)width, (int)(map_height * map_width), num_interp_pts, interp,
+                                (hipStream_t)stream, normalize != 0, eps, 1, true,
+                                plan_complete != 0));
+  return SDK_OK;
+}
+
+int sdk_mapped_avg_unpool_planned(const void* grad_output, const void* sample_map,
+                                  const void* interp_weights, void* grad_input, void* plan,
+                                  size_t plan_bytes, int32_t plan_complete, int64_t batch,
+                                  int64_t channels, int64_t height, int64_t width,
+                                  int64_t out_height, int64_t out_width, int64_t kernel_size,
+                                  int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                  sdk_stream_t stream) {
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_avg_unpool_planned: bad pooled size");
+  SDK_REQUIRE(plan, "mapped_avg_unpool_planned: NULL plan");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(grad_output, sample_map, interp_weights, grad_input, batch, channels,
+                        height, width, M, kernel_size, num_interp_pts,
+                        "mapped_avg_unpool_planned");
+  if (rc) return rc;
+  SDK_REQUIRE(M * kernel_size < ((int64_t)1 << 31), "mapped_avg_unpool_planned: too many samples");
+  const size_t need = sdk_resample_to_map_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "mapped_avg_unpool_planned: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_resample_to_map<T>(
+                                (const T*)grad_output, (const T*)sample_map,
+                                (const T*)interp_weights, (T*)grad_input, (T*)nullptr, plan,
+                                plan_bytes, planes, (int)height, (int)width,
+                                (int)(M * kernel_size), num_interp_pts, interp,
+                                (hipStream_t)stream, false, 0.0, (int)kernel_size, true,
+                                plan_complete != 0));
+  return SDK_OK;
+}
+
+int sdk_mapped_max_unpool_plan_build(const void* sample_map, void* plan, size_t plan_bytes,
+                                     int64_t height, int64_t width, int64_t out_height,
+                                     int64_t out_width, int64_t kernel_size,
+                                     int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                     sdk_stream_t stream) {
+  SDK_REQUIRE(sample_map && plan, "mapped_max_unpool_plan_build: NULL pointer");
+  SDK_REQUIRE(out_height > 0 && out_width > 0 && kernel_size >= 1 && num_interp_pts >= 0,
+              "mapped_max_unpool_plan_build: bad size");
+  int rc = check_plane(height, width, "mapped_max_unpool_plan_build");
+  if (rc) return rc;
+  const int64_t M = out_height * out_width;
+  SDK_REQUIRE(M < ((int64_t)1 << 31) &&
+                  M * kernel_size * pts(num_interp_pts) * 2 < ((int64_t)1 << 31),
+              "mapped_max_unpool_plan_build: map too large for a plan");
+  const size_t need = sdk_mapped_max_unpool_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "mapped_max_unpool_plan_build: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  SDK_DISPATCH_DTYPE(dtype, return build_unpool_windows<T>(
+                                (const T*)sample_map, plan, (int)height, (int)width,
+                                (int)out_height, (int)out_width, (int)kernel_size, num_interp_pts,
+                                interp, (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_mapped_max_unpool_planned(const void* grad_output, const int64_t* indices,
+                                  const void* sample_map, const void* interp_weights,
+                                  void* grad_input, void* plan, size_t plan_bytes, int64_t batch,
+                                  int64_t channels, int64_t height, int64_t width,
+                                  int64_t out_height, int64_t out_width, int64_t kernel_size,
+                                  int32_t num_interp_pts, int32_t interp, int32_t dtype,
+                                  sdk_stream_t stream) {
+  SDK_REQUIRE(indices && plan, "mapped_max_unpool_planned: NULL pointer");
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_unpool_planned: bad pooled size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(grad_output, sample_map, interp_weights, grad_input, batch, channels,
+                        height, width, M, kernel_size, num_interp_pts, "mapped_max_unpool_planned");
+  if (rc) return rc;
+  const size_t need = sdk_mapped_max_unpool_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "mapped_max_unpool_planned: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  SDK_REQUIRE(M * kernel_size * pts(num_interp_pts) * 2 < ((int64_t)1 << 31),
+              "mapped_max_unpool_planned: map too large for a plan");
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_REQUIRE(ceil_div(planes * M, kBlock) < ((int64_t)1 << 31),
+              "mapped_max_unpool_planned: too many elements");
+  SDK_DISPATCH_DTYPE(dtype, return launch_unpool<T>(
+                                (const T*)grad_output, indices, (const T*)sample_map,
+                                (const T*)interp_weights, (T*)grad_input, plan, plan_bytes, planes,
+                                (int)height, (int)width, (int)out_height, (int)out_width,
+                                (int)kernel_size, num_interp_pts, interp, (hipStream_t)stream,
+                                true));
 }
 
 }  // extern "C"
