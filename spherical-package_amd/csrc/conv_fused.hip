@@ -21,6 +21,7 @@
 //   A operand: A[i = l % 32][k = l / 32]        B operand: B[k = l / 32][j = l % 32]
 //   D, 16 registers v: D[i = 8*(v/4) + 4*(l/32) + v%4][j = l % 32]
 #include "conv_fused.hpp"
+#include "conv_small.hpp"
 #include "conv_plan.hpp"
 
 #include <hip/hip_runtime.h>
@@ -775,6 +776,8 @@ static int launch_smem(const char* what, Kern kern, dim3 grid, size_t smem, hipS
 int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const float* map,
                       const float* wts, const float* Wm, const float* bias, float* pix,
                       float* workspace, hipStream_t stream, const CachedPlan* cached) {
+  // images of a few channels: the packed kernel (a 32-channel chunk would be mostly padding)
+  if (small_conv_supported(g)) return small_forward(g, img, map, wts, Wm, bias, pix, stream);
   const int mm = matrix_mode(compute);
   const int slots = slots_for(g);
   const bool narrow = g.Cp <= 64;
@@ -1046,6 +1049,13 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                        const CachedPlan* cached) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
   int rc = SDK_OK;
+  if (small_conv_supported(g)) {
+    // images of a few channels: fill, then the packed scatter kernel
+    rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+    if (rc) return rc;
+    if (shared != nullptr) shared->valid = false;
+    return small_scatter(g, pix, map, wts, Wm, img, stream);
+  }
   if (planned_scatter_supported(g)) {
     const int* gate = nullptr;
     if (inverse_candidate(g)) {
@@ -1152,6 +1162,7 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
   int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
+  if (small_wgrad_supported(g)) return small_wgrad(g, pix, map, wts, img, gW, stream);
   if (planned_wgrad_supported(g)) {
     if (cached != nullptr)
       return wgrad_from_plan(g, matrix_mode(compute), cached->plan, pix, img, gW, workspace,

@@ -367,6 +367,11 @@ TILE_CASES = [
     (33, 64, 16, 40, 8, 40, 9, 0, 0),      # narrow tiles (<= 64 channels), nearest
     (64, 33, 10, 30, 10, 29, 7, 4, 1),     # 16 tap slots per sample
     (3, 16, 64, 128, 64, 128, 9, 0, 1),    # configuration 1's shape
+    # images of at most four channels: the packed kernels
+    (1, 8, 12, 20, 12, 20, 9, 0, 1),       # one channel
+    (2, 40, 14, 18, 7, 9, 25, 0, 0),       # 25 samples, two blocks of columns and of rows
+    (4, 100, 10, 16, 10, 16, 9, 2, 2),     # weighted, four row blocks, two column blocks
+    (4, 128, 9, 11, 9, 11, 25, 0, 1),      # weight gradient beyond the packed kernel's registers
 ]
 
 
