@@ -7,7 +7,9 @@ call into libsdk_mapped_ops.so.  The operators are registered in the
 ``sdk_mapped_ops`` namespace of torch.library for the CUDA (= HIP on ROCm)
 dispatch key only: calling them with CPU tensors raises, there is no CPU path.
 """
+import contextlib
 import ctypes
+import threading
 
 import torch
 
@@ -20,26 +22,54 @@ _DTYPES = {torch.float32: _capi.SDK_F32, torch.float64: _capi.SDK_F64}
 # (the tensors' type), "bf16" (bf16 operands, fp32 accumulate), "split" (fp32 operands as
 # three bf16 pieces each: fp32 accuracy from the bf16 matrix unit) or "unfused"
 # (separate im2col/col2im + GEMM kernels, the cross-check path).
-_compute_mode = _capi.SDK_COMPUTE_NATIVE
+_MODES = {"native": _capi.SDK_COMPUTE_NATIVE, "fp32": _capi.SDK_COMPUTE_NATIVE,
+          "bf16": _capi.SDK_COMPUTE_BF16, "unfused": _capi.SDK_COMPUTE_UNFUSED,
+          "split": _capi.SDK_COMPUTE_SPLIT}
+_default_mode = _capi.SDK_COMPUTE_NATIVE   # process-wide default
+_tls = threading.local()                   # per-thread override (conv_compute)
+
+
+def _mode_value(mode):
+    if mode not in _MODES:
+        raise ValueError("compute mode must be one of %s" % sorted(_MODES))
+    return _MODES[mode]
 
 
 def set_conv_compute(mode):
-    """Selects the GEMM arithmetic of the mapped (transposed) convolutions."""
-    global _compute_mode
-    modes = {"native": _capi.SDK_COMPUTE_NATIVE, "fp32": _capi.SDK_COMPUTE_NATIVE,
-             "bf16": _capi.SDK_COMPUTE_BF16, "unfused": _capi.SDK_COMPUTE_UNFUSED,
-             "split": _capi.SDK_COMPUTE_SPLIT}
-    if mode not in modes:
-        raise ValueError("compute mode must be one of %s" % sorted(modes))
-    _compute_mode = modes[mode]
+    """Sets the process-wide default arithmetic of the mapped (transposed) convolutions:
+    "native" (fp32 MFMA), "split" (fp32 operands as three bf16 pieces), "bf16" (operands
+    rounded to bf16), "unfused" (im2col + GEMM kernels)."""
+    global _default_mode
+    _default_mode = _mode_value(mode)
+
+
+def _current_mode():
+    return getattr(_tls, "mode", None) or _default_mode
 
 
 def get_conv_compute():
+    """The mode a convolution called now on this thread would use."""
     return {_capi.SDK_COMPUTE_BF16: "bf16", _capi.SDK_COMPUTE_UNFUSED: "unfused",
-            _capi.SDK_COMPUTE_SPLIT: "split"}.get(_compute_mode, "native")
+            _capi.SDK_COMPUTE_SPLIT: "split"}.get(_current_mode(), "native")
 
 
-# --------------------------------------------------------------------------- checks
+@contextlib.contextmanager
+def conv_compute(mode):
+    """Overrides the compute mode for the calls made inside the block on this thread; None
+    leaves the default in force.  The autograd functions run their backward under the mode
+    their forward saw, and the nn modules take a `compute` argument that ends up here."""
+    if mode is None:
+        yield
+        return
+    value = _mode_value(mode)
+    previous = getattr(_tls, "mode", None)
+    _tls.mode = value
+    try:
+        yield
+    finally:
+        _tls.mode = previous
+
+
 def _check(ref, **tensors):
     """ref: the tensor that decides device and dtype (first argument of the op)."""
     if not ref.is_cuda:
@@ -84,7 +114,7 @@ def _npts(sample_map, interp_weights, map_rank_unweighted):
 def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
     n = _capi.load().sdk_mapped_conv_workspace_bytes(
         batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp, _DTYPES[ref.dtype],
-        _compute_mode)
+        _current_mode())
     if n == 0:
         return None, 0
     return torch.empty(n, dtype=torch.uint8, device=ref.device), n
@@ -445,7 +475,7 @@ def mapped_conv_forward(x, sample_map, interp_weights, weight, bias, kernel_size
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         plan, nplan = _conv_plan(x, sample_map, interp_weights, H, W, K, P, int(interp))
-        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode,
+        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _current_mode(),
                 _stream(x))
         if plan is None:
             _capi.call("sdk_mapped_conv_forward", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
@@ -475,7 +505,7 @@ def mapped_conv_backward(grad_output, sample_map, interp_weights, x, weight, bia
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, H, W, OH, OW, K, P, int(interp))
         s = _stream(x)
-        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
+        dims = (B, Cin, H, W, Cout, OH, OW, K, P, int(interp), dt, _current_mode(), s)
         plan, nplan = _conv_plan(x, sample_map, interp_weights, H, W, K, P, int(interp))
         if plan is None:
             _capi.call("sdk_mapped_conv_backward", _ptr(grad_output), _ptr(sample_map),
@@ -503,7 +533,7 @@ def mapped_transposed_conv_forward(x, sample_map, interp_weights, weight, bias, 
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         plan, nplan = _conv_plan(x, sample_map, interp_weights, OH, OW, K, P, int(interp))
-        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _compute_mode,
+        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _current_mode(),
                 _stream(x))
         if plan is None:
             _capi.call("sdk_mapped_transposed_conv_forward", _ptr(x), _ptr(sample_map),
@@ -532,7 +562,7 @@ def mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, x, 
     with torch.cuda.device(x.device):
         ws, nws = _workspace(x, B, Cin, Cout, OH, OW, IH, IW, K, P, int(interp))
         s = _stream(x)
-        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _compute_mode, s)
+        dims = (B, Cin, IH, IW, Cout, OH, OW, K, P, int(interp), dt, _current_mode(), s)
         plan, nplan = _conv_plan(x, sample_map, interp_weights, OH, OW, K, P, int(interp))
         if plan is None:
             _capi.call("sdk_mapped_transposed_conv_backward", _ptr(grad_output), _ptr(sample_map),

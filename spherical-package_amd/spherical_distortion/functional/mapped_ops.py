@@ -19,7 +19,7 @@ import _spherical_distortion_ext._weighted_mapped_max_pooling as _weighted_mappe
 import _spherical_distortion_ext._weighted_mapped_transposed_convolution as _weighted_mapped_transposed_conv
 import _spherical_distortion_ext._weighted_resample as _weighted_resample
 
-from _spherical_distortion_ext._ops import ops as _sdk_ops
+from _spherical_distortion_ext._ops import conv_compute, get_conv_compute, ops as _sdk_ops
 
 from ..layer_utils import InterpolationType, check_args, check_input_map_shape
 
@@ -32,6 +32,7 @@ class MappedConvolutionFunction(torch.autograd.Function):
         ctx.save_for_backward(input, weight, bias, sample_map, interp_weights)
         ctx.kernel_size = int(kernel_size)
         ctx.interp = InterpolationType(interp)
+        ctx.compute = get_conv_compute()   # the backward runs in the arithmetic of the forward
         if interp_weights is None:
             return _mapped_conv.mapped_conv_forward(input, sample_map, weight, bias,
                                                     ctx.kernel_size, ctx.interp)
@@ -41,13 +42,14 @@ class MappedConvolutionFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         input, weight, bias, sample_map, interp_weights = ctx.saved_tensors
-        if interp_weights is None:
-            grads = _mapped_conv.mapped_conv_backward(grad_output, sample_map, input, weight, bias,
-                                                      ctx.kernel_size, ctx.interp)
-        else:
-            grads = _weighted_mapped_conv.weighted_mapped_conv_backward(
-                grad_output, sample_map, interp_weights, input, weight, bias, ctx.kernel_size,
-                ctx.interp)
+        with conv_compute(ctx.compute):
+            if interp_weights is None:
+                grads = _mapped_conv.mapped_conv_backward(grad_output, sample_map, input, weight,
+                                                          bias, ctx.kernel_size, ctx.interp)
+            else:
+                grads = _weighted_mapped_conv.weighted_mapped_conv_backward(
+                    grad_output, sample_map, interp_weights, input, weight, bias,
+                    ctx.kernel_size, ctx.interp)
         grad_input, grad_weight, grad_bias = grads
         return grad_input, grad_weight, grad_bias, None, None, None, None
 
@@ -61,6 +63,7 @@ class MappedTransposedConvolutionFunction(torch.autograd.Function):
         ctx.save_for_backward(input, sample_map, weight, bias, interp_weights)
         ctx.kernel_size = int(kernel_size)
         ctx.interp = InterpolationType(interp)
+        ctx.compute = get_conv_compute()
         if interp_weights is None:
             return _mapped_transposed_conv.mapped_transposed_conv_forward(
                 input, sample_map, weight, bias, output_height, output_width, ctx.kernel_size,
@@ -72,13 +75,14 @@ class MappedTransposedConvolutionFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         input, sample_map, weight, bias, interp_weights = ctx.saved_tensors
-        if interp_weights is None:
-            grads = _mapped_transposed_conv.mapped_transposed_conv_backward(
-                grad_output, sample_map, input, weight, bias, ctx.kernel_size, ctx.interp)
-        else:
-            grads = _weighted_mapped_transposed_conv.weighted_mapped_transposed_conv_backward(
-                grad_output, sample_map, interp_weights, input, weight, bias, ctx.kernel_size,
-                ctx.interp)
+        with conv_compute(ctx.compute):
+            if interp_weights is None:
+                grads = _mapped_transposed_conv.mapped_transposed_conv_backward(
+                    grad_output, sample_map, input, weight, bias, ctx.kernel_size, ctx.interp)
+            else:
+                grads = _weighted_mapped_transposed_conv.weighted_mapped_transposed_conv_backward(
+                    grad_output, sample_map, interp_weights, input, weight, bias,
+                    ctx.kernel_size, ctx.interp)
         grad_input, grad_weight, grad_bias = grads
         return grad_input, grad_weight, grad_bias, None, None, None, None, None, None
 
@@ -275,21 +279,25 @@ class UVResampleFunction(torch.autograd.Function):
 
 # ----------------------------------------------------------------------------- entry points
 def mapped_convolution(input, weight, bias, sample_map, kernel_size, interp,
-                       interp_weights=None):
-    """layers/functional/mapped_convolution.py:121-131."""
+                       interp_weights=None, compute=None):
+    """layers/functional/mapped_convolution.py:121-131.  compute (not in the reference): the
+    arithmetic of this call and of its backward ("native", "split", "bf16", "unfused"); None
+    takes the mode in force (set_conv_compute / conv_compute)."""
     check_args(input, sample_map, interp_weights, weight.shape[1], weight.shape[2])
-    return MappedConvolutionFunction.apply(input, weight, bias, sample_map, kernel_size, interp,
-                                           interp_weights)
+    with conv_compute(compute):
+        return MappedConvolutionFunction.apply(input, weight, bias, sample_map, kernel_size,
+                                               interp, interp_weights)
 
 
 def mapped_transposed_convolution(input, weight, bias, sample_map, output_height, output_width,
-                                  kernel_size, interp, interp_weights=None):
-    """layers/functional/mapped_convolution.py:134-148."""
+                                  kernel_size, interp, interp_weights=None, compute=None):
+    """layers/functional/mapped_convolution.py:134-148.  compute: as for mapped_convolution."""
     check_args(input, sample_map, interp_weights, weight.shape[0], weight.shape[2])
     check_input_map_shape(input, sample_map)
-    return MappedTransposedConvolutionFunction.apply(input, weight, bias, sample_map,
-                                                     output_height, output_width, kernel_size,
-                                                     interp, interp_weights)
+    with conv_compute(compute):
+        return MappedTransposedConvolutionFunction.apply(input, weight, bias, sample_map,
+                                                         output_height, output_width,
+                                                         kernel_size, interp, interp_weights)
 
 
 def mapped_max_pool(input, sample_map, kernel_size, interp, interp_weights=None):

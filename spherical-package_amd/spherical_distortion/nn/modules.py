@@ -25,15 +25,18 @@ def _init_uniform(weight, bias, fan_in):
 class MappedConvolution(nn.Module):
     """Convolution whose K taps per output pixel are read where `sample_map`
     says.  weight [out_channels, in_channels, kernel_size]; `bias=False` keeps a
-    zero bias parameter (mapped_convolution_layer.py:14-59)."""
+    zero bias parameter (mapped_convolution_layer.py:14-59).  compute (not in the reference):
+    this layer's arithmetic, "native", "split", "bf16" or "unfused"; None follows
+    set_conv_compute."""
 
     def __init__(self, in_channels, out_channels, kernel_size=1,
-                 interpolation=InterpolationType.BILINEAR, bias=True):
+                 interpolation=InterpolationType.BILINEAR, bias=True, compute=None):
         super().__init__()
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.kernel_size = kernel_size
         self.interp = interpolation
+        self.compute = compute
         self.weight = nn.Parameter(torch.empty(out_channels, in_channels, kernel_size))
         self.bias = nn.Parameter(torch.empty(out_channels))
         self.reset_parameters()
@@ -47,21 +50,22 @@ class MappedConvolution(nn.Module):
         """x [B,Cin,H,W]; sample_map [OH,OW,K,2] or, with interp_weights [OH,OW,K,P],
         [OH,OW,K,P,2]."""
         return F.mapped_convolution(x, self.weight, self.bias, sample_map, self.kernel_size,
-                                    self.interp, interp_weights)
+                                    self.interp, interp_weights, self.compute)
 
 
 class MappedTransposedConvolution(nn.Module):
     """The map has the input's H x W and points into the [oh, ow] output.
     weight [in_channels, out_channels, kernel_size]
-    (mapped_transposed_convolution_layer.py:10-56)."""
+    (mapped_transposed_convolution_layer.py:10-56).  compute: as for MappedConvolution."""
 
     def __init__(self, in_channels, out_channels, kernel_size=1,
-                 interpolation=InterpolationType.BILINEAR, bias=True):
+                 interpolation=InterpolationType.BILINEAR, bias=True, compute=None):
         super().__init__()
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.kernel_size = kernel_size
         self.interp = interpolation
+        self.compute = compute
         self.weight = nn.Parameter(torch.empty(in_channels, out_channels, kernel_size))
         self.bias = nn.Parameter(torch.empty(out_channels))
         self.reset_parameters()
@@ -73,7 +77,8 @@ class MappedTransposedConvolution(nn.Module):
 
     def forward(self, x, oh, ow, sample_map, interp_weights=None):
         return F.mapped_transposed_convolution(x, self.weight, self.bias, sample_map, oh, ow,
-                                               self.kernel_size, self.interp, interp_weights)
+                                               self.kernel_size, self.interp, interp_weights,
+                                               self.compute)
 
 
 class MappedMaxPool(nn.Module):

@@ -130,3 +130,44 @@ def test_plan_buffer_of_the_wrong_size_is_refused(ops):
     rc = lib.sdk_mapped_conv_plan_build(one, None, one, n - 1, 40, 64, 40, 64, 9, 0, 1,
                                         _capi.SDK_F32, None)
     assert rc != 0 and b"needs" in lib.sdk_last_error()
+
+
+def test_backward_runs_in_the_arithmetic_of_its_forward(ops, oracle):
+    """A layer built with compute="bf16" rounds its operands in forward and backward whatever
+    the process default says at backward time; a default layer follows the default."""
+    from spherical_distortion import nn as sdnn
+    m, iw, x, w, b, g, _ = _case(5, 72, 80, 24, 32, 24, 32, 9, 0, 1, "plain")
+    tm, tx, tg = _t(m), _t(x), _t(g)
+
+    def run(layer):
+        with torch.no_grad():
+            layer.weight.copy_(_t(w))
+            layer.bias.copy_(_t(b))
+        xin = tx.clone().requires_grad_(True)
+        y = layer(xin, tm)
+        y.backward(tg)
+        return y.detach(), xin.grad, layer.weight.grad
+
+    native = run(sdnn.MappedConvolution(72, 80, 9).to(DEV))
+    layer = sdnn.MappedConvolution(72, 80, 9, compute="bf16").to(DEV)
+    with torch.no_grad():
+        layer.weight.copy_(_t(w))
+        layer.bias.copy_(_t(b))
+    xin = tx.clone().requires_grad_(True)
+    y = layer(xin, tm)
+    ops.set_conv_compute("unfused")        # must not reach the backward of the bf16 layer
+    try:
+        y.backward(tg)
+    finally:
+        ops.set_conv_compute("native")
+    ops.set_conv_compute("bf16")
+    try:
+        want = run(sdnn.MappedConvolution(72, 80, 9).to(DEV))
+    finally:
+        ops.set_conv_compute("native")
+    assert torch.equal(y.detach(), want[0])
+    assert torch.equal(xin.grad, want[1])
+    assert relerr(layer.weight.grad.cpu().numpy(), want[2].cpu().numpy()) <= 1e-6
+    # and bf16 is visibly not the native arithmetic
+    assert not torch.equal(y.detach(), native[0])
+    assert relerr(y.detach().cpu().numpy(), native[0].cpu().numpy()) <= 1e-2

@@ -204,3 +204,32 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert "compute" in err()
     assert lib.sdk_mapped_conv_workspace_bytes(1, 3, 4, 8, 8, 8, 8, 9, 0, 1, 0, 3) == \
         lib.sdk_mapped_conv_workspace_bytes(1, 3, 4, 8, 8, 8, 8, 9, 0, 1, 0, 0)
+
+
+def test_compute_mode_override_is_scoped_and_per_thread():
+    """conv_compute() overrides the mode for the block on the calling thread only and restores
+    what was in force; set_conv_compute() sets the process default."""
+    import threading
+    from _spherical_distortion_ext import _ops
+    assert _ops.get_conv_compute() == "native"
+    with _ops.conv_compute("split"):
+        assert _ops.get_conv_compute() == "split"
+        seen = []
+        th = threading.Thread(target=lambda: seen.append(_ops.get_conv_compute()))
+        th.start()
+        th.join()
+        assert seen == ["native"]
+        with _ops.conv_compute("bf16"):
+            assert _ops.get_conv_compute() == "bf16"
+        with _ops.conv_compute(None):
+            assert _ops.get_conv_compute() == "split"
+        assert _ops.get_conv_compute() == "split"
+    assert _ops.get_conv_compute() == "native"
+    _ops.set_conv_compute("unfused")
+    try:
+        assert _ops.get_conv_compute() == "unfused"
+    finally:
+        _ops.set_conv_compute("native")
+    with pytest.raises(ValueError):
+        with _ops.conv_compute("fp8"):
+            pass
