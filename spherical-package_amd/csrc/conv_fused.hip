@@ -356,8 +356,21 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
   const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
   const int gm = tid % TM, gpart = tid / TM;
 
+  // The accumulators start at the bias of their rows, so the epilogue is stores alone (a bias
+  // read behind each store would wait for that store too: 64 round trips per workgroup).
   floatx16 acc[2][2];
   zero_acc(acc);
+  if (bias != nullptr) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + a_base + 32 * a + mfma_row(v, lane);
+        const float bv = bias[n < Cp ? n : Cp - 1];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) acc[a][b][v] = n < Cp ? bv : 0.0f;
+      }
+  }
 
   for (int k = 0; k < K; ++k) {
     if constexpr (INV && TILED) {
@@ -447,7 +460,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
     }
   }
 
-  // ---- epilogue: + bias, store (lanes along pixels: 128-byte rows)
+  // ---- epilogue: store (lanes along pixels: 128-byte rows)
   float* pix_b = pix + (size_t)blockIdx.y * Cp * M;
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -457,7 +470,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int n = n0 + a_base + 32 * a + mfma_row(v, lane);
-        if (n < Cp && m >= 0) pix_b[(size_t)n * M + m] = acc[a][b][v] + (bias ? bias[n] : 0.0f);
+        if (n < Cp && m >= 0) pix_b[(size_t)n * M + m] = acc[a][b][v];
       }
     }
 }

@@ -365,11 +365,26 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
   const int p_local = 32 * wave + j;
   const int2* rows_p = taps + (size_t)tile * K * S * 128 + p_local;
 
+  // The accumulators start at the bias of their rows (register v of lane l: row
+  // 8 (v / 4) + 4 (l / 32) + v % 4): the reads are issued here, with the window's, and the
+  // epilogue is stores alone.  (Read behind each store they serialise: on this part a wait
+  // for the load also waits for the store before it, 64 round trips per tile and wave.)
   floatx16 acc[NB];
+  if (bias != nullptr) {
 #pragma unroll
-  for (int a = 0; a < NB; ++a)
+    for (int a = 0; a < NB; ++a)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[a][v] = 0.0f;
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
+        const float bv = bias[n < Cp ? n : Cp - 1];
+        acc[a][v] = n < Cp ? bv : 0.0f;
+      }
+  } else {
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][v] = 0.0f;
+  }
 
   // weight tile of (k, chunk): TN rows of 32 values, 16-byte pieces e = tid + 256 i
   constexpr int WPT = TN * kCC / 4 / kWgThreads;   // float4 per thread: 4 (TN = 128) or 2
@@ -543,7 +558,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
       for (int u = 0; u < RB; ++u) rows[u] = rows_next[u];
     }
   }
-  // ---- epilogue: + bias, store.  Accumulator register v of lane l: row 8*(v/4) + 4*h + v%4
+  // ---- epilogue: store.  Accumulator register v of lane l: row 8*(v/4) + 4*h + v%4
   // (pixel-side channel), column j (pixel).
   const int oy = ty0 + (p_local >> pt.tx_shift), ox = tx0 + (p_local & (pt.TX() - 1));
   if (oy < pt.OH && ox < pt.OW) {
@@ -553,7 +568,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int n = n0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
-        if (n < Cp) out[(size_t)n * M] = acc[a][v] + (bias ? bias[n] : 0.0f);
+        if (n < Cp) out[(size_t)n * M] = acc[a][v];
       }
   }
 #undef SDK_LOAD_WEIGHTS
