@@ -528,6 +528,38 @@ __global__ __launch_bounds__(kBlock) void mapped_col2im_kernel(
   }
 }
 
+// Values of KB consecutive samples (first: k0; samples past K repeat the last) of one pixel of
+// an unweighted map for PC planes, v[g][j]: the coordinates of all KB samples are read
+// together, then all taps of all planes, then the blends (as PointTaps::gather forms them).
+// One round trip for the coordinates and one for the data per KB samples instead of per sample.
+template <typename T, int INTERP, int PC, int KB>
+__device__ __forceinline__ void gather_sample_batch(const T* __restrict__ base, size_t stride,
+                                                    int np, const T* __restrict__ pixel_coords,
+                                                    int k0, int K, int H, int W,
+                                                    T (&v)[KB][PC]) {
+  constexpr int N = PointTaps<T, INTERP>::N;
+  T cx[KB], cy[KB];
+#pragma unroll
+  for (int g = 0; g < KB; ++g) {
+    const int k = min(k0 + g, K - 1);
+    cx[g] = pixel_coords[2 * k];
+    cy[g] = pixel_coords[2 * k + 1];
+  }
+  PointTaps<T, INTERP> t[KB];
+  T raw[KB][PC][N];
+#pragma unroll
+  for (int g = 0; g < KB; ++g) {
+    t[g].set(cx[g], cy[g], H, W);
+#pragma unroll
+    for (int j = 0; j < PC; ++j) t[g].load(base + (size_t)(j < np ? j : 0) * stride, raw[g][j]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int g = 0; g < KB; ++g)
+#pragma unroll
+    for (int j = 0; j < PC; ++j) v[g][j] = j < np ? t[g].blend(raw[g][j]) : T(0);
+}
+
 // ---------------------------------------------------------------------------
 // mapped max pool.  Body: common/mapped_max_pool.h:13-57, :81-133 (device
 // branch: running maximum starts at -FLT_MAX for every T, index at -1).
@@ -550,17 +582,38 @@ __global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
     best[j] = T(-FLT_MAX);
     best_k[j] = -1;
   }
-  for (int k = 0; k < K; ++k) {
-    const size_t s = ((size_t)pix * K + k) * q;
-    T v[kPC];
-    gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
-                                            WEIGHTED ? wts + s : nullptr, P, H, W, v);
+  if constexpr (!WEIGHTED) {
+    // samples in batches whose reads are in flight together
+    constexpr int KB = INTERP == 0 ? 3 : 2;
+    const T* coords = map + (size_t)pix * K * 2;
+    for (int k0 = 0; k0 < K; k0 += KB) {
+      T v[KB][kPC];
+      gather_sample_batch<T, INTERP, kPC, KB>(in + (size_t)plane0 * HW, HW, np, coords, k0, K, H,
+                                              W, v);
 #pragma unroll
-    for (int j = 0; j < kPC; ++j)
-      if (v[j] > best[j]) {  // strict: first maximum wins, NaN never wins
-        best[j] = v[j];
-        best_k[j] = k;
-      }
+      for (int g = 0; g < KB; ++g)
+        if (k0 + g < K) {
+#pragma unroll
+          for (int j = 0; j < kPC; ++j)
+            if (v[g][j] > best[j]) {  // strict: first maximum wins, NaN never wins
+              best[j] = v[g][j];
+              best_k[j] = k0 + g;
+            }
+        }
+    }
+  } else {
+    for (int k = 0; k < K; ++k) {
+      const size_t s = ((size_t)pix * K + k) * q;
+      T v[kPC];
+      gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                              WEIGHTED ? wts + s : nullptr, P, H, W, v);
+#pragma unroll
+      for (int j = 0; j < kPC; ++j)
+        if (v[j] > best[j]) {  // strict: first maximum wins, NaN never wins
+          best[j] = v[j];
+          best_k[j] = k;
+        }
+    }
   }
 #pragma unroll
   for (int j = 0; j < kPC; ++j)
@@ -588,13 +641,29 @@ __global__ __launch_bounds__(kBlock) void mapped_avg_pool_kernel(
   T sum[kPC];
 #pragma unroll
   for (int j = 0; j < kPC; ++j) sum[j] = T(0);
-  for (int k = 0; k < K; ++k) {
-    const size_t s = ((size_t)pix * K + k) * q;
-    T v[kPC];
-    gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
-                                            WEIGHTED ? wts + s : nullptr, P, H, W, v);
+  if constexpr (!WEIGHTED) {
+    constexpr int KB = INTERP == 0 ? 3 : 2;
+    const T* coords = map + (size_t)pix * K * 2;
+    for (int k0 = 0; k0 < K; k0 += KB) {
+      T v[KB][kPC];
+      gather_sample_batch<T, INTERP, kPC, KB>(in + (size_t)plane0 * HW, HW, np, coords, k0, K, H,
+                                              W, v);
 #pragma unroll
-    for (int j = 0; j < kPC; ++j) sum[j] += v[j];
+      for (int g = 0; g < KB; ++g)
+        if (k0 + g < K) {
+#pragma unroll
+          for (int j = 0; j < kPC; ++j) sum[j] += v[g][j];
+        }
+    }
+  } else {
+    for (int k = 0; k < K; ++k) {
+      const size_t s = ((size_t)pix * K + k) * q;
+      T v[kPC];
+      gather_sample<T, INTERP, WEIGHTED, kPC>(in + (size_t)plane0 * HW, HW, np, map + s * 2,
+                                              WEIGHTED ? wts + s : nullptr, P, H, W, v);
+#pragma unroll
+      for (int j = 0; j < kPC; ++j) sum[j] += v[j];
+    }
   }
 #pragma unroll
   for (int j = 0; j < kPC; ++j)
