@@ -581,30 +581,6 @@ int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const v
     out_channels, int64_t out_height, int64_t out_width, int64_t kernel_size, int32_t
     num_interp_pts, int32_t interp, int32_t dtype, int32_t compute, sdk_stream_t stream);
 
-/* Pooling with a kept plan.  `plan` is what sdk_mapped_conv_plan_build wrote for this map
- * (sample_map [out_height, out_width, kernel_size, 2], num_interp_pts = 0) and this image size;
- * plan_bytes = sdk_mapped_conv_plan_bytes(height, width, out_height, out_width, kernel_size, 0,
- * interp, dtype).  The pixel tiles whose taps lie inside an LDS-sized window of the image pool
- * from that window (one coalesced read of every input element per tile instead of one gather
- * per sample), the others as in the plain entry points; values and indices are identical to
- * theirs (sums in the same order; only the sign of a zero may differ for interpolated samples).
- * Weighted maps (num_interp_pts > 0), float64, a NULL plan and geometries without a plan run
- * the plain entry point.  The reference has no counterpart
- * (ext_modules/include/layers/mapped_max_pooling_layer.h:42-62 is stateless). */
-int sdk_mapped_max_pool_planned(const void* input, const void* sample_map,
-                                const void* interp_weights, void* out, int64_t* indices,
-                                const void* plan, size_t plan_bytes, int64_t batch,
-                                int64_t channels, int64_t height, int64_t width,
-                                int64_t out_height, int64_t out_width, int64_t kernel_size,
-                                int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                                sdk_stream_t stream);
-int sdk_mapped_avg_pool_planned(const void* input, const void* sample_map,
-                                const void* interp_weights, void* out, const void* plan,
-                                size_t plan_bytes, int64_t batch, int64_t channels,
-                                int64_t height, int64_t width, int64_t out_height,
-                                int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
-                                int32_t interp, int32_t dtype, sdk_stream_t stream);
-
 /* ------------------------------------------------------------------------- *
  * Plans of the scatter direction.  The optional workspaces of
  * sdk_resample_to_map / sdk_resample_to_map_normalized, sdk_mapped_avg_unpool

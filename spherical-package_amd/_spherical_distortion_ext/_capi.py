@@ -56,8 +56,6 @@ SIGNATURES = {
     "sdk_mapped_transposed_conv_backward_input_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
     "sdk_mapped_transposed_conv_backward_weight_planned": [_vp] * 6 + [_sz, _vp, _sz] + _CONV_DIMS,
     "sdk_mapped_conv_plan_build": [_vp] * 3 + [_sz] + [_i64] * 5 + [_i32] * 3 + [_vp],
-    "sdk_mapped_max_pool_planned": [_vp] * 6 + [_sz] + [_i64] * 7 + [_i32] * 3 + [_vp],
-    "sdk_mapped_avg_pool_planned": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 3 + [_vp],
     # plans of the scatter direction
     "sdk_resample_to_map_plan_build": [_vp] * 3 + [_sz] + [_i64] * 5 + [_i32] * 3 + [_vp],
     "sdk_resample_plan_complete": [_vp, _sz, _vp, _vp],

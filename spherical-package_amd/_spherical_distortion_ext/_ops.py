@@ -347,12 +347,6 @@ def mapped_max_pool(x, sample_map, interp_weights, kernel_size, interp):
     out = torch.empty((B, C, OH, OW), dtype=x.dtype, device=x.device)
     idx = torch.empty((B, C, OH, OW), dtype=torch.int64, device=x.device)
     with torch.cuda.device(x.device):
-        plan, nplan = (None, 0) if P else _conv_plan(x, sample_map, None, H, W, K, 0, int(interp))
-        if plan is not None:
-            _capi.call("sdk_mapped_max_pool_planned", _ptr(x), _ptr(sample_map), _ptr(None),
-                       _ptr(out), _ptr(idx), _ptr(plan), nplan, B, C, H, W, OH, OW, K, 0,
-                       int(interp), _DTYPES[x.dtype], _stream(x))
-            return out, idx
         _capi.call("sdk_mapped_max_pool", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
                    _ptr(out), _ptr(idx), B, C, H, W, OH, OW, K, P, int(interp),
                    _DTYPES[x.dtype], _stream(x))
@@ -424,12 +418,6 @@ def mapped_avg_pool(x, sample_map, interp_weights, kernel_size, interp):
                            % (int(kernel_size), tuple(sample_map.shape)))
     out = torch.empty((B, C, OH, OW), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
-        plan, nplan = (None, 0) if P else _conv_plan(x, sample_map, None, H, W, K, 0, int(interp))
-        if plan is not None:
-            _capi.call("sdk_mapped_avg_pool_planned", _ptr(x), _ptr(sample_map), _ptr(None),
-                       _ptr(out), _ptr(plan), nplan, B, C, H, W, OH, OW, K, 0, int(interp),
-                       _DTYPES[x.dtype], _stream(x))
-            return out
         _capi.call("sdk_mapped_avg_pool", _ptr(x), _ptr(sample_map), _ptr(interp_weights),
                    _ptr(out), B, C, H, W, OH, OW, K, P, int(interp), _DTYPES[x.dtype], _stream(x))
     return out

@@ -15,8 +15,6 @@
 #include <cfloat>
 #include <climits>
 
-#include "conv_fused.hpp"
-#include "pool_window.hpp"
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
 
@@ -530,20 +528,6 @@ __global__ __launch_bounds__(kBlock) void mapped_col2im_kernel(
   }
 }
 
-// The pixel of this thread when a launch covers a device-side list of 128-pixel tiles of the
-// tiling pt (two tiles per workgroup of kBlock threads), or -1.
-__device__ __forceinline__ int listed_pixel(const PixelTiling& pt,
-                                            const int* __restrict__ tile_list,
-                                            const int* __restrict__ tile_count) {
-  static_assert(kBlock == 256, "two 128-pixel tiles per workgroup");
-  const int slot = blockIdx.x * 2 + (threadIdx.x >> 7);
-  if (slot >= *tile_count) return -1;
-  const int t = tile_list[slot], pl = threadIdx.x & 127;
-  const int oy = (t / pt.tiles_x) * pt.TY() + (pl >> pt.tx_shift);
-  const int ox = ((t % pt.tiles_x) << pt.tx_shift) + (pl & (pt.TX() - 1));
-  return (oy < pt.OH && ox < pt.OW) ? oy * pt.OW + ox : -1;
-}
-
 // Values of KB consecutive samples (first: k0; samples past K repeat the last) of one pixel of
 // an unweighted map for PC planes, v[g][j]: the coordinates of all KB samples are read
 // together, then all taps of all planes, then the blends (as PointTaps::gather forms them).
@@ -584,11 +568,9 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
     T* __restrict__ out, int64_t* __restrict__ idx, int planes, int H, int W, int M, int K,
-    int P, PixelTiling pt, const int* __restrict__ tile_list,
-    const int* __restrict__ tile_count) {
-  const int pix = tile_list != nullptr ? listed_pixel(pt, tile_list, tile_count)
-                                       : banded_pixel_block() * kBlock + threadIdx.x;
-  if (pix < 0 || pix >= M) return;
+    int P) {
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
+  if (pix >= M) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
   const size_t HW = (size_t)H * W;
@@ -649,11 +631,9 @@ __global__ __launch_bounds__(kBlock) void mapped_max_pool_kernel(
 template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void mapped_avg_pool_kernel(
     const T* __restrict__ in, const T* __restrict__ map, const T* __restrict__ wts,
-    T* __restrict__ out, int planes, int H, int W, int M, int K, int P, PixelTiling pt,
-    const int* __restrict__ tile_list, const int* __restrict__ tile_count) {
-  const int pix = tile_list != nullptr ? listed_pixel(pt, tile_list, tile_count)
-                                       : banded_pixel_block() * kBlock + threadIdx.x;
-  if (pix < 0 || pix >= M) return;
+    T* __restrict__ out, int planes, int H, int W, int M, int K, int P) {
+  const int pix = banded_pixel_block() * kBlock + threadIdx.x;
+  if (pix >= M) return;
   const int plane0 = blockIdx.y * kPC;
   const int np = min(kPC, planes - plane0);
   const size_t HW = (size_t)H * W;
@@ -1625,8 +1605,7 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
                                               (const T*)input, (const T*)sample_map,
                                               (const T*)interp_weights, (T*)out, indices,
                                               (int)planes, (int)height, (int)width, (int)M,
-                                              (int)kernel_size, num_interp_pts, PixelTiling(),
-                                              (const int*)nullptr, (const int*)nullptr))));
+                                              (int)kernel_size, num_interp_pts))));
   SDK_LAUNCH_CHECK("mapped_max_pool");
   return SDK_OK;
 }
@@ -1651,8 +1630,7 @@ int sdk_mapped_avg_pool(const void* input, const void* sample_map, const void* i
                                   dim3(kBlock), (hipStream_t)stream, (const T*)input,
                                   (const T*)sample_map, (const T*)interp_weights, (T*)out,
                                   (int)planes, (int)height, (int)width, (int)M, (int)kernel_size,
-                                  num_interp_pts, PixelTiling(), (const int*)nullptr,
-                                  (const int*)nullptr))));
+                                  num_interp_pts))));
   SDK_LAUNCH_CHECK("mapped_avg_pool");
   return SDK_OK;
 }
@@ -1923,118 +1901,6 @@ int sdk_mapped_max_unpool_planned(const void* grad_output, const int64_t* indice
                                 (int)height, (int)width, (int)out_height, (int)out_width,
                                 (int)kernel_size, num_interp_pts, interp, (hipStream_t)stream,
                                 true));
-}
-
-// ---------------------------------------------------------------------------
-// Pooling with a kept plan (sdk_mapped_conv_plan_build for the same map and image size): the
-// tiles whose taps stay inside their window pool from LDS (pool_window.hip), the others in the
-// per-pixel kernel over their list.  Weighted maps and float64 run the plain entry point.
-// ---------------------------------------------------------------------------
-static int pool_plan(const void* plan, size_t plan_bytes, int64_t height, int64_t width,
-                     int64_t out_height, int64_t out_width, int64_t kernel_size, int32_t interp,
-                     const char* what, CachedPlan* cp, bool* usable) {
-  ConvGeom g{};
-  g.B = 1;
-  g.Cg = g.Cp = 1;
-  g.H = (int)height;
-  g.W = (int)width;
-  g.M = (int)(out_height * out_width);
-  g.OW = (int)out_width;
-  g.K = (int)kernel_size;
-  g.P = 0;
-  g.interp = (interp == 1 || interp == 2) ? interp : 0;
-  const size_t need = cached_plan_bytes(g);
-  *usable = need != 0;
-  if (need == 0) return SDK_OK;
-  if (plan_bytes != need)
-    return fail(SDK_ERR_WORKSPACE, "%s: plan of %zu bytes, this geometry has %zu", what,
-                plan_bytes, need);
-  load_cached_plan(g, const_cast<void*>(plan), cp);
-  return SDK_OK;
-}
-
-int sdk_mapped_max_pool_planned(const void* input, const void* sample_map,
-                                const void* interp_weights, void* out, int64_t* indices,
-                                const void* plan, size_t plan_bytes, int64_t batch,
-                                int64_t channels, int64_t height, int64_t width,
-                                int64_t out_height, int64_t out_width, int64_t kernel_size,
-                                int32_t num_interp_pts, int32_t interp, int32_t dtype,
-                                sdk_stream_t stream) {
-  if (plan == nullptr || num_interp_pts != 0 || dtype != SDK_F32)
-    return sdk_mapped_max_pool(input, sample_map, interp_weights, out, indices, batch, channels,
-                               height, width, out_height, out_width, kernel_size,
-                               num_interp_pts, interp, dtype, stream);
-  SDK_REQUIRE(indices, "mapped_max_pool_planned: NULL indices");
-  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_pool_planned: bad output size");
-  const int64_t M = out_height * out_width;
-  int rc = check_mapped(input, sample_map, interp_weights, out, batch, channels, height, width, M,
-                        kernel_size, num_interp_pts, "mapped_max_pool_planned");
-  if (rc) return rc;
-  CachedPlan cp;
-  bool usable = false;
-  rc = pool_plan(plan, plan_bytes, height, width, out_height, out_width, kernel_size, interp,
-                 "mapped_max_pool_planned", &cp, &usable);
-  if (rc) return rc;
-  if (!usable)
-    return sdk_mapped_max_pool(input, sample_map, interp_weights, out, indices, batch, channels,
-                               height, width, out_height, out_width, kernel_size,
-                               num_interp_pts, interp, dtype, stream);
-  const int64_t planes = batch * channels;
-  if (planes == 0) return SDK_OK;
-  rc = window_pool((const float*)input, cp.plan, cp.lists, (float*)out, indices, planes,
-                   (int)height, (int)width, (int)kernel_size, (hipStream_t)stream);
-  if (rc) return rc;
-  const dim3 grid((unsigned)((cp.plan.tiles + 1) / 2), (unsigned)ceil_div(planes, kPC));
-  using T = float;
-  SDK_DISPATCH_INTERP(interp, 0,
-                      (launch((mapped_max_pool_kernel<T, INTERP, WEIGHTED>), grid, dim3(kBlock),
-                              (hipStream_t)stream, (const T*)input, (const T*)sample_map,
-                              (const T*)nullptr, (T*)out, indices, (int)planes, (int)height,
-                              (int)width, (int)M, (int)kernel_size, 0, cp.plan.pt,
-                              (const int*)cp.lists.rest, (const int*)(cp.lists.count + 1))));
-  SDK_LAUNCH_CHECK("mapped_max_pool_planned");
-  return SDK_OK;
-}
-
-int sdk_mapped_avg_pool_planned(const void* input, const void* sample_map,
-                                const void* interp_weights, void* out, const void* plan,
-                                size_t plan_bytes, int64_t batch, int64_t channels,
-                                int64_t height, int64_t width, int64_t out_height,
-                                int64_t out_width, int64_t kernel_size, int32_t num_interp_pts,
-                                int32_t interp, int32_t dtype, sdk_stream_t stream) {
-  if (plan == nullptr || num_interp_pts != 0 || dtype != SDK_F32)
-    return sdk_mapped_avg_pool(input, sample_map, interp_weights, out, batch, channels, height,
-                               width, out_height, out_width, kernel_size, num_interp_pts, interp,
-                               dtype, stream);
-  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_avg_pool_planned: bad output size");
-  const int64_t M = out_height * out_width;
-  int rc = check_mapped(input, sample_map, interp_weights, out, batch, channels, height, width, M,
-                        kernel_size, num_interp_pts, "mapped_avg_pool_planned");
-  if (rc) return rc;
-  CachedPlan cp;
-  bool usable = false;
-  rc = pool_plan(plan, plan_bytes, height, width, out_height, out_width, kernel_size, interp,
-                 "mapped_avg_pool_planned", &cp, &usable);
-  if (rc) return rc;
-  if (!usable)
-    return sdk_mapped_avg_pool(input, sample_map, interp_weights, out, batch, channels, height,
-                               width, out_height, out_width, kernel_size, num_interp_pts, interp,
-                               dtype, stream);
-  const int64_t planes = batch * channels;
-  if (planes == 0) return SDK_OK;
-  rc = window_pool((const float*)input, cp.plan, cp.lists, (float*)out, nullptr, planes,
-                   (int)height, (int)width, (int)kernel_size, (hipStream_t)stream);
-  if (rc) return rc;
-  const dim3 grid((unsigned)((cp.plan.tiles + 1) / 2), (unsigned)ceil_div(planes, kPC));
-  using T = float;
-  SDK_DISPATCH_INTERP(interp, 0,
-                      (launch((mapped_avg_pool_kernel<T, INTERP, WEIGHTED>), grid, dim3(kBlock),
-                              (hipStream_t)stream, (const T*)input, (const T*)sample_map,
-                              (const T*)nullptr, (T*)out, (int)planes, (int)height, (int)width,
-                              (int)M, (int)kernel_size, 0, cp.plan.pt,
-                              (const int*)cp.lists.rest, (const int*)(cp.lists.count + 1))));
-  SDK_LAUNCH_CHECK("mapped_avg_pool_planned");
-  return SDK_OK;
 }
 
 }  // extern "C"
