@@ -39,6 +39,25 @@ def _case(seed, Cin, Cout, H, W, OH, OW, K, P, interp, kind):
         sel = rng.uniform(size=cx.shape) < 0.2
         cx = np.where(sel, 5.3, cx)
         cy = np.where(sel, 4.1, cy)
+    if kind == "listed":
+        # One-row image, nearest, K = 3: the taps of a tile of 128 pixels are far apart (no box
+        # fits) and touch exactly 288 distinct elements in the first tile (a listed window, full
+        # to the last element), 289 in the second (one too many: the listed rest) and 128 + 128 +
+        # 128 = 384 in the third; the fourth names sixteen elements eight times each.
+        assert OH == 1 and K == 3 and P == 0
+        p = np.arange(OW)
+        t, q = p // 128, p % 128
+        third = np.select([t == 0, t == 1, t == 2], [q % 32, q % 33, q], q % 16)
+        cx = np.stack([q + 1000.0 * t, 300.0 + q + 1000.0 * t, 600.0 + third + 1000.0 * t], -1)
+        cx = cx.reshape(1, OW, 3) % W
+        cy = np.zeros_like(cx)
+        m = np.ascontiguousarray(np.stack([cx, cy], -1).astype(np.float32))
+        x = rng.standard_normal((2, Cin, H, W)).astype(np.float32)
+        w = (rng.standard_normal((Cout, Cin, K)) / np.sqrt(Cin * K)).astype(np.float32)
+        b = rng.standard_normal(Cout).astype(np.float32)
+        g = rng.standard_normal((2, Cout, OH, OW)).astype(np.float32)
+        bt = rng.standard_normal(Cin).astype(np.float32)
+        return m, None, x, w, b, g, bt
     if P:
         cx = cx[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
         cy = cy[..., None] + rng.uniform(-1, 1, (OH, OW, K, P))
@@ -62,6 +81,8 @@ CASES = [
     (72, 72, 20, 36, 20, 36, 6, 0, 0, "crowded"),    # inverse lists overflow: scatter fallback
     (130, 40, 27, 42, 24, 42, 10, 0, 2, "plain"),    # 12 tiles (not a multiple of 8), K = 10
     (16, 24, 30, 50, 30, 50, 7, 0, 1, "plain"),      # narrow layers: kernels that ignore the plan
+    (72, 80, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # listed windows: 288 (fits), 289, 384 elements
+    (40, 48, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # ... in the 64-channel kernels
 ]
 
 
