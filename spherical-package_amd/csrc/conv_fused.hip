@@ -752,9 +752,17 @@ static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const fl
     if (lists4 != nullptr) tl = *lists4;
     else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
     if (rc) return rc;
-    rc = window_wgrad(g, plan, tl, pix, img, gW, reinterpret_cast<float*>(base + t.window_partial),
-                      stream);
+    float* wp = reinterpret_cast<float*>(base + t.window_partial);
+    rc = window_wgrad(g, plan, tl, pix, img, gW, wp, stream);
     if (rc) return rc;
+    if (plan.big_lut != nullptr) {
+      // big tiles from their big windows (the partial sums of the first launch have been added
+      // up by then), what is left from global memory
+      rc = window_wgrad(g, plan, tl, pix, img, gW, wp, stream, true);
+      if (rc) return rc;
+      return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream,
+                           tl.rest_small, tl.count + 3);
+    }
     return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream, tl.rest,
                          tl.count + 1);
   }
@@ -819,6 +827,15 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
     rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
                      reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream);
     if (rc) return rc;
+    // big tiles from their big windows; the rest list below is then what neither kernel took
+    const bool with_big = plan.big_lut != nullptr;
+    if (with_big) {
+      rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
+                       reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream, true);
+      if (rc) return rc;
+    }
+    const int* rest_list = with_big ? tl.rest_small : tl.rest;
+    const int* rest_count = with_big ? tl.count + 3 : tl.count + 1;
     // the listed rest: 128 x 128 tiles, or 64 channels x two listed tiles for narrow layers
     const int units = (int)ceil_div(plan.tiles, TM / 128);
     const dim3 grid_t((unsigned)((units + 7) / 8 * 8 * (CpP / TN)), (unsigned)g.B);
@@ -831,7 +848,7 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
                                         g.M, g.K, g.P, CgP, CpP, slots, plan.tiles,               \
                                         (const int*)nullptr, (const float*)nullptr,               \
                                         (const int*)nullptr, (const int*)nullptr, plan.pt,        \
-                                        tl.rest, tl.count + 1)))
+                                        rest_list, rest_count)))
 #define GT(BFv)                                                  \
   do {                                                           \
     if (narrow) GT2(64, 256, BFv); else GT2(128, 128, BFv);      \
@@ -1097,6 +1114,15 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
         rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
                          reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream);
         if (rc) return rc;
+        const bool with_big = ip.plan.big_lut != nullptr;
+        if (with_big) {
+          rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
+                           reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream,
+                           true);
+          if (rc) return rc;
+        }
+        const int* rest_list = with_big ? tl.rest_small : tl.rest;
+        const int* rest_count = with_big ? tl.count + 3 : tl.count + 1;
         float* gw = reinterpret_cast<float*>(inv_ws + l.gather_weights);
         // the listed rest: 128 x 128 tiles, or 64 channels x two listed tiles for narrow images
         const bool narrow = g.Cg <= 64;
@@ -1113,7 +1139,7 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                    pix, (const float*)nullptr, (const float*)nullptr, (const float*)gw, bias,    \
                    img, g.Cp, 1, g.M, g.Cg, g.H * g.W, g.K, 0, CinP, CoutP, kInversePlanRows,    \
                    ip.plan.tiles, (const int*)ip.raw_off, (const float*)ip.raw_co,               \
-                   (const int*)ip.plan.ns, (const int*)ip.gate, ip.plan.pt, tl.rest, tl.count + 1)
+                   (const int*)ip.plan.ns, (const int*)ip.gate, ip.plan.pt, rest_list, rest_count)
 #define IT(BFv)                                                  \
   do {                                                           \
     if (narrow) IT2(64, 256, BFv); else IT2(128, 128, BFv);      \

@@ -26,7 +26,7 @@ template <int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     const float* __restrict__ map, const float* __restrict__ wts, PixelTiling pt, int K, int P,
     int H, int W, int S, int* __restrict__ hdr, int* __restrict__ ns_out,
-    int2* __restrict__ taps, const int* __restrict__ gate) {
+    int2* __restrict__ taps, const int* __restrict__ gate, int* __restrict__ big_lut) {
   if (gate != nullptr && *gate == 0) return;
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
@@ -132,6 +132,7 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
   // the window is the whole bounding box of the taps unless that exceeded the capacity
   bool whole = bb[0] > bb[1] || (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, W) <= kRegionCap;
   int listed = -1;   // >= 0: elements of a listed window
+  int big = -1;      // >= 0: elements of the tile's big window
   if (!whole) {
     // the distinct elements the tile touches may still fit: try a listed window
     set_clear(wset);
@@ -149,8 +150,9 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
       }
     }
     __syncthreads();
-    listed = set_finish(wset);
-    if (listed >= 0) {
+    const int distinct = set_finish(wset);
+    if (distinct >= 0 && distinct <= kRegionCap) {
+      listed = distinct;
       rg.ry0 = 0;
       rg.rx0 = 0;
       rg.RH = 1;
@@ -158,6 +160,8 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
       rg.RS = listed;
       rg.RSp = listed | 1;
       whole = true;
+    } else if (distinct > kRegionCap && big_lut != nullptr) {
+      big = distinct;   // too many for a window, few enough for a big one
     }
   }
   int* tile_hdr = hdr + (size_t)tile * kHdrStride;
@@ -171,12 +175,21 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
     for (int k = 0; k < K; ++k) most = max(most, ns_l[k]);
     tile_hdr[5] = most;   // the longest row list of the tile's samples
     tile_hdr[6] = listed >= 0 ? 1 : 0;
-    tile_hdr[7] = 0;
+    tile_hdr[7] = big >= 0 ? 1 : 0;
   }
   if (listed >= 0) {
     for (int e = tid; e < listed; e += kPlThreads) tile_hdr[kHdrLut + e] = wset.list[e];
   } else {
     write_region_lut(rg, H, W, tile_hdr + kHdrLut);
+  }
+  if (big >= 0) {
+    int* bl = big_lut + (size_t)tile * kBigStride;
+    if (tid == 0) bl[0] = big;
+    for (int e = tid; e < big; e += kPlThreads) {
+      const int off = wset.list[e], y = off / W;
+      bl[kBigLut + e] = off;
+      bl[kBigLut + kBigCap + e] = rg.encode(y, off - y * W, W);
+    }
   }
   for (int k = tid; k < K; k += kPlThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
 
@@ -192,8 +205,9 @@ __global__ __launch_bounds__(kPlThreads) void plan_kernel(
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
           if (t.w[i] != 0.0f) {
-            const int at = listed >= 0 ? set_rank(wset, listed, t.y[i] * W + t.x[i])
-                                       : rg.encode(t.y[i], t.x[i], W);
+            const int off = t.y[i] * W + t.x[i];
+            const int at = listed >= 0 ? set_rank(wset, listed, off)
+                           : (big >= 0 ? set_rank(wset, big, off) : rg.encode(t.y[i], t.x[i], W));
             row[(size_t)cnt * 128] = make_int2(at, __float_as_int(t.w[i]));
             ++cnt;
           }
@@ -255,7 +269,8 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     const int* __restrict__ ns, const int2* __restrict__ taps, float* __restrict__ gW,
     float* __restrict__ partial, int Cg, int H, int W, int Cp, int K, int S, PixelTiling pt,
     int tiles, int groups, int batches, int c_chunks, int n_tiles, int kblocks, int vec4,
-    const int* __restrict__ tile_list, const int* __restrict__ tile_count) {
+    const int* __restrict__ tile_list, const int* __restrict__ tile_count,
+    const int* __restrict__ big_lut) {
   constexpr bool BF16 = MM != kMmF32;     // operands enter the matrix unit as bf16 fragments
   constexpr bool SPLIT = MM == kMmSplit;  // ... three per operand, whose sum is the float
   __shared__ __align__(16) float region[kRegionCap * kRegE];
@@ -330,6 +345,9 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
     rg.RSp = rg.RS;
     // plan rows of this tile and sample block: uniform base, 32-bit lane offsets
     const char* tile_taps = reinterpret_cast<const char*>(taps + ((size_t)tile * K + k0) * S * 128);
+    // a big tile is taken like any other tile outside its window: its rows name ranks
+    const bool big_tile = big_lut != nullptr && hdr[tile * kHdrStride + 7] != 0;
+    const int* big_l = big_lut + (big_tile ? (size_t)tile * kBigStride : 0);
 
     __syncthreads();  // every wave is done with the previous tile's window, rows and column tiles
     if (tid < kcount) ns_l[tid] = ns[(size_t)tile * K + k0 + tid];
@@ -422,7 +440,9 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
             const int r = i >> 6, p = i & 63;
             while (r - r0 >= ns_l[kk]) r0 += ns_l[kk++];
             const char* row = tile_taps + (size_t)(kk * S + (r - r0)) * (128 * sizeof(int2));
-            prow[i] = *reinterpret_cast<const int2*>(row + (unsigned)(half * 64 + p) * (unsigned)sizeof(int2));
+            int2 ec = *reinterpret_cast<const int2*>(row + (unsigned)(half * 64 + p) * (unsigned)sizeof(int2));
+            if (__int_as_float(ec.y) != 0.0f) ec.x = plan_row_at(ec.x, big_tile, big_l);
+            prow[i] = ec;
           }
         }
         __syncthreads();
@@ -744,34 +764,48 @@ bool plan_supported(const ConvGeom& g) {
 
 static size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 
-size_t plan_bytes(const ConvGeom& g) {
+namespace {
+// [header][rows per sample][plan rows][big windows]
+struct PlanOffsets {
+  size_t ns, taps, big_lut, total;
+};
+PlanOffsets plan_offsets(const ConvGeom& g) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
-  return align16(tiles * kHdrStride * sizeof(int)) + align16(tiles * g.K * sizeof(int)) +
-         tiles * g.K * plan_slots(g) * 128 * sizeof(int2);
+  PlanOffsets o;
+  o.ns = align16(tiles * kHdrStride * sizeof(int));
+  o.taps = o.ns + align16(tiles * g.K * sizeof(int));
+  o.big_lut = o.taps + tiles * g.K * plan_slots(g) * 128 * sizeof(int2);
+  o.total = o.big_lut + align16(tiles * kBigStride * sizeof(int));
+  return o;
 }
+}  // namespace
+
+size_t plan_bytes(const ConvGeom& g) { return plan_offsets(g).total; }
 
 void load_plan(const ConvGeom& g, void* workspace, Plan* plan) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  const size_t tiles = (size_t)pt.tiles_x * pt.tiles_y;
+  const PlanOffsets o = plan_offsets(g);
   char* base = static_cast<char*>(workspace);
   plan->pt = pt;
-  plan->tiles = (int)tiles;
+  plan->tiles = pt.tiles_x * pt.tiles_y;
   plan->S = plan_slots(g);
   plan->hdr = reinterpret_cast<int*>(base);
-  plan->ns = reinterpret_cast<int*>(base + align16(tiles * kHdrStride * sizeof(int)));
-  plan->taps = reinterpret_cast<int2*>(base + align16(tiles * kHdrStride * sizeof(int)) +
-                                       align16(tiles * g.K * sizeof(int)));
+  plan->ns = reinterpret_cast<int*>(base + o.ns);
+  plan->taps = reinterpret_cast<int2*>(base + o.taps);
+  plan->big_lut = reinterpret_cast<int*>(base + o.big_lut);
 }
 
 int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-               hipStream_t stream, Plan* plan, const int* gate) {
+               hipStream_t stream, Plan* plan, const int* gate, bool with_big) {
   load_plan(g, workspace, plan);
+  if (!with_big) plan->big_lut = nullptr;
   SDK_DISPATCH_INTERP(g.interp, g.P,
                       (launch(plan_kernel<INTERP, WEIGHTED>, dim3((unsigned)plan->tiles),
                               dim3(kPlThreads), stream, map, wts, plan->pt, g.K, g.P, g.H, g.W,
                               plan->S, const_cast<int*>(plan->hdr), const_cast<int*>(plan->ns),
-                              const_cast<int2*>(plan->taps), gate)));
+                              const_cast<int2*>(plan->taps), gate,
+                              const_cast<int*>(plan->big_lut))));
   SDK_LAUNCH_CHECK("plan");
   return SDK_OK;
 }
@@ -849,7 +883,8 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 #define PW3(KBv, BFv, NWv)                                                                      \
   launch(planned_wgrad_kernel<KBv, BFv, NWv, false>, grid, dim3(kPlThreads), stream, pix, img,         \
          plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
-         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
+         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count, \
+         plan.big_lut)
 #define PW(KBv, BFv)                                                                            \
   do {                                                                                          \
     if (NW == 4) PW3(KBv, BFv, 4); else if (NW == 2) PW3(KBv, BFv, 2); else PW3(KBv, BFv, 1);   \
@@ -862,7 +897,8 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 #define PR3(KBv, NWv)                                                                           \
   launch(planned_wgrad_kernel<KBv, kMmF32, NWv, true>, grid, dim3(kPlThreads), stream, pix, img, \
          plan.hdr, plan.ns, plan.taps, gW, partial, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, plan.pt, \
-         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count)
+         plan.tiles, groups, (int)g.B, c_chunks, n_tiles, kb_count, vec4, tile_list, tile_count, \
+         plan.big_lut)
     if (KB == 4) PR3(4, 4); else PR3(5, 4);   // K = 10 .. 16 -> two or more blocks of 4 or 5
 #undef PR3
   } else {

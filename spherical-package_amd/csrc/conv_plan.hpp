@@ -12,6 +12,7 @@
 //   h[4]             1 when every active tap of the tile lies inside that window
 //   h[5]             the largest ns of the tile's samples (plan_kernel only)
 //   h[6]             1 for a listed window
+//   h[7]             1 for a big tile (below)
 //   h[8 + e]         flat image offset of window element e (-1: outside the image)
 //   ns[t*K + k]      rows of kernel sample k: the largest number of active taps
 //                    any pixel of the tile has for that sample
@@ -22,6 +23,16 @@
 //                    .y: float bits of the coefficient (interpolation weight times
 //                    point weight); pixels with fewer taps are padded with 0.
 // S = points per sample * taps per point bounds the rows of one sample.
+//
+// Big tiles.  A tile whose taps fit no window (h[4] would be 0) but touch at most kBigCap
+// distinct elements is described a second way, for kernels that give a window most of a CU's
+// LDS: with bl = big_lut + kBigStride * t,
+//   bl[0]                  number of distinct elements
+//   bl[8 + e]              flat image offset of element e, ascending
+//   bl[8 + kBigCap + e]    what .x of a tap on element e would be in the ordinary encoding
+// and the .x of its rows in taps is the rank of the tap's element in that list.  h[0..6] and
+// the window LUT stay what they would be without this; a kernel that does not run big tiles
+// from a big window turns a rank back into the ordinary encoding with plan_row_at below.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -38,7 +49,15 @@ struct Plan {
   const int* hdr;
   const int* ns;
   const int2* taps;
+  const int* big_lut;   // nullptr: the plan has no big tiles
 };
+
+// The ordinary encoding (window index, or -(flat offset) - 1) of a plan row's .x for a kernel
+// that treats tile t as a tile outside its window: x itself unless t is a big tile.
+// big: h[7] != 0; bl: big_lut + kBigStride * t.
+__device__ __forceinline__ int plan_row_at(int x, bool big, const int* __restrict__ bl) {
+  return big ? bl[kBigLut + kBigCap + x] : x;
+}
 
 PixelTiling plan_tiling(int OH, int OW);
 bool plan_supported(const ConvGeom& g);
@@ -46,21 +65,25 @@ size_t plan_bytes(const ConvGeom& g);
 
 // Builds the plan of (g, map, wts) in `workspace` (plan_bytes(g) bytes, 16-byte aligned).
 // gate: optional device flag; with one, the plan is built only if *gate != 0 (its only reader
-// is gated the same way).
+// is gated the same way).  with_big = false: the plan has no big tiles (plan->big_lut = nullptr).
 int build_plan(const ConvGeom& g, const float* map, const float* wts, void* workspace,
-               hipStream_t stream, Plan* plan, const int* gate = nullptr);
+               hipStream_t stream, Plan* plan, const int* gate = nullptr, bool with_big = true);
 
 // gW = sum_b pix[b] x im2col(img[b])^T from a plan; gW must be zero on entry.
 // partial: planned_wgrad_partial_bytes(g) bytes (when that is not 0) in which the workgroups
 // leave their sums for a second, summing kernel; nullptr: they add to gW themselves.
-// The plan's tiles by class, on the device (conv_window_gemm.hip): those whose taps all lie
-// inside their window, in ascending order, and the others; count[0], count[1] entries.
+// The plan's tiles by class, on the device (conv_window_gemm.hip), each in ascending order:
+// those whose taps all lie inside their window and the others (count[0], count[1] entries);
+// the others again as big tiles and the remainder (count[2], count[3]).
 struct TileLists {
   const int* inside;
   const int* rest;
+  const int* big;
+  const int* rest_small;
   const int* count;
 };
-// max_rows > 0: tiles with a sample of more than max_rows plan rows (hdr[8t+5]) go to `rest`.
+// max_rows > 0: tiles with a sample of more than max_rows plan rows (h[5]) are neither inside
+// nor big.
 size_t tile_lists_bytes(const ConvGeom& g);
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
                      int max_rows = 0);
@@ -69,11 +92,13 @@ int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, Tile
 // g: the contraction's geometry (gather side = img).  swapped: Wm is [Cg, Cp * K] instead of
 // [Cp, Cg * K].  weights: window_gemm_weight_bytes(g) bytes of scratch for the re-laid-out
 // weight matrix.  gate (optional): the kernel runs only if *gate == 0.
+// big: the same on the tiles of tl.big, from their big windows; `weights` must hold what an
+// earlier call with big = false left there (same g, mm, Wm).
 bool window_gemm_supported(const ConvGeom& g);
 size_t window_gemm_weight_bytes(const ConvGeom& g);
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                 const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
-                float* weights, const int* gate, hipStream_t stream);
+                float* weights, const int* gate, hipStream_t stream, bool big = false);
 
 // The scatter of geometry g regrouped by target as a plan over tiles of the image grid, whose
 // windows lie in the pixel grid; valid only if *gate == 0 after it was built (a target with
@@ -107,7 +132,9 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 // rows per sample: build the lists with max_rows = 4).  partial: window_wgrad_partial_bytes(g).
 bool window_wgrad_supported(const ConvGeom& g, int mm);
 size_t window_wgrad_partial_bytes(const ConvGeom& g);
+// big: the sums over the tiles of tl.big, from their big windows.
 int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
-                 const float* img, float* gW, float* partial, hipStream_t stream);
+                 const float* img, float* gW, float* partial, hipStream_t stream,
+                 bool big = false);
 
 }  // namespace sdk

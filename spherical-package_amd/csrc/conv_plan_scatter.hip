@@ -86,7 +86,8 @@ template <int NS, bool BF16>
 __global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
     const float* __restrict__ pix, const int* __restrict__ hdr, const int* __restrict__ ns,
     const int2* __restrict__ taps, const float* __restrict__ Ws, float* __restrict__ img, int Cg,
-    int H, int W, int Cp, int K, int S, int chunks, PixelTiling pt, const int* __restrict__ gate) {
+    int H, int W, int Cp, int K, int S, int chunks, PixelTiling pt, const int* __restrict__ gate,
+    const int* __restrict__ big_lut) {
   if (gate != nullptr && *gate == 0) return;   // another kernel has done the work
   // window, channel pairs interleaved: value of (channel c, element e) at
   // region[((c / 2) * RSp + e) * 2 + c % 2], so two channels share an 8-byte word
@@ -117,9 +118,14 @@ __global__ __launch_bounds__(kStThreads, 2) void planned_gemm_scatter_kernel(
   for (int k = tid; k < K; k += kStThreads) ns_l[k] = ns[(size_t)tile * K + k];
   // plan rows of this tile: uniform base, 32-bit lane offsets
   const char* tile_taps = reinterpret_cast<const char*>(taps + (size_t)tile * K * S * 128);
+  // a big tile is taken like any other tile outside its window: its rows name ranks
+  const bool big_tile = big_lut != nullptr && hdr[tile * kHdrStride + 7] != 0;
+  const int* big_l = big_lut + (big_tile ? (size_t)tile * kBigStride : 0);
   auto plan_row = [&](int k, int r) -> int2 {
     const char* row = tile_taps + (size_t)(k * S + r) * (128 * sizeof(int2));
-    return *reinterpret_cast<const int2*>(row + (unsigned)p_local * (unsigned)sizeof(int2));
+    int2 ec = *reinterpret_cast<const int2*>(row + (unsigned)p_local * (unsigned)sizeof(int2));
+    if (__int_as_float(ec.y) != 0.0f) ec.x = plan_row_at(ec.x, big_tile, big_l);
+    return ec;
   };
 
   // pixel-side operand, resident in registers.  fp32: step s holds channel 2*s + half;
@@ -308,7 +314,8 @@ int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const f
   char* plan_ws = reinterpret_cast<char*>(workspace) + ((staged_workspace_bytes(g) + 255) & ~(size_t)255);
   // a plan that only this (gated) kernel reads is built under the same gate; one that is
   // handed on to the weight gradient is built in any case
-  int rc = build_plan(g, map, wts, plan_ws, stream, &plan, shared != nullptr ? nullptr : gate);
+  int rc = build_plan(g, map, wts, plan_ws, stream, &plan, shared != nullptr ? nullptr : gate,
+                      shared != nullptr);
   if (rc) return rc;
   if (shared != nullptr) {
     shared->plan = plan;
@@ -318,7 +325,7 @@ int planned_gemm_scatter(const ConvGeom& g, bool bf16, const float* pix, const f
 #define PS(NSv, BFv)                                                                             \
   launch(planned_gemm_scatter_kernel<NSv, BFv>, grid, dim3(kStThreads), stream, pix, plan.hdr,   \
          plan.ns, plan.taps, (const float*)workspace, img, g.Cg, g.H, g.W, g.Cp, g.K, plan.S,    \
-         chunks, plan.pt, gate)
+         chunks, plan.pt, gate, plan.big_lut)
   if (bf16) { if (NS == 64) PS(64, true); else if (NS == 32) PS(32, true); else PS(16, true); }
   else { if (NS == 64) PS(64, false); else if (NS == 32) PS(32, false); else PS(16, false); }
 #undef PS

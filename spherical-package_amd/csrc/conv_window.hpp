@@ -26,6 +26,12 @@ constexpr int kRegionCap = 288;  // region elements per channel (kCC * 289 * 4 B
 // image offset of window element e (-1: outside the image).
 constexpr int kHdrLut = 8;
 constexpr int kHdrStride = kHdrLut + kRegionCap;
+// A tile whose taps fit no window of kRegionCap elements but touch at most kBigCap distinct
+// ones gets, besides its ordinary plan rows, a second set over a listed window of that size
+// ("big" tile; conv_plan.hpp), for kernels that give the window most of a CU's LDS.
+constexpr int kBigCap = 768;
+constexpr int kBigLut = 8;                         // [0] elements, [kBigLut + e] flat offset,
+constexpr int kBigStride = kBigLut + 2 * kBigCap;  // [kBigLut + kBigCap + e] ordinary encoding
 
 // Up to four taps of one sample point as (row, column, coefficient).  A tap that
 // is out of range or has zero weight gets coefficient 0 (and row = column = 0).
@@ -170,15 +176,15 @@ __device__ __forceinline__ void load_region_lut(const int* __restrict__ tile_hdr
 // of a mesh, whose indices say little about distance) may still touch few distinct image
 // elements.  The kernels that build plans collect the tile's distinct offsets in an LDS hash
 // set; when there are at most kRegionCap, the sorted list becomes the window and a tap's
-// window index is its rank in it.
+// window index is its rank in it; up to kBigCap they make the window of a big tile.
 // ---------------------------------------------------------------------------
-constexpr int kSetSlots = 1024;  // hash slots (> kRegionCap + the threads that may insert at once)
-constexpr int kSetSort = 512;    // length of the padded sorted list (power of two >= kRegionCap)
+constexpr int kSetSlots = 2048;  // hash slots (> kBigCap + the threads that may insert at once)
+constexpr int kSetSort = 1024;   // length of the padded sorted list (power of two >= kBigCap)
 
 struct WindowSet {
   int table[kSetSlots];
   int list[kSetSort];
-  int count;   // distinct offsets claimed; inserting stops once it exceeds kRegionCap
+  int count;   // distinct offsets claimed; inserting stops once it exceeds kBigCap
   int filled;
 };
 
@@ -193,8 +199,8 @@ __device__ __forceinline__ void set_clear(WindowSet& ws) {
 }
 
 __device__ __forceinline__ void set_insert(WindowSet& ws, int off) {
-  if (*reinterpret_cast<volatile int*>(&ws.count) > kRegionCap) return;
-  unsigned h = ((unsigned)off * 2654435761u) >> 22;
+  if (*reinterpret_cast<volatile int*>(&ws.count) > kBigCap) return;
+  unsigned h = ((unsigned)off * 2654435761u) >> 21;
   for (int probe = 0; probe < kSetSlots; ++probe) {
     const int prev = atomicCAS(&ws.table[h], -1, off);
     if (prev == -1) {
@@ -207,18 +213,19 @@ __device__ __forceinline__ void set_insert(WindowSet& ws, int off) {
 }
 
 // All threads, after a barrier behind the last set_insert.  Returns the number of distinct
-// offsets when they fit a window (ws.list[0 .. n) is then sorted), otherwise -1.
+// offsets when there are at most kBigCap (ws.list[0 .. n) is then sorted), otherwise -1.
 __device__ __forceinline__ int set_finish(WindowSet& ws) {
   const int n = ws.count;
-  if (n > kRegionCap) return -1;
+  if (n > kBigCap) return -1;
+  const int len = n <= kSetSort / 2 ? kSetSort / 2 : kSetSort;   // (the padding sorts to the end)
   for (int i = threadIdx.x; i < kSetSlots; i += blockDim.x) {
     const int key = ws.table[i];
     if (key != -1) ws.list[atomicAdd(&ws.filled, 1)] = key;
   }
   __syncthreads();
-  for (int k = 2; k <= kSetSort; k <<= 1) {
+  for (int k = 2; k <= len; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int i = threadIdx.x; i < kSetSort; i += blockDim.x) {
+      for (int i = threadIdx.x; i < len; i += blockDim.x) {
         const int o = i ^ j;
         if (o > i) {
           const int a = ws.list[i], b = ws.list[o];

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kWgThreads) void inverse_fill_tiled_kernel(
 __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
     const int* __restrict__ cnt, int* __restrict__ raw_off, float* __restrict__ raw_co,
     PixelTiling it, int K, int OH, int OW, int* __restrict__ hdr, int* __restrict__ ns_out,
-    int2* __restrict__ taps, const int* __restrict__ gate) {
+    int2* __restrict__ taps, const int* __restrict__ gate, int* __restrict__ big_lut) {
   if (*gate != 0) return;
   __shared__ int bb[4];
   __shared__ int ns_l[kPlanKMax];
@@ -209,6 +209,7 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
   Region rg = choose_region(bb[0], bb[1], bb[2], bb[3], ay, ax, it.TY(), it.TX(), OW);
   bool whole = bb[0] > bb[1] || (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, OW) <= kRegionCap;
   int listed = -1;   // >= 0: elements of a listed window
+  int big = -1;      // >= 0: elements of the tile's big window
   if (!whole) {
     // the distinct sources of the tile may still fit: try a listed window
     set_clear(wset);
@@ -219,8 +220,9 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
       for (int a = 0; a < n; ++a) set_insert(wset, ro[a * 128]);
     }
     __syncthreads();
-    listed = set_finish(wset);
-    if (listed >= 0) {
+    const int distinct = set_finish(wset);
+    if (distinct >= 0 && distinct <= kRegionCap) {
+      listed = distinct;
       rg.ry0 = 0;
       rg.rx0 = 0;
       rg.RH = 1;
@@ -228,6 +230,8 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
       rg.RS = listed;
       rg.RSp = listed | 1;
       whole = true;
+    } else if (distinct > kRegionCap && big_lut != nullptr) {
+      big = distinct;   // too many for a window, few enough for a big one
     }
   }
   int* tile_hdr = hdr + (size_t)tile * kHdrStride;
@@ -241,12 +245,21 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
     for (int k = 0; k < K; ++k) most = max(most, ns_l[k]);
     tile_hdr[5] = most;
     tile_hdr[6] = listed >= 0 ? 1 : 0;
-    tile_hdr[7] = 0;
+    tile_hdr[7] = big >= 0 ? 1 : 0;
   }
   if (listed >= 0) {
     for (int e = tid; e < listed; e += kWgThreads) tile_hdr[kHdrLut + e] = wset.list[e];
   } else {
     write_region_lut(rg, OH, OW, tile_hdr + kHdrLut);
+  }
+  if (big >= 0) {
+    int* bl = big_lut + (size_t)tile * kBigStride;
+    if (tid == 0) bl[0] = big;
+    for (int e = tid; e < big; e += kWgThreads) {
+      const int off = wset.list[e], y = off / OW;
+      bl[kBigLut + e] = off;
+      bl[kBigLut + kBigCap + e] = rg.encode(y, off - y * OW, OW);
+    }
   }
   for (int k = tid; k < K; k += kWgThreads) ns_out[(size_t)tile * K + k] = ns_l[k];
   for (int k = kpar; k < K; k += 2) {
@@ -260,7 +273,8 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
       if (a < n) {
         const int mm = ro[a * 128];
         const int my = mm / OW, mx = mm - my * OW;
-        const int at = listed >= 0 ? set_rank(wset, listed, mm) : rg.encode(my, mx, OW);
+        const int at = listed >= 0 ? set_rank(wset, listed, mm)
+                       : (big >= 0 ? set_rank(wset, big, mm) : rg.encode(my, mx, OW));
         v = make_int2(at, __float_as_int(rc[a * 128]));
       }
       row[(size_t)a * 128] = v;
@@ -268,68 +282,74 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
   }
 }
 
-// Splits the plan's tiles into those whose taps all lie inside their window (header value 4 != 0)
-// and the rest, both in ascending tile order.  One workgroup.
-//   lists[0 .. tiles)         tiles inside their window, count[0] of them
-//   lists[tiles .. 2*tiles)   the others, count[1] of them
+// Splits the plan's tiles by class, each list in ascending tile order.  One workgroup.
+//   lists[0 .. tiles)            tiles inside their window (header value 4 != 0), count[0] of them
+//   lists[tiles .. 2 tiles)      the others, count[1]
+//   lists[2 tiles .. 3 tiles)    those of the others that are big tiles (header value 7), count[2]
+//   lists[3 tiles .. 4 tiles)    ... and those that have none, count[3]
+// max_rows > 0: a tile with a sample of more rows is neither inside nor big.
 __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict__ hdr, int tiles,
                                                           int* __restrict__ lists,
                                                           int* __restrict__ count, int max_rows) {
-  __shared__ int wave_fit[16], wave_rest[16];
-  __shared__ int base[2];
+  __shared__ int wave_n[4][16];
+  __shared__ int base[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) base[0] = base[1] = 0;
+  if (tid < 4) base[tid] = 0;
   __syncthreads();
   for (int t0 = 0; t0 < tiles; t0 += 1024) {
     const int t = t0 + tid;
     const bool live = t < tiles;
-    const bool fit = live && hdr[t * kHdrStride + 4] != 0 && (max_rows <= 0 || hdr[t * kHdrStride + 5] <= max_rows);
-    const unsigned long long mf = __ballot(fit), mr = __ballot(live && !fit);
-    if (lane == 0) {
-      wave_fit[wave] = __popcll(mf);
-      wave_rest[wave] = __popcll(mr);
+    const bool rows_ok = live && (max_rows <= 0 || hdr[t * kHdrStride + 5] <= max_rows);
+    bool cls[4];
+    cls[0] = rows_ok && hdr[t * kHdrStride + 4] != 0;
+    cls[1] = live && !cls[0];
+    cls[2] = cls[1] && rows_ok && hdr[t * kHdrStride + 7] != 0;
+    cls[3] = cls[1] && !cls[2];
+    unsigned long long mask[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      mask[c] = __ballot(cls[c]);
+      if (lane == 0) wave_n[c][wave] = __popcll(mask[c]);
     }
     __syncthreads();
-    int of = base[0], orr = base[1];
-    for (int w = 0; w < wave; ++w) {
-      of += wave_fit[w];
-      orr += wave_rest[w];
-    }
     const unsigned long long below = (1ull << lane) - 1ull;
-    if (fit) lists[of + __popcll(mf & below)] = t;
-    else if (live) lists[tiles + orr + __popcll(mr & below)] = t;
-    __syncthreads();
-    if (tid == 0) {
-      int a = 0, b = 0;
-      for (int w = 0; w < 16; ++w) {
-        a += wave_fit[w];
-        b += wave_rest[w];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (cls[c]) {
+        int o = base[c];
+        for (int w = 0; w < wave; ++w) o += wave_n[c][w];
+        lists[(size_t)c * tiles + o + __popcll(mask[c] & below)] = t;
       }
-      base[0] += a;
-      base[1] += b;
+    }
+    __syncthreads();
+    if (tid < 4) {
+      int a = 0;
+      for (int w = 0; w < 16; ++w) a += wave_n[tid][w];
+      base[tid] += a;
     }
     __syncthreads();
   }
-  if (tid == 0) {
-    count[0] = base[0];
-    count[1] = base[1];
-  }
+  if (tid < 4) count[tid] = base[tid];
 }
 
 
-template <int MM, int NB>
-__global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
+// CAP: elements of the LDS window.  kRegionCap: the tiles of `list` lie inside their window,
+// two workgroups share a CU.  kBigCap: `list` holds big tiles, whose window is their list in
+// big_lut; it takes most of a CU's LDS and one workgroup runs per CU.
+template <int MM, int NB, int CAP>
+__global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_gemm_kernel(
     const float* __restrict__ img, const int* __restrict__ hdr, const int* __restrict__ ns,
     const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
     const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
     int H, int W, int Cp, int K, int S, int CpP, int chunks, PixelTiling pt, int tiles,
-    int n_tiles, const int* __restrict__ gate) {
+    int n_tiles, const int* __restrict__ gate, const int* __restrict__ big_lut) {
   if (gate != nullptr && *gate != 0) return;   // the plan is not valid: another kernel does the work
   constexpr bool BF16 = MM != kMmF32;
+  constexpr bool BIG = CAP > kRegionCap;
   constexpr int TN = 32 * NB;
-  __shared__ __align__(16) float region[(kRegionCap + 1) * kWE];
+  __shared__ __align__(16) float region[(CAP + 1) * kWE];
   __shared__ __align__(16) float As[2][TN * kWE];
-  __shared__ int src[kRegionCap];
+  __shared__ int src[CAP];
   __shared__ int ns_l[kPlanKMax];   // rows per sample (a scalar load here would sit in the LDS waits)
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -349,21 +369,20 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
   const size_t HW = (size_t)H * W;
   const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
 
-  Region rg;
-  rg.ry0 = hdr[tile * kHdrStride + 0];
-  rg.rx0 = hdr[tile * kHdrStride + 1];
-  rg.RH = hdr[tile * kHdrStride + 2];
-  rg.RW = hdr[tile * kHdrStride + 3];
-  rg.RS = rg.RH * rg.RW;
-  rg.RSp = rg.RS;
-  const int RS = rg.RS;
-  load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
-  if (tid < kWE) region[RS * kWE + tid] = 0.0f;   // the zero element padded rows point at
-  for (int k = tid; k < K; k += kWgThreads) ns_l[k] = ns[(size_t)tile * K + k];
-
   // this lane's pixel and its plan rows: row r of sample k at rows_p[(k * S + r) * 128]
   const int p_local = 32 * wave + j;
+  int RS;
   const int2* rows_p = taps + (size_t)tile * K * S * 128 + p_local;
+  if constexpr (BIG) {
+    const int* bl = big_lut + (size_t)tile * kBigStride;
+    RS = min(bl[0], CAP);
+    for (int e = tid; e < RS; e += kWgThreads) src[e] = bl[kBigLut + e];
+  } else {
+    RS = hdr[tile * kHdrStride + 2] * hdr[tile * kHdrStride + 3];
+    load_region_lut(hdr + (size_t)tile * kHdrStride, RS, src);
+  }
+  if (tid < kWE) region[RS * kWE + tid] = 0.0f;   // the zero element padded rows point at
+  for (int k = tid; k < K; k += kWgThreads) ns_l[k] = ns[(size_t)tile * K + k];
 
   // The accumulators start at the bias of their rows (register v of lane l: row
   // 8 (v / 4) + 4 (l / 32) + v % 4): the reads are issued here, with the window's, and the
@@ -453,7 +472,7 @@ __global__ __launch_bounds__(kWgThreads, 2) void window_gemm_kernel(
     {
       // wave w stages channels 8w .. 8w+7 of every window element; a lane owns elements
       // lane, lane + 64, ... and has all its loads in flight before the first LDS write
-      constexpr int ITER = (kRegionCap + 63) / 64;
+      constexpr int ITER = (CAP + 63) / 64;
       const int cw = c0 + 8 * wave;
       const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
       const unsigned plane = (unsigned)HW * 4u;
@@ -593,14 +612,16 @@ size_t window_gemm_weight_bytes(const ConvGeom& g) {
 
 size_t tile_lists_bytes(const ConvGeom& g) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  return ((size_t)2 * pt.tiles_x * pt.tiles_y + 2) * sizeof(int);
+  return ((size_t)4 * pt.tiles_x * pt.tiles_y + 4) * sizeof(int);
 }
 
 void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
   int* lists = static_cast<int*>(workspace);
   out->inside = lists;
   out->rest = lists + plan.tiles;
-  out->count = lists + (size_t)2 * plan.tiles;
+  out->big = lists + (size_t)2 * plan.tiles;
+  out->rest_small = lists + (size_t)3 * plan.tiles;
+  out->count = lists + (size_t)4 * plan.tiles;
 }
 
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
@@ -614,26 +635,33 @@ int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, Tile
 
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                 const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
-                float* weights, const int* gate, hipStream_t stream) {
+                float* weights, const int* gate, hipStream_t stream, bool big) {
   const int CpP = (g.Cp + 127) / 128 * 128;
   const int chunks = (g.Cg + kCC - 1) / kCC;
-  {
+  if (!big) {
     const size_t total = (size_t)g.K * chunks * CpP * kCC;
     const int blocks = (int)std::min<size_t>((total + kWgThreads - 1) / kWgThreads, 2048);
     launch(window_weight_kernel, dim3(blocks), dim3(kWgThreads), stream, Wm, weights, g.Cp, g.Cg,
            g.K, CpP, chunks, mm != kMmF32 ? 1 : 0, swapped ? 1 : 0);
     SDK_LAUNCH_CHECK("window_weight");
+  } else if (plan.big_lut == nullptr) {
+    return SDK_OK;
   }
   const bool wide = g.Cp > 64;
   const int TN = wide ? 128 : 64;
   const int n_tiles = (int)ceil_div(g.Cp, TN);
   // list entries are dealt to the XCDs in eighths: whole multiples of 8 workgroups
   const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
-#define WG2(MMv, NBv)                                                                          \
-  launch(window_gemm_kernel<MMv, NBv>, grid, dim3(kWgThreads), stream, img, plan.hdr, plan.ns, \
-         plan.taps, (const int*)tl.inside, (const int*)tl.count, (const float*)weights, bias,  \
-         pix, g.Cg, g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles,    \
-         gate)
+  const int* list = big ? tl.big : tl.inside;
+  const int* count = big ? tl.count + 2 : tl.count;
+#define WG3(MMv, NBv, CAPv)                                                                    \
+  launch(window_gemm_kernel<MMv, NBv, CAPv>, grid, dim3(kWgThreads), stream, img, plan.hdr,    \
+         plan.ns, plan.taps, list, count, (const float*)weights, bias, pix, g.Cg, g.H, g.W,    \
+         g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles, gate, plan.big_lut)
+#define WG2(MMv, NBv)                                                 \
+  do {                                                                \
+    if (big) WG3(MMv, NBv, kBigCap); else WG3(MMv, NBv, kRegionCap);  \
+  } while (0)
 #define WG1(MMv)                              \
   do {                                        \
     if (wide) WG2(MMv, 4); else WG2(MMv, 2);  \
@@ -643,13 +671,14 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   else WG1(kMmF32);
 #undef WG1
 #undef WG2
-  SDK_LAUNCH_CHECK("window_gemm");
+#undef WG3
+  SDK_LAUNCH_CHECK(big ? "window_gemm(big)" : "window_gemm");
   return SDK_OK;
 }
 
 namespace {
 struct InverseOffsets {
-  size_t gate, cnt, raw_co, raw_off, hdr, ns, taps, total;
+  size_t gate, cnt, raw_co, raw_off, hdr, ns, taps, big_lut, total;
 };
 InverseOffsets inverse_offsets(const ConvGeom& g) {
   auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
@@ -664,7 +693,8 @@ InverseOffsets inverse_offsets(const ConvGeom& g) {
   o.hdr = o.raw_off + up(rows * sizeof(int));
   o.ns = o.hdr + up(tiles * kHdrStride * sizeof(int));
   o.taps = o.ns + up(tiles * g.K * sizeof(int));
-  o.total = o.taps + up(rows * sizeof(int2));
+  o.big_lut = o.taps + up(rows * sizeof(int2));
+  o.total = o.big_lut + up(tiles * kBigStride * sizeof(int));
   return o;
 }
 }  // namespace
@@ -681,6 +711,7 @@ void load_inverse_plan(const ConvGeom& g, void* workspace, InversePlan* out) {
   out->plan.hdr = reinterpret_cast<int*>(ws + o.hdr);
   out->plan.ns = reinterpret_cast<int*>(ws + o.ns);
   out->plan.taps = reinterpret_cast<int2*>(ws + o.taps);
+  out->plan.big_lut = reinterpret_cast<int*>(ws + o.big_lut);
   out->gate = reinterpret_cast<int*>(ws + o.gate);
   out->raw_off = reinterpret_cast<int*>(ws + o.raw_off);
   out->raw_co = reinterpret_cast<float*>(ws + o.raw_co);
@@ -708,7 +739,8 @@ int build_inverse_plan(const ConvGeom& g, const float* map, const float* wts, vo
   launch(inverse_plan_kernel, dim3((unsigned)out->plan.tiles), dim3(kWgThreads), stream,
          (const int*)cnt, raw_off, raw_co, out->plan.pt, g.K, g.M / g.OW, g.OW,
          const_cast<int*>(out->plan.hdr), const_cast<int*>(out->plan.ns),
-         const_cast<int2*>(out->plan.taps), (const int*)out->gate);
+         const_cast<int2*>(out->plan.taps), (const int*)out->gate,
+         const_cast<int*>(out->plan.big_lut));
   SDK_LAUNCH_CHECK("inverse_plan");
   return SDK_OK;
 }

@@ -43,17 +43,21 @@ constexpr int kWwG = 36;   // floats per row of the pixel-side tile: 32 pixels +
 constexpr int kWwQ = 32;   // pixels per quarter tile
 constexpr int kWwRows = 4; // plan rows per sample this kernel applies
 
-template <int KP, int R>
-__global__ __launch_bounds__(kWwThreads, 2) void window_wgrad_kernel(
+// CAP: elements of the LDS window.  kRegionCap: the tiles of `list` lie inside their window.
+// kBigCap: `list` holds big tiles, whose window is their list in big_lut; one workgroup per CU.
+template <int KP, int R, int CAP>
+__global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, const int* __restrict__ list,
     const int* __restrict__ count, float* __restrict__ partial, int Cg, int H, int W, int Cp,
-    int S, PixelTiling pt, int groups, int batches, int c_chunks, int n_tiles, int vec4) {
+    int S, PixelTiling pt, int groups, int batches, int c_chunks, int n_tiles, int vec4,
+    const int* __restrict__ big_lut) {
   constexpr int K = 4 * KP + R;
-  __shared__ __align__(16) float region[(kRegionCap + 1) * kWwE];
+  constexpr bool BIG = CAP > kRegionCap;
+  __shared__ __align__(16) float region[(CAP + 1) * kWwE];
   __shared__ __align__(16) float gt[128 * kWwG];
   __shared__ __align__(16) int2 rowsL[K * kWwQ * kWwRows];
-  __shared__ int src[kRegionCap];
+  __shared__ int src[CAP];
   __shared__ int ns_l[K];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -97,25 +101,26 @@ __global__ __launch_bounds__(kWwThreads, 2) void window_wgrad_kernel(
   for (int ti = group; ti < cnt; ti += groups) {
     const int tile = list[ti];
     const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
-    Region rg;
-    rg.ry0 = hdr[tile * kHdrStride + 0];
-    rg.rx0 = hdr[tile * kHdrStride + 1];
-    rg.RH = hdr[tile * kHdrStride + 2];
-    rg.RW = hdr[tile * kHdrStride + 3];
-    rg.RS = rg.RH * rg.RW;
-    rg.RSp = rg.RS;
-    const int RS = rg.RS;
+    int RS;
     const int2* tile_taps = taps + (size_t)tile * K * S * 128;
+    const int* lut;
+    if constexpr (BIG) {
+      lut = big_lut + (size_t)tile * kBigStride;
+      RS = min(lut[0], CAP);
+    } else {
+      lut = hdr + (size_t)tile * kHdrStride;
+      RS = lut[2] * lut[3];
+    }
 
     __syncthreads();   // every wave is done with the previous tile
-    load_region_lut(hdr + (size_t)tile * kHdrStride, rg.RS, src);
+    for (int e = tid; e < RS; e += kWwThreads) src[e] = lut[kHdrLut + e];
     if (tid < K) ns_l[tid] = min(ns[(size_t)tile * K + tid], min(S, kWwRows));
     if (tid < kWwE) region[RS * kWwE + tid] = 0.0f;   // the zero element inactive rows point at
     __syncthreads();
     {
       // window: wave w stages channels 8w .. 8w+7 of every element; a lane owns elements
       // lane, lane + 64, ... and has all its loads in flight before the first LDS write
-      constexpr int ITER = (kRegionCap + 63) / 64;
+      constexpr int ITER = (CAP + 63) / 64;
       const int cw = c0 + 8 * wave;
       const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
       const unsigned plane = (unsigned)HW * 4u;
@@ -331,13 +336,15 @@ struct WwGrid {
   int c_chunks, n_tiles, groups, nreg;
   int64_t kinds, slots;
 };
-WwGrid ww_grid(const ConvGeom& g, int tiles) {
+// big: the launch over the big tiles (one workgroup per CU).
+WwGrid ww_grid(const ConvGeom& g, int tiles, bool big) {
   WwGrid w;
   w.c_chunks = (int)ceil_div(g.Cg, kCC);
   w.n_tiles = (int)ceil_div(g.Cp, 128);
   w.kinds = (int64_t)w.c_chunks * w.n_tiles * g.B;
-  // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall
-  const int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(512, w.kinds), 8) * 8);
+  // tile runs: a multiple of 8 (one set per XCD), about two workgroups per CU overall (one
+  // for the big windows)
+  const int64_t want = std::max<int64_t>(8, ceil_div(ceil_div(big ? 256 : 512, w.kinds), 8) * 8);
   w.groups = (int)std::min<int64_t>(ceil_div(tiles, 8) * 8, want);
   w.slots = (int64_t)w.groups * w.kinds;
   w.nreg = g.K * 16;
@@ -355,22 +362,30 @@ bool window_wgrad_supported(const ConvGeom& g, int mm) {
 size_t window_wgrad_partial_bytes(const ConvGeom& g) {
   if (g.B == 0 || !window_wgrad_supported(g, kMmF32)) return 0;
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  const WwGrid w = ww_grid(g, pt.tiles_x * pt.tiles_y);
-  return (size_t)w.slots * w.nreg * kWwThreads * sizeof(float);
+  const int tiles = pt.tiles_x * pt.tiles_y;
+  const WwGrid w = ww_grid(g, tiles, false), wb = ww_grid(g, tiles, true);
+  return (size_t)std::max(w.slots, wb.slots) * w.nreg * kWwThreads * sizeof(float);
 }
 
 int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
-                 const float* img, float* gW, float* partial, hipStream_t stream) {
-  const WwGrid w = ww_grid(g, plan.tiles);
+                 const float* img, float* gW, float* partial, hipStream_t stream, bool big) {
+  if (big && plan.big_lut == nullptr) return SDK_OK;
+  const WwGrid w = ww_grid(g, plan.tiles, big);
+  const int* list = big ? tl.big : tl.inside;
+  const int* count = big ? tl.count + 2 : tl.count;
   if (w.slots >= ((int64_t)1 << 31)) return fail(SDK_ERR_UNSUPPORTED, "window_wgrad: grid too large");
   const int TX = plan.pt.TX();
   const int vec4 = (g.OW % 4 == 0 && TX >= 16 && reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)w.slots);
   const int KP = g.K / 4, R = g.K % 4;
-#define WW(KPv, Rv)                                                                              \
-  launch(window_wgrad_kernel<KPv, Rv>, grid, dim3(kWwThreads), stream, pix, img, plan.hdr,       \
-         plan.ns, plan.taps, (const int*)tl.inside, (const int*)tl.count, partial, g.Cg, g.H,    \
-         g.W, g.Cp, plan.S, plan.pt, w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4)
+#define WW2(KPv, Rv, CAPv)                                                                       \
+  launch(window_wgrad_kernel<KPv, Rv, CAPv>, grid, dim3(kWwThreads), stream, pix, img, plan.hdr, \
+         plan.ns, plan.taps, list, count, partial, g.Cg, g.H, g.W, g.Cp, plan.S, plan.pt,        \
+         w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4, plan.big_lut)
+#define WW(KPv, Rv)                                                   \
+  do {                                                                \
+    if (big) WW2(KPv, Rv, kBigCap); else WW2(KPv, Rv, kRegionCap);    \
+  } while (0)
   switch (g.K) {
     case 1: WW(0, 1); break;
     case 2: WW(0, 2); break;
@@ -384,7 +399,8 @@ int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const
     default: WW(2, 2); break;
   }
 #undef WW
-  SDK_LAUNCH_CHECK("window_wgrad");
+#undef WW2
+  SDK_LAUNCH_CHECK(big ? "window_wgrad(big)" : "window_wgrad");
   const int kinds0 = w.c_chunks * w.n_tiles, total = (int)g.B * w.groups;
   const int parts = (int)std::min<int64_t>(std::min(total, 16),
                                            ceil_div(2048, (int64_t)w.nreg * kinds0));

@@ -42,12 +42,13 @@ def _case(seed, Cin, Cout, H, W, OH, OW, K, P, interp, kind):
     if kind == "listed":
         # One-row image, nearest, K = 3: the taps of a tile of 128 pixels are far apart (no box
         # fits) and touch exactly 288 distinct elements in the first tile (a listed window, full
-        # to the last element), 289 in the second (one too many: the listed rest) and 128 + 128 +
-        # 128 = 384 in the third; the fourth names sixteen elements eight times each.
+        # to the last element), 289 in the second (one too many: a big window) and 128 + 128 +
+        # 128 = 384 in the third and in every tile from the fifth on; the fourth names sixteen
+        # elements eight times each.
         assert OH == 1 and K == 3 and P == 0
         p = np.arange(OW)
         t, q = p // 128, p % 128
-        third = np.select([t == 0, t == 1, t == 2], [q % 32, q % 33, q], q % 16)
+        third = np.select([t == 0, t == 1, t == 3], [q % 32, q % 33, q % 16], q)
         cx = np.stack([q + 1000.0 * t, 300.0 + q + 1000.0 * t, 600.0 + third + 1000.0 * t], -1)
         cx = cx.reshape(1, OW, 3) % W
         cy = np.zeros_like(cx)
@@ -83,6 +84,7 @@ CASES = [
     (16, 24, 30, 50, 30, 50, 7, 0, 1, "plain"),      # narrow layers: kernels that ignore the plan
     (72, 80, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # listed windows: 288 (fits), 289, 384 elements
     (40, 48, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # ... in the 64-channel kernels
+    (72, 80, 1, 33000, 1, 4096, 3, 0, 0, "listed"),  # 30 of 32 tiles with a big window
 ]
 
 
