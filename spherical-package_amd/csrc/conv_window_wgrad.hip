@@ -45,6 +45,9 @@ constexpr int kWwRows = 4; // plan rows per sample this kernel applies
 
 // CAP: elements of the LDS window.  kRegionCap: the tiles of `list` lie inside their window.
 // kBigCap: `list` holds big tiles, whose window is their list in big_lut; one workgroup per CU.
+// With one wave per SIMD nothing else covers a global read, so that variant requests ahead what
+// it has registers for: the pixel-side tile and the plan rows of the next quarter, and the
+// offsets of the next tile's window, before a quarter's MFMAs.
 template <int KP, int R, int CAP>
 __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
@@ -57,8 +60,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   __shared__ __align__(16) float region[(CAP + 1) * kWwE];
   __shared__ __align__(16) float gt[128 * kWwG];
   __shared__ __align__(16) int2 rowsL[K * kWwQ * kWwRows];
-  __shared__ int src[CAP];
-  __shared__ int ns_l[K];
+  __shared__ int src[BIG ? 1 : CAP];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int j = lane & 31, h = lane >> 5;
@@ -97,12 +99,127 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   const bool n_ok = n0 + n_s < Cp;
   const float* pix_row = pix_b + (size_t)(n_ok ? n0 + n_s : 0) * M;
 
+  // ---- staging pieces.  Window: wave w stages channels 8w .. 8w+7 of every element; a lane
+  // owns elements lane, lane + 64, ... and has all its loads in flight before the first LDS write.
+  constexpr int ITER = (CAP + 63) / 64;
+  const int cw = c0 + 8 * wave;
+  const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
+  const unsigned plane = (unsigned)HW * 4u;
+  // wv[it][i] = channel cw + i of the element at flat offset wo[it] (-1: none)
+  auto fetch_window = [&](const int (&wo)[ITER], float (&wv)[ITER][8]) {
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (BIG) {
+          // No element of a listed window is missing, slots past its end are never stored, and
+          // the columns of channels past Cg are dropped with the sums: plain loads from a
+          // valid address, nothing that could become a branch around a load.
+          wv[it][i] = *reinterpret_cast<const float*>(
+              cbase + (unsigned)min(i, Cg - 1 - min(cw, Cg - 1)) * plane +
+              (unsigned)max(wo[it], 0) * 4u);
+        } else {
+          const bool ok = wo[it] >= 0 && cw + i < Cg;
+          const float d = *reinterpret_cast<const float*>(
+              cbase + (ok ? (unsigned)i * plane + (unsigned)wo[it] * 4u : 0u));
+          wv[it][i] = ok ? d : 0.0f;
+        }
+      }
+    }
+  };
+  auto store_window = [&](int RS, const float (&wv)[ITER][8]) {
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int e = lane + 64 * it;
+      if (e < RS) {
+        float4* d4 = reinterpret_cast<float4*>(region + e * kWwE + 8 * wave);
+        d4[0] = make_float4(wv[it][0], wv[it][1], wv[it][2], wv[it][3]);
+        d4[1] = make_float4(wv[it][4], wv[it][5], wv[it][6], wv[it][7]);
+      }
+    }
+  };
+  // Quarter q of a tile: this thread's 16 values of the pixel-side tile (row n_s, pixels
+  // 16 hr_s .. + 15) and its share of the plan rows, entry idx = tid + 256 u = (k, r, m), with
+  // the rows its sample has (the row itself is read whether it exists or not, clamped to S).
+  constexpr int TOTAL = K * kWwRows * kWwQ;
+  constexpr int NR = (TOTAL + kWwThreads - 1) / kWwThreads;
+  auto fetch_quarter = [&](int tile_, int q_, float4 (&gq)[4], int2 (&pr)[NR], int (&pn)[NR]) {
+    const int ty0_ = (tile_ / pt.tiles_x) * pt.TY(), tx0_ = (tile_ % pt.tiles_x) << pt.tx_shift;
+    const int p0 = kWwQ * q_ + 16 * hr_s;
+    if (vec4) {
+      const int oy = ty0_ + (p0 >> pt.tx_shift), ox = tx0_ + (p0 & (pt.TX() - 1));
+      const float* rowp = pix_row + (size_t)oy * pt.OW + ox;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        gq[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (n_ok && oy < pt.OH && ox + 4 * i < pt.OW)
+          gq[i] = *reinterpret_cast<const float4*>(rowp + 4 * i);
+      }
+    } else {
+      float f[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int p = p0 + i;
+        const int oy = ty0_ + (p >> pt.tx_shift), ox = tx0_ + (p & (pt.TX() - 1));
+        const bool ok = n_ok && oy < pt.OH && ox < pt.OW;
+        const float d = pix_row[ok ? (size_t)oy * pt.OW + ox : 0];
+        f[i] = ok ? d : 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) gq[i] = make_float4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+    }
+    const int2* tt = taps + (size_t)tile_ * K * S * 128;
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {
+      const int idx = min(kWwThreads * u + tid, TOTAL - 1);
+      const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
+      pr[u] = tt[((size_t)k * S + min(r, S - 1)) * 128 + kWwQ * q_ + m];
+      pn[u] = ns[(size_t)tile_ * K + k];
+    }
+  };
+  auto store_quarter = [&](int RS, const float4 (&gq)[4], const int2 (&pr)[NR],
+                           const int (&pn)[NR]) {
+    float4* dst = reinterpret_cast<float4*>(gt + n_s * kWwG + 16 * hr_s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = gq[i];
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {
+      const int idx = kWwThreads * u + tid;
+      if (idx < TOTAL) {
+        const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
+        const bool on = r < min(pn[u], min(S, kWwRows)) && __int_as_float(pr[u].y) != 0.0f;
+        rowsL[(k * kWwQ + m) * kWwRows + r] =
+            make_int2((on ? pr[u].x : RS) * (kWwE * 4), on ? pr[u].y : 0);
+      }
+    }
+  };
+  // what the big variant holds ahead: the coming quarter, the offsets of the next tile's window
+  float4 pg[4];
+  int2 pr[NR];
+  int pn[NR];
+  int wo[BIG ? ITER : 1];
+  // offsets of the window elements this lane stages for big tile `tile_`
+  auto fetch_offsets = [&](int tile_) {
+    const int* bl = big_lut + (size_t)tile_ * kBigStride;
+    const int RSn = min(bl[0], CAP);
+#pragma unroll
+    for (int it = 0; it < (BIG ? ITER : 1); ++it) {
+      const int e = lane + 64 * it;
+      wo[it] = e < RSn ? bl[kBigLut + e] : -1;
+    }
+  };
+
   const int cnt = *count;
+  if constexpr (BIG) {
+    if (group < cnt) {
+      const int first = list[group];
+      fetch_offsets(first);
+      fetch_quarter(first, 0, pg, pr, pn);
+    }
+  }
   for (int ti = group; ti < cnt; ti += groups) {
     const int tile = list[ti];
-    const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
     int RS;
-    const int2* tile_taps = taps + (size_t)tile * K * S * 128;
     const int* lut;
     if constexpr (BIG) {
       lut = big_lut + (size_t)tile * kBigStride;
@@ -111,93 +228,49 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
       lut = hdr + (size_t)tile * kHdrStride;
       RS = lut[2] * lut[3];
     }
+    const bool has_next = ti + groups < cnt;
+    const int tile_next = has_next ? list[ti + groups] : tile;
 
     __syncthreads();   // every wave is done with the previous tile
-    for (int e = tid; e < RS; e += kWwThreads) src[e] = lut[kHdrLut + e];
-    if (tid < K) ns_l[tid] = min(ns[(size_t)tile * K + tid], min(S, kWwRows));
     if (tid < kWwE) region[RS * kWwE + tid] = 0.0f;   // the zero element inactive rows point at
-    __syncthreads();
-    {
-      // window: wave w stages channels 8w .. 8w+7 of every element; a lane owns elements
-      // lane, lane + 64, ... and has all its loads in flight before the first LDS write
-      constexpr int ITER = (CAP + 63) / 64;
-      const int cw = c0 + 8 * wave;
-      const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
-      const unsigned plane = (unsigned)HW * 4u;
-      float v[ITER][8];
+    if constexpr (BIG) {
+      float sv[ITER][8];
+      fetch_window(wo, sv);
+      store_window(RS, sv);
+    } else {
+      for (int e = tid; e < RS; e += kWwThreads) src[e] = lut[kHdrLut + e];
+      __syncthreads();
+      int so[ITER];
+      float sv[ITER][8];
 #pragma unroll
       for (int it = 0; it < ITER; ++it) {
         const int e = lane + 64 * it;
-        const int o = e < RS ? src[e] : -1;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const bool ok = o >= 0 && cw + i < Cg;
-          const float d = *reinterpret_cast<const float*>(
-              cbase + (ok ? (unsigned)i * plane + (unsigned)o * 4u : 0u));
-          v[it][i] = ok ? d : 0.0f;
-        }
+        so[it] = e < RS ? src[e] : -1;
       }
-#pragma unroll
-      for (int it = 0; it < ITER; ++it) {
-        const int e = lane + 64 * it;
-        if (e < RS) {
-          float4* d4 = reinterpret_cast<float4*>(region + e * kWwE + 8 * wave);
-          d4[0] = make_float4(v[it][0], v[it][1], v[it][2], v[it][3]);
-          d4[1] = make_float4(v[it][4], v[it][5], v[it][6], v[it][7]);
-        }
-      }
+      fetch_window(so, sv);
+      store_window(RS, sv);
     }
 
 #pragma unroll 1
     for (int q = 0; q < 4; ++q) {
       if (q > 0) __syncthreads();   // the previous quarter's reads of gt / rowsL are done
-      // ---- pixel-side tile of the quarter: gt[n][m], m = 16 hr + i
-      {
-        const int p0 = kWwQ * q + 16 * hr_s;
-        float4 gq[4];
-        if (vec4) {
-          const int oy = ty0 + (p0 >> pt.tx_shift), ox = tx0 + (p0 & (pt.TX() - 1));
-          const float* rowp = pix_row + (size_t)oy * pt.OW + ox;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            gq[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (n_ok && oy < pt.OH && ox + 4 * i < pt.OW)
-              gq[i] = *reinterpret_cast<const float4*>(rowp + 4 * i);
-          }
-        } else {
-          float f[16];
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int p = p0 + i;
-            const int oy = ty0 + (p >> pt.tx_shift), ox = tx0 + (p & (pt.TX() - 1));
-            const bool ok = n_ok && oy < pt.OH && ox < pt.OW;
-            const float d = pix_row[ok ? (size_t)oy * pt.OW + ox : 0];
-            f[i] = ok ? d : 0.0f;
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) gq[i] = make_float4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
-        }
-        float4* dst = reinterpret_cast<float4*>(gt + n_s * kWwG + 16 * hr_s);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = gq[i];
-      }
-      // ---- plan rows of the quarter: rowsL[(k * 32 + m) * 4 + r] = (window byte offset, coefficient)
-      {
-        constexpr int TOTAL = K * kWwRows * kWwQ;
-#pragma unroll
-        for (int i0 = 0; i0 < TOTAL; i0 += kWwThreads) {
-          const int idx = i0 + tid;
-          if (idx < TOTAL) {
-            const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
-            int2 ec = make_int2(0, 0);
-            if (r < ns_l[k]) ec = tile_taps[((size_t)k * S + r) * 128 + kWwQ * q + m];
-            const bool on = __int_as_float(ec.y) != 0.0f;
-            rowsL[(k * kWwQ + m) * kWwRows + r] =
-                make_int2((on ? ec.x : RS) * (kWwE * 4), on ? ec.y : 0);
-          }
-        }
+      if constexpr (BIG) {
+        store_quarter(RS, pg, pr, pn);
+      } else {
+        // ---- pixel-side tile of the quarter: gt[n][m], m = 16 hr + i; plan rows of the
+        // quarter: rowsL[(k * 32 + m) * 4 + r] = (window byte offset, coefficient)
+        fetch_quarter(tile, q, pg, pr, pn);
+        store_quarter(RS, pg, pr, pn);
       }
       __syncthreads();   // (for q == 0 this also publishes the window)
+      if constexpr (BIG) {
+        // requests for what comes next, answered while this quarter's MFMAs run
+        if (q < 3) fetch_quarter(tile, q + 1, pg, pr, pn);
+        else if (has_next) {
+          fetch_quarter(tile_next, 0, pg, pr, pn);
+          fetch_offsets(tile_next);
+        }
+      }
 
       // ---- 16 MFMA steps over the quarter's pixels m = 16 h + s, as a three-stage pipeline:
       // while the MFMAs of step s issue, the window values of step s + 1 and the plan rows of
