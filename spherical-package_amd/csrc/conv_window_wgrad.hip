@@ -57,6 +57,9 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
     const int* __restrict__ big_lut) {
   constexpr int K = 4 * KP + R;
   constexpr bool BIG = CAP > kRegionCap;
+  // (with two workgroups per CU the registers are not there: the requests spill and the kernel
+  // takes half as long again)
+  constexpr bool PIPE = BIG;
   __shared__ __align__(16) float region[(CAP + 1) * kWwE];
   __shared__ __align__(16) float gt[128 * kWwG];
   __shared__ __align__(16) int2 rowsL[K * kWwQ * kWwRows];
@@ -210,10 +213,10 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   };
 
   const int cnt = *count;
-  if constexpr (BIG) {
+  if constexpr (PIPE) {
     if (group < cnt) {
       const int first = list[group];
-      fetch_offsets(first);
+      if constexpr (BIG) fetch_offsets(first);
       fetch_quarter(first, 0, pg, pr, pn);
     }
   }
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
 #pragma unroll 1
     for (int q = 0; q < 4; ++q) {
       if (q > 0) __syncthreads();   // the previous quarter's reads of gt / rowsL are done
-      if constexpr (BIG) {
+      if constexpr (PIPE) {
         store_quarter(RS, pg, pr, pn);
       } else {
         // ---- pixel-side tile of the quarter: gt[n][m], m = 16 hr + i; plan rows of the
@@ -263,12 +266,12 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
         store_quarter(RS, pg, pr, pn);
       }
       __syncthreads();   // (for q == 0 this also publishes the window)
-      if constexpr (BIG) {
+      if constexpr (PIPE) {
         // requests for what comes next, answered while this quarter's MFMAs run
         if (q < 3) fetch_quarter(tile, q + 1, pg, pr, pn);
         else if (has_next) {
           fetch_quarter(tile_next, 0, pg, pr, pn);
-          fetch_offsets(tile_next);
+          if constexpr (BIG) fetch_offsets(tile_next);
         }
       }
 
