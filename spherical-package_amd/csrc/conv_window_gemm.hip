@@ -443,8 +443,9 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
     _Pragma("unroll") for (int u = 0; u < RB; ++u)                                \
       dst[u] = rows_p[((size_t)(kv) * S + min((r0v) + u, S - 1)) * 128];          \
   } while (0)
-  // col[] += the taps of up to four rows
-#define SDK_GATHER_ROWS(src, r0v)                                                 \
+  // col[] += the taps of up to four rows (FIRST: col[] = ..., the product of the first row
+  // instead of a register clear and a multiply-add)
+#define SDK_GATHER_ROWS(src, r0v, FIRST)                                          \
   do {                                                                            \
     int e[RB];                                                                    \
     float co[RB];                                                                 \
@@ -458,7 +459,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
       const float d[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w,        \
                            d2.x, d2.y, d2.z, d2.w, d3.x, d3.y, d3.z, d3.w};       \
       _Pragma("unroll") for (int i = 0; i < 16; ++i)                              \
-        colv[i] = __builtin_fmaf(co[u], d[i], colv[i]);                           \
+        colv[i] = (FIRST) && u == 0 ? co[u] * d[i] : __builtin_fmaf(co[u], d[i], colv[i]); \
     }                                                                             \
   } while (0)
 
@@ -523,14 +524,12 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
 
       // ---- gather: col[c][pixel j] for this lane's 16 channels of the chunk
       float colv[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) colv[i] = 0.0f;
-      SDK_GATHER_ROWS(rows, 0);
+      SDK_GATHER_ROWS(rows, 0, true);
       if (n_rows > RB) {
         for (int r0 = RB; r0 < n_rows; r0 += RB) {
           int2 more[RB];
           SDK_LOAD_ROWS(more, k, r0);
-          SDK_GATHER_ROWS(more, r0);
+          SDK_GATHER_ROWS(more, r0, false);
         }
       }
       // ---- contraction
