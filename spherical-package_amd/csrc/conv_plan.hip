@@ -328,6 +328,7 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
   int buf = 0;
   // all tiles, or the listed ones (tile_list[i], i < *tile_count)
   const int n_listed = tile_list != nullptr ? *tile_count : tiles;
+  if (n_listed == 0) return;   // (the summing kernel sees the same count and adds nothing)
   for (int ti = group; ti < n_listed; ti += groups) {
     const int tile = tile_list != nullptr ? tile_list[ti] : ti;
     const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
@@ -715,7 +716,9 @@ __global__ __launch_bounds__(kPlThreads, 2) void planned_wgrad_kernel(
 // batches * groups workgroups of that kind.  The index arithmetic mirrors the kernel's.
 __global__ __launch_bounds__(kPlThreads) void wgrad_reduce_kernel(
     const float* __restrict__ partial, float* __restrict__ gW, int Cg, int Cp, int K, int KB,
-    int NW, int groups, int batches, int c_chunks, int n_tiles, int kblocks) {
+    int NW, int groups, int batches, int c_chunks, int n_tiles, int kblocks,
+    const int* __restrict__ tile_count) {
+  if (tile_count != nullptr && *tile_count == 0) return;   // nothing was summed
   const int tid = threadIdx.x, kkv = blockIdx.x, kk = kkv >> 4, v = kkv & 15;
   const int kb = blockIdx.y % kblocks, nt = (blockIdx.y / kblocks) % n_tiles;
   const int cc = blockIdx.y / (kblocks * n_tiles);
@@ -913,7 +916,7 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
     const int parts = (int)std::min<int64_t>(std::min(total, 16), ceil_div(2048, (int64_t)KB * 16 * kinds0));
     launch(wgrad_reduce_kernel, dim3((unsigned)(KB * 16), (unsigned)kinds0, (unsigned)std::max(parts, 1)),
            dim3(kPlThreads), stream, (const float*)partial, gW, g.Cg, g.Cp, g.K, KB, NW, groups,
-           (int)g.B, c_chunks, n_tiles, kb_count);
+           (int)g.B, c_chunks, n_tiles, kb_count, tile_list != nullptr ? tile_count : nullptr);
     SDK_LAUNCH_CHECK("wgrad_reduce");
   }
   return SDK_OK;

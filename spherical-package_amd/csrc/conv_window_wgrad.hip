@@ -213,6 +213,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   };
 
   const int cnt = *count;
+  if (cnt == 0) return;   // (the summing kernel sees the same count and adds nothing)
   if constexpr (PIPE) {
     if (group < cnt) {
       const int first = list[group];
@@ -380,7 +381,8 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
 // row tile), over every z-th of the batches * groups workgroups of that kind.
 __global__ __launch_bounds__(kWwThreads) void window_wgrad_reduce_kernel(
     const float* __restrict__ partial, float* __restrict__ gW, int Cg, int Cp, int K, int KP,
-    int R, int groups, int batches, int c_chunks, int n_tiles) {
+    int R, int groups, int batches, int c_chunks, int n_tiles, const int* __restrict__ count) {
+  if (*count == 0) return;   // nothing was summed
   const int tid = threadIdx.x, reg = blockIdx.x;
   const int nt = blockIdx.y % n_tiles, cc = blockIdx.y / n_tiles;
   const int kinds = c_chunks * n_tiles * batches;
@@ -482,7 +484,7 @@ int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const
                                            ceil_div(2048, (int64_t)w.nreg * kinds0));
   launch(window_wgrad_reduce_kernel, dim3((unsigned)w.nreg, (unsigned)kinds0, (unsigned)std::max(parts, 1)),
          dim3(kWwThreads), stream, (const float*)partial, gW, g.Cg, g.Cp, g.K, KP, R, w.groups,
-         (int)g.B, w.c_chunks, w.n_tiles);
+         (int)g.B, w.c_chunks, w.n_tiles, count);
   SDK_LAUNCH_CHECK("window_wgrad_reduce");
   return SDK_OK;
 }
