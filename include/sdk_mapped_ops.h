@@ -435,7 +435,13 @@ int sdk_bias_grad(const void* grad_output, void* grad_bias, int64_t batch, int64
  * Replaces `_mapped_convolution.mapped_conv_backward` /
  * `_weighted_mapped_convolution.weighted_mapped_conv_backward`, which return the three
  * tensors from one call (ext_modules/include/layers/mapped_convolution_layer.h:89-134,
- *  weighted_mapped_convolution_layer.h:103-153). */
+ *  weighted_mapped_convolution_layer.h:103-153).
+ * When grad_output holds 384 MiB or more, the bias gradient (bound by HBM) runs on a stream of
+ * the library's own, forked from `stream` before the two contractions (bound by the matrix
+ * unit) and joined behind them; everything the call launches is complete when the work queued
+ * on `stream` behind the call starts.  While `stream` is being captured into a graph, and for
+ * smaller tensors, all of it runs on `stream`.  The same holds for
+ * sdk_mapped_transposed_conv_backward. */
 int sdk_mapped_conv_backward(const void* grad_output, const void* sample_map,
                              const void* interp_weights, const void* input, const void* weight,
                              void* grad_input, void* grad_weight, void* grad_bias,

@@ -4,6 +4,8 @@
 // request, otherwise to the generic im2col/col2im + GEMM path.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "conv_fused.hpp"
 #include "conv_internal.hpp"
 #include "sdk_host.hpp"
@@ -104,6 +106,67 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
   return SDK_OK;
 }
 
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// The bias gradient of a combined backward call reads grad_output once and is bound by HBM; the
+// two contractions beside it are bound by the matrix unit and leave HBM idle.  It runs on a
+// stream of the library's own (default priority), forked from the caller's stream before the
+// contractions and joined behind them, so that its waves take the slots the contraction
+// workgroups leave free.  One side stream and event pair per device, created at the first
+// call; if that fails (or the call is being captured into a graph) the bias gradient simply
+// runs on the caller's stream, as it does when grad_output is small.
+// ---------------------------------------------------------------------------
+namespace {
+// grad_output of at least this many bytes (a bias gradient of about 0.1 ms) goes to the side stream
+constexpr int64_t kSideStreamBytes = (int64_t)384 << 20;
+inline bool side_worth(int64_t batch, int64_t channels, int64_t pixels, int32_t dtype) {
+  return batch * channels * pixels * (dtype == SDK_F64 ? 8 : 4) >= kSideStreamBytes;
+}
+struct SideStream {
+  bool tried = false, ok = false;
+  hipStream_t s = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+};
+constexpr int kMaxDevices = 64;
+SideStream g_side[kMaxDevices];
+std::mutex g_side_mutex;
+
+// Runs `work(stream_to_use)` forked from `stream`; returns with *joined = the event the caller's
+// stream must wait for afterwards (nullptr: the work ran on the caller's stream).
+// worth: whether the work is long enough to pay for the fork and the join (about 50 us of
+// stream synchronisation, measured on a 64 us convolution step and on a 1.8 ms one).
+template <typename Work>
+int fork_side(hipStream_t stream, hipEvent_t* joined, bool worth, Work work) {
+  *joined = nullptr;
+  if (!worth) return work(stream);
+  int dev = -1;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices ||
+      hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return work(stream);
+  }
+  std::lock_guard<std::mutex> lock(g_side_mutex);
+  SideStream& ss = g_side[dev];
+  if (!ss.tried) {
+    ss.tried = true;
+    ss.ok = hipStreamCreateWithFlags(&ss.s, hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) == hipSuccess &&
+            hipEventCreateWithFlags(&ss.join, hipEventDisableTiming) == hipSuccess;
+    if (!ss.ok) (void)hipGetLastError();
+  }
+  if (!ss.ok || hipEventRecord(ss.fork, stream) != hipSuccess ||
+      hipStreamWaitEvent(ss.s, ss.fork, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return work(stream);
+  }
+  const int rc = work(ss.s);
+  if (hipEventRecord(ss.join, ss.s) != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "backward: cannot record the side stream's event");
+  *joined = ss.join;
+  return rc;
+}
 }  // namespace
 
 extern "C" {
@@ -281,14 +344,24 @@ static int impl_mapped_conv_backward(const void* grad_output, const void* sample
   if (rc) return rc;
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
+  hipEvent_t joined = nullptr;
+  rc = fork_side((hipStream_t)stream, &joined, side_worth(batch, out_channels, M, dtype),
+                 [&](hipStream_t s) {
+    return bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, s,
+                     s != (hipStream_t)stream);
+  });
   SharedPlan shared;   // the tap plan of the map is built once for both contractions
-  rc = run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
-           nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared, plan);
-  if (rc) return rc;
-  rc = run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
-           nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, &shared, plan);
-  if (rc) return rc;
-  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, stream);
+  if (rc == SDK_OK)
+    rc = run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights,
+             weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared,
+             plan);
+  if (rc == SDK_OK)
+    rc = run(what, GATHER_WGRAD, g, dtype, compute, grad_output, sample_map, interp_weights, input,
+             nullptr, grad_weight, workspace, workspace_bytes, (hipStream_t)stream, &shared, plan);
+  // (joined also after an error: the caller's stream must not run ahead of the side stream)
+  if (joined != nullptr && hipStreamWaitEvent((hipStream_t)stream, joined, 0) != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "%s: cannot join the side stream", what);
+  return rc;
 }
 
 static int impl_mapped_transposed_conv_backward(const void* grad_output, const void* sample_map,
@@ -301,19 +374,30 @@ static int impl_mapped_transposed_conv_backward(const void* grad_output, const v
                                         int64_t kernel_size, int32_t num_interp_pts,
                                         int32_t interp, int32_t dtype, int32_t compute,
                                         sdk_stream_t stream, PlanArg plan) {
-  int rc = impl_mapped_transposed_conv_backward_input(
-      grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes,
-      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
-      num_interp_pts, interp, dtype, compute, stream, plan);
-  if (rc) return rc;
-  rc = impl_mapped_transposed_conv_backward_weight(
-      grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes,
-      batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
-      num_interp_pts, interp, dtype, compute, stream, plan);
-  if (rc) return rc;
-  SDK_REQUIRE(grad_bias, "mapped_transposed_conv_backward: NULL pointer");
-  return sdk_bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype,
-                       stream);
+  const char* what = "mapped_transposed_conv_backward";
+  SDK_REQUIRE(grad_output && grad_bias, "%s: NULL pointer", what);
+  SDK_REQUIRE(out_height >= 1 && out_width >= 1 && out_height * out_width < ((int64_t)1 << 31),
+              "%s: bad output size", what);
+  hipEvent_t joined = nullptr;
+  int rc = fork_side((hipStream_t)stream, &joined,
+                     side_worth(batch, out_channels, out_height * out_width, dtype),
+                     [&](hipStream_t s) {
+    return bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype, s,
+                     s != (hipStream_t)stream);
+  });
+  if (rc == SDK_OK)
+    rc = impl_mapped_transposed_conv_backward_input(
+        grad_output, sample_map, interp_weights, weight, grad_input, workspace, workspace_bytes,
+        batch, in_channels, in_height, in_width, out_channels, out_height, out_width,
+        kernel_size, num_interp_pts, interp, dtype, compute, stream, plan);
+  if (rc == SDK_OK)
+    rc = impl_mapped_transposed_conv_backward_weight(
+        grad_output, sample_map, interp_weights, input, grad_weight, workspace, workspace_bytes,
+        batch, in_channels, in_height, in_width, out_channels, out_height, out_width, kernel_size,
+        num_interp_pts, interp, dtype, compute, stream, plan);
+  if (joined != nullptr && hipStreamWaitEvent((hipStream_t)stream, joined, 0) != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "%s: cannot join the side stream", what);
+  return rc;
 }
 
 

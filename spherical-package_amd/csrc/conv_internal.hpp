@@ -16,6 +16,10 @@ inline int matrix_mode(int compute) {
 }
 
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream);
+// grad_bias[c] = sum over batch and pixels (sdk_bias_grad).  beside_contractions: the variant
+// that uses no LDS, for a launch that runs concurrently with the contraction kernels.
+int bias_grad(const void* grad_output, void* grad_bias, int64_t batch, int64_t channels,
+              int64_t pixels, int32_t dtype, hipStream_t stream, bool beside_contractions);
 // gate: optional device flag; with one, the fill runs only if *gate != 0.
 int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
 
