@@ -487,7 +487,8 @@ template <int INTERP, bool WEIGHTED, int TC, int TM, bool BF16>
 __global__ __launch_bounds__(kThreads) void gemm_scatter_kernel(
     const float* __restrict__ pix, const float* __restrict__ map, const float* __restrict__ wts,
     const float* __restrict__ Wsc, float* __restrict__ img, int Cg, int H, int W, int Cp, int M,
-    int K, int P, int CgP, int CpP, int slots, int m_tiles) {
+    int K, int P, int CgP, int CpP, int slots, int m_tiles, const int* __restrict__ gate) {
+  if (gate != nullptr && *gate == 0) return;   // another kernel has done the work
   extern __shared__ __align__(16) unsigned char smem[];
   float* Bs = reinterpret_cast<float*>(smem);             // [kKC][TM]  pix chunk
   float* As = Bs + kKC * TM;                               // [kKC][TC]  weight chunk
@@ -688,6 +689,8 @@ bool fused_supported(const ConvGeom& g) {
 
 static bool inverse_candidate(const ConvGeom& g);
 static size_t inverse_bytes(const ConvGeom& g);
+static bool scatter_tries_inverse(const ConvGeom& g);
+static size_t inverse_ws_offset(const ConvGeom& g);
 // Tail of the workspace used by the weight gradient: partial sums of the plan-driven kernel,
 // those of the window kernel, the tile lists.
 struct WgradTail {
@@ -724,8 +727,7 @@ size_t fused_workspace_bytes(const ConvGeom& g) {
   size_t need = std::max((size_t)g.K * CpP * CgP * sizeof(float), staged_workspace_bytes(g));
   if (gather_from_window(g)) need = std::max(need, gather_layout(g).total);
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
-  if (planned_scatter_supported(g) && inverse_candidate(g))
-    need = ((need + 255) & ~(size_t)255) + inverse_bytes(g);
+  if (scatter_tries_inverse(g)) need = std::max(need, inverse_ws_offset(g) + inverse_bytes(g));
   // last: the weight gradient's tile lists and partial sums (the plan and, in a combined
   // backward call, everything before it are still in use when they are written)
   return ((need + 255) & ~(size_t)255) + wgrad_tail(g).total;
@@ -1014,6 +1016,22 @@ static size_t inverse_bytes(const ConvGeom& g) {
   return off[6];
 }
 
+// The scatter runs as a gather over an inverse map or plan whenever one can be built: always
+// beside the plan-driven scatter kernel (its fallback when a target has too many sources), and
+// through the window kernels also where that kernel does not reach (more than 128 pixel-side
+// channels), with the atomic scatter kernel as the fallback.
+static bool scatter_tries_inverse(const ConvGeom& g) {
+  return inverse_candidate(g) && (planned_scatter_supported(g) || scatter_from_window(g));
+}
+// Where the inverse structures start in the workspace: behind the weight copies of the fallback
+// kernels and the tap plan.
+static size_t inverse_ws_offset(const ConvGeom& g) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  const size_t weights = std::max((size_t)g.K * round_up(g.Cp, 128) * round_up(g.Cg, 128) * sizeof(float),
+                                  staged_workspace_bytes(g));
+  return up(up(weights) + (plan_supported(g) ? plan_bytes(g) : 0));
+}
+
 static int build_inverse(const ConvGeom& g, const float* map, const float* wts, char* ws,
                          hipStream_t stream, InverseMap* inv) {
   size_t off[7];
@@ -1086,14 +1104,16 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     if (shared != nullptr) shared->valid = false;
     return small_scatter(g, pix, map, wts, Wm, img, stream);
   }
-  if (planned_scatter_supported(g)) {
+  const bool planned_fb = planned_scatter_supported(g);
+  const int* generic_gate = nullptr;   // gate of the atomic scatter kernel at the end
+  bool filled = false;
+  if (scatter_tries_inverse(g)) {
     const int* gate = nullptr;
-    if (inverse_candidate(g)) {
+    {
       // Try the scatter as a gather over the inverse map.  The inverse is built on the device;
       // if a target collects more sources than its rows hold, the gather kernel exits at once
       // and the fill and the scatter kernel below run instead (and vice versa).
-      const size_t base = ((staged_workspace_bytes(g) + 255) & ~(size_t)255) + plan_bytes(g);
-      char* inv_ws = reinterpret_cast<char*>(workspace) + ((base + 255) & ~(size_t)255);
+      char* inv_ws = reinterpret_cast<char*>(workspace) + inverse_ws_offset(g);
       if (scatter_from_window(g)) {
         // the inverse lists as a plan: image tiles whose sources stay inside a window of the
         // pixel grid gather from LDS, the others from global memory
@@ -1160,18 +1180,29 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     }
     rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream, gate);
     if (rc) return rc;
+    filled = true;
+    generic_gate = gate;
+  }
+  if (planned_fb) {
+    if (!filled) {
+      rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+      if (rc) return rc;
+    }
     if (cached != nullptr && shared != nullptr) {
       // the weight gradient of this call takes the cached plan; the scatter kernel (which runs
       // only if the gate is raised) builds its own
       shared->plan = cached->plan;
       shared->valid = true;
-      return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream,
+      return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, generic_gate, stream,
                                   nullptr);
     }
-    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, gate, stream, shared);
+    return planned_gemm_scatter(g, bf16, pix, map, wts, Wm, img, workspace, generic_gate, stream,
+                                shared);
   }
-  rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
-  if (rc) return rc;
+  if (!filled) {
+    rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+    if (rc) return rc;
+  }
   const int slots = slots_for(g);
   const bool narrow = g.Cg <= 64;
   const int TC = narrow ? 64 : 128, TM = narrow ? 256 : 128;
@@ -1187,7 +1218,7 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
                                         gemm_scatter_kernel<INTERP, WEIGHTED, TCv, TMv, BFv>, grid, \
                                         smem, stream, pix, map, wts, (const float*)workspace,  \
                                         img, g.Cg, g.H, g.W, g.Cp, g.M, g.K, g.P, CgP, CpP,    \
-                                        slots, m_tiles)))
+                                        slots, m_tiles, generic_gate)))
   if (bf16) { if (narrow) GS(64, 256, true); else GS(128, 128, true); }
   else { if (narrow) GS(64, 256, false); else GS(128, 128, false); }
 #undef GS

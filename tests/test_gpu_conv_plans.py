@@ -85,6 +85,8 @@ CASES = [
     (72, 80, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # listed windows: 288 (fits), 289, 384 elements
     (40, 48, 1, 4500, 1, 512, 3, 0, 0, "listed"),    # ... in the 64-channel kernels
     (72, 80, 1, 33000, 1, 4096, 3, 0, 0, "listed"),  # 30 of 32 tiles with a big window
+    (72, 80, 64, 96, 32, 48, 9, 0, 1, "plain"),      # stride 2: every tile's box is 19 x 35, all big
+    (72, 136, 48, 64, 24, 32, 9, 2, 2, "plain"),     # ... weighted, more than 128 pixel-side channels
 ]
 
 
