@@ -720,7 +720,7 @@ static GatherLayout gather_layout(const ConvGeom& g) {
   l.total = l.window_weights + up(window_gemm_weight_bytes(g));
   return l;
 }
-static bool gather_from_window(const ConvGeom& g) { return window_gemm_supported(g) && g.Cp > 32; }
+static bool gather_from_window(const ConvGeom& g) { return window_gemm_supported(g); }
 
 size_t fused_workspace_bytes(const ConvGeom& g) {
   const int CpP = round_up(g.Cp, 128), CgP = round_up(g.Cg, 128);
@@ -989,7 +989,7 @@ static ConvGeom inverse_geom(const ConvGeom& g) {
   return r;
 }
 static bool scatter_from_window(const ConvGeom& g) {
-  return g.Cg > 32 && g.M % g.OW == 0 && window_gemm_supported(inverse_geom(g)) &&
+  return g.M % g.OW == 0 && window_gemm_supported(inverse_geom(g)) &&
          (int64_t)g.H * g.W * g.K < ((int64_t)1 << 31);
 }
 // Scratch of the scatter run from the inverse plan (behind the forward plan's region).

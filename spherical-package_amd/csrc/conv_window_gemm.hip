@@ -406,8 +406,8 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
   }
 
   // weight tile of (k, chunk): TN rows of 32 values, 16-byte pieces e = tid + 256 i
-  constexpr int WPT = TN * kCC / 4 / kWgThreads;   // float4 per thread: 4 (TN = 128) or 2
-  static_assert(WPT == 4 || WPT == 2, "weight tile of 128 or 64 rows");
+  constexpr int WPT = TN * kCC / 4 / kWgThreads;   // float4 per thread: 4 (TN = 128), 2 or 1
+  static_assert(WPT == 4 || WPT == 2 || WPT == 1, "weight tile of 128, 64 or 32 rows");
   float4 w0, w1, w2, w3;   // (named registers: an array here ends up in scratch memory)
   w0 = w1 = w2 = w3 = make_float4(0.f, 0.f, 0.f, 0.f);
 #define SDK_LOAD_WEIGHTS(kv, chunkv)                                              \
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
     const float4* srcw = reinterpret_cast<const float4*>(                         \
         Wp + (((size_t)(kv) * chunks + (chunkv)) * CpP + n0) * kCC) + tid;        \
     w0 = srcw[0];                                                                 \
-    w1 = srcw[kWgThreads];                                                        \
+    if constexpr (WPT >= 2) w1 = srcw[kWgThreads];                                \
     if constexpr (WPT == 4) {                                                     \
       w2 = srcw[2 * kWgThreads];                                                  \
       w3 = srcw[3 * kWgThreads];                                                  \
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
   do {                                                                            \
     float* dstw = &As[bufv][(tid >> 3) * kWE + 4 * (tid & 7)];                    \
     *reinterpret_cast<float4*>(dstw) = w0;                                        \
-    *reinterpret_cast<float4*>(dstw + 32 * kWE) = w1;                             \
+    if constexpr (WPT >= 2) *reinterpret_cast<float4*>(dstw + 32 * kWE) = w1;     \
     if constexpr (WPT == 4) {                                                     \
       *reinterpret_cast<float4*>(dstw + 64 * kWE) = w2;                           \
       *reinterpret_cast<float4*>(dstw + 96 * kWE) = w3;                           \
@@ -599,7 +599,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
 
 
 bool window_gemm_supported(const ConvGeom& g) {
-  return plan_supported(g) && g.Cp > 32 && g.B <= 65535 &&
+  return plan_supported(g) && g.Cp >= 1 && g.B <= 65535 &&
          (int64_t)g.H * g.W <= ((int64_t)1 << 24);
 }
 
@@ -646,8 +646,8 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   } else if (plan.big_lut == nullptr) {
     return SDK_OK;
   }
-  const bool wide = g.Cp > 64;
-  const int TN = wide ? 128 : 64;
+  const bool wide = g.Cp > 64, thin = g.Cp <= 32;
+  const int TN = wide ? 128 : (thin ? 32 : 64);
   const int n_tiles = (int)ceil_div(g.Cp, TN);
   // list entries are dealt to the XCDs in eighths: whole multiples of 8 workgroups
   const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
@@ -661,9 +661,9 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   do {                                                                \
     if (big) WG3(MMv, NBv, kBigCap); else WG3(MMv, NBv, kRegionCap);  \
   } while (0)
-#define WG1(MMv)                              \
-  do {                                        \
-    if (wide) WG2(MMv, 4); else WG2(MMv, 2);  \
+#define WG1(MMv)                                                            \
+  do {                                                                      \
+    if (wide) WG2(MMv, 4); else if (thin) WG2(MMv, 1); else WG2(MMv, 2);    \
   } while (0)
   if (mm == kMmBf16) WG1(kMmBf16);
   else if (mm == kMmSplit) WG1(kMmSplit);
