@@ -755,12 +755,12 @@ static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const fl
     else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
     if (rc) return rc;
     float* wp = reinterpret_cast<float*>(base + t.window_partial);
-    rc = window_wgrad(g, plan, tl, pix, img, gW, wp, stream);
+    rc = window_wgrad(g, mm, plan, tl, pix, img, gW, wp, stream);
     if (rc) return rc;
     if (plan.big_lut != nullptr) {
       // big tiles from their big windows (the partial sums of the first launch have been added
       // up by then), what is left from global memory
-      rc = window_wgrad(g, plan, tl, pix, img, gW, wp, stream, true);
+      rc = window_wgrad(g, mm, plan, tl, pix, img, gW, wp, stream, true);
       if (rc) return rc;
       return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream,
                            tl.rest_small, tl.count + 3);

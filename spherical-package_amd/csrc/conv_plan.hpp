@@ -128,13 +128,13 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
                   const int* tile_list = nullptr, const int* tile_count = nullptr);
 
 // The same sums over the tiles of tl.inside, from an LDS window with the column values built
-// straight into MFMA operands (conv_window_wgrad.hip; fp32 MFMA, K <= 10, at most four plan
-// rows per sample: build the lists with max_rows = 4).  partial: window_wgrad_partial_bytes(g).
+// straight into MFMA operands (conv_window_wgrad.hip; K <= 10, at most four plan rows per
+// sample: build the lists with max_rows = 4; mm: the matrix arithmetic).  partial: window_wgrad_partial_bytes(g).
 bool window_wgrad_supported(const ConvGeom& g, int mm);
 size_t window_wgrad_partial_bytes(const ConvGeom& g);
 // big: the sums over the tiles of tl.big, from their big windows.
-int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
-                 const float* img, float* gW, float* partial, hipStream_t stream,
-                 bool big = false);
+int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
+                 const float* pix, const float* img, float* gW, float* partial,
+                 hipStream_t stream, bool big = false);
 
 }  // namespace sdk

@@ -48,7 +48,7 @@ constexpr int kWwRows = 4; // plan rows per sample this kernel applies
 // With one wave per SIMD nothing else covers a global read, so that variant requests ahead what
 // it has registers for: the pixel-side tile and the plan rows of the next quarter, and the
 // offsets of the next tile's window, before a quarter's MFMAs.
-template <int KP, int R, int CAP>
+template <int KP, int R, int CAP, int MM>
 __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, const int* __restrict__ list,
@@ -276,6 +276,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
         }
       }
 
+      if constexpr (MM == kMmF32) {
       // ---- 16 MFMA steps over the quarter's pixels m = 16 h + s, as a three-stage pipeline:
       // while the MFMAs of step s issue, the window values of step s + 1 and the plan rows of
       // step s + 2 are in flight, so no LDS round trip stands between two steps' MFMAs.
@@ -358,6 +359,78 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
 #undef SDK_ROWS_ISSUE
 #undef SDK_VALS_ISSUE
 #undef SDK_BLEND
+      } else {
+        // ---- bf16 matrix unit (operands rounded to bf16, or split into three bf16 pieces):
+        // one instruction contracts 16 pixels, lane (j, h) supplying its row / channel for the
+        // eight pixels 8 h .. 8 h + 7 of the group.  A lane therefore builds eight column values
+        // per sample and instruction from the window (the same reads and multiply-adds per
+        // pixel as above) and takes its eight values of a row of the pixel-side tile as two
+        // 16-byte reads.  The matrix unit is a small part of the time here; the kernel is bound
+        // by the operand construction.
+        constexpr int KW = KP + R;
+#pragma unroll 1
+        for (int grp = 0; grp < 2; ++grp) {
+          const int m0 = 16 * grp + 8 * h;   // first of this lane's eight pixels of the quarter
+          Bf16Frag b16[KW];
+          Bf16Split b3[MM == kMmSplit ? KW : 1];
+#pragma unroll
+          for (int c = 0; c < KW; ++c) {
+            const int k = c < KP ? wave * KP + c : 4 * KP + (c - KP);
+            const int4* rp = reinterpret_cast<const int4*>(rowsL + (k * kWwQ + m0) * kWwRows);
+            float bv[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const int4 r01 = rp[2 * i], r23 = rp[2 * i + 1];
+              const float v0 = *reinterpret_cast<const float*>(regb + r01.x);
+              const float v1 = *reinterpret_cast<const float*>(regb + r01.z);
+              const float v2 = *reinterpret_cast<const float*>(regb + r23.x);
+              const float v3 = *reinterpret_cast<const float*>(regb + r23.z);
+              float t = __int_as_float(r01.y) * v0;
+              t = __builtin_fmaf(__int_as_float(r01.w), v1, t);
+              t = __builtin_fmaf(__int_as_float(r23.y), v2, t);
+              bv[i] = __builtin_fmaf(__int_as_float(r23.w), v3, t);
+            }
+            if constexpr (MM == kMmSplit) b3[c] = split_bf16x8(bv);
+            else b16[c] = pack_bf16x8(bv);
+          }
+          // A fragments: rows 32 a + j (and 32 wave + j for the remaining samples)
+          auto a_values = [&](int row, float (&f)[8]) {
+            const float4* ap = reinterpret_cast<const float4*>(gt + row * kWwG + m0);
+            const float4 lo = ap[0], hi = ap[1];
+            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+            f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+          };
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            if constexpr (KP > 0) {
+              float f[8];
+              a_values(32 * a + j, f);
+              if constexpr (MM == kMmSplit) {
+                const Bf16Split a3 = split_bf16x8(f);
+#pragma unroll
+                for (int kk = 0; kk < KP; ++kk) accF[kk][a] = mfma_split(a3, b3[kk], accF[kk][a]);
+              } else {
+                const Bf16Frag a16 = pack_bf16x8(f);
+#pragma unroll
+                for (int kk = 0; kk < KP; ++kk) accF[kk][a] = mfma_bf16(a16, b16[kk], accF[kk][a]);
+              }
+            }
+          }
+          if constexpr (R > 0) {
+            float f[8];
+            a_values(32 * wave + j, f);
+            if constexpr (MM == kMmSplit) {
+              const Bf16Split a3 = split_bf16x8(f);
+#pragma unroll
+              for (int r = 0; r < R; ++r) accR[r] = mfma_split(a3, b3[KP + r], accR[r]);
+            } else {
+              const Bf16Frag a16 = pack_bf16x8(f);
+#pragma unroll
+              for (int r = 0; r < R; ++r) accR[r] = mfma_bf16(a16, b16[KP + r], accR[r]);
+            }
+          }
+        }
+      }
     }
   }
 
@@ -433,7 +506,8 @@ WwGrid ww_grid(const ConvGeom& g, int tiles, bool big) {
 bool window_wgrad_supported(const ConvGeom& g, int mm) {
   // (every wave multiplies four 32-row blocks: with 64 rows or fewer half of that is padding,
   // and the plan-driven kernel, which splits the pixels instead, is the faster one)
-  return mm == kMmF32 && planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 64 &&
+  (void)mm;   // every matrix arithmetic
+  return planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 64 &&
          (int64_t)g.H * g.W <= ((int64_t)1 << 24);
 }
 
@@ -445,8 +519,9 @@ size_t window_wgrad_partial_bytes(const ConvGeom& g) {
   return (size_t)std::max(w.slots, wb.slots) * w.nreg * kWwThreads * sizeof(float);
 }
 
-int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* pix,
-                 const float* img, float* gW, float* partial, hipStream_t stream, bool big) {
+int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
+                 const float* pix, const float* img, float* gW, float* partial,
+                 hipStream_t stream, bool big) {
   if (big && plan.big_lut == nullptr) return SDK_OK;
   const WwGrid w = ww_grid(g, plan.tiles, big);
   const int* list = big ? tl.big : tl.inside;
@@ -456,10 +531,16 @@ int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const
   const int vec4 = (g.OW % 4 == 0 && TX >= 16 && reinterpret_cast<uintptr_t>(pix) % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)w.slots);
   const int KP = g.K / 4, R = g.K % 4;
-#define WW2(KPv, Rv, CAPv)                                                                       \
-  launch(window_wgrad_kernel<KPv, Rv, CAPv>, grid, dim3(kWwThreads), stream, pix, img, plan.hdr, \
-         plan.ns, plan.taps, list, count, partial, g.Cg, g.H, g.W, g.Cp, plan.S, plan.pt,        \
-         w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4, plan.big_lut)
+#define WW3(KPv, Rv, CAPv, MMv)                                                                  \
+  launch(window_wgrad_kernel<KPv, Rv, CAPv, MMv>, grid, dim3(kWwThreads), stream, pix, img,      \
+         plan.hdr, plan.ns, plan.taps, list, count, partial, g.Cg, g.H, g.W, g.Cp, plan.S,       \
+         plan.pt, w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4, plan.big_lut)
+#define WW2(KPv, Rv, CAPv)                                                       \
+  do {                                                                           \
+    if (mm == kMmBf16) WW3(KPv, Rv, CAPv, kMmBf16);                              \
+    else if (mm == kMmSplit) WW3(KPv, Rv, CAPv, kMmSplit);                       \
+    else WW3(KPv, Rv, CAPv, kMmF32);                                             \
+  } while (0)
 #define WW(KPv, Rv)                                                   \
   do {                                                                \
     if (big) WW2(KPv, Rv, kBigCap); else WW2(KPv, Rv, kRegionCap);    \
@@ -478,6 +559,7 @@ int window_wgrad(const ConvGeom& g, const Plan& plan, const TileLists& tl, const
   }
 #undef WW
 #undef WW2
+#undef WW3
   SDK_LAUNCH_CHECK(big ? "window_wgrad(big)" : "window_wgrad");
   const int kinds0 = w.c_chunks * w.n_tiles, total = (int)g.B * w.groups;
   const int parts = (int)std::min<int64_t>(std::min(total, 16),
