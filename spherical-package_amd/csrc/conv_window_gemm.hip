@@ -336,7 +336,10 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
 // CAP: elements of the LDS window.  kRegionCap: the tiles of `list` lie inside their window,
 // two workgroups share a CU.  kBigCap: `list` holds big tiles, whose window is their list in
 // big_lut; it takes most of a CU's LDS and one workgroup runs per CU.
-template <int MM, int NB, int CAP>
+// XR: plan rows beyond the first four that are requested ahead as well (0 or 2).  The lists of
+// an inverse plan are as long as targets have sources: at unit scale a third of the samples
+// of a weighted bispherical map have six rows somewhere in a tile.
+template <int MM, int NB, int CAP, int XR>
 __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_gemm_kernel(
     const float* __restrict__ img, const int* __restrict__ hdr, const int* __restrict__ ns,
     const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
@@ -438,22 +441,25 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
   // its latency.  Samples with more than four rows fetch the others when they need them.
   constexpr int RB = 4;
   int2 rows[RB], rows_next[RB];
-#define SDK_LOAD_ROWS(dst, kv, r0v)                                               \
+  int2 xrows[XR > 0 ? XR : 1], xrows_next[XR > 0 ? XR : 1];
+#define SDK_LOAD_ROWS_N(dst, kv, r0v, NR)                                         \
   do {                                                                            \
-    _Pragma("unroll") for (int u = 0; u < RB; ++u)                                \
+    _Pragma("unroll") for (int u = 0; u < (NR); ++u)                              \
       dst[u] = rows_p[((size_t)(kv) * S + min((r0v) + u, S - 1)) * 128];          \
   } while (0)
+#define SDK_LOAD_ROWS(dst, kv, r0v) SDK_LOAD_ROWS_N(dst, kv, r0v, RB)
   // col[] += the taps of up to four rows (FIRST: col[] = ..., the product of the first row
   // instead of a register clear and a multiply-add)
-#define SDK_GATHER_ROWS(src, r0v, FIRST)                                          \
+#define SDK_GATHER_ROWS(src, r0v, FIRST) SDK_GATHER_ROWS_N(src, r0v, FIRST, RB)
+#define SDK_GATHER_ROWS_N(src, r0v, FIRST, NR)                                    \
   do {                                                                            \
     int e[RB];                                                                    \
     float co[RB];                                                                 \
-    _Pragma("unroll") for (int u = 0; u < RB; ++u) {                              \
+    _Pragma("unroll") for (int u = 0; u < (NR); ++u) {                            \
       co[u] = (r0v) + u < n_rows ? __int_as_float(src[u].y) : 0.0f;               \
       e[u] = co[u] != 0.0f ? src[u].x : RS;                                       \
     }                                                                             \
-    _Pragma("unroll") for (int u = 0; u < RB; ++u) {                              \
+    _Pragma("unroll") for (int u = 0; u < (NR); ++u) {                            \
       const float4* rp = reinterpret_cast<const float4*>(region + e[u] * kWE + 16 * h); \
       const float4 d0 = rp[0], d1 = rp[1], d2 = rp[2], d3 = rp[3];                \
       const float d[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w,        \
@@ -467,6 +473,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
   SDK_LOAD_WEIGHTS(0, 0);
   int n_rows = ns[(size_t)tile * K];
   SDK_LOAD_ROWS(rows, 0, 0);
+  if constexpr (XR > 0) SDK_LOAD_ROWS_N(xrows, 0, RB, XR);
   for (int chunk = 0; chunk < chunks; ++chunk) {
     const int c0 = chunk * kCC;
     __syncthreads();   // every wave is done with the previous chunk's window (and src is built)
@@ -519,6 +526,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
       const int chunk_n = last_k ? (chunk + 1 < chunks ? chunk + 1 : 0) : chunk;
       SDK_LOAD_WEIGHTS(kn, chunk_n);
       SDK_LOAD_ROWS(rows_next, kn, 0);
+      if constexpr (XR > 0) SDK_LOAD_ROWS_N(xrows_next, kn, RB, XR);
       const int n_rows_next = __builtin_amdgcn_readfirstlane(ns_l[kn]);
       asm volatile("" ::: "memory");   // the requests stay here, ahead of the gather and the MFMAs
 
@@ -526,7 +534,8 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
       float colv[16];
       SDK_GATHER_ROWS(rows, 0, true);
       if (n_rows > RB) {
-        for (int r0 = RB; r0 < n_rows; r0 += RB) {
+        if constexpr (XR > 0) SDK_GATHER_ROWS_N(xrows, RB, false, XR);
+        for (int r0 = RB + XR; r0 < n_rows; r0 += RB) {
           int2 more[RB];
           SDK_LOAD_ROWS(more, k, r0);
           SDK_GATHER_ROWS(more, r0, false);
@@ -574,6 +583,10 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
       n_rows = n_rows_next;
 #pragma unroll
       for (int u = 0; u < RB; ++u) rows[u] = rows_next[u];
+      if constexpr (XR > 0) {
+#pragma unroll
+        for (int u = 0; u < XR; ++u) xrows[u] = xrows_next[u];
+      }
     }
   }
   // ---- epilogue: store.  Accumulator register v of lane l: row 8*(v/4) + 4*h + v%4
@@ -592,7 +605,9 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
 #undef SDK_LOAD_WEIGHTS
 #undef SDK_STORE_WEIGHTS
 #undef SDK_LOAD_ROWS
+#undef SDK_LOAD_ROWS_N
 #undef SDK_GATHER_ROWS
+#undef SDK_GATHER_ROWS_N
 }
 
 }  // namespace
@@ -653,10 +668,17 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
   const int* list = big ? tl.big : tl.inside;
   const int* count = big ? tl.count + 2 : tl.count;
-#define WG3(MMv, NBv, CAPv)                                                                    \
-  launch(window_gemm_kernel<MMv, NBv, CAPv>, grid, dim3(kWgThreads), stream, img, plan.hdr,    \
-         plan.ns, plan.taps, list, count, (const float*)weights, bias, pix, g.Cg, g.H, g.W,    \
-         g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles, gate, plan.big_lut)
+  // (an inverse plan is what this function is given with swapped weights)
+  const bool more_rows = swapped && plan.S > 4;
+#define WG4(MMv, NBv, CAPv, XRv)                                                               \
+  launch(window_gemm_kernel<MMv, NBv, CAPv, XRv>, grid, dim3(kWgThreads), stream, img,         \
+         plan.hdr, plan.ns, plan.taps, list, count, (const float*)weights, bias, pix, g.Cg,    \
+         g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles, gate,         \
+         plan.big_lut)
+#define WG3(MMv, NBv, CAPv)                                                    \
+  do {                                                                         \
+    if (more_rows) WG4(MMv, NBv, CAPv, 2); else WG4(MMv, NBv, CAPv, 0);        \
+  } while (0)
 #define WG2(MMv, NBv)                                                 \
   do {                                                                \
     if (big) WG3(MMv, NBv, kBigCap); else WG3(MMv, NBv, kRegionCap);  \
@@ -671,6 +693,7 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
 #undef WG1
 #undef WG2
 #undef WG3
+#undef WG4
   SDK_LAUNCH_CHECK(big ? "window_gemm(big)" : "window_gemm");
   return SDK_OK;
 }
