@@ -17,6 +17,11 @@
 // v_mfma_f32_32x32x2_f32; each wavefront owns a 64 x 64 block of the 128 x 128
 // (or 64 x 256) workgroup tile as 2 x 2 MFMA accumulators.
 //
+// These kernels read their operands from global memory.  For a map that has a tap plan
+// (conv_plan.hpp) the drivers at the end of this file run them only on the tiles that the
+// plan's LDS-window kernels (conv_window_gemm.hip, conv_window_wgrad.hip) leave over, and as
+// the device-side fallback of the inverse plan.
+//
 // MFMA 32x32x2 f32 register layout used below (wave64, lane l):
 //   A operand: A[i = l % 32][k = l / 32]        B operand: B[k = l / 32][j = l % 32]
 //   D, 16 registers v: D[i = 8*(v/4) + 4*(l/32) + v%4][j = l % 32]
