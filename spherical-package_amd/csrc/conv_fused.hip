@@ -838,7 +838,7 @@ int fused_gather_gemm(const ConvGeom& g, int compute, const float* img, const fl
     const bool with_big = plan.big_lut != nullptr;
     if (with_big) {
       rc = window_gemm(g, mm, plan, tl, img, Wm, false, bias, pix,
-                       reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream, true);
+                       reinterpret_cast<float*>(ws + l.window_weights), nullptr, stream, kListBig);
       if (rc) return rc;
     }
     const int* rest_list = with_big ? tl.rest_small : tl.rest;
@@ -1133,17 +1133,24 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
         } else {
           rc = build_inverse_plan(g, map, wts, inv_ws + l.inverse, stream, &ip);
           if (rc) return rc;
-          rc = build_tile_lists(ip.plan, inv_ws + l.lists, stream, &tl);
+          rc = build_tile_lists(ip.plan, inv_ws + l.lists, stream, &tl, 0, kProductCap);
           if (rc) return rc;
         }
-        rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
-                         reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream);
+        float* ww = reinterpret_cast<float*>(inv_ws + l.window_weights);
+        // image tiles with few sources (the image finer than the pixel grid) in the product
+        // form where it exists, all others inside their window in the gather form
+        const bool product = window_product_supported(r, mm);
+        rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img, ww, ip.gate, stream,
+                         product ? kListInsideLarge : kListInside);
         if (rc) return rc;
+        if (product) {
+          rc = window_product(r, ip.plan, tl, pix, bias, img, ww, ip.gate, stream);
+          if (rc) return rc;
+        }
         const bool with_big = ip.plan.big_lut != nullptr;
         if (with_big) {
-          rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img,
-                           reinterpret_cast<float*>(inv_ws + l.window_weights), ip.gate, stream,
-                           true);
+          rc = window_gemm(r, mm, ip.plan, tl, pix, Wm, true, bias, img, ww, ip.gate, stream,
+                           kListBig);
           if (rc) return rc;
         }
         const int* rest_list = with_big ? tl.rest_small : tl.rest;
@@ -1334,7 +1341,8 @@ int build_cached_plan(const ConvGeom& g, const float* map, const float* wts, voi
   if (l.has_inverse) {
     rc = build_inverse_plan(g, map, wts, b + l.inverse, stream, &cp.inverse);
     if (rc) return rc;
-    rc = build_tile_lists(cp.inverse.plan, b + l.inverse_lists, stream, &cp.inverse_lists, 0);
+    rc = build_tile_lists(cp.inverse.plan, b + l.inverse_lists, stream, &cp.inverse_lists, 0,
+                          kProductCap);
     if (rc) return rc;
   }
   return SDK_OK;

@@ -74,31 +74,49 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
 // leave their sums for a second, summing kernel; nullptr: they add to gW themselves.
 // The plan's tiles by class, on the device (conv_window_gemm.hip), each in ascending order:
 // those whose taps all lie inside their window and the others (count[0], count[1] entries);
-// the others again as big tiles and the remainder (count[2], count[3]).
+// the others again as big tiles and the remainder (count[2], count[3]); and, when the lists
+// were built with small_cap > 0 (kProductCap for an inverse plan, whose small windows can run
+// in the product form below), `inside` again as the tiles with a window of at most small_cap
+// elements and the remainder (count[4], count[5]).
 struct TileLists {
   const int* inside;
   const int* rest;
   const int* big;
   const int* rest_small;
+  const int* product;
+  const int* inside_large;
   const int* count;
 };
 // max_rows > 0: tiles with a sample of more than max_rows plan rows (h[5]) are neither inside
 // nor big.
 size_t tile_lists_bytes(const ConvGeom& g);
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
-                     int max_rows = 0);
+                     int max_rows = 0, int small_cap = 0);
 
 // pix[b] = Wm x im2col(img[b]) + bias on the tiles of tl.inside, gathered from an LDS window.
 // g: the contraction's geometry (gather side = img).  swapped: Wm is [Cg, Cp * K] instead of
 // [Cp, Cg * K].  weights: window_gemm_weight_bytes(g) bytes of scratch for the re-laid-out
 // weight matrix.  gate (optional): the kernel runs only if *gate == 0.
-// big: the same on the tiles of tl.big, from their big windows; `weights` must hold what an
-// earlier call with big = false left there (same g, mm, Wm).
+// kListBig: `weights` must hold what an earlier call for one of the other lists left there
+// (same g, mm, Wm).
 bool window_gemm_supported(const ConvGeom& g);
 size_t window_gemm_weight_bytes(const ConvGeom& g);
+// which: the tiles of tl.inside, tl.big, or tl.inside_large (what window_product leaves).
+constexpr int kListInside = 0, kListBig = 1, kListInsideLarge = 2;
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                 const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
-                float* weights, const int* gate, hipStream_t stream, bool big = false);
+                float* weights, const int* gate, hipStream_t stream, int which = kListInside);
+
+// Product form of the same contraction for the tiles of tl.product of an inverse plan (image
+// tiles whose sources are at most kProductCap pixels: up-sampling and strided maps): per sample
+// the weights are applied at the source pixels and the image pixels gather the products from
+// LDS, which is half the matrix work of gathering first or less.  fp32 MFMA; g.Cg <= 256.
+// weights: what window_gemm(..., kListInsideLarge) left for the same g, Wm.
+constexpr int kProductCap = 64;
+bool window_product_supported(const ConvGeom& g, int mm);
+int window_product(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* img,
+                   const float* bias, float* pix, const float* weights, const int* gate,
+                   hipStream_t stream);
 
 // The scatter of geometry g regrouped by target as a plan over tiles of the image grid, whose
 // windows lie in the pixel grid; valid only if *gate == 0 after it was built (a target with

@@ -210,7 +210,11 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
   bool whole = bb[0] > bb[1] || (bb[1] - bb[0] + 1) * min(bb[3] - bb[2] + 1, OW) <= kRegionCap;
   int listed = -1;   // >= 0: elements of a listed window
   int big = -1;      // >= 0: elements of the tile's big window
-  if (!whole) {
+  // A box that fits may still hold far more pixels than the tile has sources (the sources of an
+  // up-sampling map on a mesh: 60 of them spread over a few hundred indices): the sorted list
+  // of the distinct sources then makes the smaller window, small enough for the product form.
+  const bool sparse_box = whole && bb[0] <= bb[1] && rg.RS > kProductCap;
+  if (!whole || sparse_box) {
     // the distinct sources of the tile may still fit: try a listed window
     set_clear(wset);
     __syncthreads();
@@ -221,7 +225,9 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
     }
     __syncthreads();
     const int distinct = set_finish(wset);
-    if (distinct >= 0 && distinct <= kRegionCap) {
+    if (sparse_box && (distinct < 0 || distinct > kProductCap)) {
+      // the box stays
+    } else if (distinct >= 0 && distinct <= kRegionCap) {
       listed = distinct;
       rg.ry0 = 0;
       rg.rx0 = 0;
@@ -286,35 +292,45 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
 //   lists[0 .. tiles)            tiles inside their window (header value 4 != 0), count[0] of them
 //   lists[tiles .. 2 tiles)      the others, count[1]
 //   lists[2 tiles .. 3 tiles)    those of the others that are big tiles (header value 7), count[2]
-//   lists[3 tiles .. 4 tiles)    ... and those that have none, count[3]
+//   lists[3 tiles .. 4 tiles)    ... and those that are not, count[3]
+//   lists[4 tiles .. 5 tiles)    small_cap > 0: the tiles of the first list whose window has at
+//                                most small_cap elements, count[4]
+//   lists[5 tiles .. 6 tiles)    ... and the others of the first list, count[5]
 // max_rows > 0: a tile with a sample of more rows is neither inside nor big.
 __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict__ hdr, int tiles,
                                                           int* __restrict__ lists,
-                                                          int* __restrict__ count, int max_rows) {
-  __shared__ int wave_n[4][16];
-  __shared__ int base[4];
+                                                          int* __restrict__ count, int max_rows,
+                                                          int small_cap) {
+  constexpr int NC = 6;
+  __shared__ int wave_n[NC][16];
+  __shared__ int base[NC];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid < 4) base[tid] = 0;
+  if (tid < NC) base[tid] = 0;
   __syncthreads();
   for (int t0 = 0; t0 < tiles; t0 += 1024) {
     const int t = t0 + tid;
     const bool live = t < tiles;
     const bool rows_ok = live && (max_rows <= 0 || hdr[t * kHdrStride + 5] <= max_rows);
-    bool cls[4];
-    cls[0] = rows_ok && hdr[t * kHdrStride + 4] != 0;
-    cls[1] = live && !cls[0];
+    const bool fit = rows_ok && hdr[t * kHdrStride + 4] != 0;
+    const bool small = fit && small_cap > 0 &&
+                       hdr[t * kHdrStride + 2] * hdr[t * kHdrStride + 3] <= small_cap;
+    bool cls[NC];
+    cls[0] = fit;
+    cls[1] = live && !fit;
     cls[2] = cls[1] && rows_ok && hdr[t * kHdrStride + 7] != 0;
     cls[3] = cls[1] && !cls[2];
-    unsigned long long mask[4];
+    cls[4] = small;
+    cls[5] = fit && !small;
+    unsigned long long mask[NC];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < NC; ++c) {
       mask[c] = __ballot(cls[c]);
       if (lane == 0) wave_n[c][wave] = __popcll(mask[c]);
     }
     __syncthreads();
     const unsigned long long below = (1ull << lane) - 1ull;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < NC; ++c) {
       if (cls[c]) {
         int o = base[c];
         for (int w = 0; w < wave; ++w) o += wave_n[c][w];
@@ -322,14 +338,14 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
       }
     }
     __syncthreads();
-    if (tid < 4) {
+    if (tid < NC) {
       int a = 0;
       for (int w = 0; w < 16; ++w) a += wave_n[tid][w];
       base[tid] += a;
     }
     __syncthreads();
   }
-  if (tid < 4) count[tid] = base[tid];
+  if (tid < NC) count[tid] = base[tid];
 }
 
 
@@ -610,6 +626,223 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
 #undef SDK_GATHER_ROWS_N
 }
 
+
+// ---------------------------------------------------------------------------
+// Product form.  In the inverse direction of an up-sampling or strided map the image is finer
+// than the pixel grid: the 128 image pixels of a tile draw on few source pixels (a quarter as
+// many at stride 2, plus a border), and gathering first means contracting all 128 of them
+// against every sample.  Here, per sample k,
+//
+//   T_k[s][n] = sum_c W[n, (c, k)] * src[c][s]          for the tile's source pixels s  (MFMA)
+//   out[n][u] += sum_r coefficient(u, k, r) * T_k[source(u, k, r)][n]                   (LDS)
+//
+// The window of source pixels (at most kProductCap = 64, every channel) stays in LDS for the
+// whole tile and feeds the MFMAs as it lies: no operand is built.  T_k goes through LDS, and a
+// thread gathers, for its image pixel and 64 of the 128 produced channels, the rows its plan
+// rows name (window index, coefficient).
+//
+//   workgroup = one image tile x 128 produced channels x one batch element
+//   MFMA role:   wave w = source pixels 32 (w % 2) .. + 31 x produced channels 64 (w / 2) .. + 63
+//   gather role: thread t = image pixel t % 128 of the tile, produced channels 64 (t / 128) .. + 63
+//
+// CH: 32-channel chunks of the gathered tensor the window holds (2, 4 or 8).
+// ---------------------------------------------------------------------------
+
+template <int CH, int NBP>
+__global__ __launch_bounds__(kWgThreads, CH <= 4 ? 2 : 1) void window_product_kernel(
+    const float* __restrict__ img, const int* __restrict__ hdr, const int* __restrict__ ns,
+    const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
+    const float* __restrict__ Wp, const float* __restrict__ bias, float* __restrict__ pix, int Cg,
+    int H, int W, int Cp, int K, int S, int CpP, int chunks, PixelTiling pt, int n_tiles,
+    const int* __restrict__ gate) {
+  if (gate != nullptr && *gate != 0) return;
+  constexpr int XS = 32 * CH + 4;   // floats per source pixel in the window
+  constexpr int kPrT = 64 * NBP + 4;   // floats per row of T: the channels + 4 of skew
+  // Two copies of T for the 64-channel form: the products of sample k + 1 are written while
+  // other waves still gather sample k, and one barrier per sample is enough.
+  constexpr int TB = NBP == 1 ? 2 : 1;
+  constexpr int TSZ = (kProductCap + 1) * kPrT;   // (+ a row of zeros)
+  __shared__ __align__(16) float X[kProductCap * XS];
+  __shared__ __align__(16) float Tl[TB * TSZ];
+  __shared__ int src[kProductCap];
+  __shared__ int ns_l[kPlanKMax];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int j = lane & 31, h = lane >> 5;
+  const int cnt = *count;
+  const int per = (cnt + 7) >> 3;
+  const int wg = blockIdx.x / n_tiles;
+  const int slot = (wg & 7) * per + (wg >> 3);
+  if ((wg >> 3) >= per || slot >= cnt) return;
+  const int tile = list[slot];
+  constexpr int TN = 64 * NBP, HN = TN / 2;   // channels per workgroup, per wave pair / thread
+  const int n0 = (blockIdx.x % n_tiles) * TN;
+  const int ty0 = (tile / pt.tiles_x) * pt.TY(), tx0 = (tile % pt.tiles_x) << pt.tx_shift;
+  const int M = pt.OH * pt.OW;
+  const size_t HW = (size_t)H * W;
+  const float* img_b = img + (size_t)blockIdx.y * Cg * HW;
+
+  const int RS = min(hdr[tile * kHdrStride + 2] * hdr[tile * kHdrStride + 3], kProductCap);
+  load_region_lut(hdr + (size_t)tile * kHdrStride, RS, src);
+  for (int k = tid; k < K; k += kWgThreads) ns_l[k] = ns[(size_t)tile * K + k];
+  for (int i = tid; i < TB * kPrT; i += kWgThreads)
+    Tl[(i / kPrT) * TSZ + kProductCap * kPrT + i % kPrT] = 0.0f;
+  __syncthreads();
+  {
+    // window: lane = source pixel, wave w = channels 8w .. 8w+7 of every chunk; the channels of
+    // a chunk lie in the order the MFMA steps take them (as in window_gemm_kernel)
+    const int o = lane < RS ? src[lane] : -1;
+    for (int chunk = 0; chunk < chunks; ++chunk) {
+      const int cw = chunk * kCC + 8 * wave;
+      const char* cbase = reinterpret_cast<const char*>(img_b + (size_t)min(cw, Cg - 1) * HW);
+      const unsigned plane = (unsigned)HW * 4u;
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const bool ok = o >= 0 && cw + i < Cg;
+        const float d = *reinterpret_cast<const float*>(
+            cbase + (ok ? (unsigned)i * plane + (unsigned)o * 4u : 0u));
+        v[i] = ok ? d : 0.0f;
+      }
+      float* dst = X + lane * XS + chunk * kCC;
+      *reinterpret_cast<float4*>(dst + 4 * wave) = make_float4(v[0], v[2], v[4], v[6]);
+      *reinterpret_cast<float4*>(dst + 16 + 4 * wave) = make_float4(v[1], v[3], v[5], v[7]);
+    }
+  }
+
+  // gather role
+  const int p_local = tid & 127, hh = tid >> 7;
+  const int2* rows_p = taps + (size_t)tile * K * S * 128 + p_local;
+  float oacc[HN];
+#pragma unroll
+  for (int i = 0; i < HN; ++i) {
+    const int n = n0 + HN * hh + i;
+    oacc[i] = (bias != nullptr && n < Cp) ? bias[n] : 0.0f;
+  }
+  // MFMA role
+  const int pb = wave & 1, cb = wave >> 1;
+  const float* xrow = X + (32 * pb + j) * XS + 16 * h;
+  // weights of (k, chunk), rows n0 + HN cb + 32 a + j, this lane's 16 values: 4 x 16 bytes
+  auto weight_ptr = [&](int k, int chunk, int a) {
+    return reinterpret_cast<const float4*>(
+        Wp + (((size_t)k * chunks + chunk) * CpP + n0 + HN * cb + 32 * a + j) * kCC + 16 * h);
+  };
+  // Weights come from global memory (the L2) straight into A operands.  Where the registers
+  // allow it (WS) all of a sample's weights are requested a whole sample ahead; otherwise one
+  // chunk ahead, which at 16 MFMAs per block and chunk does not always cover the read.
+  constexpr bool WS = NBP == 1 && CH <= 4;
+  constexpr int WC = WS ? CH : 1;
+  float4 wa[WC][NBP][4], wn[WC][NBP][4];
+#pragma unroll
+  for (int c = 0; c < WC; ++c)
+#pragma unroll
+    for (int a = 0; a < NBP; ++a)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) wa[c][a][q] = weight_ptr(0, min(c, chunks - 1), a)[q];
+  __syncthreads();   // the window is complete
+
+  for (int k = 0; k < K; ++k) {
+    const int n_rows = ns_l[k];
+    int2 rows[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) rows[u] = rows_p[((size_t)k * S + min(u, S - 1)) * 128];
+    floatx16 acc[NBP];
+#pragma unroll
+    for (int a = 0; a < NBP; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][v] = 0.0f;
+#define SDK_PRODUCT_CHUNK(chunkv, wv)                                                        \
+  do {                                                                                        \
+    const float4* xp = reinterpret_cast<const float4*>(xrow + (chunkv) * kCC);                \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                           \
+      const float4 b = xp[q];                                                                 \
+      _Pragma("unroll") for (int a = 0; a < NBP; ++a) {                                       \
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[a][q].x, b.x, acc[a], 0, 0, 0);      \
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[a][q].y, b.y, acc[a], 0, 0, 0);      \
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[a][q].z, b.z, acc[a], 0, 0, 0);      \
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[a][q].w, b.w, acc[a], 0, 0, 0);      \
+      }                                                                                       \
+    }                                                                                         \
+  } while (0)
+    if constexpr (WS) {
+      const int kn = k + 1 < K ? k + 1 : 0;   // (after the last sample: the first again, unused)
+#pragma unroll
+      for (int c = 0; c < WC; ++c)
+#pragma unroll
+        for (int a = 0; a < NBP; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wn[c][a][q] = weight_ptr(kn, min(c, chunks - 1), a)[q];
+#pragma unroll
+      for (int c = 0; c < WC; ++c)
+        if (c < chunks) SDK_PRODUCT_CHUNK(c, wa[c]);
+#pragma unroll
+      for (int c = 0; c < WC; ++c)
+#pragma unroll
+        for (int a = 0; a < NBP; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wa[c][a][q] = wn[c][a][q];
+    } else {
+      for (int chunk = 0; chunk < chunks; ++chunk) {
+        // the next weights (of the next sample after the last chunk; the first ones again at the end)
+        const bool last_c = chunk + 1 == chunks;
+        const int kn = last_c ? (k + 1 < K ? k + 1 : 0) : k, cn = last_c ? 0 : chunk + 1;
+#pragma unroll
+        for (int a = 0; a < NBP; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wn[0][a][q] = weight_ptr(kn, cn, a)[q];
+        SDK_PRODUCT_CHUNK(chunk, wa[0]);
+#pragma unroll
+        for (int a = 0; a < NBP; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wa[0][a][q] = wn[0][a][q];
+      }
+    }
+#undef SDK_PRODUCT_CHUNK
+    if (TB == 1 && k > 0) __syncthreads();   // the gather of the sample before is done with T
+    float* Tk = Tl + (TB == 2 ? (k & 1) * TSZ : 0);
+    // T[s][n]: accumulator register v of lane (j, h): row n = 8 (v / 4) + 4 h + v % 4, column s = j
+    {
+      float* trow = Tk + (32 * pb + j) * kPrT + HN * cb + 4 * h;
+#pragma unroll
+      for (int a = 0; a < NBP; ++a)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+          *reinterpret_cast<float4*>(trow + 32 * a + 8 * g4) =
+              make_float4(acc[a][4 * g4], acc[a][4 * g4 + 1], acc[a][4 * g4 + 2], acc[a][4 * g4 + 3]);
+    }
+    __syncthreads();
+    // gather: rows of this thread's image pixel (a row past the sample's count or of weight 0
+    // reads the row of zeros)
+    auto add_row = [&](int2 ec) {
+      const float co = __int_as_float(ec.y);
+      const int e = co != 0.0f ? min(ec.x, kProductCap - 1) : kProductCap;
+      const float4* tp = reinterpret_cast<const float4*>(Tk + e * kPrT + HN * hh);
+#pragma unroll
+      for (int i = 0; i < HN / 4; ++i) {
+        const float4 t = tp[i];
+        oacc[4 * i + 0] = __builtin_fmaf(co, t.x, oacc[4 * i + 0]);
+        oacc[4 * i + 1] = __builtin_fmaf(co, t.y, oacc[4 * i + 1]);
+        oacc[4 * i + 2] = __builtin_fmaf(co, t.z, oacc[4 * i + 2]);
+        oacc[4 * i + 3] = __builtin_fmaf(co, t.w, oacc[4 * i + 3]);
+      }
+    };
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (u < n_rows) add_row(rows[u]);
+    for (int r = 4; r < n_rows; ++r) add_row(rows_p[((size_t)k * S + r) * 128]);
+  }
+  // ---- store
+  const int oy = ty0 + (p_local >> pt.tx_shift), ox = tx0 + (p_local & (pt.TX() - 1));
+  if (oy < pt.OH && ox < pt.OW) {
+    float* out = pix + (size_t)blockIdx.y * Cp * M + (size_t)oy * pt.OW + ox;
+#pragma unroll
+    for (int i = 0; i < HN; ++i) {
+      const int n = n0 + HN * hh + i;
+      if (n < Cp) out[(size_t)n * M] = oacc[i];
+    }
+  }
+}
+
 }  // namespace
 
 
@@ -626,7 +859,7 @@ size_t window_gemm_weight_bytes(const ConvGeom& g) {
 
 size_t tile_lists_bytes(const ConvGeom& g) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  return ((size_t)4 * pt.tiles_x * pt.tiles_y + 4) * sizeof(int);
+  return ((size_t)6 * pt.tiles_x * pt.tiles_y + 8) * sizeof(int);
 }
 
 void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
@@ -635,30 +868,33 @@ void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
   out->rest = lists + plan.tiles;
   out->big = lists + (size_t)2 * plan.tiles;
   out->rest_small = lists + (size_t)3 * plan.tiles;
-  out->count = lists + (size_t)4 * plan.tiles;
+  out->product = lists + (size_t)4 * plan.tiles;
+  out->inside_large = lists + (size_t)5 * plan.tiles;
+  out->count = lists + (size_t)6 * plan.tiles;
 }
 
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,
-                     int max_rows) {
+                     int max_rows, int small_cap) {
   load_tile_lists(plan, workspace, out);
   launch(tile_lists_kernel, dim3(1), dim3(1024), stream, plan.hdr, plan.tiles,
-         const_cast<int*>(out->inside), const_cast<int*>(out->count), max_rows);
+         const_cast<int*>(out->inside), const_cast<int*>(out->count), max_rows, small_cap);
   SDK_LAUNCH_CHECK("tile_lists");
   return SDK_OK;
 }
 
 int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                 const float* img, const float* Wm, bool swapped, const float* bias, float* pix,
-                float* weights, const int* gate, hipStream_t stream, bool big) {
+                float* weights, const int* gate, hipStream_t stream, int which) {
   const int CpP = (g.Cp + 127) / 128 * 128;
   const int chunks = (g.Cg + kCC - 1) / kCC;
+  const bool big = which == kListBig;
   if (!big) {
     const size_t total = (size_t)g.K * chunks * CpP * kCC;
     const int blocks = (int)std::min<size_t>((total + kWgThreads - 1) / kWgThreads, 2048);
     launch(window_weight_kernel, dim3(blocks), dim3(kWgThreads), stream, Wm, weights, g.Cp, g.Cg,
            g.K, CpP, chunks, mm != kMmF32 ? 1 : 0, swapped ? 1 : 0);
     SDK_LAUNCH_CHECK("window_weight");
-  } else if (plan.big_lut == nullptr) {
+  } else if (big && plan.big_lut == nullptr) {
     return SDK_OK;
   }
   const bool wide = g.Cp > 64, thin = g.Cp <= 32;
@@ -666,10 +902,12 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   const int n_tiles = (int)ceil_div(g.Cp, TN);
   // list entries are dealt to the XCDs in eighths: whole multiples of 8 workgroups
   const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
-  const int* list = big ? tl.big : tl.inside;
-  const int* count = big ? tl.count + 2 : tl.count;
+  const int* list = big ? tl.big : (which == kListInsideLarge ? tl.inside_large : tl.inside);
+  const int* count = big ? tl.count + 2 : (which == kListInsideLarge ? tl.count + 5 : tl.count);
   // (an inverse plan is what this function is given with swapped weights)
-  const bool more_rows = swapped && plan.S > 4;
+  // (wide layers only: with fewer MFMAs per sample the two extra requests cost more than the
+  // exposed reads they save; configuration 5's up-sampling layer 0.35 -> 0.38 ms)
+  const bool more_rows = swapped && plan.S > 4 && wide;
 #define WG4(MMv, NBv, CAPv, XRv)                                                               \
   launch(window_gemm_kernel<MMv, NBv, CAPv, XRv>, grid, dim3(kWgThreads), stream, img,         \
          plan.hdr, plan.ns, plan.taps, list, count, (const float*)weights, bias, pix, g.Cg,    \
@@ -695,6 +933,33 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
 #undef WG3
 #undef WG4
   SDK_LAUNCH_CHECK(big ? "window_gemm(big)" : "window_gemm");
+  return SDK_OK;
+}
+
+bool window_product_supported(const ConvGeom& g, int mm) {
+  return mm == kMmF32 && window_gemm_supported(g) && g.Cg <= 256;
+}
+
+int window_product(const ConvGeom& g, const Plan& plan, const TileLists& tl, const float* img,
+                   const float* bias, float* pix, const float* weights, const int* gate,
+                   hipStream_t stream) {
+  const int CpP = (g.Cp + 127) / 128 * 128;
+  const int chunks = (g.Cg + kCC - 1) / kCC;
+  const bool wide = g.Cp > 64;
+  const int n_tiles = (int)ceil_div(g.Cp, wide ? 128 : 64);
+  const dim3 grid((unsigned)((plan.tiles + 7) / 8 * 8 * n_tiles), (unsigned)g.B);
+#define WP2(CHv, NBPv)                                                                        \
+  launch(window_product_kernel<CHv, NBPv>, grid, dim3(kWgThreads), stream, img, plan.hdr,     \
+         plan.ns, plan.taps, tl.product, tl.count + 4, weights, bias, pix, g.Cg, g.H, g.W,    \
+         g.Cp, g.K, plan.S, CpP, chunks, plan.pt, n_tiles, gate)
+#define WP(CHv)                                     \
+  do {                                              \
+    if (wide) WP2(CHv, 2); else WP2(CHv, 1);        \
+  } while (0)
+  if (chunks <= 2) WP(2); else if (chunks <= 4) WP(4); else WP(8);
+#undef WP
+#undef WP2
+  SDK_LAUNCH_CHECK("window_product");
   return SDK_OK;
 }
 
