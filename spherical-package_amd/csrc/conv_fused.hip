@@ -773,6 +773,22 @@ static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const fl
     return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream, tl.rest,
                          tl.count + 1);
   }
+  if (window_wgrad_narrow_supported(g, mm) && window_wgrad_partial_bytes(g) != 0) {
+    // narrow layers with one plan row per sample: the tiles inside their window from the
+    // window, the others from global memory
+    const WgradTail t = wgrad_tail(g);
+    char* base = wgrad_tail_base(g, workspace);
+    TileLists tl;
+    int rc = SDK_OK;
+    if (lists4 != nullptr) tl = *lists4;
+    else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
+    if (rc) return rc;
+    rc = window_wgrad_narrow(g, plan, tl, pix, img, gW,
+                             reinterpret_cast<float*>(base + t.window_partial), stream);
+    if (rc) return rc;
+    return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream, tl.rest,
+                         tl.count + 1);
+  }
   return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream);
 }
 

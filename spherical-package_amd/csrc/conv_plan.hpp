@@ -149,6 +149,15 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 // straight into MFMA operands (conv_window_wgrad.hip; K <= 10, at most four plan rows per
 // sample: build the lists with max_rows = 4; mm: the matrix arithmetic).  partial: window_wgrad_partial_bytes(g).
 bool window_wgrad_supported(const ConvGeom& g, int mm);
+// ... and for layers of at most 64 pixel-side channels with nearest taps and no interpolation
+// weights (float32 matrix arithmetic): the tiles of tl.inside; partial:
+// window_wgrad_narrow_partial_bytes(g), which window_wgrad_partial_bytes(g) returns for them.
+bool window_wgrad_narrow_supported(const ConvGeom& g, int mm);
+size_t window_wgrad_narrow_partial_bytes(const ConvGeom& g);
+int window_wgrad_narrow(const ConvGeom& g, const Plan& plan, const TileLists& tl,
+                        const float* pix, const float* img, float* gW, float* partial,
+                        hipStream_t stream);
+
 size_t window_wgrad_partial_bytes(const ConvGeom& g);
 // big: the sums over the tiles of tl.big, from their big windows.
 int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,

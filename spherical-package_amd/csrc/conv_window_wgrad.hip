@@ -512,6 +512,8 @@ bool window_wgrad_supported(const ConvGeom& g, int mm) {
 }
 
 size_t window_wgrad_partial_bytes(const ConvGeom& g) {
+  if (g.B != 0 && window_wgrad_narrow_supported(g, kMmF32))
+    return window_wgrad_narrow_partial_bytes(g);
   if (g.B == 0 || !window_wgrad_supported(g, kMmF32)) return 0;
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const int tiles = pt.tiles_x * pt.tiles_y;
