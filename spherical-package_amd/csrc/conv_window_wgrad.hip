@@ -214,14 +214,17 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
 
   const int cnt = *count;
   if (cnt == 0) return;   // (the summing kernel sees the same count and adds nothing)
+  // The workgroups of one XCD take neighbouring tiles of the list at the same time: their
+  // windows share cache lines, which then meet in that XCD's L2.
+  const int first_ti = (group & 7) * (groups >> 3) + (group >> 3);
   if constexpr (PIPE) {
-    if (group < cnt) {
-      const int first = list[group];
+    if (first_ti < cnt) {
+      const int first = list[first_ti];
       if constexpr (BIG) fetch_offsets(first);
       fetch_quarter(first, 0, pg, pr, pn);
     }
   }
-  for (int ti = group; ti < cnt; ti += groups) {
+  for (int ti = first_ti; ti < cnt; ti += groups) {
     const int tile = list[ti];
     int RS;
     const int* lut;
