@@ -216,27 +216,29 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const T* __restrict__ go
   const T* p = gout + ((size_t)b * C + c) * M;
   constexpr int V = 16 / (int)sizeof(T);   // elements per 16-byte load
   T acc = T(0);
-  int e = beg;
-  if (((reinterpret_cast<uintptr_t>(p) + (size_t)beg * sizeof(T)) & 15) == 0) {
-    T a0 = T(0), a1 = T(0), a2 = T(0), a3 = T(0);
-    const int nv = (end - beg) / V;
-    for (int i = threadIdx.x; i < nv; i += 256) {
-      if constexpr (V == 4) {
-        const float4 v = reinterpret_cast<const float4*>(p + beg)[i];
-        a0 += v.x;
-        a1 += v.y;
-        a2 += v.z;
-        a3 += v.w;
-      } else {
-        const double2 v = reinterpret_cast<const double2*>(p + beg)[i];
-        a0 += v.x;
-        a1 += v.y;
-      }
+  // elements up to the first 16-byte boundary (planes whose size is not a multiple of four
+  // elements start anywhere), 16-byte loads from there, then what is left
+  const int mis = (int)(((reinterpret_cast<uintptr_t>(p) + (size_t)beg * sizeof(T)) & 15) / sizeof(T));
+  const int head = min(end - beg, mis ? V - mis : 0);
+  if ((int)threadIdx.x < head) acc += p[beg + threadIdx.x];
+  const int vbeg = beg + head;
+  T a0 = T(0), a1 = T(0), a2 = T(0), a3 = T(0);
+  const int nv = (end - vbeg) / V;
+  for (int i = threadIdx.x; i < nv; i += 256) {
+    if constexpr (V == 4) {
+      const float4 v = reinterpret_cast<const float4*>(p + vbeg)[i];
+      a0 += v.x;
+      a1 += v.y;
+      a2 += v.z;
+      a3 += v.w;
+    } else {
+      const double2 v = reinterpret_cast<const double2*>(p + vbeg)[i];
+      a0 += v.x;
+      a1 += v.y;
     }
-    acc = (a0 + a1) + (a2 + a3);
-    e = beg + nv * V;
   }
-  for (int i = e + threadIdx.x; i < end; i += 256) acc += p[i];
+  acc += (a0 + a1) + (a2 + a3);
+  for (int i = vbeg + nv * V + threadIdx.x; i < end; i += 256) acc += p[i];
   // wave64 butterfly, then one LDS slot per wave (or one atomic per wave)
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
   if constexpr (NOLDS) {

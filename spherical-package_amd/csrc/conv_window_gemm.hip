@@ -355,7 +355,10 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
 // XR: plan rows beyond the first four that are requested ahead as well (0 or 2).  The lists of
 // an inverse plan are as long as targets have sources: at unit scale a third of the samples
 // of a weighted bispherical map have six rows somewhere in a tile.
-template <int MM, int NB, int CAP, int XR>
+// RBT: plan rows requested and applied together: 4, or 1 for plans whose samples have a single
+// row (nearest taps without interpolation weights; three rows of padding would cost three
+// quarters of the gather's LDS reads and multiply-adds).
+template <int MM, int NB, int CAP, int XR, int RBT = 4>
 __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_gemm_kernel(
     const float* __restrict__ img, const int* __restrict__ hdr, const int* __restrict__ ns,
     const int2* __restrict__ taps, const int* __restrict__ list, const int* __restrict__ count,
@@ -455,7 +458,7 @@ __global__ __launch_bounds__(kWgThreads, CAP > kRegionCap ? 1 : 2) void window_g
   // conditions (rows past the sample's count re-read its last slot and are masked when they
   // are used), so that no branch and no wait sits between a request and the MFMAs that cover
   // its latency.  Samples with more than four rows fetch the others when they need them.
-  constexpr int RB = 4;
+  constexpr int RB = RBT;
   int2 rows[RB], rows_next[RB];
   int2 xrows[XR > 0 ? XR : 1], xrows_next[XR > 0 ? XR : 1];
 #define SDK_LOAD_ROWS_N(dst, kv, r0v, NR)                                         \
@@ -917,9 +920,16 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   do {                                                                         \
     if (more_rows) WG4(MMv, NBv, CAPv, 2); else WG4(MMv, NBv, CAPv, 0);        \
   } while (0)
+#define WG1R(MMv, NBv)                                                                         \
+  launch(window_gemm_kernel<MMv, NBv, kRegionCap, 0, 1>, grid, dim3(kWgThreads), stream, img,  \
+         plan.hdr, plan.ns, plan.taps, list, count, (const float*)weights, bias, pix, g.Cg,    \
+         g.H, g.W, g.Cp, g.K, plan.S, CpP, chunks, plan.pt, plan.tiles, n_tiles, gate,         \
+         plan.big_lut)
 #define WG2(MMv, NBv)                                                 \
   do {                                                                \
-    if (big) WG3(MMv, NBv, kBigCap); else WG3(MMv, NBv, kRegionCap);  \
+    if (big) WG3(MMv, NBv, kBigCap);                                  \
+    else if (plan.S == 1) WG1R(MMv, NBv);                             \
+    else WG3(MMv, NBv, kRegionCap);                                   \
   } while (0)
 #define WG1(MMv)                                                            \
   do {                                                                      \
@@ -929,6 +939,7 @@ int window_gemm(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl
   else if (mm == kMmSplit) WG1(kMmSplit);
   else WG1(kMmF32);
 #undef WG1
+#undef WG1R
 #undef WG2
 #undef WG3
 #undef WG4

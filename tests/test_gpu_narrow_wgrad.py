@@ -64,3 +64,24 @@ def test_workgroups_that_walk_several_tiles(ops, oracle, Cout, K):
     wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, 0, None)
     assert relerr(gw.cpu().numpy(), ww) <= 1e-4
     assert relerr(gi.cpu().numpy(), wi) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("M", [1, 3, 5, 642, 1023, 4098, 20007])
+def test_bias_gradient_on_planes_of_any_size(M, dtype):
+    """Planes whose size is not a multiple of four elements start at any alignment: the sum
+    takes the elements up to a 16-byte boundary singly, then 16-byte loads."""
+    from _spherical_distortion_ext import _capi
+    lib = _capi.load()
+    rng = np.random.default_rng(M)
+    g = rng.standard_normal((3, 5, M)).astype(dtype)
+    tg = torch.from_numpy(g).to(DEV)
+    out = torch.empty(5, dtype=tg.dtype, device=DEV)
+    code = _capi.SDK_F32 if dtype == np.float32 else _capi.SDK_F64
+    rc = lib.sdk_bias_grad(tg.data_ptr(), out.data_ptr(), 3, 5, M, code, None)
+    assert rc == 0, lib.sdk_last_error()
+    torch.cuda.synchronize()
+    want = g.astype(np.float64).sum(axis=(0, 2))
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    scale = np.abs(g.astype(np.float64)).sum(axis=(0, 2)).max()
+    assert np.abs(out.cpu().numpy() - want).max() <= tol * scale
