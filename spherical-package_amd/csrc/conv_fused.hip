@@ -783,11 +783,34 @@ static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const fl
     if (lists4 != nullptr) tl = *lists4;
     else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
     if (rc) return rc;
-    rc = window_wgrad_narrow(g, plan, tl, pix, img, gW,
-                             reinterpret_cast<float*>(base + t.window_partial), stream);
+    float* wp = reinterpret_cast<float*>(base + t.window_partial);
+    rc = window_wgrad_narrow(g, plan, tl, pix, img, gW, wp, stream);
     if (rc) return rc;
+    if (window_wgrad_big_supported(g, mm) && plan.big_lut != nullptr) {
+      rc = window_wgrad(g, mm, plan, tl, pix, img, gW, wp, stream, true);
+      if (rc) return rc;
+      return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream,
+                           tl.rest_small, tl.count + 3);
+    }
     return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream, tl.rest,
                          tl.count + 1);
+  }
+  if (window_wgrad_big_supported(g, mm) && window_wgrad_partial_bytes(g) != 0 &&
+      plan.big_lut != nullptr) {
+    // at most 64 pixel-side channels: the big tiles from their big windows, every other tile
+    // in the plan-driven kernel
+    const WgradTail t = wgrad_tail(g);
+    char* base = wgrad_tail_base(g, workspace);
+    TileLists tl;
+    int rc = SDK_OK;
+    if (lists4 != nullptr) tl = *lists4;
+    else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
+    if (rc) return rc;
+    rc = window_wgrad(g, mm, plan, tl, pix, img, gW,
+                      reinterpret_cast<float*>(base + t.window_partial), stream, true);
+    if (rc) return rc;
+    return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream,
+                         tl.not_big, tl.count + 6);
   }
   return planned_wgrad(g, mm, plan, pix, img, gW, wgrad_partial(g, workspace), stream);
 }

@@ -77,7 +77,8 @@ int build_plan(const ConvGeom& g, const float* map, const float* wts, void* work
 // the others again as big tiles and the remainder (count[2], count[3]); and, when the lists
 // were built with small_cap > 0 (kProductCap for an inverse plan, whose small windows can run
 // in the product form below), `inside` again as the tiles with a window of at most small_cap
-// elements and the remainder (count[4], count[5]).
+// elements and the remainder (count[4], count[5]); and every tile that is not a big tile
+// (count[6]).
 struct TileLists {
   const int* inside;
   const int* rest;
@@ -85,6 +86,7 @@ struct TileLists {
   const int* rest_small;
   const int* product;
   const int* inside_large;
+  const int* not_big;
   const int* count;
 };
 // max_rows > 0: tiles with a sample of more than max_rows plan rows (h[5]) are neither inside
@@ -149,6 +151,9 @@ int planned_wgrad(const ConvGeom& g, int mm, const Plan& plan, const float* pix,
 // straight into MFMA operands (conv_window_wgrad.hip; K <= 10, at most four plan rows per
 // sample: build the lists with max_rows = 4; mm: the matrix arithmetic).  partial: window_wgrad_partial_bytes(g).
 bool window_wgrad_supported(const ConvGeom& g, int mm);
+// ... for the big tiles alone (window_wgrad(..., big = true)): also layers of at most 64
+// pixel-side channels, whose other tiles are faster in the plan-driven kernel.
+bool window_wgrad_big_supported(const ConvGeom& g, int mm);
 // ... and for layers of at most 64 pixel-side channels with nearest taps and no interpolation
 // weights (float32 matrix arithmetic): the tiles of tl.inside; partial:
 // window_wgrad_narrow_partial_bytes(g), which window_wgrad_partial_bytes(g) returns for them.

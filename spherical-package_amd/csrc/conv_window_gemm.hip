@@ -296,12 +296,13 @@ __global__ __launch_bounds__(kWgThreads) void inverse_plan_kernel(
 //   lists[4 tiles .. 5 tiles)    small_cap > 0: the tiles of the first list whose window has at
 //                                most small_cap elements, count[4]
 //   lists[5 tiles .. 6 tiles)    ... and the others of the first list, count[5]
+//   lists[6 tiles .. 7 tiles)    every tile that is not in the third list, count[6]
 // max_rows > 0: a tile with a sample of more rows is neither inside nor big.
 __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict__ hdr, int tiles,
                                                           int* __restrict__ lists,
                                                           int* __restrict__ count, int max_rows,
                                                           int small_cap) {
-  constexpr int NC = 6;
+  constexpr int NC = 7;
   __shared__ int wave_n[NC][16];
   __shared__ int base[NC];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -321,6 +322,7 @@ __global__ __launch_bounds__(1024) void tile_lists_kernel(const int* __restrict_
     cls[3] = cls[1] && !cls[2];
     cls[4] = small;
     cls[5] = fit && !small;
+    cls[6] = live && !cls[2];
     unsigned long long mask[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -862,7 +864,7 @@ size_t window_gemm_weight_bytes(const ConvGeom& g) {
 
 size_t tile_lists_bytes(const ConvGeom& g) {
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
-  return ((size_t)6 * pt.tiles_x * pt.tiles_y + 8) * sizeof(int);
+  return ((size_t)7 * pt.tiles_x * pt.tiles_y + 8) * sizeof(int);
 }
 
 void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
@@ -873,7 +875,8 @@ void load_tile_lists(const Plan& plan, void* workspace, TileLists* out) {
   out->rest_small = lists + (size_t)3 * plan.tiles;
   out->product = lists + (size_t)4 * plan.tiles;
   out->inside_large = lists + (size_t)5 * plan.tiles;
-  out->count = lists + (size_t)6 * plan.tiles;
+  out->not_big = lists + (size_t)6 * plan.tiles;
+  out->count = lists + (size_t)7 * plan.tiles;
 }
 
 int build_tile_lists(const Plan& plan, void* workspace, hipStream_t stream, TileLists* out,

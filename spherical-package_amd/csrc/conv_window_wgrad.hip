@@ -506,22 +506,33 @@ WwGrid ww_grid(const ConvGeom& g, int tiles, bool big) {
 }
 }  // namespace
 
-bool window_wgrad_supported(const ConvGeom& g, int mm) {
-  // (every wave multiplies four 32-row blocks: with 64 rows or fewer half of that is padding,
-  // and the plan-driven kernel, which splits the pixels instead, is the faster one)
+bool window_wgrad_big_supported(const ConvGeom& g, int mm) {
   (void)mm;   // every matrix arithmetic
-  return planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp > 64 &&
+  return planned_wgrad_supported(g) && g.K >= 1 && g.K <= 10 && g.Cp >= 1 &&
          (int64_t)g.H * g.W <= ((int64_t)1 << 24);
 }
 
+bool window_wgrad_supported(const ConvGeom& g, int mm) {
+  // (every wave multiplies four 32-row blocks: with 64 rows or fewer half of that is padding.
+  // On tiles inside an ordinary window the plan-driven kernel, which splits the pixels
+  // instead, is then the faster one; on big tiles, which it reads from global memory, the
+  // padded window kernel still is, down to a few rows: 3 x 3 bilinear at stride 2 on a
+  // 64 x 128 grid, 4 x 128 -> 64 channels: 346 against 162 us; 128 -> 13 channels: the whole
+  // backward call 0.49 against 0.29 ms.)
+  return window_wgrad_big_supported(g, mm) && g.Cp > 64;
+}
+
 size_t window_wgrad_partial_bytes(const ConvGeom& g) {
-  if (g.B != 0 && window_wgrad_narrow_supported(g, kMmF32))
-    return window_wgrad_narrow_partial_bytes(g);
-  if (g.B == 0 || !window_wgrad_supported(g, kMmF32)) return 0;
+  if (g.B == 0) return 0;
+  // (one buffer serves whichever window kernels the call runs, one after the other)
+  const size_t narrow =
+      window_wgrad_narrow_supported(g, kMmF32) ? window_wgrad_narrow_partial_bytes(g) : 0;
+  if (!window_wgrad_big_supported(g, kMmF32)) return narrow;
   const PixelTiling pt = plan_tiling(g.M / g.OW, g.OW);
   const int tiles = pt.tiles_x * pt.tiles_y;
   const WwGrid w = ww_grid(g, tiles, false), wb = ww_grid(g, tiles, true);
-  return (size_t)std::max(w.slots, wb.slots) * w.nreg * kWwThreads * sizeof(float);
+  return std::max(narrow,
+                  (size_t)std::max(w.slots, wb.slots) * w.nreg * kWwThreads * sizeof(float));
 }
 
 int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,

@@ -87,6 +87,9 @@ CASES = [
     (72, 80, 1, 33000, 1, 4096, 3, 0, 0, "listed"),  # 30 of 32 tiles with a big window
     (72, 80, 64, 96, 32, 48, 9, 0, 1, "plain"),      # stride 2: every tile's box is 19 x 35, all big
     (72, 136, 48, 64, 24, 32, 9, 2, 2, "plain"),     # ... weighted, more than 128 pixel-side channels
+    (72, 48, 64, 96, 32, 48, 9, 0, 1, "plain"),      # ... 48 output channels: big tiles from the window,
+    (72, 40, 64, 96, 32, 48, 9, 0, 0, "plain"),      #     the others from the plan; nearest taps
+    (72, 13, 64, 96, 32, 48, 9, 0, 1, "plain"),      #     13 output channels
 ]
 
 
