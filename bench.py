@@ -280,7 +280,14 @@ def bench_pool3(torch, ops, timer, steps, warmup):
     ms_af, _ = timer.run(lambda: ops.mapped_avg_pool(x, m, None, K, 0), steps, warmup)
     ms_ab, _ = timer.run(lambda: ops.mapped_avg_unpool(g, m, None, H, W, K, 0), steps, warmup)
     avg_bytes = _nbytes(x, m, val)
-    return {"pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f,
+    # what a plain copy of the same input reaches on this GPU (the tensor library's copy kernel,
+    # read + write): the rate a memory-bound kernel can be held against beside the published peak
+    y = torch.empty_like(x)
+    ms_c, _ = timer.run(lambda: y.copy_(x), steps, warmup)
+    copy_ref = dict(ms=ms_c, **_roof("hbm", 2 * _nbytes(x), ms_c))
+    del y
+    return {"copy_reference": copy_ref,
+            "pool_forward": dict(ms=ms_f, **_roof("hbm", fwd_bytes, ms_f,
                                                   traffic=_measured_traffic("mapped_max_pool"))),
             "pool_backward": dict(ms=ms_b, **_roof("hbm", bwd_bytes, ms_b,
                                                    traffic=_measured_traffic("mapped_max_unpool"))),
