@@ -725,13 +725,25 @@ __global__ __launch_bounds__(kPlThreads) void wgrad_reduce_kernel(
   const int kinds = c_chunks * n_tiles * kblocks * batches;
   const int total = batches * groups;
   const size_t per_wg = (size_t)KB * 16 * kPlThreads;
-  float s = 0.0f;
-  for (int i = blockIdx.z; i < total; i += gridDim.z) {
-    const int b = i / groups, grp = i % groups;
+  // four reads in flight per thread (a plain loop waits for each in turn)
+  auto at = [&](int i) {
+    const int ic = min(i, total - 1);
+    const int b = ic / groups, grp = ic % groups;
     const int kind = ((b * c_chunks + cc) * n_tiles + nt) * kblocks + kb;
     const size_t wg = ((size_t)(grp >> 3) * kinds + kind) * 8 + (grp & 7);
-    s += partial[wg * per_wg + (size_t)kkv * kPlThreads + tid];
+    const float val = partial[wg * per_wg + (size_t)kkv * kPlThreads + tid];
+    return i < total ? val : 0.0f;
+  };
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  const int step = gridDim.z;
+  for (int i = blockIdx.z; i < total; i += 4 * step) {
+    const float v0 = at(i), v1 = at(i + step), v2 = at(i + 2 * step), v3 = at(i + 3 * step);
+    s0 += v0;
+    s1 += v1;
+    s2 += v2;
+    s3 += v3;
   }
+  const float s = (s0 + s1) + (s2 + s3);
   const int wave = tid >> 6, lane = tid & 63, nl = lane & 31, h = lane >> 5;
   const int c = cc * kCC + nl;
   const int n = nt * (32 * NW) + 32 * (wave % NW) + 8 * (v >> 2) + 4 * h + (v & 3);
