@@ -65,7 +65,8 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   __shared__ __align__(16) int2 rowsL[K * kWwQ * kWwRows];
   __shared__ int src[BIG ? 1 : CAP];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (a scalar for the compiler)
   const int j = lane & 31, h = lane >> 5;
   // Workgroup ids go round-robin over the 8 XCDs.  All workgroups of one tile run (every
   // batch element and channel chunk) read the same plan rows, those of one batch element the
@@ -114,30 +115,31 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
     for (int it = 0; it < ITER; ++it) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        if constexpr (BIG) {
-          // No element of a listed window is missing, slots past its end are never stored, and
-          // the columns of channels past Cg are dropped with the sums: plain loads from a
-          // valid address, nothing that could become a branch around a load.
-          wv[it][i] = *reinterpret_cast<const float*>(
-              cbase + (unsigned)min(i, Cg - 1 - min(cw, Cg - 1)) * plane +
-              (unsigned)max(wo[it], 0) * 4u);
-        } else {
-          const bool ok = wo[it] >= 0 && cw + i < Cg;
-          const float d = *reinterpret_cast<const float*>(
-              cbase + (ok ? (unsigned)i * plane + (unsigned)wo[it] * 4u : 0u));
-          wv[it][i] = ok ? d : 0.0f;
-        }
+        // Plain loads from a valid address, nothing that could become a branch around a load
+        // (with a condition on the load the generated code took one of the eight of every
+        // round behind a branch and waited for it there: five round trips per window instead
+        // of one).  Slots past the window's end are never stored, the columns of channels
+        // past Cg are dropped with the sums, and elements a box window has outside the image
+        // (offset -1) are zeroed where they are stored.
+        const unsigned ch = __builtin_amdgcn_readfirstlane(
+            (unsigned)min(i, Cg - 1 - min(cw, Cg - 1)) * plane);
+        wv[it][i] = *reinterpret_cast<const float*>(cbase + ch + (unsigned)max(wo[it], 0) * 4u);
       }
     }
   };
-  auto store_window = [&](int RS, const float (&wv)[ITER][8]) {
+  auto store_window = [&](int RS, const int (&wo)[ITER], const float (&wv)[ITER][8]) {
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
       const int e = lane + 64 * it;
       if (e < RS) {
         float4* d4 = reinterpret_cast<float4*>(region + e * kWwE + 8 * wave);
-        d4[0] = make_float4(wv[it][0], wv[it][1], wv[it][2], wv[it][3]);
-        d4[1] = make_float4(wv[it][4], wv[it][5], wv[it][6], wv[it][7]);
+        if (wo[it] >= 0) {
+          d4[0] = make_float4(wv[it][0], wv[it][1], wv[it][2], wv[it][3]);
+          d4[1] = make_float4(wv[it][4], wv[it][5], wv[it][6], wv[it][7]);
+        } else {
+          d4[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+          d4[1] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
       }
     }
   };
@@ -146,6 +148,14 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
   // the rows its sample has (the row itself is read whether it exists or not, clamped to S).
   constexpr int TOTAL = K * kWwRows * kWwQ;
   constexpr int NR = (TOTAL + kWwThreads - 1) / kWwThreads;
+  unsigned row_off[NR], row_k[NR];
+#pragma unroll
+  for (int u = 0; u < NR; ++u) {
+    const int idx = min(kWwThreads * u + tid, TOTAL - 1);
+    const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
+    row_k[u] = k;
+    row_off[u] = (k * S + min(r, S - 1)) * 128 + m;
+  }
   auto fetch_quarter = [&](int tile_, int q_, float4 (&gq)[4], int2 (&pr)[NR], int (&pn)[NR]) {
     const int ty0_ = (tile_ / pt.tiles_x) * pt.TY(), tx0_ = (tile_ % pt.tiles_x) << pt.tx_shift;
     const int p0 = kWwQ * q_ + 16 * hr_s;
@@ -171,13 +181,13 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
 #pragma unroll
       for (int i = 0; i < 4; ++i) gq[i] = make_float4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
     }
-    const int2* tt = taps + (size_t)tile_ * K * S * 128;
+    // (uniform bases, per-thread constant offsets: no 64-bit address arithmetic per entry)
+    const int2* tp = taps + ((size_t)tile_ * K * S * 128 + kWwQ * q_);
+    const int* np = ns + (size_t)tile_ * K;
 #pragma unroll
     for (int u = 0; u < NR; ++u) {
-      const int idx = min(kWwThreads * u + tid, TOTAL - 1);
-      const int k = idx >> 7, r = (idx >> 5) & 3, m = idx & 31;
-      pr[u] = tt[((size_t)k * S + min(r, S - 1)) * 128 + kWwQ * q_ + m];
-      pn[u] = ns[(size_t)tile_ * K + k];
+      pr[u] = tp[row_off[u]];
+      pn[u] = np[row_k[u]];
     }
   };
   auto store_quarter = [&](int RS, const float4 (&gq)[4], const int2 (&pr)[NR],
@@ -243,7 +253,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
     if constexpr (BIG) {
       float sv[ITER][8];
       fetch_window(wo, sv);
-      store_window(RS, sv);
+      store_window(RS, wo, sv);
     } else {
       for (int e = tid; e < RS; e += kWwThreads) src[e] = lut[kHdrLut + e];
       __syncthreads();
@@ -255,7 +265,7 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
         so[it] = e < RS ? src[e] : -1;
       }
       fetch_window(so, sv);
-      store_window(RS, sv);
+      store_window(RS, so, sv);
     }
 
 #pragma unroll 1
