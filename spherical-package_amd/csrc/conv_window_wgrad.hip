@@ -48,7 +48,9 @@ constexpr int kWwRows = 4; // plan rows per sample this kernel applies
 // With one wave per SIMD nothing else covers a global read, so that variant requests ahead what
 // it has registers for: the pixel-side tile and the plan rows of the next quarter, and the
 // offsets of the next tile's window, before a quarter's MFMAs.
-template <int KP, int R, int CAP, int MM>
+// ONE: every sample of the plan has a single row (nearest taps without interpolation weights);
+// the step loop then reads and applies that row alone instead of four, three of them padding.
+template <int KP, int R, int CAP, int MM, bool ONE = false>
 __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, const int* __restrict__ list,
@@ -304,30 +306,41 @@ __global__ __launch_bounds__(kWwThreads, CAP > kRegionCap ? 1 : 2) void window_w
     _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
       const int k = c < KP ? wave * KP + c : 4 * KP + (c - KP);                      \
       const int4* rp = reinterpret_cast<const int4*>(rows_h + (k * kWwQ + st) * kWwRows); \
-      R01[c] = rp[0];                                                                \
-      R23[c] = rp[1];                                                                \
+      if constexpr (ONE) {                                                           \
+        const int2 r0 = *reinterpret_cast<const int2*>(rp);                          \
+        R01[c].x = r0.x;                                                             \
+        R01[c].y = r0.y;                                                             \
+      } else {                                                                       \
+        R01[c] = rp[0];                                                              \
+        R23[c] = rp[1];                                                              \
+      }                                                                              \
     }                                                                                \
   } while (0)
 #define SDK_VALS_ISSUE()                                                             \
   do {                                                                               \
     _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
       val[c][0] = *reinterpret_cast<const float*>(regb + R01[c].x);                  \
-      val[c][1] = *reinterpret_cast<const float*>(regb + R01[c].z);                  \
-      val[c][2] = *reinterpret_cast<const float*>(regb + R23[c].x);                  \
-      val[c][3] = *reinterpret_cast<const float*>(regb + R23[c].z);                  \
       co[c][0] = __int_as_float(R01[c].y);                                           \
-      co[c][1] = __int_as_float(R01[c].w);                                           \
-      co[c][2] = __int_as_float(R23[c].y);                                           \
-      co[c][3] = __int_as_float(R23[c].w);                                           \
+      if constexpr (!ONE) {                                                          \
+        val[c][1] = *reinterpret_cast<const float*>(regb + R01[c].z);                \
+        val[c][2] = *reinterpret_cast<const float*>(regb + R23[c].x);                \
+        val[c][3] = *reinterpret_cast<const float*>(regb + R23[c].z);                \
+        co[c][1] = __int_as_float(R01[c].w);                                         \
+        co[c][2] = __int_as_float(R23[c].y);                                         \
+        co[c][3] = __int_as_float(R23[c].w);                                         \
+      }                                                                              \
     }                                                                                \
   } while (0)
 #define SDK_BLEND(dst)                                                               \
   do {                                                                               \
     _Pragma("unroll") for (int c = 0; c < KW; ++c) {                                 \
       float bv = co[c][0] * val[c][0];                                               \
-      bv = __builtin_fmaf(co[c][1], val[c][1], bv);                                  \
-      bv = __builtin_fmaf(co[c][2], val[c][2], bv);                                  \
-      dst[c] = __builtin_fmaf(co[c][3], val[c][3], bv);                              \
+      if constexpr (!ONE) {                                                          \
+        bv = __builtin_fmaf(co[c][1], val[c][1], bv);                                \
+        bv = __builtin_fmaf(co[c][2], val[c][2], bv);                                \
+        bv = __builtin_fmaf(co[c][3], val[c][3], bv);                                \
+      }                                                                              \
+      dst[c] = bv;                                                                   \
     }                                                                                \
   } while (0)
       SDK_ROWS_ISSUE(0);
@@ -573,10 +586,15 @@ int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& t
   launch(window_wgrad_kernel<KPv, Rv, CAPv, MMv>, grid, dim3(kWwThreads), stream, pix, img,      \
          plan.hdr, plan.ns, plan.taps, list, count, partial, g.Cg, g.H, g.W, g.Cp, plan.S,       \
          plan.pt, w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4, plan.big_lut)
+#define WW3ONE(KPv, Rv, CAPv)                                                                    \
+  launch(window_wgrad_kernel<KPv, Rv, CAPv, kMmF32, true>, grid, dim3(kWwThreads), stream, pix,   \
+         img, plan.hdr, plan.ns, plan.taps, list, count, partial, g.Cg, g.H, g.W, g.Cp, plan.S,   \
+         plan.pt, w.groups, (int)g.B, w.c_chunks, w.n_tiles, vec4, plan.big_lut)
 #define WW2(KPv, Rv, CAPv)                                                       \
   do {                                                                           \
     if (mm == kMmBf16) WW3(KPv, Rv, CAPv, kMmBf16);                              \
     else if (mm == kMmSplit) WW3(KPv, Rv, CAPv, kMmSplit);                       \
+    else if (plan.S == 1) WW3ONE(KPv, Rv, CAPv);                                 \
     else WW3(KPv, Rv, CAPv, kMmF32);                                             \
   } while (0)
 #define WW(KPv, Rv)                                                   \
@@ -598,6 +616,7 @@ int window_wgrad(const ConvGeom& g, int mm, const Plan& plan, const TileLists& t
 #undef WW
 #undef WW2
 #undef WW3
+#undef WW3ONE
   SDK_LAUNCH_CHECK(big ? "window_wgrad(big)" : "window_wgrad");
   const int kinds0 = w.c_chunks * w.n_tiles, total = (int)g.B * w.groups;
   const int parts = (int)std::min<int64_t>(std::min(total, 16),
