@@ -90,6 +90,8 @@ CASES = [
     (72, 48, 64, 96, 32, 48, 9, 0, 1, "plain"),      # ... 48 output channels: big tiles from the window,
     (72, 40, 64, 96, 32, 48, 9, 0, 0, "plain"),      #     the others from the plan; nearest taps
     (72, 13, 64, 96, 32, 48, 9, 0, 1, "plain"),      #     13 output channels
+    (72, 80, 64, 96, 32, 48, 9, 0, 0, "plain"),      # stride 2, nearest taps, wide: one row per sample in big windows
+    (72, 80, 40, 64, 40, 64, 9, 0, 0, "plain"),      # ... and in ordinary ones
 ]
 
 
