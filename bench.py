@@ -212,8 +212,25 @@ def bench_conv1(torch, ops, timer, steps, warmup):
         ops.mapped_conv_forward(x, m, None, w, b, K, interp)
         ops.mapped_conv_backward(g, m, None, x, w, b, K, interp)
     ms_s, _ = timer.run(step, steps, warmup)
-    return {"conv1_latency": {"forward_us": round(ms_f * 1e3, 1),
-                              "forward_backward_us": round(ms_s * 1e3, 1)}}
+    out = {"forward_us": round(ms_f * 1e3, 1), "forward_backward_us": round(ms_s * 1e3, 1)}
+    # the same step captured into a HIP graph and replayed (the library launches kernels only and
+    # allocates nothing, so a caller bound by launches can do this): time per replay
+    try:
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        ms_g, _ = timer.run(graph.replay, steps, warmup)
+        out["forward_backward_graph_replay_us"] = round(ms_g * 1e3, 1)
+    except Exception as e:  # reported, not fatal: the eager figures above stand
+        out["forward_backward_graph_replay_us"] = None
+        out["graph_error"] = str(e)[:200]
+    return {"conv1_latency": out}
 
 
 def bench_resample2(torch, ops, timer, steps, warmup):
