@@ -223,3 +223,56 @@ def test_uv_resampling_voting_and_generated_maps(ops, oracle, seed):
     got = _n(ops.mapped_avg_pool(_t(x), m, None, kh * kw, 2))
     want = oracle.mapped_avg_pool(x, mo, kh * kw, 2)
     assert relerr(got, want) <= 1e-9
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_fused_kernels_against_the_unfused_path_on_random_layers(ops, seed):
+    """Twenty random layers per seed (nearest, bilinear and bispherical taps, 1 to 12 samples,
+    3 to 136 output channels, unit stride and stride 2, one-row grids of thousands of pixels,
+    batches that make workgroups walk several tiles): the plan-driven and window kernels against
+    the im2col + GEMM path of the same library, which shares none of their code.  The oracle
+    pins both elsewhere; here the point is breadth at no CPU cost."""
+    rng = np.random.default_rng(seed)
+
+    def err(a, b):
+        return float((a - b).abs().max() / max(b.abs().max().item(), 1e-30))
+
+    for case in range(20):
+        interp = int(rng.choice([0, 0, 1, 2]))
+        K = int(rng.integers(1, 13))
+        Cin = int(rng.choice([5, 16, 33, 64, 72, 100, 130, 256]))
+        Cout = int(rng.choice([3, 8, 13, 32, 33, 48, 64, 65, 96, 128, 136]))
+        B = int(rng.choice([1, 2, 3, 8]))
+        stride = int(rng.choice([1, 1, 2]))
+        OH, OW = int(rng.integers(1, 40)), int(rng.integers(16, 90))
+        if rng.uniform() < 0.2:
+            OH, OW = 1, int(rng.integers(200, 3000))
+        H, W = OH * stride + int(rng.integers(0, 3)), OW * stride + int(rng.integers(0, 3))
+        ys, xs = np.meshgrid(np.arange(OH), np.arange(OW), indexing="ij")
+        dy, dx = rng.integers(-2, 3, K), rng.integers(-3, 4, K)
+        spread = float(rng.choice([0.4, 0.4, 3.0]))
+        cx = stride * xs[..., None] + dx + rng.uniform(-spread, spread, (OH, OW, K))
+        cy = stride * ys[..., None] + dy + rng.uniform(-spread, spread, (OH, OW, K))
+        if OH == 1:
+            cy = np.zeros_like(cy)
+        m = _t(np.stack([cx, cy], -1).astype(np.float32))
+        x = torch.randn(B, Cin, H, W, device=DEV)
+        g = torch.randn(B, Cout, OH, OW, device=DEV)
+        w = torch.randn(Cout, Cin, K, device=DEV) / np.sqrt(Cin * K)
+        b = torch.randn(Cout, device=DEV)
+        bt = torch.randn(Cin, device=DEV)
+        res = {}
+        try:
+            for mode in ("native", "unfused"):
+                ops.set_conv_compute(mode)
+                y = ops.mapped_conv_forward(x, m, None, w, b, K, interp)
+                gi, gw, gb = ops.mapped_conv_backward(g, m, None, x, w, b, K, interp)
+                yt = ops.mapped_transposed_conv_forward(g, m, None, w, bt, H, W, K, interp)
+                res[mode] = (y, gi, gw, gb, yt)
+        finally:
+            ops.set_conv_compute("native")
+        what = dict(seed=seed, case=case, interp=interp, K=K, Cin=Cin, Cout=Cout, B=B,
+                    stride=stride, OH=OH, OW=OW, H=H, W=W, spread=spread)
+        for name, a, r in zip(("forward", "grad_input", "grad_weight", "grad_bias", "transposed"),
+                              res["native"], res["unfused"]):
+            assert err(a, r) <= BWD, (name, what)
