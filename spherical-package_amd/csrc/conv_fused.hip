@@ -784,7 +784,7 @@ static int wgrad_from_plan(const ConvGeom& g, int mm, const Plan& plan, const fl
     else rc = build_tile_lists(plan, base + t.lists, stream, &tl, 4);
     if (rc) return rc;
     float* wp = reinterpret_cast<float*>(base + t.window_partial);
-    rc = window_wgrad_narrow(g, plan, tl, pix, img, gW, wp, stream);
+    rc = window_wgrad_narrow(g, mm, plan, tl, pix, img, gW, wp, stream);
     if (rc) return rc;
     if (window_wgrad_big_supported(g, mm) && plan.big_lut != nullptr) {
       rc = window_wgrad(g, mm, plan, tl, pix, img, gW, wp, stream, true);

@@ -155,11 +155,11 @@ bool window_wgrad_supported(const ConvGeom& g, int mm);
 // pixel-side channels, whose other tiles are faster in the plan-driven kernel.
 bool window_wgrad_big_supported(const ConvGeom& g, int mm);
 // ... and for layers of at most 64 pixel-side channels with nearest taps and no interpolation
-// weights (float32 matrix arithmetic): the tiles of tl.inside; partial:
+// weights (mm: the matrix arithmetic): the tiles of tl.inside; partial:
 // window_wgrad_narrow_partial_bytes(g), which window_wgrad_partial_bytes(g) returns for them.
 bool window_wgrad_narrow_supported(const ConvGeom& g, int mm);
 size_t window_wgrad_narrow_partial_bytes(const ConvGeom& g);
-int window_wgrad_narrow(const ConvGeom& g, const Plan& plan, const TileLists& tl,
+int window_wgrad_narrow(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                         const float* pix, const float* img, float* gW, float* partial,
                         hipStream_t stream);
 

@@ -44,7 +44,7 @@ constexpr int kWnE = 36;   // floats per window element: 32 channels + 4 of skew
 constexpr int kWnH = 64;   // pixels per stage: half a tile
 constexpr int kWnG = 68;   // floats per row of the pixel-side tile: 64 pixels + 4 of skew
 
-template <int KF, int R, int NBW>
+template <int KF, int R, int NBW, int MM>
 __global__ __launch_bounds__(kWnThreads, 2) void window_wgrad_narrow_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const int* __restrict__ hdr,
     const int* __restrict__ ns, const int2* __restrict__ taps, const int* __restrict__ list,
@@ -244,92 +244,164 @@ __global__ __launch_bounds__(kWnThreads, 2) void window_wgrad_narrow_kernel(
       }
       if (q == 0 || has_next) fetch_half(q == 0 ? tile : tile_next, q ^ 1);
 
-      // ---- eight groups of four MFMA steps; plan rows two groups ahead, values one.  A wave's
-      // share of the remaining samples (row block blk_w, steps phase + NPH t of every group)
-      // is addressed through per-wave base pointers, so all waves run the same code.
-      {
-        constexpr int KFa = KF > 0 ? KF : 1, Ra = R > 0 ? R : 1;
-        const unsigned short* rows_h = rowsL + 32 * h;
-        const unsigned short* rows_r = rows_h + 4 * KF * kWnH + phase;
-        const float* gt_r = gt + (32 * blk_w + j) * kWnG + 32 * h + phase;
-        uint2 Rn[KFa];             // four steps' offsets of a full sample, 16 bits each
-        unsigned Rr[Ra][TPG];      // offsets of this wave's steps of a remaining sample
-        float val[KFa][4], valr[Ra][TPG];
-        auto rows_issue = [&](int grp) {
-          const int gq = grp < 8 ? grp : 7;
+      if constexpr (MM == kMmF32) {
+        // ---- eight groups of four MFMA steps; plan rows two groups ahead, values one.  A wave's
+        // share of the remaining samples (row block blk_w, steps phase + NPH t of every group)
+        // is addressed through per-wave base pointers, so all waves run the same code.
+        {
+          constexpr int KFa = KF > 0 ? KF : 1, Ra = R > 0 ? R : 1;
+          const unsigned short* rows_h = rowsL + 32 * h;
+          const unsigned short* rows_r = rows_h + 4 * KF * kWnH + phase;
+          const float* gt_r = gt + (32 * blk_w + j) * kWnG + 32 * h + phase;
+          uint2 Rn[KFa];             // four steps' offsets of a full sample, 16 bits each
+          unsigned Rr[Ra][TPG];      // offsets of this wave's steps of a remaining sample
+          float val[KFa][4], valr[Ra][TPG];
+          auto rows_issue = [&](int grp) {
+            const int gq = grp < 8 ? grp : 7;
 #pragma unroll
-          for (int i = 0; i < KF; ++i)
-            Rn[i] = *reinterpret_cast<const uint2*>(rows_h + (4 * i + wave) * kWnH + 4 * gq);
+            for (int i = 0; i < KF; ++i)
+              Rn[i] = *reinterpret_cast<const uint2*>(rows_h + (4 * i + wave) * kWnH + 4 * gq);
 #pragma unroll
-          for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int t = 0; t < TPG; ++t) Rr[r][t] = rows_r[r * kWnH + 4 * gq + NPH * t];
-        };
-        auto at = [&](const uint2& w, int step) {
-          const unsigned d = step < 2 ? w.x : w.y;
-          return *reinterpret_cast<const float*>(regb + ((step & 1) ? d >> 16 : d & 0xffffu));
-        };
-        auto vals_issue = [&]() {
+              for (int t = 0; t < TPG; ++t) Rr[r][t] = rows_r[r * kWnH + 4 * gq + NPH * t];
+          };
+          auto at = [&](const uint2& w, int step) {
+            const unsigned d = step < 2 ? w.x : w.y;
+            return *reinterpret_cast<const float*>(regb + ((step & 1) ? d >> 16 : d & 0xffffu));
+          };
+          auto vals_issue = [&]() {
 #pragma unroll
-          for (int i = 0; i < KF; ++i)
+            for (int i = 0; i < KF; ++i)
 #pragma unroll
-            for (int st = 0; st < 4; ++st) val[i][st] = at(Rn[i], st);
+              for (int st = 0; st < 4; ++st) val[i][st] = at(Rn[i], st);
 #pragma unroll
-          for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int t = 0; t < TPG; ++t)
-              valr[r][t] = *reinterpret_cast<const float*>(regb + Rr[r][t]);
-        };
-        rows_issue(0);
-        vals_issue();    // group 0
-        rows_issue(1);
+              for (int t = 0; t < TPG; ++t)
+                valr[r][t] = *reinterpret_cast<const float*>(regb + Rr[r][t]);
+          };
+          rows_issue(0);
+          vals_issue();    // group 0
+          rows_issue(1);
 #pragma unroll
-        for (int grp = 0; grp < 8; ++grp) {
-          float4 A[NBW];
-          float Ar[TPG];
+          for (int grp = 0; grp < 8; ++grp) {
+            float4 A[NBW];
+            float Ar[TPG];
 #pragma unroll
-          for (int a = 0; a < NBW; ++a)
-            A[a] = *reinterpret_cast<const float4*>(gt + (32 * a + j) * kWnG + 32 * h + 4 * grp);
-          if constexpr (R > 0) {
-#pragma unroll
-            for (int t = 0; t < TPG; ++t) Ar[t] = gt_r[4 * grp + NPH * t];
-          }
-          float b[KFa][4], br[Ra][TPG];
-#pragma unroll
-          for (int i = 0; i < KF; ++i)
-#pragma unroll
-            for (int s = 0; s < 4; ++s) b[i][s] = val[i][s];
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < TPG; ++t) br[r][t] = valr[r][t];
-          if (grp < 7) {
-            vals_issue();            // group grp + 1
-            rows_issue(grp + 2);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int s = 0; s < 4; ++s) {
-#pragma unroll
-            for (int i = 0; i < KF; ++i) {
-#pragma unroll
-              for (int a = 0; a < NBW; ++a) {
-                const float av = s == 0 ? A[a].x : (s == 1 ? A[a].y : (s == 2 ? A[a].z : A[a].w));
-                acc[i * NBW + a] =
-                    __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[i][s], acc[i * NBW + a], 0, 0, 0);
-              }
-            }
+            for (int a = 0; a < NBW; ++a)
+              A[a] = *reinterpret_cast<const float4*>(gt + (32 * a + j) * kWnG + 32 * h + 4 * grp);
             if constexpr (R > 0) {
-              if (s % NPH == NPH - 1) {
-                const int t = s / NPH;
 #pragma unroll
-                for (int r = 0; r < R; ++r)
-                  acc[KF * NBW + r] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                      Ar[t], br[r][t], acc[KF * NBW + r], 0, 0, 0);
+              for (int t = 0; t < TPG; ++t) Ar[t] = gt_r[4 * grp + NPH * t];
+            }
+            float b[KFa][4], br[Ra][TPG];
+#pragma unroll
+            for (int i = 0; i < KF; ++i)
+#pragma unroll
+              for (int s = 0; s < 4; ++s) b[i][s] = val[i][s];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+              for (int t = 0; t < TPG; ++t) br[r][t] = valr[r][t];
+            if (grp < 7) {
+              vals_issue();            // group grp + 1
+              rows_issue(grp + 2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+              for (int i = 0; i < KF; ++i) {
+#pragma unroll
+                for (int a = 0; a < NBW; ++a) {
+                  const float av = s == 0 ? A[a].x : (s == 1 ? A[a].y : (s == 2 ? A[a].z : A[a].w));
+                  acc[i * NBW + a] =
+                      __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[i][s], acc[i * NBW + a], 0, 0, 0);
+                }
+              }
+              if constexpr (R > 0) {
+                if (s % NPH == NPH - 1) {
+                  const int t = s / NPH;
+#pragma unroll
+                  for (int r = 0; r < R; ++r)
+                    acc[KF * NBW + r] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        Ar[t], br[r][t], acc[KF * NBW + r], 0, 0, 0);
+                }
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      } else {
+        // ---- bf16 matrix unit (operands rounded to bf16, or split into three bf16 pieces): one
+        // instruction contracts 16 pixels, lane (j, h) supplying its row / channel for the eight
+        // pixels 8 h .. 8 h + 7 of a group of 16.  A lane reads its eight window offsets of a
+        // sample as one 16-byte read and the eight values after them; a wave's share of the
+        // remaining samples is row block blk_w on every NPH-th group.
+        const unsigned short* rows_g = rowsL + 8 * h;
+#pragma unroll 1
+        for (int grp = 0; grp < 4; ++grp) {
+          auto b_values = [&](int k, float (&f)[8]) {
+            const uint4 w = *reinterpret_cast<const uint4*>(rows_g + k * kWnH + 16 * grp);
+            const unsigned d[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              f[2 * i] = *reinterpret_cast<const float*>(regb + (d[i] & 0xffffu));
+              f[2 * i + 1] = *reinterpret_cast<const float*>(regb + (d[i] >> 16));
+            }
+          };
+          auto a_values = [&](int row, float (&f)[8]) {
+            const float4* ap = reinterpret_cast<const float4*>(gt + row * kWnG + 16 * grp + 8 * h);
+            const float4 lo = ap[0], hi = ap[1];
+            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+            f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+          };
+          Bf16Frag a16[NBW];
+          Bf16Split a3[MM == kMmSplit ? NBW : 1];
+          const bool mine = R > 0 && (grp % NPH) == phase;   // this group carries the wave's share
+          if (KF > 0 || mine) {
+#pragma unroll
+            for (int a = 0; a < NBW; ++a) {
+              float f[8];
+              a_values(32 * a + j, f);
+              if constexpr (MM == kMmSplit) a3[a] = split_bf16x8(f);
+              else a16[a] = pack_bf16x8(f);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < KF; ++i) {
+            float f[8];
+            b_values(4 * i + wave, f);
+            if constexpr (MM == kMmSplit) {
+              const Bf16Split b3 = split_bf16x8(f);
+#pragma unroll
+              for (int a = 0; a < NBW; ++a) acc[i * NBW + a] = mfma_split(a3[a], b3, acc[i * NBW + a]);
+            } else {
+              const Bf16Frag b16 = pack_bf16x8(f);
+#pragma unroll
+              for (int a = 0; a < NBW; ++a) acc[i * NBW + a] = mfma_bf16(a16[a], b16, acc[i * NBW + a]);
+            }
+          }
+          if (mine) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              float f[8];
+              b_values(4 * KF + r, f);
+              if constexpr (MM == kMmSplit) {
+                const Bf16Split b3 = split_bf16x8(f);
+                // (the row block is the wave's: a select between the two fragments)
+                acc[KF * NBW + r] = NBW == 1 || blk_w == 0
+                                        ? mfma_split(a3[0], b3, acc[KF * NBW + r])
+                                        : mfma_split(a3[NBW - 1], b3, acc[KF * NBW + r]);
+              } else {
+                const Bf16Frag b16 = pack_bf16x8(f);
+                acc[KF * NBW + r] = NBW == 1 || blk_w == 0
+                                        ? mfma_bf16(a16[0], b16, acc[KF * NBW + r])
+                                        : mfma_bf16(a16[NBW - 1], b16, acc[KF * NBW + r]);
               }
             }
           }
-          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -409,7 +481,8 @@ WnGrid wn_grid(const ConvGeom& g, int tiles) {
 
 bool window_wgrad_narrow_supported(const ConvGeom& g, int mm) {
   // (nearest taps without interpolation weights: one plan row per sample, coefficient one)
-  if (!(planned_wgrad_supported(g) && mm == kMmF32 && g.interp == 0 && g.P == 0 && g.K >= 1 &&
+  (void)mm;   // every matrix arithmetic
+  if (!(planned_wgrad_supported(g) && g.interp == 0 && g.P == 0 && g.K >= 1 &&
         g.K <= 10 && g.Cp <= 64 && (int64_t)g.H * g.W <= ((int64_t)1 << 24)))
     return false;
   // a thread's run of sixteen pixels of the pixel-side tile lies in one row of the grid and in
@@ -423,7 +496,7 @@ size_t window_wgrad_narrow_partial_bytes(const ConvGeom& g) {
   return (size_t)w.slots * w.nreg * kWnThreads * sizeof(float);
 }
 
-int window_wgrad_narrow(const ConvGeom& g, const Plan& plan, const TileLists& tl,
+int window_wgrad_narrow(const ConvGeom& g, int mm, const Plan& plan, const TileLists& tl,
                         const float* pix, const float* img, float* gW, float* partial,
                         hipStream_t stream) {
   const WnGrid w = wn_grid(g, plan.tiles);
@@ -431,10 +504,16 @@ int window_wgrad_narrow(const ConvGeom& g, const Plan& plan, const TileLists& tl
     return fail(SDK_ERR_UNSUPPORTED, "window_wgrad_narrow: grid too large");
   const int NBW = g.Cp > 32 ? 2 : 1;
   const dim3 grid((unsigned)w.slots);
-#define WN2(KFv, Rv, NBWv)                                                                      \
-  launch(window_wgrad_narrow_kernel<KFv, Rv, NBWv>, grid, dim3(kWnThreads), stream, pix, img,   \
-         plan.hdr, plan.ns, plan.taps, tl.inside, tl.count, partial, g.Cg, g.H, g.W, g.Cp,      \
+#define WN3(KFv, Rv, NBWv, MMv)                                                                \
+  launch(window_wgrad_narrow_kernel<KFv, Rv, NBWv, MMv>, grid, dim3(kWnThreads), stream, pix,   \
+         img, plan.hdr, plan.ns, plan.taps, tl.inside, tl.count, partial, g.Cg, g.H, g.W, g.Cp, \
          plan.pt, w.groups, (int)g.B, w.c_chunks)
+#define WN2(KFv, Rv, NBWv)                                       \
+  do {                                                           \
+    if (mm == kMmBf16) WN3(KFv, Rv, NBWv, kMmBf16);              \
+    else if (mm == kMmSplit) WN3(KFv, Rv, NBWv, kMmSplit);       \
+    else WN3(KFv, Rv, NBWv, kMmF32);                             \
+  } while (0)
 #define WN(KFv, Rv)                                        \
   do {                                                     \
     if (NBW == 2) WN2(KFv, Rv, 2); else WN2(KFv, Rv, 1);   \
@@ -453,6 +532,7 @@ int window_wgrad_narrow(const ConvGeom& g, const Plan& plan, const TileLists& tl
   }
 #undef WN
 #undef WN2
+#undef WN3
   SDK_LAUNCH_CHECK("window_wgrad_narrow");
   const int total = (int)g.B * w.groups;
   const int parts = (int)std::min<int64_t>(std::min(total, 16),

@@ -42,25 +42,36 @@ def _nearest_case(seed, B, Cin, Cout, H, W, K):
     return m, x, w, b, g
 
 
+@pytest.mark.parametrize("mode", ["native", "split", "bf16"])
 @pytest.mark.parametrize("Cout", [24, 48])
 @pytest.mark.parametrize("K", range(1, 11))
-def test_every_kernel_size_and_block_width(ops, oracle, K, Cout):
+def test_every_kernel_size_and_block_width(ops, oracle, K, Cout, mode):
     m, x, w, b, g = _nearest_case(100 * K + Cout, 2, 40, Cout, 20, 37, K)
-    gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), None, _t(x), _t(w), _t(b), K, 0)
+    ops.set_conv_compute(mode)
+    try:
+        gi, gw, gb = ops.mapped_conv_backward(_t(g), _t(m), None, _t(x), _t(w), _t(b), K, 0)
+    finally:
+        ops.set_conv_compute("native")
     wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, 0, None)
-    assert relerr(gw.cpu().numpy(), ww) <= 1e-4
-    assert relerr(gi.cpu().numpy(), wi) <= 1e-4
+    tol = 1e-2 if mode == "bf16" else 1e-4
+    assert relerr(gw.cpu().numpy(), ww) <= tol
+    assert relerr(gi.cpu().numpy(), wi) <= tol
     assert relerr(gb.cpu().numpy(), wb) <= 1e-4
 
 
+@pytest.mark.parametrize("mode", ["native", "split"])
 @pytest.mark.parametrize("Cout,K", [(40, 7), (8, 9), (64, 4)])
-def test_workgroups_that_walk_several_tiles(ops, oracle, Cout, K):
+def test_workgroups_that_walk_several_tiles(ops, oracle, Cout, K, mode):
     # 8 batch elements x 8 chunks of image channels: eight workgroups per kind share the 24
     # tiles of the 48 x 64 grid, three each
     m, x, w, b, g = _nearest_case(7 + Cout + K, 8, 256, Cout, 48, 64, K)
     tm = _t(m)
-    for rep in range(2):                       # second call: the plan comes from the cache
-        gi, gw, gb = ops.mapped_conv_backward(_t(g), tm, None, _t(x), _t(w), _t(b), K, 0)
+    ops.set_conv_compute(mode)
+    try:
+        for rep in range(2):                   # second call: the plan comes from the cache
+            gi, gw, gb = ops.mapped_conv_backward(_t(g), tm, None, _t(x), _t(w), _t(b), K, 0)
+    finally:
+        ops.set_conv_compute("native")
     wi, ww, wb = oracle.mapped_conv_backward(g, m, x, w, b, K, 0, None)
     assert relerr(gw.cpu().numpy(), ww) <= 1e-4
     assert relerr(gi.cpu().numpy(), wi) <= 1e-4
