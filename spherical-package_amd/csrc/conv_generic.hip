@@ -224,14 +224,26 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const T* __restrict__ go
   const int vbeg = beg + head;
   T a0 = T(0), a1 = T(0), a2 = T(0), a3 = T(0);
   const int nv = (end - vbeg) / V;
-  for (int i = threadIdx.x; i < nv; i += 256) {
-    if constexpr (V == 4) {
-      const float4 v = reinterpret_cast<const float4*>(p + vbeg)[i];
+  if constexpr (V == 4) {
+    // four loads in flight per thread (one per iteration waits for each in turn)
+    const float4* pv = reinterpret_cast<const float4*>(p + vbeg);
+    int i = threadIdx.x;
+    for (; i + 768 < nv; i += 1024) {
+      const float4 v0 = pv[i], v1 = pv[i + 256], v2 = pv[i + 512], v3 = pv[i + 768];
+      a0 += (v0.x + v1.x) + (v2.x + v3.x);
+      a1 += (v0.y + v1.y) + (v2.y + v3.y);
+      a2 += (v0.z + v1.z) + (v2.z + v3.z);
+      a3 += (v0.w + v1.w) + (v2.w + v3.w);
+    }
+    for (; i < nv; i += 256) {
+      const float4 v = pv[i];
       a0 += v.x;
       a1 += v.y;
       a2 += v.z;
       a3 += v.w;
-    } else {
+    }
+  } else {
+    for (int i = threadIdx.x; i < nv; i += 256) {
       const double2 v = reinterpret_cast<const double2*>(p + vbeg)[i];
       a0 += v.x;
       a1 += v.y;
