@@ -603,14 +603,22 @@ int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const v
  *   sdk_resample_to_map_workspace_bytes(height, width, dtype).  kernel_size = 1
  *   for a resampling map [map_height, map_width, (P,) 2]; for average
  *   unpooling pass the pooled grid as map_height x map_width and the map's K.
- * sdk_resample_plan_complete: synchronises `stream` and sets *complete to 1
- *   when every target's list holds all its sources (at most 16 each).  The
- *   planned calls take that as plan_complete: with 1 they launch the gather
- *   alone (sample_map / interp_weights are then not read by
- *   sdk_resample_to_map_planned and may be NULL); with 0 they also launch the
- *   gated fallback (fill, atomic scatter, division), which runs only if the
- *   plan is incomplete.  Passing 1 for an incomplete plan drops the sources
- *   that did not fit.
+ *   An average-unpooling plan also holds, behind the lists, the pooled window
+ *   of every image tile (as sdk_mapped_max_unpool's plan does): where every
+ *   window has at most 8192 pooled pixels the planned call sums each tile in
+ *   LDS from its window and the lists are neither filled nor read; otherwise
+ *   it gathers through the lists.
+ * sdk_resample_plan_complete: synchronises `stream` and sets *complete to a
+ *   bit mask.  Bit 0 (value 1): the planned call needs no fallback (every
+ *   target's list holds all its sources, at most 16 each, or the lists are not
+ *   used).  Bit 1 (value 2): the tiled average unpooling runs.  The planned
+ *   calls take that mask as plan_complete: with bit 0 set they launch the
+ *   gather (or the tiled kernel) alone (sample_map / interp_weights are then
+ *   not read by sdk_resample_to_map_planned and may be NULL; the average
+ *   unpooling always reads them); with 0 they launch every stage, each gated on
+ *   the device, and the fallback (fill, atomic scatter, division) runs only if
+ *   the plan is incomplete.  Passing a set bit for a plan that did not report
+ *   it gives wrong results (sources that did not fit are dropped).
  * sdk_resample_to_map_planned: normalize = 0 is sdk_resample_to_map (weight_sum
  *   optional), normalize = 1 sdk_resample_to_map_normalized (weight_sum
  *   required, eps used).

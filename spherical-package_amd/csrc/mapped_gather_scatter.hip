@@ -173,7 +173,8 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void resample_inverse_fill_kernel(
     const T* __restrict__ map, const T* __restrict__ wts, int H, int W, int MP, int P,
     int* __restrict__ cnt, int* __restrict__ src, T* __restrict__ co, int* __restrict__ gate,
-    int group) {
+    int group, const int* __restrict__ only_if) {
+  if (only_if != nullptr && *only_if == 0) return;   // the lists are not needed
   const int pix = blockIdx.x * kBlock + threadIdx.x;
   if (pix >= MP) return;
   const int q = WEIGHTED ? P : 1;
@@ -206,7 +207,9 @@ template <typename T, int PC>
 __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
     const T* __restrict__ in, const int* __restrict__ cnt, const int* __restrict__ src,
     const T* __restrict__ co, T* __restrict__ out, T* __restrict__ wsum, int planes, int HW,
-    int MP, const int* __restrict__ gate, int normalize, T eps, int group) {
+    int MP, const int* __restrict__ gate, int normalize, T eps, int group,
+    const int* __restrict__ skip) {
+  if (skip != nullptr && *skip != 0) return;   // the tiled kernel has written the output
   if (*gate != 0) return;
   const int u = banded_pixel_block() * kBlock + threadIdx.x;
   if (u >= HW) return;
@@ -741,6 +744,7 @@ constexpr int kUpTile = 1 << kUpTileLog2;   // image pixels per workgroup
 constexpr int kUpPer = kUpTile / kBlock;    // ... and per thread
 constexpr int kUpWindow = 8192;   // pooled pixels a tile may have to look at
 constexpr int kUpBytes = 32768;   // LDS of the tile accumulators: kUpTile x planes per pass
+constexpr int kUpAhead = 3;       // pooled pixels of a lane whose reads are in flight together
 
 struct UnpoolTiling {
   int H, W, tw_shift, tiles_x, tiles_y;
@@ -957,6 +961,164 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
   }
 }
 
+// Average unpooling by image tile: the tiling and the windows of unpool_tiles_kernel, but every
+// pooled pixel of the window hands value / K to all K of its samples, so the taps of a sample
+// are worked out once for the planes of a pass and no index is read.  A lane walks the samples
+// of its own pooled pixel (neighbouring lanes then add to different image pixels).  Runs only
+// where flags[0] says that every window fits (avg_unpool_verdict_kernel); the sums of a pixel
+// are divided by K once, at the store, like the list gather does.
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void avg_unpool_tiles_kernel(
+    const T* __restrict__ gout, const T* __restrict__ map, const T* __restrict__ wts,
+    const int* __restrict__ win, const int* __restrict__ flags, T* __restrict__ gin,
+    UnpoolTiling ut, int planes, int planes_per_group, int M, int OW, int K, int P) {
+  if (flags[0] == 0) return;
+  constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));   // planes per pass
+  __shared__ T acc[PLMAX * kUpTile];
+  const int tid = threadIdx.x, tile = blockIdx.x;
+  const size_t HW = (size_t)ut.H * ut.W;
+  const int p_begin = blockIdx.y * planes_per_group;
+  const int p_end = min(planes, p_begin + planes_per_group);
+  const int ty0 = (tile / ut.tiles_x) * ut.TH(), tx0 = (tile % ut.tiles_x) << ut.tw_shift;
+  const int q = WEIGHTED ? P : 1;
+  const int* w = win + (size_t)tile * 8;
+  const int anchor = w[0] - 1;
+  int WH = 0, WW = 0, wy0 = 0, wx0 = 0;
+  if (anchor >= 0) {
+    const int ay = anchor / OW, ax = anchor % OW;
+    WH = w[1] + w[2] + 1;
+    const bool full = w[3] + w[4] + 1 >= OW;   // all around: columns as they are
+    WW = full ? OW : w[3] + w[4] + 1;
+    wy0 = ay - w[1];
+    wx0 = full ? 0 : ax - w[3];
+    wx0 += wx0 < 0 ? OW : 0;
+  }
+  const int WN = WH * WW;   // <= kUpWindow (flags[0])
+  const float rcp_ww = WW > 0 ? 1.0f / (float)WW : 0.0f;
+  const T inv_k = T(1) / T(K);
+  int u[kUpPer];
+#pragma unroll
+  for (int j = 0; j < kUpPer; ++j) {
+    const int L = (((tid >> 6) * kUpPer + j) << 6) + (tid & 63);
+    const int y = ty0 + (L >> ut.tw_shift), x = tx0 + (L & (ut.TW() - 1));
+    u[j] = (y < ut.H && x < ut.W) ? y * ut.W + x : -1;
+  }
+#pragma unroll
+  for (int j = 0; j < kUpPer; ++j)
+#pragma unroll
+    for (int pl = 0; pl < PLMAX; ++pl)
+      acc[pl * kUpTile + (((tid >> 6) * kUpPer + j) << 6) + (tid & 63)] = T(0);
+  __syncthreads();
+  for (int p0 = p_begin; p0 < p_end; p0 += PLMAX) {
+    const int np = min(PLMAX, p_end - p0);
+    // kUpAhead pooled pixels per lane and round: their values and first coordinates are all
+    // requested before the first of them is worked on
+    for (int o0 = tid; o0 < WN; o0 += kUpAhead * kBlock) {
+      size_t s0[kUpAhead];
+      T gv[kUpAhead][PLMAX], cx0[kUpAhead], cy0[kUpAhead];
+#pragma unroll
+      for (int j = 0; j < kUpAhead; ++j) {
+        const int o = o0 + j * kBlock < WN ? o0 + j * kBlock : o0;   // past the end: read again
+        const int r = (int)(((float)o + 0.5f) * rcp_ww);    // o / WW (o < 2^13: exact)
+        int ox = wx0 + (o - r * WW);
+        ox -= ox >= OW ? OW : 0;
+        const int m = (wy0 + r) * OW + ox;
+        const size_t at = (size_t)p0 * M + m;
+#pragma unroll
+        for (int pl = 0; pl < PLMAX; ++pl)
+          gv[j][pl] = gout[at + (size_t)(pl < np ? pl : 0) * M];
+        s0[j] = (size_t)m * K * q;   // the pixel's first map point
+        cx0[j] = map[s0[j] * 2];
+        cy0[j] = map[s0[j] * 2 + 1];
+      }
+      const int pts_n = K * q;
+#pragma unroll
+      for (int j = 0; j < kUpAhead; ++j) {
+        if (o0 + j * kBlock >= WN) break;
+        T cx = cx0[j], cy = cy0[j];
+        for (int s = 0; s < pts_n; ++s) {
+          const T x_now = cx, y_now = cy;
+          const size_t sn = s0[j] + min(s + 1, pts_n - 1);   // the next point, a turn ahead
+          cx = map[sn * 2];
+          cy = map[sn * 2 + 1];
+          PointTaps<T, INTERP> taps;
+          taps.set(x_now, y_now, ut.H, ut.W);
+          const T wv = WEIGHTED ? wts[s0[j] + s] : T(1);
+#pragma unroll
+          for (int n = 0; n < PointTaps<T, INTERP>::N; ++n) {
+            const int ry = taps.ty[n] - ty0, rx = taps.tx[n] - tx0;
+            if (taps.off[n] >= 0 && (unsigned)ry < (unsigned)ut.TH() &&
+                (unsigned)rx < (unsigned)ut.TW()) {
+              const int cell = (ry << ut.tw_shift) + rx;
+              const T c = INTERP == 0 ? wv : taps.w[n] * wv;
+              if constexpr (sizeof(T) == 4) {
+                int offs[PLMAX];
+                float vals[PLMAX];
+#pragma unroll
+                for (int pl = 0; pl < PLMAX; ++pl) {
+                  offs[pl] = pl * kUpTile + cell;
+                  vals[pl] = c * gv[j][pl];
+                }
+                lds_add_f32_batch<PLMAX>(reinterpret_cast<float*>(acc), offs, vals);
+              } else {
+#pragma unroll
+                for (int pl = 0; pl < PLMAX; ++pl)
+                  lds_add(acc + pl * kUpTile + cell, c * gv[j][pl]);
+              }
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // store the tile and clear it for the next pass
+#pragma unroll
+    for (int j = 0; j < kUpPer; ++j) {
+#pragma unroll
+      for (int pl = 0; pl < PLMAX; ++pl) {
+        T* cell = acc + pl * kUpTile + (((tid >> 6) * kUpPer + j) << 6) + (tid & 63);
+        const T v = *cell;
+        *cell = T(0);
+        if (u[j] >= 0 && pl < np) gin[(size_t)(p0 + pl) * HW + u[j]] = v * inv_k;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Flags of the tiled average unpooling, in front of its tile windows: [0] every window fits
+// the tiled kernel, [1] the opposite (the inverse lists are needed), [2] the gate of the atomic
+// fallback.  Stage 0 (after the windows): [0] and [1].  Stage 1 (after the lists, whose own
+// gate counts the sources that found a list full): [2] = that gate where the lists are used;
+// the word after the lists' gate receives a copy of [0].
+__global__ __launch_bounds__(kBlock) void avg_unpool_verdict_kernel(
+    const int* __restrict__ win, int tiles, int OW, int* __restrict__ flags,
+    int* __restrict__ lists_gate, int stage) {
+  if (stage == 1) {
+    if (threadIdx.x == 0) {
+      flags[2] = flags[0] != 0 ? 0 : lists_gate[0];
+      lists_gate[1] = flags[0];   // for the host: sdk_resample_plan_complete
+    }
+    return;
+  }
+  __shared__ int too_big;
+  if (threadIdx.x == 0) too_big = 0;
+  __syncthreads();
+  for (int t = threadIdx.x; t < tiles; t += kBlock) {
+    const int* w = win + (size_t)t * 8;
+    if (w[0] > 0) {
+      const int64_t WH = (int64_t)w[1] + w[2] + 1;
+      const int64_t WW = min((int64_t)w[3] + w[4] + 1, (int64_t)OW);
+      if (WH * WW > kUpWindow) too_big = 1;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    flags[0] = too_big ? 0 : 1;
+    flags[1] = too_big ? 1 : 0;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Host-side launch helpers.
 // ---------------------------------------------------------------------------
@@ -1000,62 +1162,127 @@ static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
   return off[3] + up((size_t)HW * kInvSlots * esz);
 }
 
+static UnpoolTiling unpool_tiling(int H, int W);
+static size_t unpool_layout(const UnpoolTiling& ut);
+template <typename T>
+static int build_unpool_windows(const T* map, void* workspace, int H, int W, int OH, int OW, int K,
+                                int P, int interp, hipStream_t stream);
+
+// Average unpooling (group = K > 1 samples per pooled pixel, pooled rows of OW pixels) can run
+// tiled over the image when the workspace has room for the tile windows behind the lists.
+static bool avg_unpool_tiled(int H, int W, int MP, int group, int OW, int P, size_t esz,
+                             int64_t planes, size_t lists_bytes, size_t workspace_bytes) {
+  if (group <= 1 || OW <= 0 || (MP / group) % OW != 0) return false;
+  const UnpoolTiling ut = unpool_tiling(H, W);
+  return workspace_bytes >= lists_bytes + unpool_layout(ut) &&
+         (int64_t)ut.tiles_x * ut.tiles_y < ((int64_t)1 << 27) && planes < ((int64_t)1 << 31);
+}
+
 // Inverts a map into `workspace` (inverse_layout bytes): per target pixel the list of its
 // (source, coefficient) pairs, and the gate word that counts sources that found their list full.
+// For average unpooling with room for them (avg_unpool_tiled) the tile windows and their flags
+// follow the lists, and the lists are filled only where a window is too large for the tiled
+// kernel.
 template <typename T>
-static int build_inverse_lists(const T* map, const T* wts, void* workspace, int H, int W, int MP,
-                               int P, int interp, int group, hipStream_t stream) {
+static int build_inverse_lists(const T* map, const T* wts, void* workspace, size_t workspace_bytes,
+                               int H, int W, int MP, int P, int interp, int group, int OW,
+                               hipStream_t stream) {
   size_t off[4];
-  inverse_layout((int64_t)H * W, sizeof(T), off);
+  const size_t lists_bytes = inverse_layout((int64_t)H * W, sizeof(T), off);
   char* ws = static_cast<char*>(workspace);
   int* g = reinterpret_cast<int*>(ws + off[0]);
   int* cnt = reinterpret_cast<int*>(ws + off[1]);
   int* src = reinterpret_cast<int*>(ws + off[2]);
   T* co = reinterpret_cast<T*>(ws + off[3]);
-  int rc = zero_fill(ws, off[2], stream);
+  int* flags = nullptr;
+  if (avg_unpool_tiled(H, W, MP, group, OW, P, sizeof(T), 0, lists_bytes, workspace_bytes)) {
+    flags = reinterpret_cast<int*>(ws + lists_bytes);
+    const UnpoolTiling ut = unpool_tiling(H, W);
+    const int rc = build_unpool_windows<T>(map, ws + lists_bytes, H, W, MP / group / OW, OW, group,
+                                           P, interp, stream);
+    if (rc != SDK_OK) return rc;
+    launch(avg_unpool_verdict_kernel, dim3(1), dim3(kBlock), stream, (const int*)(flags + 64),
+           ut.tiles_x * ut.tiles_y, OW, flags, g, 0);
+    SDK_LAUNCH_CHECK("mapped_avg_unpool(windows)");
+  }
+  int rc;
+  if (flags) {   // the gate, read by the caller whatever happens; the counters where needed
+    rc = zero_fill(ws, off[1], stream);
+    if (rc == SDK_OK) rc = zero_fill_gated(ws + off[1], off[2] - off[1], stream, flags + 1);
+  } else {
+    rc = zero_fill(ws, off[2], stream);
+  }
   if (rc != SDK_OK) return rc;
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((resample_inverse_fill_kernel<T, INTERP, WEIGHTED>),
                               dim3((unsigned)ceil_div(MP, kBlock)), dim3(kBlock), stream, map,
-                              wts, H, W, MP, P, cnt, src, co, g, group)));
+                              wts, H, W, MP, P, cnt, src, co, g, group,
+                              (const int*)(flags ? flags + 1 : nullptr))));
   SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
+  if (flags) {
+    launch(avg_unpool_verdict_kernel, dim3(1), dim3(kBlock), stream, (const int*)(flags + 64), 0,
+           OW, flags, g, 1);
+    SDK_LAUNCH_CHECK("mapped_avg_unpool(gate)");
+  }
   return SDK_OK;
 }
 
 // prebuilt: `workspace` already holds the lists of this map (build_inverse_lists);
-// complete: ... and the caller knows that its gate is 0, so the fallback launches are left out.
+// complete: ... and the caller knows (sdk_resample_plan_complete) that its gate is 0 (bit 0),
+// so the fallback launches are left out, and that the tiled average unpooling runs (bit 1), so
+// the list gather is left out as well.
+// OW > 0 (average unpooling): width of the pooled grid.
 template <typename T>
 static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* out, T* wsum,
                                   void* workspace, size_t workspace_bytes, int64_t planes, int H,
                                   int W, int MP, int P, int interp, hipStream_t stream,
                                   bool normalize = false, double eps = 0.0, int group = 1,
-                                  bool prebuilt = false, bool complete = false) {
+                                  bool prebuilt = false, int complete = 0, int OW = 0) {
   const int HW = H * W;
   const int* gate = nullptr;   // non-null: device flag, != 0 means "use the atomic scatter"
   size_t off[4];
-  if (workspace != nullptr && workspace_bytes >= inverse_layout(HW, sizeof(T), off)) {
+  const size_t lists_bytes = inverse_layout(HW, sizeof(T), off);
+  if (workspace != nullptr && workspace_bytes >= lists_bytes) {
     char* ws = static_cast<char*>(workspace);
     int* g = reinterpret_cast<int*>(ws + off[0]);
     int* cnt = reinterpret_cast<int*>(ws + off[1]);
     int* src = reinterpret_cast<int*>(ws + off[2]);
     T* co = reinterpret_cast<T*>(ws + off[3]);
+    const bool tiled = !normalize && wsum == nullptr &&
+                       avg_unpool_tiled(H, W, MP, group, OW, P, sizeof(T), planes, lists_bytes, workspace_bytes);
+    const int* flags = tiled ? reinterpret_cast<const int*>(ws + lists_bytes) : nullptr;
     if (!prebuilt) {
-      const int rc = build_inverse_lists<T>(map, wts, workspace, H, W, MP, P, interp, group, stream);
+      const int rc = build_inverse_lists<T>(map, wts, workspace, tiled ? workspace_bytes : lists_bytes,
+                                            H, W, MP, P, interp, group, OW, stream);
       if (rc != SDK_OK) return rc;
     }
-    if (planes > 0 || wsum) {
+    if (tiled && planes > 0) {
+      const UnpoolTiling ut = unpool_tiling(H, W);
+      const int64_t tiles = (int64_t)ut.tiles_x * ut.tiles_y;
+      constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));
+      const int64_t groups = std::max<int64_t>(1, std::min<int64_t>(ceil_div(planes, PLMAX),
+                                                                    ceil_div(16384, tiles)));
+      const int64_t per_group = ceil_div(ceil_div(planes, groups), PLMAX) * PLMAX;
+      const dim3 grid_t((unsigned)tiles, (unsigned)ceil_div(planes, per_group));   // <= 16384 rows
+      SDK_DISPATCH_INTERP(interp, P,
+                          (launch((avg_unpool_tiles_kernel<T, INTERP, WEIGHTED>), grid_t,
+                                  dim3(kBlock), stream, in, map, wts, flags + 64, flags, out, ut,
+                                  (int)planes, (int)per_group, MP / group, OW, group, P)));
+      SDK_LAUNCH_CHECK("mapped_avg_unpool(tiles)");
+    }
+    if ((planes > 0 || wsum) && !(tiled && prebuilt && (complete & 2))) {
       const int pc = planes_per_thread(planes);
 #define RIG(PCv)                                                                                 \
   launch(resample_inverse_gather_kernel<T, PCv>,                                                 \
          dim3(banded_grid_x(HW), (unsigned)std::max<int64_t>(1, ceil_div(planes, PCv))),         \
          dim3(kBlock), stream, in, (const int*)cnt, (const int*)src, (const T*)co, out, wsum,    \
-         (int)planes, HW, MP, (const int*)g, normalize ? 1 : 0, (T)eps, group)
+         (int)planes, HW, MP, (const int*)g, normalize ? 1 : 0, (T)eps, group, flags)
       if (pc == 8) RIG(8); else if (pc == 4) RIG(4); else RIG(2);
 #undef RIG
       SDK_LAUNCH_CHECK("resample_to_map(inverse gather)");
     }
-    gate = g;
-    if (prebuilt && complete) return SDK_OK;
+    gate = tiled ? flags + 2 : g;
+    if (prebuilt && (complete & 1)) return SDK_OK;
   }
   // the scatter: fills, then one launch for all planes and (an extra grid row) the weight sum
   const size_t out_bytes = sizeof(T) * (size_t)planes * H * W, sum_bytes = sizeof(T) * (size_t)H * W;
@@ -1404,7 +1631,9 @@ int sdk_resample_from_map(const void* image, const void* sample_map, const void*
 size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_t dtype) {
   if (height < 1 || width < 1 || height * width >= ((int64_t)1 << 31)) return 0;
   size_t off[4];
-  return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off);
+  // the inverse lists, then the tile windows of the tiled average unpooling
+  return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off) +
+         unpool_layout(unpool_tiling((int)height, (int)width));
 }
 
 static int resample_to_map_entry(const void* input, const void* sample_map,
@@ -1654,7 +1883,8 @@ int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
                                 (const T*)interp_weights, (T*)grad_input, (T*)nullptr, workspace,
                                 workspace_bytes, planes, (int)height, (int)width,
                                 (int)(M * kernel_size), num_interp_pts, interp,
-                                (hipStream_t)stream, false, 0.0, (int)kernel_size));
+                                (hipStream_t)stream, false, 0.0, (int)kernel_size, false, 0,
+                                (int)out_width));
   return SDK_OK;
 }
 
@@ -1763,21 +1993,22 @@ int sdk_resample_to_map_plan_build(const void* sample_map, const void* interp_we
     return fail(SDK_ERR_WORKSPACE, "resample_to_map_plan_build: plan of %zu bytes, need %zu",
                 plan_bytes, need);
   SDK_DISPATCH_DTYPE(dtype, return build_inverse_lists<T>(
-                                (const T*)sample_map, (const T*)interp_weights, plan, (int)height,
-                                (int)width, (int)(map_height * map_width * kernel_size),
-                                num_interp_pts, interp, (int)kernel_size, (hipStream_t)stream));
+                                (const T*)sample_map, (const T*)interp_weights, plan, plan_bytes,
+                                (int)height, (int)width,
+                                (int)(map_height * map_width * kernel_size), num_interp_pts,
+                                interp, (int)kernel_size, (int)map_width, (hipStream_t)stream));
   return SDK_OK;
 }
 
 int sdk_resample_plan_complete(const void* plan, size_t plan_bytes, sdk_stream_t stream,
                                int32_t* complete) {
   SDK_REQUIRE(plan && complete && plan_bytes >= 256, "resample_plan_complete: bad argument");
-  int gate = 1;
-  hipError_t e = hipMemcpyAsync(&gate, plan, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream);
+  int gate[2] = {1, 0};   // sources that found a list full; "the tiled average unpooling runs"
+  hipError_t e = hipMemcpyAsync(gate, plan, sizeof(gate), hipMemcpyDeviceToHost, (hipStream_t)stream);
   if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
   if (e != hipSuccess)
     return fail(SDK_ERR_DEVICE, "resample_plan_complete: %s", hipGetErrorString(e));
-  *complete = gate == 0 ? 1 : 0;
+  *complete = (gate[0] == 0 ? 1 : 0) | (gate[1] != 0 ? 2 : 0);
   return SDK_OK;
 }
 
@@ -1843,7 +2074,7 @@ int sdk_mapped_avg_unpool_planned(const void* grad_output, const void* sample_ma
                                 plan_bytes, planes, (int)height, (int)width,
                                 (int)(M * kernel_size), num_interp_pts, interp,
                                 (hipStream_t)stream, false, 0.0, (int)kernel_size, true,
-                                plan_complete != 0));
+                                plan_complete, (int)out_width));
   return SDK_OK;
 }
 

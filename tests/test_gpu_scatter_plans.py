@@ -139,13 +139,50 @@ def test_avg_unpool_planned(capi, oracle, P, interp):
     flag = ctypes.c_int32(-1)
     capi.call("sdk_resample_plan_complete", _p(plan), n, _stream(),
               ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
-    # (K * P * 4 = 40 taps per pooled pixel overfill some lists of the weighted case)
-    assert flag.value == (1 if P == 0 else 0)
+    # every tile's window of the pooled grid is small here, so the call runs tiled over the
+    # image and the lists (which K * P * 4 = 40 taps per pooled pixel would overfill in the
+    # weighted case) are not needed
+    assert flag.value == 3          # no fallback needed (1), the tiled kernel runs (2)
     want = oracle.mapped_avg_unpool(g, m, H, W, K, interp, iw)
     for complete in sorted({int(flag.value), 0}):
         out = torch.full((B, C, H, W), float("nan"), device=DEV)
         capi.call("sdk_mapped_avg_unpool_planned", _p(tg), _p(tm), _p(tiw), _p(out), _p(plan), n,
                   complete, B, C, H, W, OH, OW, K, P, interp, F32, _stream())
+        assert relerr(_n(out), want) <= 1e-5
+
+
+@pytest.mark.parametrize("K,want_flag", [(2, 1), (8, 0)])
+def test_avg_unpool_of_a_scattered_map(capi, oracle, K, want_flag):
+    """Samples anywhere in the image: every image tile is reached from all over the pooled grid
+    (96 x 96 > 8192 pooled pixels per window), so the tiled kernel stands back and the call
+    gathers through the lists (K = 2, nearest taps: about 4.5 sources per image pixel) or, where those
+    overflow (K = 8: about 18), falls back to the atomic scatter; planned with either
+    plan_complete value, and unplanned with the call's own workspace and without one."""
+    rng = np.random.default_rng(5 + K)
+    OH, OW, H, W = 96, 96, 64, 64
+    m = np.stack([rng.uniform(-0.4, W - 0.6, (OH, OW, K)),
+                  rng.uniform(-0.4, H - 0.6, (OH, OW, K))], -1).astype(np.float32)
+    g = rng.standard_normal((2, 3, OH, OW)).astype(np.float32)
+    tm, tg = _t(m), _t(g)
+    B, C = g.shape[:2]
+    n = capi.load().sdk_resample_to_map_workspace_bytes(H, W, F32)
+    plan = torch.empty(n, dtype=torch.uint8, device=DEV)
+    capi.call("sdk_resample_to_map_plan_build", _p(tm), None, _p(plan), n, OH, OW, H, W, K, 0,
+              0, F32, _stream())
+    flag = ctypes.c_int32(-1)
+    capi.call("sdk_resample_plan_complete", _p(plan), n, _stream(),
+              ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+    assert flag.value == want_flag
+    want = oracle.mapped_avg_unpool(g, m, H, W, K, 0, None)
+    for complete in sorted({int(flag.value), 0}):
+        out = torch.full((B, C, H, W), float("nan"), device=DEV)
+        capi.call("sdk_mapped_avg_unpool_planned", _p(tg), _p(tm), None, _p(out), _p(plan), n,
+                  complete, B, C, H, W, OH, OW, K, 0, 0, F32, _stream())
+        assert relerr(_n(out), want) <= 1e-5
+    for ws, nws in ((torch.empty(n, dtype=torch.uint8, device=DEV), n), (None, 0)):
+        out = torch.full((B, C, H, W), float("nan"), device=DEV)
+        capi.call("sdk_mapped_avg_unpool", _p(tg), _p(tm), None, _p(out), _p(ws), nws, B, C, H, W,
+                  OH, OW, K, 0, 0, F32, _stream())
         assert relerr(_n(out), want) <= 1e-5
 
 
