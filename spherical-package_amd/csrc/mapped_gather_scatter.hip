@@ -961,7 +961,9 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
   }
 }
 
-// Average unpooling by image tile: the tiling and the windows of unpool_tiles_kernel, but every
+// Average unpooling by image tile (body: common/mapped_avg_pool.h:42-69, :109-143, every
+// sample of a pooled pixel receiving grad_output / K through the resampling scatter of
+// core/resample.h): the tiling and the windows of unpool_tiles_kernel, but every
 // pooled pixel of the window hands value / K to all K of its samples, so the taps of a sample
 // are worked out once for the planes of a pass and no index is read.  A lane walks the samples
 // of its own pooled pixel (neighbouring lanes then add to different image pixels).  Runs only
@@ -995,7 +997,6 @@ __global__ __launch_bounds__(kBlock) void avg_unpool_tiles_kernel(
   }
   const int WN = WH * WW;   // <= kUpWindow (flags[0])
   const float rcp_ww = WW > 0 ? 1.0f / (float)WW : 0.0f;
-  const T inv_k = T(1) / T(K);
   int u[kUpPer];
 #pragma unroll
   for (int j = 0; j < kUpPer; ++j) {
@@ -1079,7 +1080,7 @@ __global__ __launch_bounds__(kBlock) void avg_unpool_tiles_kernel(
         T* cell = acc + pl * kUpTile + (((tid >> 6) * kUpPer + j) << 6) + (tid & 63);
         const T v = *cell;
         *cell = T(0);
-        if (u[j] >= 0 && pl < np) gin[(size_t)(p0 + pl) * HW + u[j]] = v * inv_k;
+        if (u[j] >= 0 && pl < np) gin[(size_t)(p0 + pl) * HW + u[j]] = v / T(K);
       }
     }
     __syncthreads();
