@@ -44,7 +44,9 @@ def set_conv_compute(mode):
 
 
 def _current_mode():
-    return getattr(_tls, "mode", None) or _default_mode
+    # SDK_COMPUTE_NATIVE is 0: an override is "set" when it is not None, whatever its value
+    mode = getattr(_tls, "mode", None)
+    return _default_mode if mode is None else mode
 
 
 def get_conv_compute():
@@ -126,25 +128,78 @@ def _workspace(ref, batch, cin, cout, img_h, img_w, map_h, map_w, K, P, interp):
 # (and the point weights') storage address, offset, version counter, shape and the geometry, and
 # holds the storages, so an address cannot be handed to another tensor while its entry lives;
 # in-place changes of a map bump its version and miss.
+#
+# The cache evicts the least recently used entry beyond `_PLAN_CACHE_MAX` (a hit moves its
+# entry to the end).  Three kinds of call go past it, to the entry points that build what they
+# need in the call's own workspace: a map without a version counter (a tensor created under
+# torch.inference_mode(): an in-place change of it could not be seen), a key that misses while
+# the current stream is being captured into a graph (the build would only be recorded, the
+# entry would look built to an eager call before the first replay, and its buffer would belong
+# to the graph's private pool), and everything when the cache is switched off.
 _PLAN_CACHE = {}
 _PLAN_CACHE_MAX = 16
 _plan_cache_enabled = True
+_NO_KEY = object()   # _tensor_key of a tensor whose changes cannot be tracked
 
 
-def set_conv_plan_cache(enabled):
+class _PlanEntry:
+    """A kept plan: the buffer, its size, the storages of the map it was built from, the
+    stream that used it last (every call reads the plan, and the max-unpool call rewrites the
+    plan's gate word, so a call on another stream is ordered behind the last user) and the
+    `complete` verdict of a scatter plan."""
+    __slots__ = ("plan", "nbytes", "keep", "stream", "complete")
+
+    def __init__(self, plan, nbytes, keep, stream, complete=0):
+        self.plan, self.nbytes, self.keep, self.stream, self.complete = \
+            plan, nbytes, keep, stream, complete
+
+
+def set_conv_plan_cache(enabled, max_entries=None):
     """Keeps (default) or rebuilds per call what the operators derive from a map alone: the
     plans of the mapped (transposed) convolutions, the inverted maps of resample_to_map and
-    average unpooling, the tile windows of max unpooling."""
-    global _plan_cache_enabled
+    average unpooling, the tile windows of max unpooling.  max_entries: how many plans are
+    kept (least recently used dropped first; default 16, one per (map, geometry) in use)."""
+    global _plan_cache_enabled, _PLAN_CACHE_MAX
     _plan_cache_enabled = bool(enabled)
+    if max_entries is not None:
+        if int(max_entries) < 1:
+            raise ValueError("max_entries must be at least 1")
+        _PLAN_CACHE_MAX = int(max_entries)
     if not enabled:
         _PLAN_CACHE.clear()
+    while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
+        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
 
 
 def _tensor_key(t):
     if t is None:
         return None
+    if t.is_inference():
+        return _NO_KEY
     return (t.untyped_storage().data_ptr(), t.storage_offset(), t._version, tuple(t.shape))
+
+
+def _cache_lookup(key, cur):
+    """The entry of `key`, made the most recently used one and ordered behind its last user
+    on another stream; None on a miss."""
+    ent = _PLAN_CACHE.pop(key, None)
+    if ent is None:
+        return None
+    _PLAN_CACHE[key] = ent
+    if ent.stream != cur:
+        cur.wait_stream(ent.stream)
+        ent.stream = cur
+    return ent
+
+
+def _cache_insert(key, ent):
+    while len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
+        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
+    _PLAN_CACHE[key] = ent
+
+
+def _uncacheable(*keys):
+    return any(k is _NO_KEY for k in keys)
 
 
 def _conv_plan(ref, sample_map, interp_weights, img_h, img_w, K, P, interp):
@@ -153,14 +208,16 @@ def _conv_plan(ref, sample_map, interp_weights, img_h, img_w, K, P, interp):
     if not _plan_cache_enabled or ref.dtype != torch.float32:
         return None, 0
     MH, MW = int(sample_map.shape[0]), int(sample_map.shape[1])
-    key = (ref.device, _tensor_key(sample_map), _tensor_key(interp_weights), int(img_h),
-           int(img_w), int(K), int(P), int(interp))
-    ent = _PLAN_CACHE.get(key)
+    km, kw = _tensor_key(sample_map), _tensor_key(interp_weights)
+    if _uncacheable(km, kw):
+        return None, 0
+    key = (ref.device, km, kw, int(img_h), int(img_w), int(K), int(P), int(interp))
     cur = torch.cuda.current_stream(ref.device)
+    ent = _cache_lookup(key, cur)
     if ent is not None:
-        if ent[3] != cur:
-            cur.wait_stream(ent[3])   # built on another stream: order this call behind the build
-        return ent[0], ent[1]
+        return ent.plan, ent.nbytes
+    if torch.cuda.is_current_stream_capturing():
+        return None, 0
     n = _capi.load().sdk_mapped_conv_plan_bytes(int(img_h), int(img_w), MH, MW, int(K), int(P),
                                                 int(interp), _capi.SDK_F32)
     if n == 0:
@@ -169,11 +226,9 @@ def _conv_plan(ref, sample_map, interp_weights, img_h, img_w, K, P, interp):
     _capi.call("sdk_mapped_conv_plan_build", _ptr(sample_map), _ptr(interp_weights), _ptr(plan), n,
                int(img_h), int(img_w), MH, MW, int(K), int(P), int(interp), _capi.SDK_F32,
                _stream(ref))
-    while len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
-        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
     keep = (sample_map.untyped_storage(),
             None if interp_weights is None else interp_weights.untyped_storage())
-    _PLAN_CACHE[key] = (plan, n, keep, cur)
+    _cache_insert(key, _PlanEntry(plan, n, keep, cur))
     return plan, n
 
 
@@ -188,14 +243,16 @@ def _scatter_plan(kind, ref, sample_map, interp_weights, out_h, out_w, K, P, int
     if not _plan_cache_enabled:
         return None, 0, 0
     dt = _DTYPES[ref.dtype]
-    key = (kind, ref.device, dt, _tensor_key(sample_map), _tensor_key(interp_weights),
-           int(out_h), int(out_w), int(K), int(P), int(interp))
-    ent = _PLAN_CACHE.get(key)
+    km, kw = _tensor_key(sample_map), _tensor_key(interp_weights)
+    if _uncacheable(km, kw):
+        return None, 0, 0
+    key = (kind, ref.device, dt, km, kw, int(out_h), int(out_w), int(K), int(P), int(interp))
     cur = torch.cuda.current_stream(ref.device)
+    ent = _cache_lookup(key, cur)
     if ent is not None:
-        if ent[3] != cur:
-            cur.wait_stream(ent[3])
-        return ent[0], ent[1], ent[4]
+        return ent.plan, ent.nbytes, ent.complete
+    if torch.cuda.is_current_stream_capturing():
+        return None, 0, 0
     lib = _capi.load()
     query = ("sdk_mapped_max_unpool_workspace_bytes" if kind == "max_unpool"
              else "sdk_resample_to_map_workspace_bytes")
@@ -212,16 +269,13 @@ def _scatter_plan(kind, ref, sample_map, interp_weights, out_h, out_w, K, P, int
         _capi.call("sdk_resample_to_map_plan_build", _ptr(sample_map), _ptr(interp_weights),
                    _ptr(plan), n, MH, MW, int(out_h), int(out_w), int(K), int(P), int(interp), dt,
                    _stream(ref))
-        if not torch.cuda.is_current_stream_capturing():
-            flag = ctypes.c_int32(0)
-            _capi.call("sdk_resample_plan_complete", _ptr(plan), n, _stream(ref),
-                       ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
-            complete = int(flag.value)
-    while len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
-        _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
+        flag = ctypes.c_int32(0)
+        _capi.call("sdk_resample_plan_complete", _ptr(plan), n, _stream(ref),
+                   ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+        complete = int(flag.value)
     keep = (sample_map.untyped_storage(),
             None if interp_weights is None else interp_weights.untyped_storage())
-    _PLAN_CACHE[key] = (plan, n, keep, cur, complete)
+    _cache_insert(key, _PlanEntry(plan, n, keep, cur, complete))
     return plan, n, complete
 
 

@@ -54,10 +54,22 @@ struct PlanArg {
   size_t bytes = 0;
 };
 
+// The size check of a caller's plan buffer, also made up front by the combined backward calls
+// so that a refused call has launched nothing.
+int check_plan(const char* what, const ConvGeom& g, int dtype, int compute, PlanArg plan) {
+  if (plan.buffer == nullptr || dtype != SDK_F32 || compute == SDK_COMPUTE_UNFUSED ||
+      !fused_supported(g))
+    return SDK_OK;
+  const size_t need = cached_plan_bytes(g);
+  if (need == 0 || plan.bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "%s: the plan buffer has %zu bytes, this geometry's plan %zu",
+                what, plan.bytes, need);
+  return SDK_OK;
+}
+
 int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, const void* in0,
         const void* map, const void* wts, const void* in1, const void* bias, void* out, void* ws,
-        size_t ws_bytes, hipStream_t stream, SharedPlan* shared = nullptr,
-        PlanArg plan = PlanArg()) {
+        size_t ws_bytes, hipStream_t stream, SharedPlan* shared, PlanArg plan) {
   if (g.B == 0 && op != GATHER_WGRAD) return SDK_OK;
   if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && fused_supported(g)) {
     int rc = check_workspace(what, fused_workspace_bytes(g), ws, ws_bytes);
@@ -65,10 +77,8 @@ int run(const char* what, Op op, const ConvGeom& g, int dtype, int compute, cons
     CachedPlan cached;
     const CachedPlan* cp = nullptr;
     if (plan.buffer != nullptr) {
-      const size_t need = cached_plan_bytes(g);
-      if (need == 0 || plan.bytes < need)
-        return fail(SDK_ERR_WORKSPACE, "%s: the plan buffer has %zu bytes, this geometry's plan %zu",
-                    what, plan.bytes, need);
+      rc = check_plan(what, g, dtype, compute, plan);
+      if (rc) return rc;
       load_cached_plan(g, plan.buffer, &cached);
       cp = &cached;
     }
@@ -298,7 +308,7 @@ static int impl_mapped_transposed_conv_backward_input(const void* grad_output, c
   ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)in_width};
   return run(what, GATHER_GEMM, g, dtype, compute, grad_output, sample_map, interp_weights, weight,
-             nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream);
+             nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, nullptr, plan);
 }
 
 static int impl_mapped_transposed_conv_backward_weight(const void* grad_output, const void* sample_map,
@@ -344,6 +354,8 @@ static int impl_mapped_conv_backward(const void* grad_output, const void* sample
   if (rc) return rc;
   ConvGeom g{batch, (int)in_channels, (int)height, (int)width, (int)out_channels, (int)M,
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
+  rc = check_plan(what, g, dtype, compute, plan);
+  if (rc) return rc;
   hipEvent_t joined = nullptr;
   rc = fork_side((hipStream_t)stream, &joined, side_worth(batch, out_channels, M, dtype),
                  [&](hipStream_t s) {
@@ -378,8 +390,20 @@ static int impl_mapped_transposed_conv_backward(const void* grad_output, const v
   SDK_REQUIRE(grad_output && grad_bias, "%s: NULL pointer", what);
   SDK_REQUIRE(out_height >= 1 && out_width >= 1 && out_height * out_width < ((int64_t)1 << 31),
               "%s: bad output size", what);
+  SDK_REQUIRE(in_height >= 1 && in_width >= 1, "%s: bad input size", what);
+  int rc = check_common(what, batch, out_channels, out_height, out_width, in_channels,
+                        in_height * in_width, kernel_size, num_interp_pts, interp_weights, dtype,
+                        compute);
+  if (rc) return rc;
+  {
+    ConvGeom g{batch, (int)out_channels, (int)out_height, (int)out_width, (int)in_channels,
+               (int)(in_height * in_width), (int)kernel_size, num_interp_pts, interp,
+               (int)in_width};
+    rc = check_plan(what, g, dtype, compute, plan);
+    if (rc) return rc;
+  }
   hipEvent_t joined = nullptr;
-  int rc = fork_side((hipStream_t)stream, &joined,
+  rc = fork_side((hipStream_t)stream, &joined,
                      side_worth(batch, out_channels, out_height * out_width, dtype),
                      [&](hipStream_t s) {
     return bias_grad(grad_output, grad_bias, batch, out_channels, out_height * out_width, dtype, s,

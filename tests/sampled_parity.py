@@ -11,6 +11,12 @@ on those pixels:
                                                grad_output that is zero outside pix
   backward, dense g  grad_input[:, :, tgt]   = oracle_backward_input(g[src], map[src])[tgt]
                                                where src = every map pixel with a tap in tgt
+                     grad_weight[ns][:, cs]  = oracle_backward(g[:, ns], map, x[:, cs])'s
+                                               grad_weight: an entry (n, c, k) of the weight
+                                               gradient sums over batch and pixels only, so
+                                               the oracle on channel subsets of x and g (whole
+                                               map, every pixel) returns the full evaluation's
+                                               entries for those channels
 
 No formula is restated here: only the oracle's own entry points are called, on sliced maps.
 """
@@ -100,7 +106,9 @@ class ConvOracle:
     cfg: dict of numpy arrays as workloads.config4 / config5 return them."""
 
     def __init__(self, oracle, cfg, n_random, n_targets, seed=0, rows=(0, 1, -2, -1),
-                 cols=(0, -1)):
+                 cols=(0, -1), n_weight_channels=0):
+        """n_weight_channels: how many output and input channels (first, last and random ones
+        between) the dense weight gradient is evaluated on by the oracle; 0 leaves it out."""
         self.cfg = cfg
         m, iw = cfg["sample_map"], cfg.get("interp_weights")
         x, w, b, g = cfg["x"], cfg["weight"], cfg["bias"], cfg["grad_output"]
@@ -119,6 +127,20 @@ class ConvOracle:
         ms, ws = slice_map(m, iw, self.sources)
         gi = oracle.mapped_conv_backward_input(at(g, self.sources), ms, x.shape, w, K, it, ws)
         self.grad_input_dense = at(gi, self.targets)
+        # dense grad_output, grad_weight on channel subsets
+        self.w_out = self.w_in = None
+        if n_weight_channels:
+            rng = np.random.default_rng(seed + 2)
+
+            def pick(n):
+                k = min(int(n_weight_channels), n)
+                mid = rng.choice(np.arange(1, n - 1), size=max(k - 2, 0), replace=False) \
+                    if n > 2 else np.zeros(0, np.int64)
+                return np.unique(np.concatenate([[0, n - 1], mid]).astype(np.int64))[:max(k, 1)]
+            self.w_out, self.w_in = pick(w.shape[0]), pick(w.shape[1])
+            _, self.grad_weight_dense, _ = oracle.mapped_conv_backward(
+                np.ascontiguousarray(g[:, self.w_out]), m, np.ascontiguousarray(x[:, self.w_in]),
+                np.ascontiguousarray(w[self.w_out][:, self.w_in]), b[self.w_out], K, it, iw)
 
     def check_forward(self, y):
         return relerr(at(y, self.pix), self.forward)
@@ -132,3 +154,9 @@ class ConvOracle:
     def check_backward_dense(self, gi):
         """gi: the GPU's grad_input for the configuration's dense grad_output."""
         return relerr(at(gi, self.targets), self.grad_input_dense)
+
+    def check_weight_dense(self, gw):
+        """gw: the GPU's grad_weight [Cout, Cin, K] for the dense grad_output, compared on
+        the channel subsets the oracle evaluated."""
+        gw = gw.detach().cpu().numpy() if hasattr(gw, "detach") else np.asarray(gw)
+        return relerr(gw[self.w_out][:, self.w_in], self.grad_weight_dense)

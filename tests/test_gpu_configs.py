@@ -67,7 +67,8 @@ def test_configuration2_reduced(ops, oracle):
     norm, wsum = ops.resample_to_map_normalized(_t(want), _t(m), None, H, W, it, 1e-12)
     want_sum = oracle.resample_to_map(np.ones((1, 1) + want.shape[2:], np.float32), m, H, W, it)[0, 0]
     assert relerr(_n(wsum), want_sum) <= BWD
-    assert relerr(_n(norm), want_back / (want_sum + np.float32(1e-12))) <= 1e-3
+    # non-negative weights: the quotient's error stays at n * eps * max|value| (scatter bound)
+    assert relerr(_n(norm), want_back / (want_sum + np.float32(1e-12))) <= BWD
     # nearest-neighbour gather: bit-exact
     near = _n(ops.resample_from_map(_t(x), _t(m), None, 0))
     assert np.array_equal(near, oracle.resample_from_map(x, m, 0))

@@ -114,13 +114,18 @@ def test_planned_calls_match_plain_calls_and_the_oracle(ops, oracle, tc, mode):
                 # its input lives on the map's grid, its output is H x W
                 yt = ops.mapped_transposed_conv_forward(_t(g), tm, tiw, _t(w), _t(bt), H, W, K,
                                                         interp)
-            res[cached] = [t.cpu().numpy() for t in (y, gi, gw, gb, yt)]
+                # ... and its backward: cotangent on the H x W image, input = g on the grid
+                tgi, tgw, tgb = ops.mapped_transposed_conv_backward(_t(x), tm, tiw, _t(g), _t(w),
+                                                                    _t(bt), K, interp)
+            res[cached] = [t.cpu().numpy() for t in (y, gi, gw, gb, yt, tgi, tgw, tgb)]
     finally:
         ops.set_conv_plan_cache(True)
         ops.set_conv_compute("native")
-    y0, gi0, gw0, gb0, yt0 = res[False]
-    y1, gi1, gw1, gb1, yt1 = res[True]
+    y0, gi0, gw0, gb0, yt0, tgi0, tgw0, tgb0 = res[False]
+    y1, gi1, gw1, gb1, yt1, tgi1, tgw1, tgb1 = res[True]
     assert np.array_equal(y0, y1)
+    assert np.array_equal(tgi0, tgi1)          # a gather in either case: the same bits
+    assert relerr(tgw1, tgw0) <= 1e-6 and relerr(tgb1, tgb0) <= 1e-6
     if kind == "crowded" or Cin <= 64:
         # scatter fallback (float atomics) / narrow layers (source lists in the order the
         # atomics were served): the summation order varies from run to run
@@ -136,6 +141,8 @@ def test_planned_calls_match_plain_calls_and_the_oracle(ops, oracle, tc, mode):
     assert relerr(gi1, wi) <= tol_b and relerr(gw1, ww) <= tol_b
     assert relerr(yt1, oracle.mapped_transposed_conv_forward(g, m, w, bt, H, W, K, interp,
                                                              iw)) <= tol_b
+    ti, tw, tb = oracle.mapped_transposed_conv_backward(x, m, g, w, bt, K, interp, iw)
+    assert relerr(tgi1, ti) <= tol_b and relerr(tgw1, tw) <= tol_b and relerr(tgb1, tb) <= tol_b
 
 
 def test_cache_misses_after_an_in_place_change_of_the_map(ops, oracle):
@@ -160,6 +167,88 @@ def test_plan_buffer_of_the_wrong_size_is_refused(ops):
     rc = lib.sdk_mapped_conv_plan_build(one, None, one, n - 1, 40, 64, 40, 64, 9, 0, 1,
                                         _capi.SDK_F32, None)
     assert rc != 0 and b"needs" in lib.sdk_last_error()
+
+
+def test_every_planned_entry_point_refuses_a_plan_that_is_too_small(ops):
+    """All eight *_planned entry points check plan_bytes against the geometry's plan before
+    they launch anything (the combined backward calls before their bias gradient too)."""
+    from _spherical_distortion_ext import _capi
+    lib = _capi.load()
+    B, Cin, Cout, H, W, K = 1, 72, 80, 40, 64, 9
+    n = lib.sdk_mapped_conv_plan_bytes(H, W, H, W, K, 0, 1, _capi.SDK_F32)
+    nws = lib.sdk_mapped_conv_workspace_bytes(B, Cin, Cout, H, W, H, W, K, 0, 1, _capi.SDK_F32, 0)
+    buf = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=DEV)
+    m, x, y = buf(H, W, K, 2), buf(B, Cin, H, W), buf(B, Cout, H, W)
+    w, wt, b = buf(Cout, Cin, K), buf(Cin, Cout, K), buf(Cout)
+    gw, gb = buf(Cout, Cin, K), buf(Cout)
+    ws = torch.empty(nws, dtype=torch.uint8, device=DEV)
+    plan = torch.empty(n, dtype=torch.uint8, device=DEV)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    dims = (B, Cin, H, W, Cout, H, W, K, 0, 1, _capi.SDK_F32, 0, None)
+    tail = (P(ws), nws, P(plan), n - 256)
+    calls = {
+        "sdk_mapped_conv_forward_planned": (P(x), P(m), None, P(w), P(b), P(y)),
+        "sdk_mapped_conv_backward_input_planned": (P(y), P(m), None, P(w), P(x)),
+        "sdk_mapped_conv_backward_weight_planned": (P(y), P(m), None, P(x), P(gw)),
+        "sdk_mapped_conv_backward_planned": (P(y), P(m), None, P(x), P(w), P(x), P(gw), P(gb)),
+        # transposed layer Cin -> Cout over the same map: input on the grid, output H x W
+        "sdk_mapped_transposed_conv_forward_planned": (P(x), P(m), None, P(wt), P(b), P(y)),
+        "sdk_mapped_transposed_conv_backward_input_planned": (P(y), P(m), None, P(wt), P(x)),
+        "sdk_mapped_transposed_conv_backward_weight_planned": (P(y), P(m), None, P(x), P(gw)),
+        "sdk_mapped_transposed_conv_backward_planned": (P(y), P(m), None, P(x), P(wt), P(x), P(gw),
+                                                        P(gb)),
+    }
+    for name, args in calls.items():
+        rc = getattr(lib, name)(*args, *tail, *dims)
+        assert rc == -3, (name, rc, lib.sdk_last_error())
+        assert b"plan buffer" in lib.sdk_last_error(), name
+    torch.cuda.synchronize()
+    assert float(gb.abs().max()) == 0.0       # no bias gradient was launched by a refused call
+
+
+def test_maps_made_under_inference_mode_go_past_the_cache(ops, oracle):
+    """A tensor created under torch.inference_mode() has no version counter; the cached
+    operators take the uncached entry points for it instead of failing."""
+    Cin, Cout, H, W, OH, OW, K, P, interp, kind = CASES[0]
+    m, iw, x, w, b, g, _ = _case(11, *CASES[0])
+    before = len(ops._PLAN_CACHE)
+    with torch.inference_mode():
+        tm = _t(m)
+        assert tm.is_inference()
+        y = ops.mapped_conv_forward(_t(x), tm, None, _t(w), _t(b), K, interp).cpu().numpy()
+        pooled, idx = ops.mapped_max_pool(_t(x), tm, None, K, interp)
+        back = ops.mapped_max_unpool(pooled, idx, tm, None, H, W, K, interp).cpu().numpy()
+        up = ops.resample_to_map(_t(x), _t(m[:, :, 0]), None, H, W, interp).cpu().numpy()
+    assert len(ops._PLAN_CACHE) == before
+    assert relerr(y, oracle.mapped_conv_forward(x, m, w, b, K, interp, None)) <= 1e-5
+    pv, pi = oracle.mapped_max_pool(x, m, K, interp)
+    assert np.array_equal(idx.cpu().numpy(), pi)
+    assert relerr(back, oracle.mapped_max_unpool(pv, pi, m, H, W, K, interp)) <= 1e-4
+    assert relerr(up, oracle.resample_to_map(x, m[:, :, 0], H, W, interp)) <= 1e-4
+
+
+def test_a_plan_is_not_built_under_graph_capture(ops):
+    """A key that misses while the stream is being captured takes the uncached entry points:
+    nothing is inserted into the cache, and the replayed graph gives the eager result."""
+    Cin, Cout, H, W, OH, OW, K, P, interp, kind = CASES[0]
+    m, iw, x, w, b, g, _ = _case(13, *CASES[0])
+    tx, tw, tb = _t(x), _t(w), _t(b)
+    tm = _t(m)
+    eager = ops.mapped_conv_forward(tx, _t(m), None, tw, tb, K, interp)   # another map tensor
+    before = len(ops._PLAN_CACHE)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        out = torch.empty_like(eager)
+        with torch.cuda.graph(graph, stream=side):
+            out.copy_(ops.mapped_conv_forward(tx, tm, None, tw, tb, K, interp))
+    assert len(ops._PLAN_CACHE) == before
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
 
 
 def test_backward_runs_in_the_arithmetic_of_its_forward(ops, oracle):

@@ -94,7 +94,9 @@ def test_resample_to_map_crowded_targets_and_no_workspace(ops, oracle, interp, w
     ones = oracle.resample_to_map(np.ones((1, 1, MH, MW), dt), m, H, W, interp, iw)[0, 0]
     gotn, wsum = ops.resample_to_map_normalized(_t(y), _t(m), _t(iw), H, W, interp, 1e-12)
     assert relerr(_n(wsum), ones) <= 1e-4
-    assert relerr(_n(gotn), want / (ones + dt(1e-12))) <= 1e-3
+    # weights are non-negative, so numerator and weight sum each carry n * eps relative to
+    # the weight sum and the quotient n * eps * max|y|: the scatter tolerance holds for it
+    assert relerr(_n(gotn), want / (ones + dt(1e-12))) <= 1e-4
     assert relerr(_n(ops.resample_to_map(_t(y), _t(m), _t(iw), H, W, interp)), want) <= 1e-4
     # the same call through the C ABI without workspace
     ty, tm, tw = _t(y), _t(m), _t(iw)
@@ -108,7 +110,7 @@ def test_resample_to_map_crowded_targets_and_no_workspace(ops, oracle, interp, w
                ops._ptr(out), ops._ptr(wsum2), None, 0, 1e-12, B, C, MH, MW, H, W,
                P if weighted else 0, interp, 0, ops._stream(ty))
     assert relerr(_n(wsum2), ones) <= 1e-4
-    assert relerr(_n(out), want / (ones + dt(1e-12))) <= 1e-3
+    assert relerr(_n(out), want / (ones + dt(1e-12))) <= 1e-4
 
 
 @pytest.mark.parametrize("case", CASES, ids=_ids)

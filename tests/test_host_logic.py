@@ -233,3 +233,85 @@ def test_compute_mode_override_is_scoped_and_per_thread():
     with pytest.raises(ValueError):
         with _ops.conv_compute("fp8"):
             pass
+
+
+def test_native_override_under_a_non_native_default():
+    """"native" is the C ABI's value 0: an override to it must still count as an override,
+    and a mode recorded by a forward ("native") must be what conv_compute() restores for its
+    backward after the process default has changed."""
+    from _spherical_distortion_ext import _ops
+    _ops.set_conv_compute("bf16")
+    try:
+        assert _ops.get_conv_compute() == "bf16"
+        with _ops.conv_compute("native"):
+            assert _ops.get_conv_compute() == "native"
+            with _ops.conv_compute("split"):
+                assert _ops.get_conv_compute() == "split"
+            assert _ops.get_conv_compute() == "native"
+        assert _ops.get_conv_compute() == "bf16"
+    finally:
+        _ops.set_conv_compute("native")
+    # a forward that ran in native mode, its backward after the default moved to bf16
+    recorded = _ops.get_conv_compute()
+    assert recorded == "native"
+    _ops.set_conv_compute("bf16")
+    try:
+        with _ops.conv_compute(recorded):
+            assert _ops.get_conv_compute() == "native"
+            assert _ops._current_mode() == 0
+    finally:
+        _ops.set_conv_compute("native")
+
+
+def test_tensor_key_of_tensors_without_a_version_counter():
+    """A tensor made under torch.inference_mode() has no version counter: the plan cache
+    cannot see its in-place changes, so it gets the no-key marker and the operators go
+    past the cache for it."""
+    from _spherical_distortion_ext import _ops
+    plain = torch.zeros(4, 5, 3, 2)
+    key = _ops._tensor_key(plain)
+    assert key == (plain.untyped_storage().data_ptr(), 0, plain._version, (4, 5, 3, 2))
+    plain.add_(1)
+    assert _ops._tensor_key(plain) != key           # an in-place change misses
+    assert _ops._tensor_key(None) is None
+    with torch.inference_mode():
+        inf = torch.zeros(4, 5, 3, 2)
+    assert inf.is_inference()
+    assert _ops._tensor_key(inf) is _ops._NO_KEY
+    assert _ops._uncacheable(key, _ops._NO_KEY) and not _ops._uncacheable(key, None)
+
+
+def test_plan_cache_evicts_the_least_recently_used_entry():
+    from _spherical_distortion_ext import _ops
+
+    class Stream:          # stands in for a torch stream: identity and wait_stream only
+        def __init__(self):
+            self.waited = []
+
+        def wait_stream(self, other):
+            self.waited.append(other)
+
+    s0, s1 = Stream(), Stream()
+    saved, saved_max = dict(_ops._PLAN_CACHE), _ops._PLAN_CACHE_MAX
+    _ops._PLAN_CACHE.clear()
+    try:
+        _ops.set_conv_plan_cache(True, max_entries=3)
+        for k in "abc":
+            _ops._cache_insert(k, _ops._PlanEntry(k.upper(), 1, None, s0))
+        assert _ops._cache_lookup("a", s0).plan == "A" and s0.waited == []
+        _ops._cache_insert("d", _ops._PlanEntry("D", 1, None, s0))     # evicts b, not a
+        assert list(_ops._PLAN_CACHE) == ["c", "a", "d"]
+        assert _ops._cache_lookup("b", s0) is None
+        # a user on another stream is ordered behind the last user, which it then becomes
+        ent = _ops._cache_lookup("c", s1)
+        assert s1.waited == [s0] and ent.stream is s1
+        assert _ops._cache_lookup("c", s1) is ent and s1.waited == [s0]
+        assert _ops._cache_lookup("c", s0) is ent and s0.waited == [s1]
+        _ops.set_conv_plan_cache(True, max_entries=1)
+        assert list(_ops._PLAN_CACHE) == ["c"]
+        with pytest.raises(ValueError):
+            _ops.set_conv_plan_cache(True, max_entries=0)
+    finally:
+        _ops._PLAN_CACHE.clear()
+        _ops._PLAN_CACHE.update(saved)
+        _ops._PLAN_CACHE_MAX = saved_max
