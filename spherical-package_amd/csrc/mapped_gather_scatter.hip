@@ -15,6 +15,7 @@
 #include <cfloat>
 #include <climits>
 
+#include "pool_band.hpp"
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
 
@@ -1826,6 +1827,13 @@ int sdk_mapped_max_pool(const void* input, const void* sample_map, const void* i
   if (rc) return rc;
   const int64_t planes = batch * channels;
   if (planes == 0) return SDK_OK;
+  if (dtype == SDK_F32 && num_interp_pts == 0 && interp != 1 && interp != 2 &&
+      pool_band_launch(false, (const float*)input, (const float*)sample_map, (float*)out, indices,
+                       planes, (int)height, (int)width, (int)out_height, (int)out_width,
+                       (int)kernel_size, (hipStream_t)stream)) {
+    SDK_LAUNCH_CHECK("mapped_max_pool");
+    return SDK_OK;
+  }
   const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_DTYPE(
       dtype,
@@ -1852,6 +1860,13 @@ int sdk_mapped_avg_pool(const void* input, const void* sample_map, const void* i
   if (rc) return rc;
   const int64_t planes = batch * channels;
   if (planes == 0) return SDK_OK;
+  if (dtype == SDK_F32 && num_interp_pts == 0 && interp != 1 && interp != 2 &&
+      pool_band_launch(true, (const float*)input, (const float*)sample_map, (float*)out, nullptr,
+                       planes, (int)height, (int)width, (int)out_height, (int)out_width,
+                       (int)kernel_size, (hipStream_t)stream)) {
+    SDK_LAUNCH_CHECK("mapped_avg_pool");
+    return SDK_OK;
+  }
   const dim3 grid(banded_grid_x(M), (unsigned)ceil_div(planes, kPC));
   SDK_DISPATCH_DTYPE(
       dtype,
