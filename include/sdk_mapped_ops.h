@@ -320,14 +320,16 @@ int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
  *
  * `workspace` is optional device scratch of sdk_mapped_max_unpool_workspace_bytes()
  * bytes (it depends on the input plane and the element size only).  With it the
- * call inverts the sample map once and runs as a gather: every input pixel sums
- * the pooled pixels whose index names a sample that reaches it, and is written
- * once with a plain store.  Without it (NULL, or too small), or when the map or
- * the indices do not fit that scheme (more than 32 taps reach one input pixel,
- * the pooled pixels that can reach one tile of the input are spread too far
- * apart, or an index names a sample of another pooled pixel than its own), the
- * call zero-fills grad_input and scatters with atomic adds, as the reference
- * does; the choice is made on the device, the result is the same.
+ * call works by pieces of the input plane, whole rows (float32, single nearest
+ * taps, kernel_size 4 or 9, width a multiple of 4) or tiles: the pooled pixels
+ * that can reach a piece are found from the map, their contributions are summed
+ * in on-chip memory and every input pixel is written once with a plain store.
+ * Without it (NULL, or too small), or when the map or the indices do not fit
+ * that scheme (the pooled pixels that can reach one piece of the input are too
+ * many or spread too far apart, or an index names a sample of another pooled
+ * pixel than its own), the call zero-fills grad_input and scatters with atomic
+ * adds, as the reference does; the choice is made on the device, the result is
+ * the same.
  * Replaces `_mapped_max_pooling.mapped_max_unpool` /
  * `_weighted_mapped_max_pooling.weighted_mapped_max_unpool`
  * (ext_modules/include/layers/mapped_max_pooling_layer.h:64-88,
@@ -343,8 +345,9 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
 /* sdk_mapped_max_unpool for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same arguments and results as sdk_mapped_max_unpool without the workspace pair:
- * the tile-window scratch (256 + 32 bytes per 2048-pixel tile of the input plane) is a
- * 262 400-byte array inside the library, one copy per GPU, held until the process ends.  The
+ * the scratch (256 + 32 bytes per 2048-pixel tile of the input plane for the tile windows,
+ * 32 KB for the row-band table behind them) is a 295 168-byte array inside the library, one
+ * copy per GPU, held until the process ends.  The
  * call allocates and frees nothing.  Limit: the input plane may have at most
  * SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES tiles, ceil(width / TW) * ceil(height / (2048 / TW))
  * with TW = 128 (wider for planes lower than 16 rows, narrower for planes under 65 columns),

@@ -774,7 +774,8 @@ __device__ __forceinline__ void grow_window(int* w, int up, int down, int left, 
 template <typename T, int INTERP, bool WEIGHTED, bool GROW>
 __global__ __launch_bounds__(kBlock) void unpool_window_kernel(
     const T* __restrict__ map, int64_t samples, int P, int K, int OW, UnpoolTiling ut,
-    int* __restrict__ win) {
+    int* __restrict__ win, const int* __restrict__ skip) {
+  if (skip != nullptr && skip[0] != 0) return;   // the row-band kernels do this call
   __shared__ int s_tile[kWinSlots];
   __shared__ int s_ext[kWinSlots][4];
   if (GROW) {
@@ -836,8 +837,8 @@ __global__ __launch_bounds__(kBlock) void unpool_tiles_kernel(
     const T* __restrict__ gout, const int64_t* __restrict__ idx, const T* __restrict__ map,
     const T* __restrict__ wts, const int* __restrict__ win, T* __restrict__ gin,
     int* __restrict__ gate, UnpoolTiling ut, int planes, int planes_per_group, int M, int OW,
-    int K, int P, int64_t map_elems) {
-  if (*gate != 0) return;
+    int K, int P, int64_t map_elems, const int* __restrict__ skip) {
+  if (*gate != 0 || (skip != nullptr && skip[0] != 0)) return;
   constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));   // planes per pass
   __shared__ T acc[PLMAX * kUpTile];
   const int tid = threadIdx.x, tile = blockIdx.x;
@@ -974,8 +975,9 @@ template <typename T, int INTERP, bool WEIGHTED>
 __global__ __launch_bounds__(kBlock) void avg_unpool_tiles_kernel(
     const T* __restrict__ gout, const T* __restrict__ map, const T* __restrict__ wts,
     const int* __restrict__ win, const int* __restrict__ flags, T* __restrict__ gin,
-    UnpoolTiling ut, int planes, int planes_per_group, int M, int OW, int K, int P) {
-  if (flags[0] == 0) return;
+    UnpoolTiling ut, int planes, int planes_per_group, int M, int OW, int K, int P,
+    const int* __restrict__ skip) {
+  if (flags[0] == 0 || (skip != nullptr && skip[0] != 0)) return;
   constexpr int PLMAX = kUpBytes / (kUpTile * (int)sizeof(T));   // planes per pass
   __shared__ T acc[PLMAX * kUpTile];
   const int tid = threadIdx.x, tile = blockIdx.x;
@@ -1093,9 +1095,11 @@ __global__ __launch_bounds__(kBlock) void avg_unpool_tiles_kernel(
 // fallback.  Stage 0 (after the windows): [0] and [1].  Stage 1 (after the lists, whose own
 // gate counts the sources that found a list full): [2] = that gate where the lists are used;
 // the word after the lists' gate receives a copy of [0].
+// bands: the row-band table of these windows, or nullptr; where its verdict word says that the
+// band kernels do the call, the windows (which may not have been built then) are not looked at.
 __global__ __launch_bounds__(kBlock) void avg_unpool_verdict_kernel(
     const int* __restrict__ win, int tiles, int OW, int* __restrict__ flags,
-    int* __restrict__ lists_gate, int stage) {
+    int* __restrict__ lists_gate, int stage, const int* __restrict__ bands) {
   if (stage == 1) {
     if (threadIdx.x == 0) {
       flags[2] = flags[0] != 0 ? 0 : lists_gate[0];
@@ -1106,6 +1110,7 @@ __global__ __launch_bounds__(kBlock) void avg_unpool_verdict_kernel(
   __shared__ int too_big;
   if (threadIdx.x == 0) too_big = 0;
   __syncthreads();
+  if (bands != nullptr && bands[0] != 0) tiles = 0;
   for (int t = threadIdx.x; t < tiles; t += kBlock) {
     const int* w = win + (size_t)t * 8;
     if (w[0] > 0) {
@@ -1166,9 +1171,12 @@ static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
 
 static UnpoolTiling unpool_tiling(int H, int W);
 static size_t unpool_layout(const UnpoolTiling& ut);
+static size_t unpool_layout_with_bands(const UnpoolTiling& ut);
 template <typename T>
-static int build_unpool_windows(const T* map, void* workspace, int H, int W, int OH, int OW, int K,
-                                int P, int interp, hipStream_t stream);
+static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, int interp);
+template <typename T>
+static int build_unpool_windows(const T* map, void* workspace, size_t workspace_bytes, int H, int W,
+                                int OH, int OW, int K, int P, int interp, hipStream_t stream);
 
 // Average unpooling (group = K > 1 samples per pooled pixel, pooled rows of OW pixels) can run
 // tiled over the image when the workspace has room for the tile windows behind the lists.
@@ -1200,11 +1208,16 @@ static int build_inverse_lists(const T* map, const T* wts, void* workspace, size
   if (avg_unpool_tiled(H, W, MP, group, OW, P, sizeof(T), 0, lists_bytes, workspace_bytes)) {
     flags = reinterpret_cast<int*>(ws + lists_bytes);
     const UnpoolTiling ut = unpool_tiling(H, W);
-    const int rc = build_unpool_windows<T>(map, ws + lists_bytes, H, W, MP / group / OW, OW, group,
-                                           P, interp, stream);
+    const size_t region = workspace_bytes - lists_bytes;
+    const int rc = build_unpool_windows<T>(map, ws + lists_bytes, region, H, W, MP / group / OW,
+                                           OW, group, P, interp, stream);
     if (rc != SDK_OK) return rc;
+    const int* bands = nullptr;
+    if (region >= unpool_layout_with_bands(ut) &&
+        unpool_bands_possible<T>(H, W, MP / group / OW, OW, group, P, interp))
+      bands = reinterpret_cast<const int*>(ws + lists_bytes + unpool_layout(ut));
     launch(avg_unpool_verdict_kernel, dim3(1), dim3(kBlock), stream, (const int*)(flags + 64),
-           ut.tiles_x * ut.tiles_y, OW, flags, g, 0);
+           ut.tiles_x * ut.tiles_y, OW, flags, g, 0, bands);
     SDK_LAUNCH_CHECK("mapped_avg_unpool(windows)");
   }
   int rc;
@@ -1223,7 +1236,7 @@ static int build_inverse_lists(const T* map, const T* wts, void* workspace, size
   SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
   if (flags) {
     launch(avg_unpool_verdict_kernel, dim3(1), dim3(kBlock), stream, (const int*)(flags + 64), 0,
-           OW, flags, g, 1);
+           OW, flags, g, 1, (const int*)nullptr);
     SDK_LAUNCH_CHECK("mapped_avg_unpool(gate)");
   }
   return SDK_OK;
@@ -1253,10 +1266,25 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
     const bool tiled = !normalize && wsum == nullptr &&
                        avg_unpool_tiled(H, W, MP, group, OW, P, sizeof(T), planes, lists_bytes, workspace_bytes);
     const int* flags = tiled ? reinterpret_cast<const int*>(ws + lists_bytes) : nullptr;
+    // the row-band form of the tiled average unpooling: the table behind the tile windows
+    const int* bands = nullptr;
+    if (tiled) {
+      const UnpoolTiling ut = unpool_tiling(H, W);
+      if (workspace_bytes - lists_bytes >= unpool_layout_with_bands(ut) &&
+          unpool_bands_possible<T>(H, W, MP / group / OW, OW, group, P, interp))
+        bands = reinterpret_cast<const int*>(ws + lists_bytes + unpool_layout(ut));
+    }
     if (!prebuilt) {
       const int rc = build_inverse_lists<T>(map, wts, workspace, tiled ? workspace_bytes : lists_bytes,
                                             H, W, MP, P, interp, group, OW, stream);
       if (rc != SDK_OK) return rc;
+    }
+    if (bands != nullptr && planes > 0) {
+      if constexpr (sizeof(T) == 4) {
+        unpool_band_launch(true, (const float*)in, nullptr, (const float*)map, (float*)out, bands,
+                           nullptr, planes, H, W, MP / group / OW, OW, group, stream);
+        SDK_LAUNCH_CHECK("mapped_avg_unpool(bands)");
+      }
     }
     if (tiled && planes > 0) {
       const UnpoolTiling ut = unpool_tiling(H, W);
@@ -1269,7 +1297,7 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
       SDK_DISPATCH_INTERP(interp, P,
                           (launch((avg_unpool_tiles_kernel<T, INTERP, WEIGHTED>), grid_t,
                                   dim3(kBlock), stream, in, map, wts, flags + 64, flags, out, ut,
-                                  (int)planes, (int)per_group, MP / group, OW, group, P)));
+                                  (int)planes, (int)per_group, MP / group, OW, group, P, bands)));
       SDK_LAUNCH_CHECK("mapped_avg_unpool(tiles)");
     }
     if ((planes > 0 || wsum) && !(tiled && prebuilt && (complete & 2))) {
@@ -1447,25 +1475,48 @@ static size_t unpool_layout(const UnpoolTiling& ut) {
   return 256 + (size_t)ut.tiles_x * ut.tiles_y * 8 * sizeof(int);
 }
 
-// The tile windows of the tiled unpool (a function of the map alone) into `workspace`
-// (unpool_layout bytes), gate word cleared.
+// ... followed, when the workspace has room for it, by the table of the row-band kernels
+// (pool_band.hpp), whose first word is the device-side verdict "the band kernels do this map".
+static size_t unpool_layout_with_bands(const UnpoolTiling& ut) {
+  return unpool_layout(ut) + unpool_band_table_bytes(ut.H, ut.W);
+}
+
+// Whether the row-band kernels take this element type, interpolation and shape at all.
 template <typename T>
-static int build_unpool_windows(const T* map, void* workspace, int H, int W, int OH, int OW, int K,
-                                int P, int interp, hipStream_t stream) {
+static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, int interp) {
+  return sizeof(T) == 4 && P == 0 && interp != 1 && interp != 2 &&
+         unpool_band_shape(H, W, OH, OW, K);
+}
+
+// The tile windows of the tiled unpool (a function of the map alone) into `workspace`
+// (unpool_layout bytes), gate word cleared; with workspace_bytes >= unpool_layout_with_bands
+// the band table as well; where its verdict is 1 every call on this map runs the band kernels
+// and the window kernels return at once.
+template <typename T>
+static int build_unpool_windows(const T* map, void* workspace, size_t workspace_bytes, int H, int W,
+                                int OH, int OW, int K, int P, int interp, hipStream_t stream) {
   const UnpoolTiling ut = unpool_tiling(H, W);
   char* ws = static_cast<char*>(workspace);
   int* win = reinterpret_cast<int*>(ws + 256);
-  int rc = zero_fill(ws, unpool_layout(ut), stream);
+  const bool with_table = workspace_bytes >= unpool_layout_with_bands(ut);
+  int rc = zero_fill(ws, with_table ? unpool_layout_with_bands(ut) : unpool_layout(ut), stream);
   if (rc != SDK_OK) return rc;
+  const int* skip = nullptr;
+  if (with_table && unpool_bands_possible<T>(H, W, OH, OW, K, P, interp)) {
+    int* table = reinterpret_cast<int*>(ws + unpool_layout(ut));
+    unpool_band_build((const float*)map, table, H, W, OH, OW, K, stream);
+    SDK_LAUNCH_CHECK("mapped_max_unpool(band table)");
+    skip = table;
+  }
   const int64_t samples = (int64_t)OH * OW * K;
   const dim3 grid_s((unsigned)ceil_div(samples, kBlock));
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((unpool_window_kernel<T, INTERP, WEIGHTED, false>), grid_s,
-                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win, skip)));
   SDK_LAUNCH_CHECK("mapped_max_unpool(anchors)");
   SDK_DISPATCH_INTERP(interp, P,
                       (launch((unpool_window_kernel<T, INTERP, WEIGHTED, true>), grid_s,
-                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win)));
+                              dim3(kBlock), stream, map, samples, P, K, OW, ut, win, skip)));
   SDK_LAUNCH_CHECK("mapped_max_unpool(windows)");
   return SDK_OK;
 }
@@ -1495,19 +1546,33 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
     char* ws = static_cast<char*>(workspace);
     int* g = reinterpret_cast<int*>(ws);
     int* win = reinterpret_cast<int*>(ws + 256);
+    // the row-band kernels, where the workspace holds their table and they take the call
+    const int* bands = nullptr;
+    if (workspace_bytes >= unpool_layout_with_bands(ut) &&
+        unpool_bands_possible<T>(H, W, OH, OW, K, P, interp))
+      bands = reinterpret_cast<const int*>(ws + unpool_layout(ut));
     int rc;
     if (prebuilt) {
-      // the windows are there; the gate word is this call's own (the tile kernel raises it)
+      // the windows are there; the gate word is this call's own (the kernels raise it)
       rc = zero_fill(ws, 256, stream);
     } else {
-      rc = build_unpool_windows<T>(map, workspace, H, W, OH, OW, K, P, interp, stream);
+      rc = build_unpool_windows<T>(map, workspace, workspace_bytes, H, W, OH, OW, K, P, interp,
+                                   stream);
     }
     if (rc != SDK_OK) return rc;
+    if (bands != nullptr) {
+      if constexpr (sizeof(T) == 4) {
+        unpool_band_launch(false, (const float*)gout, indices, (const float*)map, (float*)gin,
+                           bands, g, planes, H, W, OH, OW, K, stream);
+        SDK_LAUNCH_CHECK("mapped_max_unpool(bands)");
+      }
+    }
     const dim3 grid_t((unsigned)tiles, (unsigned)groups);
     SDK_DISPATCH_INTERP(interp, P,
                         (launch((unpool_tiles_kernel<T, INTERP, WEIGHTED>), grid_t, dim3(kBlock),
                                 stream, gout, indices, map, wts, (const int*)win, gin, g, ut,
-                                (int)planes, (int)per_group, (int)M, OW, K, P, map_elems)));
+                                (int)planes, (int)per_group, (int)M, OW, K, P, map_elems,
+                                bands)));
     SDK_LAUNCH_CHECK("mapped_max_unpool(tiles)");
     gate = g;
   }
@@ -1570,7 +1635,9 @@ using namespace sdk;
 // that pointer is what the fill kernel and the unpool kernels receive.
 // ---------------------------------------------------------------------------
 static constexpr int kStaticUnpoolTiles = SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES;   // of 2048 pixels
-static constexpr size_t kStaticUnpoolBytes = 256 + (size_t)kStaticUnpoolTiles * 8 * sizeof(int);
+// tile windows, then 32 KB for the row-band table (planes of up to 4000 rows of bands)
+static constexpr size_t kStaticUnpoolBytes = 256 + (size_t)kStaticUnpoolTiles * 8 * sizeof(int) +
+                                             32768;
 static __device__ __align__(256) unsigned char scratch[kStaticUnpoolBytes];
 
 static constexpr int kMaxDevices = 64;
@@ -1635,7 +1702,7 @@ size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_
   size_t off[4];
   // the inverse lists, then the tile windows of the tiled average unpooling
   return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off) +
-         unpool_layout(unpool_tiling((int)height, (int)width));
+         unpool_layout_with_bands(unpool_tiling((int)height, (int)width));
 }
 
 static int resample_to_map_entry(const void* input, const void* sample_map,
@@ -1907,7 +1974,7 @@ int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
 size_t sdk_mapped_max_unpool_workspace_bytes(int64_t height, int64_t width, int32_t dtype) {
   if (height < 1 || width < 1 || height * width >= ((int64_t)1 << 31)) return 0;
   (void)dtype;
-  return unpool_layout(unpool_tiling((int)height, (int)width));
+  return unpool_layout_with_bands(unpool_tiling((int)height, (int)width));
 }
 
 int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,
@@ -1943,7 +2010,7 @@ int sdk_mapped_max_unpool_static(const void* grad_output, const int64_t* indices
   SDK_REQUIRE(height >= 1 && width >= 1 && height * width < ((int64_t)1 << 31),
               "mapped_max_unpool_static: bad plane size");
   const size_t need = unpool_layout(unpool_tiling((int)height, (int)width));
-  if (need > kStaticUnpoolBytes)
+  if (need > 256 + (size_t)kStaticUnpoolTiles * 8 * sizeof(int))
     return fail(SDK_ERR_WORKSPACE,
                 "mapped_max_unpool_static: a %lld x %lld plane needs %zu bytes of tile windows, "
                 "the built-in scratch holds %zu (%d tiles of %d pixels); use sdk_mapped_max_unpool "
@@ -2113,7 +2180,7 @@ int sdk_mapped_max_unpool_plan_build(const void* sample_map, void* plan, size_t 
     return fail(SDK_ERR_WORKSPACE, "mapped_max_unpool_plan_build: plan of %zu bytes, need %zu",
                 plan_bytes, need);
   SDK_DISPATCH_DTYPE(dtype, return build_unpool_windows<T>(
-                                (const T*)sample_map, plan, (int)height, (int)width,
+                                (const T*)sample_map, plan, plan_bytes, (int)height, (int)width,
                                 (int)out_height, (int)out_width, (int)kernel_size, num_interp_pts,
                                 interp, (hipStream_t)stream));
   return SDK_OK;

@@ -264,6 +264,250 @@ bool dispatch_ipt(int ipt, const float* in, const float* map, float* out, int64_
   return false;
 }
 
+
+// ---------------------------------------------------------------------------
+// Unpooling by image row bands (max: common/mapped_max_pool.h:60-78, :136-171; average:
+// common/mapped_avg_pool.h:42-68, :107-140).  A workgroup owns RB whole image rows and a
+// range of planes, sums what reaches those rows in LDS and stores every element once, 16 bytes
+// at a time: no zero fill, no atomics in memory.  What can reach a band is fixed by the map:
+// a table (built once per map by unpool_band_rows_kernel, kept in the caller's workspace or
+// plan) holds per band the range of pooled rows with a tap in it.  A thread owns up to kUbIpt
+// pooled pixels of that range; the positions of their K taps inside the band are worked out
+// once, packed two to a register, and serve every plane, so per plane a pooled pixel costs
+// one index read, one gradient read, a select by the winning sample and one LDS add.
+//
+// table: [0] 1 when every band's range fits (kUbIpt * 256 pooled pixels), else 0 (the caller
+// then takes its other route); [8 + 2b] last pooled row of band b + 1 (0: nothing reaches
+// it); [9 + 2b] kUbBig - first pooled row.  Both grow by atomicMax from a zero fill.
+// ---------------------------------------------------------------------------
+constexpr int kUbIpt = 8;
+constexpr int kUbLdsBytes = 32 * 1024;
+constexpr int kUbLdsFloats = kUbLdsBytes / 4;
+constexpr int kUbBig = 1 << 30;
+constexpr unsigned kUbNone = 0xFFFFu;
+
+__global__ __launch_bounds__(kBandBlock) void unpool_band_rows_kernel(
+    const float* __restrict__ map, int M, int OW, int K, int H, int W, int RB,
+    int* __restrict__ table) {
+  const int pix = blockIdx.x * kBandBlock + threadIdx.x;
+  if (pix >= M) return;
+  const int r = pix / OW;
+  const float2* coords = reinterpret_cast<const float2*>(map) + (size_t)pix * K;
+  int bmin = INT_MAX, bmax = -1;
+  for (int k = 0; k < K; ++k) {
+    const float2 c = coords[k];
+    PointTaps<float, 0> tp;
+    tp.set(c.x, c.y, H, W);
+    if (tp.off[0] >= 0) {
+      bmin = min(bmin, tp.ty[0] / RB);
+      bmax = max(bmax, tp.ty[0] / RB);
+    }
+  }
+  // every band between the first and the last one touched (a superset does no harm: a pooled
+  // pixel of the range without a tap in the band adds nothing)
+  for (int b = bmin; b <= bmax; ++b) {
+    int* e = table + 8 + 2 * b;
+    if (e[0] < r + 1) atomicMax(&e[0], r + 1);
+    if (e[1] < kUbBig - r) atomicMax(&e[1], kUbBig - r);
+  }
+}
+
+__global__ __launch_bounds__(kBandBlock) void unpool_band_verdict_kernel(int* __restrict__ table,
+                                                                        int nbands, int OW) {
+  __shared__ int bad;
+  if (threadIdx.x == 0) bad = 0;
+  __syncthreads();
+  for (int b = threadIdx.x; b < nbands; b += kBandBlock) {
+    const int hi1 = table[8 + 2 * b];
+    if (hi1 > 0) {
+      const int lo = kUbBig - table[9 + 2 * b];
+      if ((int64_t)(hi1 - lo) * OW > (int64_t)kUbIpt * kBandBlock) bad = 1;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) table[0] = bad ? 0 : 1;
+}
+
+// One 64-bit compare-and-swap loop that adds (a, b) to an aligned pair of floats in LDS.
+__device__ __forceinline__ void lds_add_f32x2(float2* addr, float a, float b) {
+  unsigned long long* ip = reinterpret_cast<unsigned long long*>(addr);
+  unsigned long long old = __hip_atomic_load(ip, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  while (true) {
+    const unsigned long long assumed = old;
+    old = atomicCAS(ip, assumed, add_pair(assumed, a, b));
+    if (old == assumed) break;
+  }
+}
+
+// Piece v (four floats) of a band row run, past the caches; one 16-byte store where the
+// tensor is 16-byte aligned (aligned: the same for every thread of the launch).
+__device__ __forceinline__ void store_piece(float* dst, int v, vec4 val, int aligned) {
+  if (aligned) {
+    __builtin_nontemporal_store(val, reinterpret_cast<vec4*>(dst) + v);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) __builtin_nontemporal_store(val[e], dst + 4 * v + e);
+  }
+}
+
+// Tap k of a pooled pixel from its packed taps, by a chain of selects.  Each word passes
+// through an empty asm first: seen as plain array elements, the compiler turns the chain into
+// one load at a computed address and the whole array moves from registers to private memory.
+template <int K>
+__device__ __forceinline__ unsigned packed_tap(const unsigned (&offp)[(K + 1) / 2], int k) {
+  unsigned w = offp[0];
+  asm volatile("" : "+v"(w));
+#pragma unroll
+  for (int h = 1; h < (K + 1) / 2; ++h) {
+    unsigned x = offp[h];
+    asm volatile("" : "+v"(x));
+    w = (k >> 1) == h ? x : w;
+  }
+  return (k & 1) ? (w >> 16) : (w & 0xFFFFu);
+}
+
+// gate: raised (and the caller's atomic route then redoes the call) when an index names a
+// sample of another pooled pixel than its own, which mapped_max_pool never writes but the
+// scatter accepts: such a sample may reach a band whose range does not hold the pixel.
+//
+// Two planes per pass.  The LDS adds are compare-and-swap loops (the native float add to LDS
+// runs at a fraction of their rate on this GPU: 788 against 198 us for the average unpooling
+// of an 8 x 64 x 128 x 256 gradient), one after the other (issued as a batch, with the taps
+// outside the band masked or sent to a spare word, they were slower).  Max unpooling keeps the two planes apart (their
+// winners differ); average unpooling interleaves them, (plane 0, plane 1) per band element,
+// and adds both with one 64-bit swap per tap.
+template <bool AVG, int K>
+__global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
+    const float* __restrict__ gout, const int64_t* __restrict__ idx, const float* __restrict__ map,
+    float* __restrict__ gin, const int* __restrict__ table, int* __restrict__ gate, int planes,
+    int H, int W, int OW, int M, int RB, int nbands, int chunks, int map_elems, int aligned) {
+  if (table[0] == 0) return;
+  constexpr int PG = 2;
+  __shared__ __attribute__((aligned(16))) float acc[kUbLdsFloats];
+  constexpr int KH = (K + 1) / 2;
+  const int t = threadIdx.x;
+  const int xcd = blockIdx.x & 7, within = blockIdx.x >> 3;
+  const int band = within % nbands;
+  const int chunk = (within / nbands) * 8 + xcd;
+  if (chunk >= chunks) return;
+  const int p_begin = (int)((int64_t)chunk * planes / chunks);
+  const int p_end = (int)((int64_t)(chunk + 1) * planes / chunks);
+  const size_t HW = (size_t)H * W;
+  const int y0 = band * RB;
+  const int band_rows = min(RB, H - y0);
+  const int band_elems = band_rows * W;       // <= kUbLdsFloats / PG, W % 4 == 0
+  const int n_vec = band_elems / 4;
+  const int hi1 = table[8 + 2 * band];
+  const int lo = hi1 > 0 ? kUbBig - table[9 + 2 * band] : 0;
+  const int npw = hi1 > 0 ? (hi1 - lo) * OW : 0;   // pooled pixels that may reach the band
+  const int pw0 = lo * OW;
+
+  unsigned offp[kUbIpt][KH];
+#pragma unroll
+  for (int j = 0; j < kUbIpt; ++j) {
+    const int i = t + kBandBlock * j;
+    const int pix = pw0 + min(i, max(npw - 1, 0));
+    const float2* coords = reinterpret_cast<const float2*>(map) + (size_t)pix * K;
+#pragma unroll
+    for (int h = 0; h < KH; ++h) {
+      unsigned half[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int k = 2 * h + e;
+        half[e] = kUbNone;
+        if (k < K) {
+          const float2 c = coords[k];
+          PointTaps<float, 0> tp;
+          tp.set(c.x, c.y, H, W);
+          const int ry = tp.ty[0] - y0;
+          if (i < npw && tp.off[0] >= 0 && (unsigned)ry < (unsigned)band_rows)
+            half[e] = (unsigned)(ry * W + tp.tx[0]);
+        }
+      }
+      offp[j][h] = half[0] | (half[1] << 16);
+    }
+  }
+  vec4* acc4 = reinterpret_cast<vec4*>(acc);
+  for (int v = t; v < PG * n_vec; v += kBandBlock) acc4[v] = vec4{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+  // Stores the band sums of the planes q, q + 1 (the second only below p_end) and clears them.
+  auto store_pass = [&](int q) {
+    for (int v = t; v < n_vec; v += kBandBlock) {
+      vec4 a, b;
+      if constexpr (AVG) {
+        const vec4 lo4 = acc4[2 * v], hi4 = acc4[2 * v + 1];   // (p0, p1) of four elements
+        acc4[2 * v] = vec4{0.f, 0.f, 0.f, 0.f};
+        acc4[2 * v + 1] = vec4{0.f, 0.f, 0.f, 0.f};
+        a = vec4{lo4[0], lo4[2], hi4[0], hi4[2]} / float(K);
+        b = vec4{lo4[1], lo4[3], hi4[1], hi4[3]} / float(K);
+      } else {
+        a = acc4[v];
+        b = acc4[n_vec + v];
+        acc4[v] = vec4{0.f, 0.f, 0.f, 0.f};
+        acc4[n_vec + v] = vec4{0.f, 0.f, 0.f, 0.f};
+      }
+      store_piece(gin + (size_t)q * HW + (size_t)y0 * W, v, a, aligned);
+      if (q + 1 < p_end) store_piece(gin + (size_t)(q + 1) * HW + (size_t)y0 * W, v, b, aligned);
+    }
+  };
+
+  bool stray = false;
+  for (int p = p_begin; p < p_end; p += PG) {
+    // this pass's indices and gradients are requested first; the previous pass is stored
+    // while they are on their way
+    int64_t sv[kUbIpt][PG];
+    float gv[kUbIpt][PG];
+#pragma unroll
+    for (int j = 0; j < kUbIpt; ++j) {
+      const int i = t + kBandBlock * j;
+      const size_t at = (size_t)pw0 + min(i, max(npw - 1, 0));
+#pragma unroll
+      for (int g = 0; g < PG; ++g) {
+        const size_t e = (size_t)min(p + g, p_end - 1) * M + at;
+        if constexpr (!AVG) sv[j][g] = idx[e];
+        gv[j][g] = gout[e];
+      }
+    }
+    if (p > p_begin) {
+      store_pass(p - PG);
+      __syncthreads();
+    }
+    const bool two = p + 1 < p_end;
+#pragma unroll
+    for (int j = 0; j < kUbIpt; ++j) {
+      const int i = t + kBandBlock * j;
+      if (i >= npw) continue;
+      if constexpr (AVG) {
+        float2* acc2 = reinterpret_cast<float2*>(acc);
+        const float gb = two ? gv[j][1] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const unsigned o16 = (offp[j][k >> 1] >> ((k & 1) * 16)) & 0xFFFFu;
+          if (o16 != kUbNone) lds_add_f32x2(acc2 + o16, gv[j][0], gb);
+        }
+      } else {
+        const int first = (pw0 + i) * K * 2;   // map element of the pixel's first sample
+#pragma unroll
+        for (int g = 0; g < PG; ++g) {
+          if (g == 1 && !two) continue;
+          const int64_t s64 = sv[j][g];
+          const bool live = s64 >= 0 && s64 + 2 <= (int64_t)map_elems;   // others add nothing
+          const int d = (int)s64 - first;
+          const bool mine = d >= 0 && d < 2 * K && (d & 1) == 0;
+          stray |= live && !mine;
+          if (live && mine) {
+            const unsigned o16 = packed_tap<K>(offp[j], d >> 1);
+            if (o16 != kUbNone) lds_add_f32(acc + g * band_elems + o16, gv[j][g]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  store_pass(p_begin + (p_end - p_begin - 1) / PG * PG);   // the last pass
+  if (stray) atomicAdd(gate, 1);
+}
+
 }  // namespace
 
 bool pool_band_launch(bool avg, const float* in, const float* map, float* out, int64_t* idx,
@@ -290,6 +534,60 @@ bool pool_band_launch(bool avg, const float* in, const float* map, float* out, i
                : dispatch_ipt<false, 9>(ipt, in, map, out, idx, (int)planes, H, W, OW, M, R, stream);
   return avg ? dispatch_ipt<true, 4>(ipt, in, map, out, idx, (int)planes, H, W, OW, M, R, stream)
              : dispatch_ipt<false, 4>(ipt, in, map, out, idx, (int)planes, H, W, OW, M, R, stream);
+}
+
+// Image rows per unpooling band: two planes of RB rows in the 32 KB of a workgroup's sums.
+static int unpool_band_rows_per_band(int W) {
+  if (W % 4 != 0) return 0;
+  for (int rb : {16, 8, 4, 2, 1})
+    if ((int64_t)rb * W * 2 <= kUbLdsFloats) return rb;
+  return 0;
+}
+
+bool unpool_band_shape(int H, int W, int OH, int OW, int K) {
+  return unpool_band_rows_per_band(W) > 0 && (K == 4 || K == 9) &&
+         (int64_t)OH * OW * K * 2 < ((int64_t)1 << 31);
+}
+
+size_t unpool_band_table_bytes(int H, int W) {
+  const int rb = unpool_band_rows_per_band(W);
+  const int64_t nbands = rb > 0 ? ceil_div(H, rb) : 0;
+  return (size_t)(8 + 2 * nbands) * sizeof(int);   // the verdict word is there for every plane
+}
+
+void unpool_band_build(const float* map, int* table, int H, int W, int OH, int OW, int K,
+                       hipStream_t stream) {
+  const int rb = unpool_band_rows_per_band(W);
+  const int M = OH * OW;
+  launch(unpool_band_rows_kernel, dim3((unsigned)ceil_div(M, kBandBlock)), dim3(kBandBlock), stream,
+         map, M, OW, K, H, W, rb, table);
+  launch(unpool_band_verdict_kernel, dim3(1), dim3(kBandBlock), stream, table,
+         (int)ceil_div(H, rb), OW);
+}
+
+void unpool_band_launch(bool avg, const float* gout, const int64_t* idx, const float* map,
+                        float* gin, const int* table, int* gate, int64_t planes, int H, int W,
+                        int OH, int OW, int K, hipStream_t stream) {
+  const int rb = unpool_band_rows_per_band(W);
+  const int nbands = (int)ceil_div(H, rb);
+  // one round of resident workgroups (three per CU for max unpooling, whose registers allow
+  // no more, four for average unpooling; measured: 102 against 112 us and 107 against 115 us
+  // on an 8 x 64 x 256 x 512 image), chunks in eighths (one per XCD), at least two planes each
+  int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(planes / 2, (avg ? 1024 : 768) / nbands));
+  chunks = std::max(8, chunks / 8 * 8);
+  chunks = (int)std::min<int64_t>(chunks, planes);
+  const unsigned grid = 8u * (unsigned)nbands * (unsigned)ceil_div(chunks, 8);
+  const int M = OH * OW;
+#define UB(AVGv, Kv)                                                                          \
+  launch(unpool_band_kernel<AVGv, Kv>, dim3(grid), dim3(kBandBlock), stream, gout, idx, map, \
+         gin, table, gate, (int)planes, H, W, OW, M, rb, nbands, chunks, M * K * 2,               \
+         ((uintptr_t)gin & 15) == 0 ? 1 : 0)
+  if (K == 9) {
+    if (avg) UB(true, 9); else UB(false, 9);
+  } else {
+    if (avg) UB(true, 4); else UB(false, 4);
+  }
+#undef UB
 }
 
 }  // namespace sdk

@@ -12,4 +12,21 @@ namespace sdk {
 bool pool_band_launch(bool avg, const float* in, const float* map, float* out, int64_t* idx,
                       int64_t planes, int H, int W, int OH, int OW, int K, hipStream_t stream);
 
+// Unpooling by image row bands (float32, single nearest taps, K = 4 or 9, image width a
+// multiple of 4 and at most 4096).  unpool_band_shape says whether
+// the kernels take the shape at all.  The table (unpool_band_table_bytes, zero-filled by the
+// caller, then unpool_band_build) depends on the map alone; its first word is the device-side
+// verdict: 1 when the band kernels will do the call, 0 when they return at once and the
+// caller's other route has to run (it stays 0 when unpool_band_build is never called).
+bool unpool_band_shape(int H, int W, int OH, int OW, int K);
+size_t unpool_band_table_bytes(int H, int W);
+void unpool_band_build(const float* map, int* table, int H, int W, int OH, int OW, int K,
+                       hipStream_t stream);
+// avg: every sample of a pooled pixel receives grad_output / K (idx unused); else the sample the
+// index names receives grad_output.  gate: raised when an index names a sample of another
+// pooled pixel than its own (the caller then redoes the call with its atomic route).
+void unpool_band_launch(bool avg, const float* gout, const int64_t* idx, const float* map,
+                        float* gin, const int* table, int* gate, int64_t planes, int H, int W,
+                        int OH, int OW, int K, hipStream_t stream);
+
 }  // namespace sdk
