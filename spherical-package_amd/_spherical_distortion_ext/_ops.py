@@ -6,9 +6,16 @@ allocates the outputs with torch, fetches the current HIP stream and makes one
 call into libsdk_mapped_ops.so.  The operators are registered in the
 ``sdk_mapped_ops`` namespace of torch.library for the CUDA (= HIP on ROCm)
 dispatch key only: calling them with CPU tensors raises, there is no CPU path.
+
+The schemas are defined here.  Where libsdk_torch_ops.so is built (csrc/torch_ops.cpp, the
+same checks, allocation, stream fetch and plan cache in C++), it is loaded and implements the
+operators it names; the functions below implement the others, and all of them when that
+library is absent or the environment says SDK_TORCH_OPS=python.  The compute mode, the plan
+cache switches and the unpool workspace switch set here reach both.
 """
 import contextlib
 import ctypes
+import os
 import threading
 
 import torch
@@ -35,12 +42,19 @@ def _mode_value(mode):
     return _MODES[mode]
 
 
+# libsdk_torch_ops.so as a ctypes handle (its control functions) once it is loaded, else None
+_native = None
+_NATIVE_OPS = frozenset()
+
+
 def set_conv_compute(mode):
     """Sets the process-wide default arithmetic of the mapped (transposed) convolutions:
     "native" (fp32 MFMA), "split" (fp32 operands as three bf16 pieces), "bf16" (operands
     rounded to bf16), "unfused" (im2col + GEMM kernels)."""
     global _default_mode
     _default_mode = _mode_value(mode)
+    if _native is not None:
+        _native.sdk_torch_set_default_mode(_default_mode)
 
 
 def _current_mode():
@@ -66,10 +80,14 @@ def conv_compute(mode):
     value = _mode_value(mode)
     previous = getattr(_tls, "mode", None)
     _tls.mode = value
+    if _native is not None:
+        _native.sdk_torch_set_thread_mode(value)
     try:
         yield
     finally:
         _tls.mode = previous
+        if _native is not None:
+            _native.sdk_torch_set_thread_mode(-1 if previous is None else previous)
 
 
 def _check(ref, **tensors):
@@ -169,6 +187,16 @@ def set_conv_plan_cache(enabled, max_entries=None):
         _PLAN_CACHE.clear()
     while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
         _PLAN_CACHE.pop(next(iter(_PLAN_CACHE)))
+    if _native is not None:
+        _native.sdk_torch_set_plan_cache(1 if enabled else 0, _PLAN_CACHE_MAX)
+
+
+def plan_cache_size():
+    """Plans kept at the moment, by the compiled operator layer and by this module."""
+    n = len(_PLAN_CACHE)
+    if _native is not None:
+        n += int(_native.sdk_torch_plan_cache_size())
+    return n
 
 
 def _tensor_key(t):
@@ -388,6 +416,8 @@ def set_unpool_workspace(enabled):
     as a gather; without it the call is the zero fill + atomic scatter."""
     global _UNPOOL_WORKSPACE
     _UNPOOL_WORKSPACE = bool(enabled)
+    if _native is not None:
+        _native.sdk_torch_set_unpool_workspace(1 if enabled else 0)
 
 
 def mapped_max_pool(x, sample_map, interp_weights, kernel_size, interp):
@@ -815,9 +845,38 @@ _SCHEMAS = (
      mapped_transposed_conv_backward),
 )
 
+def _load_native():
+    """Loads the compiled operator layer when it is built (its static registration implements
+    the operators it names for the CUDA key) and returns (ctypes handle, operator names)."""
+    path = os.path.join(os.path.dirname(_capi.LIB_PATH), "libsdk_torch_ops.so")
+    if os.environ.get("SDK_TORCH_OPS", "") == "python" or not os.path.exists(path):
+        return None, frozenset()
+    _capi.load()
+    torch.ops.load_library(path)
+    lib = ctypes.CDLL(path)
+    lib.sdk_torch_native_ops.restype = ctypes.c_char_p
+    lib.sdk_torch_set_thread_mode.restype = ctypes.c_int
+    lib.sdk_torch_plan_cache_size.restype = ctypes.c_int
+    lib.sdk_torch_current_mode.restype = ctypes.c_int
+    for name in ("sdk_torch_set_default_mode", "sdk_torch_set_plan_cache",
+                 "sdk_torch_set_unpool_workspace"):
+        getattr(lib, name).restype = None
+    return lib, frozenset(lib.sdk_torch_native_ops().decode().split(","))
+
+
 _library = torch.library.Library(_NS, "DEF")
 for _name, _schema, _fn in _SCHEMAS:
     _library.define(_name + _schema)
-    _library.impl(_name, _fn, "CUDA")
+_native, _NATIVE_OPS = _load_native()
+for _name, _schema, _fn in _SCHEMAS:
+    if _name not in _NATIVE_OPS:
+        _library.impl(_name, _fn, "CUDA")
 
+
+# The functions above stay reachable under their own names in PYTHON_IMPL; where the compiled
+# layer implements an operator, the module-level name is the registered operator itself, so
+# that callers of this module and callers of torch.ops.sdk_mapped_ops run the same code.
 ops = getattr(torch.ops, _NS)
+PYTHON_IMPL = {_name: _fn for _name, _schema, _fn in _SCHEMAS}
+for _name in _NATIVE_OPS:
+    globals()[_name] = getattr(ops, _name)
