@@ -207,6 +207,43 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_fill_kernel(
   }
 }
 
+// Sorts every target's list by source (then by coefficient bits), in place.  The fill appends
+// in the order its atomics are served, so entry s of neighbouring targets names unrelated
+// sources; sorted, neighbouring targets read neighbouring sources with the same instruction
+// (fewer cache lines per read), and the sum of a target no longer depends on scheduling.
+// One thread per target; lists are short (kInvSlots at most): selection sort on global memory.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void resample_inverse_sort_kernel(
+    const int* __restrict__ cnt, int* __restrict__ src, T* __restrict__ co, int HW,
+    const int* __restrict__ gate, const int* __restrict__ only_if) {
+  if (only_if != nullptr && *only_if == 0) return;
+  if (*gate != 0) return;   // some list overflowed: the call scatters instead
+  const int u = blockIdx.x * kBlock + threadIdx.x;
+  if (u >= HW) return;
+  const int n = min(cnt[u], kInvSlots);
+  for (int i = 0; i + 1 < n; ++i) {
+    int best = i, bs = src[(size_t)i * HW + u];
+    T bc = co[(size_t)i * HW + u];
+    const int first_s = bs;
+    const T first_c = bc;
+    for (int j = i + 1; j < n; ++j) {
+      const int sj = src[(size_t)j * HW + u];
+      const T cj = co[(size_t)j * HW + u];
+      if (sj < bs || (sj == bs && cj < bc)) {
+        best = j;
+        bs = sj;
+        bc = cj;
+      }
+    }
+    if (best != i) {
+      src[(size_t)best * HW + u] = first_s;
+      co[(size_t)best * HW + u] = first_c;
+      src[(size_t)i * HW + u] = bs;
+      co[(size_t)i * HW + u] = bc;
+    }
+  }
+}
+
 template <typename T, int PC>
 __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
     const T* __restrict__ in, const int* __restrict__ cnt, const int* __restrict__ src,
@@ -225,13 +262,35 @@ __global__ __launch_bounds__(kBlock) void resample_inverse_gather_kernel(
 #pragma unroll
   for (int j = 0; j < PC; ++j) acc[j] = T(0);
   T wtot = T(0);
-  for (int s = 0; s < n; ++s) {
-    const int m = src[(size_t)s * HW + u];
-    const T c = co[(size_t)s * HW + u];
-    wtot += c;
+  // List entries in batches of four: the four (source, coefficient) reads of a lane are in
+  // flight together, then its 4 * PC value reads, so a wave pays two round trips per batch
+  // instead of two per entry (a wave runs as long as its longest list).  Entries past a
+  // lane's own count are read from their slot all the same (the slot exists, its content is
+  // not used) and select a zero contribution; the sum keeps the ascending entry order.
+  for (int s0 = 0; __any(s0 < n); s0 += 4) {
+    int m[4];
+    T c[4];
+    bool on[4];
 #pragma unroll
-    for (int j = 0; j < PC; ++j)
-      acc[j] += c * in[(size_t)(plane0 + (j < np ? j : 0)) * in_plane + m];
+    for (int i = 0; i < 4; ++i) {
+      on[i] = s0 + i < n;
+      const size_t at = (size_t)min(s0 + i, kInvSlots - 1) * HW + u;
+      m[i] = src[at];
+      c[i] = co[at];
+    }
+    T v[4][PC];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const size_t mi = on[i] ? (size_t)m[i] : 0;
+#pragma unroll
+      for (int j = 0; j < PC; ++j) v[i][j] = in[(size_t)(plane0 + (j < np ? j : 0)) * in_plane + mi];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      wtot += on[i] ? c[i] : T(0);
+#pragma unroll
+      for (int j = 0; j < PC; ++j) acc[j] += on[i] ? c[i] * v[i][j] : T(0);
+    }
   }
   // average unpooling hands every sample value / group: divided once here, after the sum
   if (group > 1) {
@@ -1237,6 +1296,10 @@ static int build_inverse_lists(const T* map, const T* wts, void* workspace, size
                               wts, H, W, MP, P, cnt, src, co, g, group,
                               (const int*)(flags ? flags + 1 : nullptr))));
   SDK_LAUNCH_CHECK("resample_to_map(inverse fill)");
+  launch(resample_inverse_sort_kernel<T>, dim3((unsigned)ceil_div((int64_t)H * W, kBlock)),
+         dim3(kBlock), stream, (const int*)cnt, src, co, H * W, (const int*)g,
+         (const int*)(flags ? flags + 1 : nullptr));
+  SDK_LAUNCH_CHECK("resample_to_map(inverse sort)");
   if (flags) {
     launch(avg_unpool_verdict_kernel, dim3(1), dim3(kBlock), stream, (const int*)(flags + 64), 0,
            OW, flags, g, 1, (const int*)nullptr);
