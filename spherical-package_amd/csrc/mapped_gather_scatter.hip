@@ -105,9 +105,60 @@ __global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
   const size_t HW = (size_t)H * W;
   const int q = WEIGHTED ? P : 1;
   T acc[PC];
-  gather_sample<T, INTERP, WEIGHTED, PC>(image + (size_t)plane0 * HW, HW, np,
-                                         map + (size_t)pix * q * 2,
-                                         WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W, acc);
+  if constexpr (INTERP != 0 && !WEIGHTED) {
+    // The two taps of an image row are neighbours in memory: one read of two elements (from
+    // any element boundary) fetches both, which halves the read instructions and, where
+    // neighbouring lanes lie about two pixels apart and the reads are bound by the requests
+    // the vector cache takes per cycle, the time with them.  The pair starts at column
+    // clamp(x1, 0, W - 2); a tap takes the element of its own column from it.  Only the
+    // wrapped neighbour of the last column (bispherical) is not in its pair and is read on its
+    // own.  The blend is PointTaps::blend, on the same values.
+    if (W >= 2) {
+      PointTaps<T, INTERP> t;
+      t.set(map[(size_t)pix * 2], map[(size_t)pix * 2 + 1], H, W);
+      typedef T pair_t __attribute__((ext_vector_type(2)));
+      const int cb = min(max(t.tx[0], 0), W - 2);
+      const int r1 = min(max(t.ty[0], 0), H - 1), r2 = min(max(t.ty[2], 0), H - 1);
+      const size_t o1 = (size_t)r1 * W + cb, o2 = (size_t)r2 * W + cb;
+      const bool wrapped = INTERP == 2 && t.tx[1] != t.tx[0] + 1;   // x1 = W - 1, x2 = 0
+      const T* base = image + (size_t)plane0 * HW;
+      pair_t top[PC], bot[PC];
+      T wrap_top[PC], wrap_bot[PC];
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        const T* plane = base + (size_t)(j < np ? j : 0) * HW;
+        __builtin_memcpy(&top[j], plane + o1, sizeof(pair_t));   // (element alignment only)
+        __builtin_memcpy(&bot[j], plane + o2, sizeof(pair_t));
+      }
+      if (__any(wrapped)) {
+#pragma unroll
+        for (int j = 0; j < PC; ++j) {
+          const T* plane = base + (size_t)(j < np ? j : 0) * HW;
+          wrap_top[j] = plane[(size_t)r1 * W];
+          wrap_bot[j] = plane[(size_t)r2 * W];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const bool first0 = t.tx[0] == cb, first1 = t.tx[1] == cb;
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        T raw[4];
+        raw[0] = first0 ? top[j].x : top[j].y;
+        raw[2] = first0 ? bot[j].x : bot[j].y;
+        raw[1] = wrapped ? wrap_top[j] : (first1 ? top[j].x : top[j].y);
+        raw[3] = wrapped ? wrap_bot[j] : (first1 ? bot[j].x : bot[j].y);
+        acc[j] = j < np ? t.blend(raw) : T(0);
+      }
+    } else {
+      gather_sample<T, INTERP, WEIGHTED, PC>(image + (size_t)plane0 * HW, HW, np,
+                                             map + (size_t)pix * 2, nullptr, P, H, W, acc);
+    }
+  } else {
+    gather_sample<T, INTERP, WEIGHTED, PC>(image + (size_t)plane0 * HW, HW, np,
+                                           map + (size_t)pix * q * 2,
+                                           WEIGHTED ? wts + (size_t)pix * q : nullptr, P, H, W,
+                                           acc);
+  }
 #pragma unroll
   for (int j = 0; j < PC; ++j)
     if (j < np) out[(size_t)(plane0 + j) * MP + pix] = acc[j];
