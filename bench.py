@@ -48,7 +48,12 @@ class Timer:
     def __init__(self, torch):
         self.torch = torch
 
-    def run(self, fn, steps, warmup):
+    def run(self, fn, steps, warmup, reps=1):
+        """Mean and minimum time of one call of fn over `steps` timed regions of `reps` calls
+        each.  reps > 1 is for calls of a few tens of microseconds, where the event pair
+        itself (a few microseconds of command processing between the marker and the kernel)
+        would be a visible part of a region holding one call; the calls of a region are issued
+        back to back on the stream, so a region's time over reps is what one launch takes."""
         t = self.torch
         for _ in range(warmup):
             fn()
@@ -57,10 +62,11 @@ class Timer:
                for _ in range(steps)]
         for a, b in evs:
             a.record()
-            fn()
+            for _ in range(reps):
+                fn()
             b.record()
         t.cuda.synchronize()
-        ms = [a.elapsed_time(b) for a, b in evs]
+        ms = [a.elapsed_time(b) / reps for a, b in evs]
         return float(np.mean(ms)), float(np.min(ms))
 
 
@@ -265,7 +271,7 @@ def bench_conv1(torch, ops, timer, steps, warmup):
     return {"conv1_latency": out}
 
 
-def bench_resample2(torch, ops, timer, steps, warmup):
+def bench_resample2(torch, ops, timer, steps, warmup, reps=8):
     import workloads
     cfg = workloads.config2()
     dev = "cuda:0"
@@ -273,9 +279,9 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     m = torch.from_numpy(cfg["sample_map"]).to(dev)
     H, W = cfg["out_shape"]
     patches = ops.resample_from_map(x, m, None, 1)
-    ms_g, _ = timer.run(lambda: ops.resample_from_map(x, m, None, 1), steps, warmup)
+    ms_g, _ = timer.run(lambda: ops.resample_from_map(x, m, None, 1), steps, warmup, reps=8)
     ms_s, _ = timer.run(lambda: ops.resample_to_map_normalized(patches, m, None, H, W, 1, 1e-12),
-                        steps, warmup)
+                        steps, warmup, reps=8)
     gather_bytes = _nbytes(x, m, patches)
     scatter_bytes = _nbytes(patches, m, x) + H * W * 4.0
     # the UV way back: every image pixel reads its face's patch at (u, v); and its adjoint
@@ -284,12 +290,12 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     B, C = x.shape[:2]
     NT, TP = m.shape[0], cfg["patch"]
     tex = patches.view(B, C, NT, TP, TP)
-    ms_uf, _ = timer.run(lambda: ops.resample_from_uv_maps(tex, quad, uv, 1), steps, warmup)
+    ms_uf, _ = timer.run(lambda: ops.resample_from_uv_maps(tex, quad, uv, 1), steps, warmup, reps=8)
     ms_ub, _ = timer.run(lambda: ops.resample_to_uv_maps(x, quad, uv, NT, TP, TP, 1), steps,
-                         warmup)
+                         warmup, reps=8)
     uv_bytes = _nbytes(tex, quad, uv, x)
     # the kernel map of configuration 4's image, generated on the device (bytes = the map)
-    ms_map, _ = timer.run(lambda: ops.equirect_kernel_map(256, 512, 3, 3), steps, warmup)
+    ms_map, _ = timer.run(lambda: ops.equirect_kernel_map(256, 512, 3, 3), steps, warmup, reps=8)
     map_bytes = 256 * 512 * 9 * 2 * 4.0
     # voting resample: a 13-class label image halved in size, four sources per output pixel
     gen = torch.Generator().manual_seed(7)
@@ -297,7 +303,7 @@ def bench_resample2(torch, ops, timer, steps, warmup):
     yy, xx = torch.meshgrid(torch.arange(H) // 2, torch.arange(W) // 2, indexing="ij")
     vmap = torch.stack([xx, yy], -1).contiguous().to(dev)
     ms_v, _ = timer.run(lambda: ops.voting_resample_to_map(labels, vmap, H // 2, W // 2, 13),
-                        steps, warmup)
+                        steps, warmup, reps=8)
     vote_bytes = _nbytes(labels, vmap) + B * (H // 2) * (W // 2) * 8.0
     return {"voting_resample": dict(ms=ms_v, **_roof("hbm", vote_bytes, ms_v)),
             "map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
@@ -311,7 +317,7 @@ def bench_resample2(torch, ops, timer, steps, warmup):
                                                        traffic=_measured_traffic("resample_to_map")))}
 
 
-def bench_pool3(torch, ops, timer, steps, warmup):
+def bench_pool3(torch, ops, timer, steps, warmup, reps=8):
     import workloads
     cfg = workloads.config3()
     dev = "cuda:0"
@@ -321,18 +327,18 @@ def bench_pool3(torch, ops, timer, steps, warmup):
     K = cfg["kernel_size"]
     H, W = x.shape[2:]
     val, idx = ops.mapped_max_pool(x, m, None, K, 0)
-    ms_f, _ = timer.run(lambda: ops.mapped_max_pool(x, m, None, K, 0), steps, warmup)
-    ms_b, _ = timer.run(lambda: ops.mapped_max_unpool(g, idx, m, None, H, W, K, 0), steps, warmup)
+    ms_f, _ = timer.run(lambda: ops.mapped_max_pool(x, m, None, K, 0), steps, warmup, reps=8)
+    ms_b, _ = timer.run(lambda: ops.mapped_max_unpool(g, idx, m, None, H, W, K, 0), steps, warmup, reps=8)
     fwd_bytes = _nbytes(x, m, val, idx)
     bwd_bytes = _nbytes(g, idx, m, x)
     # average pooling on the same input and map: no index tensor on either side
-    ms_af, _ = timer.run(lambda: ops.mapped_avg_pool(x, m, None, K, 0), steps, warmup)
-    ms_ab, _ = timer.run(lambda: ops.mapped_avg_unpool(g, m, None, H, W, K, 0), steps, warmup)
+    ms_af, _ = timer.run(lambda: ops.mapped_avg_pool(x, m, None, K, 0), steps, warmup, reps=8)
+    ms_ab, _ = timer.run(lambda: ops.mapped_avg_unpool(g, m, None, H, W, K, 0), steps, warmup, reps=8)
     avg_bytes = _nbytes(x, m, val)
     # what a plain copy of the same input reaches on this GPU (the tensor library's copy kernel,
     # read + write): the rate a memory-bound kernel can be held against beside the published peak
     y = torch.empty_like(x)
-    ms_c, _ = timer.run(lambda: y.copy_(x), steps, warmup)
+    ms_c, _ = timer.run(lambda: y.copy_(x), steps, warmup, reps=8)
     copy_ref = dict(ms=ms_c, **_roof("hbm", 2 * _nbytes(x), ms_c))
     del y
     return {"copy_reference": copy_ref,
