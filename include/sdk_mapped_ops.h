@@ -629,6 +629,14 @@ int sdk_mapped_transposed_conv_backward_planned(const void* grad_output, const v
  *   sdk_mapped_max_unpool_workspace_bytes(height, width, dtype).  The first
  *   256 bytes of this plan are the call's fallback flag and are rewritten by
  *   every planned call: calls that share one plan must not overlap.
+ * sdk_mapped_max_unpool_plan_bands: synchronises `stream` and sets *bands to 1
+ *   if the plan's map lets one kernel do the whole call (float32, unweighted
+ *   nearest taps, every pooled row reaching few image rows), else to 0.
+ * sdk_mapped_max_unpool_planned_bands: sdk_mapped_max_unpool_planned for a plan
+ *   on which that query returned 1 (with 0 the result is undefined): the same
+ *   result with two launches in place of five.  Unweighted maps only, so it
+ *   takes no interp_weights / num_interp_pts.  It leaves the plan's flag
+ *   cleared itself instead of clearing it up front.
  * ------------------------------------------------------------------------- */
 int sdk_resample_to_map_plan_build(const void* sample_map, const void* interp_weights, void* plan,
                                    size_t plan_bytes, int64_t map_height, int64_t map_width,
@@ -663,6 +671,15 @@ int sdk_mapped_max_unpool_planned(const void* grad_output, const int64_t* indice
                                   int64_t out_height, int64_t out_width, int64_t kernel_size,
                                   int32_t num_interp_pts, int32_t interp, int32_t dtype,
                                   sdk_stream_t stream);
+int sdk_mapped_max_unpool_plan_bands(const void* plan, size_t plan_bytes, int64_t height,
+                                     int64_t width, int32_t dtype, sdk_stream_t stream,
+                                     int32_t* bands);
+int sdk_mapped_max_unpool_planned_bands(const void* grad_output, const int64_t* indices,
+                                        const void* sample_map, void* grad_input, void* plan,
+                                        size_t plan_bytes, int64_t batch, int64_t channels,
+                                        int64_t height, int64_t width, int64_t out_height,
+                                        int64_t out_width, int64_t kernel_size, int32_t interp,
+                                        int32_t dtype, sdk_stream_t stream);
 
 #ifdef __cplusplus
 }

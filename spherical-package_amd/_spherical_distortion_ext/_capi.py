@@ -64,6 +64,8 @@ SIGNATURES = {
     "sdk_mapped_avg_unpool_planned": [_vp] * 5 + [_sz, _i32] + [_i64] * 7 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_unpool_plan_build": [_vp, _vp, _sz] + [_i64] * 5 + [_i32] * 3 + [_vp],
     "sdk_mapped_max_unpool_planned": [_vp] * 6 + [_sz] + [_i64] * 7 + [_i32] * 3 + [_vp],
+    "sdk_mapped_max_unpool_plan_bands": [_vp, _sz, _i64, _i64, _i32, _vp, _vp],
+    "sdk_mapped_max_unpool_planned_bands": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 2 + [_vp],
 }
 OTHER_SYMBOLS = ("sdk_last_error", "sdk_version", "sdk_mapped_conv_workspace_bytes",
                  "sdk_resample_to_map_workspace_bytes", "sdk_mapped_max_unpool_workspace_bytes",

@@ -267,7 +267,8 @@ def _scatter_plan(kind, ref, sample_map, interp_weights, out_h, out_w, K, P, int
     kind "resample" / "avg_unpool": the inverted map (sdk_resample_to_map_plan_build; K = 1 for
     a resampling map), complete = 1 when every target's list holds all its sources, checked
     once after the build (not under stream capture, where the check's synchronisation is not
-    allowed).  kind "max_unpool": the tile windows (sdk_mapped_max_unpool_plan_build)."""
+    allowed).  kind "max_unpool": the tile windows (sdk_mapped_max_unpool_plan_build), complete = 1
+    when the row-band kernel does every call on the plan (sdk_mapped_max_unpool_plan_bands)."""
     if not _plan_cache_enabled:
         return None, 0, 0
     dt = _DTYPES[ref.dtype]
@@ -293,6 +294,10 @@ def _scatter_plan(kind, ref, sample_map, interp_weights, out_h, out_w, K, P, int
     if kind == "max_unpool":
         _capi.call("sdk_mapped_max_unpool_plan_build", _ptr(sample_map), _ptr(plan), n, int(out_h),
                    int(out_w), MH, MW, int(K), int(P), int(interp), dt, _stream(ref))
+        flag = ctypes.c_int32(0)
+        _capi.call("sdk_mapped_max_unpool_plan_bands", _ptr(plan), n, int(out_h), int(out_w), dt,
+                   _stream(ref), ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+        complete = int(flag.value)
     else:
         _capi.call("sdk_resample_to_map_plan_build", _ptr(sample_map), _ptr(interp_weights),
                    _ptr(plan), n, MH, MW, int(out_h), int(out_w), int(K), int(P), int(interp), dt,
@@ -452,8 +457,14 @@ def mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, in_h, i
                       device=grad_output.device)
     with torch.cuda.device(grad_output.device):
         if _UNPOOL_WORKSPACE:
-            plan, nplan, _ = _scatter_plan("max_unpool", grad_output, sample_map, interp_weights,
-                                           in_h, in_w, kernel_size, P, interp)
+            plan, nplan, bands = _scatter_plan("max_unpool", grad_output, sample_map,
+                                               interp_weights, in_h, in_w, kernel_size, P, interp)
+            if plan is not None and bands:
+                _capi.call("sdk_mapped_max_unpool_planned_bands", _ptr(grad_output),
+                           _ptr(idx_mask), _ptr(sample_map), _ptr(gin), _ptr(plan), nplan, B, C,
+                           int(in_h), int(in_w), OH, OW, int(kernel_size), int(interp),
+                           _DTYPES[grad_output.dtype], _stream(grad_output))
+                return gin
             if plan is not None:
                 _capi.call("sdk_mapped_max_unpool_planned", _ptr(grad_output), _ptr(idx_mask),
                            _ptr(sample_map), _ptr(interp_weights), _ptr(gin), _ptr(plan), nplan,

@@ -808,6 +808,41 @@ __global__ __launch_bounds__(kBlock) void mapped_max_unpool_kernel(
   }
 }
 
+// After the row-band unpool of a call whose plan is known to run it: the band kernel has written
+// every image pixel and added every sample whose index lies among its own pooled pixel's
+// samples; it raised gate[0] if it met an index that names another pixel's sample ("stray":
+// never produced by the pooling, allowed by the operator).  This kernel adds those samples
+// where they point, as mapped_max_unpool_kernel would have, and the workgroup that finishes
+// last clears gate[0] for the next call on the plan (gate[1] counts finished workgroups).
+template <typename T, int INTERP, bool WEIGHTED>
+__global__ __launch_bounds__(kBlock) void mapped_max_unpool_stray_kernel(
+    const T* __restrict__ gout, const int64_t* __restrict__ idx, const T* __restrict__ map,
+    const T* __restrict__ wts, T* __restrict__ gin, size_t total, int H, int W, int M, int K,
+    int P, int64_t map_elems, int* gate) {
+  if (*(volatile int*)gate == 0) return;
+  const int q = WEIGHTED ? P : 1;
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / (size_t)M;
+    const int64_t pix = (int64_t)(i - plane * (size_t)M);
+    const int64_t s = idx[i];
+    if (s < 0 || s + 2 * q > map_elems) continue;
+    const int64_t d = s - pix * K * q * 2;
+    if (d >= 0 && d < (int64_t)2 * K * q && (d & 1) == 0) continue;   // the band kernel's own
+    const T val[1] = {gout[i]};
+    scatter_sample<T, INTERP, WEIGHTED, 1>(gin + plane * (size_t)H * W, 0, 1, map + s,
+                                           WEIGHTED ? wts + s / 2 : nullptr, P, H, W, val);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    if (atomicAdd(gate + 1, 1) == (int)gridDim.x - 1) {
+      gate[1] = 0;
+      gate[0] = 0;
+    }
+  }
+}
+
 // The adjoint of the unpool: every pooled element reads the image at the sample its index
 // names (same index convention, same range rule: an index outside the map reads nothing).
 // This is the gradient of unpooling with respect to the pooled values; the reference's own
@@ -1642,7 +1677,7 @@ template <typename T>
 static int launch_unpool(const T* gout, const int64_t* indices, const T* map, const T* wts, T* gin,
                          void* workspace, size_t workspace_bytes, int64_t planes, int H, int W,
                          int OH, int OW, int K, int P, int interp, hipStream_t stream,
-                         bool prebuilt = false) {
+                         bool prebuilt = false, bool bands_known = false) {
   const int64_t HW = (int64_t)H * W, M = (int64_t)OH * OW;
   const int q = pts(P);
   const size_t total = (size_t)planes * M;
@@ -1669,6 +1704,28 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
         unpool_bands_possible<T>(H, W, OH, OW, K, P, interp))
       bands = reinterpret_cast<const int*>(ws + unpool_layout(ut));
     int rc;
+    if (bands_known) {
+      // The caller has read the plan's verdict (sdk_mapped_max_unpool_plan_bands): the band
+      // kernel does the call, and the one kernel after it runs only for indices that name
+      // another pixel's sample.  The gate word is zero between calls (the plan build clears
+      // it, the stray kernel clears it again after use).
+      if constexpr (sizeof(T) == 4) {
+        if (bands == nullptr)
+          return fail(SDK_ERR_INVALID_ARGUMENT, "mapped_max_unpool_planned_bands: no band table for this shape");
+        unpool_band_launch(false, (const float*)gout, indices, (const float*)map, (float*)gin,
+                           bands, g, planes, H, W, OH, OW, K, stream);
+        SDK_LAUNCH_CHECK("mapped_max_unpool(bands)");
+        const int64_t blocks = std::min<int64_t>(ceil_div((int64_t)total, kBlock), 4096);
+        SDK_DISPATCH_INTERP(interp, P,
+                            (launch((mapped_max_unpool_stray_kernel<T, INTERP, WEIGHTED>),
+                                    dim3((unsigned)blocks), dim3(kBlock), stream, gout, indices,
+                                    map, wts, gin, total, H, W, (int)M, K, P, map_elems, g)));
+        SDK_LAUNCH_CHECK("mapped_max_unpool(stray)");
+        return SDK_OK;
+      } else {
+        return fail(SDK_ERR_INVALID_ARGUMENT, "mapped_max_unpool_planned_bands: no band table for this type");
+      }
+    }
     if (prebuilt) {
       // the windows are there; the gate word is this call's own (the kernels raise it)
       rc = zero_fill(ws, 256, stream);
@@ -2332,6 +2389,58 @@ int sdk_mapped_max_unpool_planned(const void* grad_output, const int64_t* indice
                                 (int)height, (int)width, (int)out_height, (int)out_width,
                                 (int)kernel_size, num_interp_pts, interp, (hipStream_t)stream,
                                 true));
+}
+
+int sdk_mapped_max_unpool_plan_bands(const void* plan, size_t plan_bytes, int64_t height,
+                                     int64_t width, int32_t dtype, sdk_stream_t stream,
+                                     int32_t* bands) {
+  SDK_REQUIRE(plan && bands, "mapped_max_unpool_plan_bands: NULL pointer");
+  int rc = check_plane(height, width, "mapped_max_unpool_plan_bands");
+  if (rc) return rc;
+  const size_t need = sdk_mapped_max_unpool_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "mapped_max_unpool_plan_bands: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  *bands = 0;
+  const UnpoolTiling ut = unpool_tiling((int)height, (int)width);
+  if (dtype != SDK_F32 || plan_bytes < unpool_layout_with_bands(ut)) return SDK_OK;
+  int verdict = 0;
+  hipError_t e = hipMemcpyAsync(&verdict, static_cast<const char*>(plan) + unpool_layout(ut),
+                                sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream);
+  if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+  if (e != hipSuccess)
+    return fail(SDK_ERR_DEVICE, "mapped_max_unpool_plan_bands: %s", hipGetErrorString(e));
+  *bands = verdict != 0 ? 1 : 0;
+  return SDK_OK;
+}
+
+int sdk_mapped_max_unpool_planned_bands(const void* grad_output, const int64_t* indices,
+                                        const void* sample_map, void* grad_input, void* plan,
+                                        size_t plan_bytes, int64_t batch, int64_t channels,
+                                        int64_t height, int64_t width, int64_t out_height,
+                                        int64_t out_width, int64_t kernel_size, int32_t interp,
+                                        int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(indices && plan, "mapped_max_unpool_planned_bands: NULL pointer");
+  SDK_REQUIRE(out_height > 0 && out_width > 0, "mapped_max_unpool_planned_bands: bad pooled size");
+  const int64_t M = out_height * out_width;
+  int rc = check_mapped(grad_output, sample_map, nullptr, grad_input, batch, channels, height,
+                        width, M, kernel_size, 0, "mapped_max_unpool_planned_bands");
+  if (rc) return rc;
+  const size_t need = sdk_mapped_max_unpool_workspace_bytes(height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "mapped_max_unpool_planned_bands: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  SDK_REQUIRE(M * kernel_size * 2 < ((int64_t)1 << 31),
+              "mapped_max_unpool_planned_bands: map too large for a plan");
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_REQUIRE(ceil_div(planes * M, kBlock) < ((int64_t)1 << 31),
+              "mapped_max_unpool_planned_bands: too many elements");
+  SDK_DISPATCH_DTYPE(dtype, return launch_unpool<T>(
+                                (const T*)grad_output, indices, (const T*)sample_map,
+                                (const T*)nullptr, (T*)grad_input, plan, plan_bytes, planes,
+                                (int)height, (int)width, (int)out_height, (int)out_width,
+                                (int)kernel_size, 0, interp, (hipStream_t)stream, true, true));
 }
 
 }  // extern "C"

@@ -255,7 +255,9 @@ PlanRef scatter_plan(Kind kind, const Tensor& ref, const Tensor& map, const OptT
         if (kind == kMaxUnpool) {
           SDK_CALL(sdk_mapped_max_unpool_plan_build, map.data_ptr(), buf, n, out_h, out_w, MH, MW,
                    K, (int32_t)P, (int32_t)interp, dt, stream);
-          return 0;
+          int32_t bands = 0;
+          SDK_CALL(sdk_mapped_max_unpool_plan_bands, buf, n, out_h, out_w, dt, stream, &bands);
+          return (int)bands;
         }
         SDK_CALL(sdk_resample_to_map_plan_build, map.data_ptr(), cptr(wts), buf, n, MH, MW, out_h,
                  out_w, K, (int32_t)P, (int32_t)interp, dt, stream);
@@ -398,6 +400,12 @@ Tensor mapped_max_unpool(const Tensor& g, const Tensor& idx, const Tensor& map,
   hipStream_t s = stream_of(g);
   if (g_unpool_workspace) {
     PlanRef plan = scatter_plan(kMaxUnpool, g, map, wts, in_h, in_w, kernel_size, P, interp, s);
+    if (plan.plan.defined() && plan.complete) {
+      SDK_CALL(sdk_mapped_max_unpool_planned_bands, g.data_ptr(), idx.data_ptr<int64_t>(),
+               map.data_ptr(), gin.data_ptr(), plan.ptr(), plan.nbytes, B, C, in_h, in_w, OH, OW,
+               kernel_size, (int32_t)interp, dt, s);
+      return gin;
+    }
     if (plan.plan.defined()) {
       SDK_CALL(sdk_mapped_max_unpool_planned, g.data_ptr(), idx.data_ptr<int64_t>(), map.data_ptr(),
                cptr(wts), gin.data_ptr(), plan.ptr(), plan.nbytes, B, C, in_h, in_w, OH, OW,

@@ -190,3 +190,58 @@ def test_band_unpooling_stands_back_for_what_it_does_not_take(ops, capi, oracle)
         got, gate = _max_unpool(capi, tg, bad, tm, H, W, K, how)
         assert how == "static" or gate > 0
         assert relerr(got, oracle.mapped_max_unpool(g, ref_idx, m, H, W, K, 0)) <= 1e-4
+
+
+def test_planned_bands_call_matches_the_planned_call(ops, capi, oracle):
+    """sdk_mapped_max_unpool_plan_bands says whether one kernel does a plan's calls;
+    sdk_mapped_max_unpool_planned_bands then gives the planned call's result with the flag left
+    clear for the next call: indices from the pooling, then indices that name other pixels'
+    samples (added behind the band kernel), then the first again on the same plan."""
+    B, C, H, W, OH, OW, K = 2, 5, 32, 128, 16, 64, 9
+    rng = np.random.default_rng(21)
+    m = _grid_map(OH, OW, H, W, K, rng)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    g = rng.standard_normal((B, C, OH, OW)).astype(np.float32)
+    tm, tg = _t(m), _t(g)
+    _, idx = ops.mapped_max_pool(_t(x), tm, None, K, 0)
+    bad = torch.roll(idx, shifts=(2, 7), dims=(2, 3)).contiguous()
+    bad[0, 0, 0, 0] = -1
+    bad[1, 2, 3, 3] = OH * OW * K * 2 + 6
+    bad[1, 1, 5, 5] = int(bad[1, 1, 5, 5]) | 1        # an odd index: y of one sample, x of the next
+    ref_bad = _n(bad).copy()
+    ref_bad[1, 2, 3, 3] = -1
+    lib = capi.load()
+    n = lib.sdk_mapped_max_unpool_workspace_bytes(H, W, F32)
+    ws = torch.empty(n, dtype=torch.uint8, device=DEV)
+    capi.call("sdk_mapped_max_unpool_plan_build", _p(tm), _p(ws), n, H, W, OH, OW, K, 0, 0, F32,
+              _stream())
+    flag = ctypes.c_int32(-1)
+    capi.call("sdk_mapped_max_unpool_plan_bands", _p(ws), n, H, W, F32, _stream(),
+              ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+    assert flag.value == 1
+    buf = torch.empty((B, C, H, W), device=DEV)
+    for which, ref_idx in ((idx, _n(idx)), (bad, ref_bad), (idx, _n(idx)), (bad, ref_bad)):
+        buf.fill_(float("nan"))
+        capi.call("sdk_mapped_max_unpool_planned_bands", _p(tg), _p(which), _p(tm), _p(buf), _p(ws),
+                  n, B, C, H, W, OH, OW, K, 0, F32, _stream())
+        torch.cuda.synchronize()
+        assert int(ws[:8].view(torch.int32)[0]) == 0 and int(ws[:8].view(torch.int32)[1]) == 0
+        assert relerr(_n(buf), oracle.mapped_max_unpool(g, ref_idx, m, H, W, K, 0)) <= 1e-4
+    # a map the bands do not take: the query says so (and the operator layer then makes the
+    # ordinary planned call)
+    OH2, OW2 = 100, 120
+    m2 = np.stack([rng.uniform(-0.4, W - 0.6, (OH2, OW2, K)),
+                   rng.uniform(-0.4, H - 0.6, (OH2, OW2, K))], -1).astype(np.float32)
+    capi.call("sdk_mapped_max_unpool_plan_build", _p(_t(m2)), _p(ws), n, H, W, OH2, OW2, K, 0, 0,
+              F32, _stream())
+    capi.call("sdk_mapped_max_unpool_plan_bands", _p(ws), n, H, W, F32, _stream(),
+              ctypes.cast(ctypes.byref(flag), ctypes.c_void_p))
+    assert flag.value == 0
+    g2 = rng.standard_normal((B, C, OH2, OW2)).astype(np.float32)
+    _, idx2 = ops.mapped_max_pool(_t(x), _t(m2), None, K, 0)
+    got = ops.mapped_max_unpool(_t(g2), idx2, _t(m2), None, H, W, K, 0)
+    assert relerr(_n(got), oracle.mapped_max_unpool(g2, _n(idx2), m2, H, W, K, 0)) <= 1e-4
+    # and through the operator layer on the first map (the band variant is what it calls)
+    for which, ref_idx in ((idx, _n(idx)), (bad, ref_bad), (idx, _n(idx))):
+        got = ops.mapped_max_unpool(tg, which, tm, None, H, W, K, 0)
+        assert relerr(_n(got), oracle.mapped_max_unpool(g, ref_idx, m, H, W, K, 0)) <= 1e-4
