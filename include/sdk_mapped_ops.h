@@ -346,7 +346,7 @@ int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same arguments and results as sdk_mapped_max_unpool without the workspace pair:
  * the scratch (256 + 32 bytes per 2048-pixel tile of the input plane for the tile windows,
- * 32 KB for the row-band table behind them) is a 295 168-byte array inside the library, one
+ * 48 KB for the row-band table behind them) is a 311 552-byte array inside the library, one
  * copy per GPU, held until the process ends.  The
  * call allocates and frees nothing.  Limit: the input plane may have at most
  * SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES tiles, ceil(width / TW) * ceil(height / (2048 / TW))

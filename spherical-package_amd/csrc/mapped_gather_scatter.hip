@@ -1324,7 +1324,8 @@ template <typename T>
 static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, int interp);
 template <typename T>
 static int build_unpool_windows(const T* map, void* workspace, size_t workspace_bytes, int H, int W,
-                                int OH, int OW, int K, int P, int interp, hipStream_t stream);
+                                int OH, int OW, int K, int P, int interp, hipStream_t stream,
+                                unsigned* seen = nullptr);
 
 // Average unpooling (group = K > 1 samples per pooled pixel, pooled rows of OW pixels) can run
 // tiled over the image when the workspace has room for the tile windows behind the lists.
@@ -1357,8 +1358,11 @@ static int build_inverse_lists(const T* map, const T* wts, void* workspace, size
     flags = reinterpret_cast<int*>(ws + lists_bytes);
     const UnpoolTiling ut = unpool_tiling(H, W);
     const size_t region = workspace_bytes - lists_bytes;
-    const int rc = build_unpool_windows<T>(map, ws + lists_bytes, region, H, W, MP / group / OW,
-                                           OW, group, P, interp, stream);
+    // the lists' counters, not yet in use, lend themselves to the band table's build
+    int rc = zero_fill(ws + off[1], off[2] - off[1], stream);
+    if (rc != SDK_OK) return rc;
+    rc = build_unpool_windows<T>(map, ws + lists_bytes, region, H, W, MP / group / OW, OW, group,
+                                 P, interp, stream, reinterpret_cast<unsigned*>(cnt));
     if (rc != SDK_OK) return rc;
     const int* bands = nullptr;
     if (region >= unpool_layout_with_bands(ut) &&
@@ -1644,9 +1648,11 @@ static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, in
 // (unpool_layout bytes), gate word cleared; with workspace_bytes >= unpool_layout_with_bands
 // the band table as well; where its verdict is 1 every call on this map runs the band kernels
 // and the window kernels return at once.
+// seen: scratch for the band table's build (unpool_band_build), or nullptr.
 template <typename T>
 static int build_unpool_windows(const T* map, void* workspace, size_t workspace_bytes, int H, int W,
-                                int OH, int OW, int K, int P, int interp, hipStream_t stream) {
+                                int OH, int OW, int K, int P, int interp, hipStream_t stream,
+                                unsigned* seen) {
   const UnpoolTiling ut = unpool_tiling(H, W);
   char* ws = static_cast<char*>(workspace);
   int* win = reinterpret_cast<int*>(ws + 256);
@@ -1656,7 +1662,7 @@ static int build_unpool_windows(const T* map, void* workspace, size_t workspace_
   const int* skip = nullptr;
   if (with_table && unpool_bands_possible<T>(H, W, OH, OW, K, P, interp)) {
     int* table = reinterpret_cast<int*>(ws + unpool_layout(ut));
-    unpool_band_build((const float*)map, table, H, W, OH, OW, K, stream);
+    unpool_band_build((const float*)map, table, H, W, OH, OW, K, stream, seen);
     SDK_LAUNCH_CHECK("mapped_max_unpool(band table)");
     skip = table;
   }
@@ -1809,9 +1815,9 @@ using namespace sdk;
 // that pointer is what the fill kernel and the unpool kernels receive.
 // ---------------------------------------------------------------------------
 static constexpr int kStaticUnpoolTiles = SDK_MAPPED_MAX_UNPOOL_STATIC_MAX_TILES;   // of 2048 pixels
-// tile windows, then 32 KB for the row-band table (planes of up to 4000 rows of bands)
+// tile windows, then 48 KB for the row-band table (planes of up to 4000 rows of bands)
 static constexpr size_t kStaticUnpoolBytes = 256 + (size_t)kStaticUnpoolTiles * 8 * sizeof(int) +
-                                             32768;
+                                             49152;
 static __device__ __align__(256) unsigned char scratch[kStaticUnpoolBytes];
 
 static constexpr int kMaxDevices = 64;

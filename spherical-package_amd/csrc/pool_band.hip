@@ -277,19 +277,25 @@ bool dispatch_ipt(int ipt, const float* in, const float* map, float* out, int64_
 // one index read, one gradient read, a select by the winning sample and one LDS add.
 //
 // table: [0] 1 when every band's range fits (kUbIpt * 256 pooled pixels), else 0 (the caller
-// then takes its other route); [8 + 2b] last pooled row of band b + 1 (0: nothing reaches
-// it); [9 + 2b] kUbBig - first pooled row.  Both grow by atomicMax from a zero fill.
+// then takes its other route); [3] 1 when the build looked for pooled pixels that have the
+// same sample k at the same image pixel; [8 + 2b] last pooled row of band b + 1 (0: nothing
+// reaches it); [9 + 2b] kUbBig - first pooled row; [8 + 2 nbands + b] raised when two such
+// pooled pixels meet in band b (where [3] is set and this is 0, average unpooling adds
+// band b sample by sample without atomics).  All grow by atomicMax from a zero fill.
 // ---------------------------------------------------------------------------
-constexpr int kUbIpt = 8;
+constexpr int kUbWindowPixels = 2048;   // pooled pixels a band's range may hold
 constexpr int kUbLdsBytes = 32 * 1024;
 constexpr int kUbLdsFloats = kUbLdsBytes / 4;
 constexpr int kUbBig = 1 << 30;
 constexpr unsigned kUbNone = 0xFFFFu;
 
+// seen: nullptr, or one zeroed word per image pixel; bit k is set by the first pooled pixel
+// whose sample k lands there, and a second one marks the band.
 __global__ __launch_bounds__(kBandBlock) void unpool_band_rows_kernel(
-    const float* __restrict__ map, int M, int OW, int K, int H, int W, int RB,
-    int* __restrict__ table) {
+    const float* __restrict__ map, int M, int OW, int K, int H, int W, int RB, int nbands,
+    int* __restrict__ table, unsigned* __restrict__ seen) {
   const int pix = blockIdx.x * kBandBlock + threadIdx.x;
+  if (pix == 0) table[3] = seen != nullptr ? 1 : 0;
   if (pix >= M) return;
   const int r = pix / OW;
   const float2* coords = reinterpret_cast<const float2*>(map) + (size_t)pix * K;
@@ -301,6 +307,11 @@ __global__ __launch_bounds__(kBandBlock) void unpool_band_rows_kernel(
     if (tp.off[0] >= 0) {
       bmin = min(bmin, tp.ty[0] / RB);
       bmax = max(bmax, tp.ty[0] / RB);
+      if (seen != nullptr) {
+        const unsigned bit = 1u << k;
+        if (atomicOr(seen + tp.off[0], bit) & bit)
+          atomicMax(&table[8 + 2 * nbands + tp.ty[0] / RB], 1);
+      }
     }
   }
   // every band between the first and the last one touched (a superset does no harm: a pooled
@@ -321,7 +332,7 @@ __global__ __launch_bounds__(kBandBlock) void unpool_band_verdict_kernel(int* __
     const int hi1 = table[8 + 2 * b];
     if (hi1 > 0) {
       const int lo = kUbBig - table[9 + 2 * b];
-      if ((int64_t)(hi1 - lo) * OW > (int64_t)kUbIpt * kBandBlock) bad = 1;
+      if ((int64_t)(hi1 - lo) * OW > kUbWindowPixels) bad = 1;
     }
   }
   __syncthreads();
@@ -375,14 +386,25 @@ __device__ __forceinline__ unsigned packed_tap(const unsigned (&offp)[(K + 1) / 
 // of an 8 x 64 x 128 x 256 gradient), one after the other (issued as a batch, with the taps
 // outside the band masked or sent to a spare word, they were slower).  Max unpooling keeps the two planes apart (their
 // winners differ); average unpooling interleaves them, (plane 0, plane 1) per band element,
-// and adds both with one 64-bit swap per tap.
+// and adds both with one 64-bit swap per tap.  In a band where the table says that sample k of
+// different pooled pixels never shares an image pixel, average unpooling needs no atomics at
+// all: the samples are added one k at a time, a barrier between them, every lane reading,
+// adding to and writing back elements no other lane touches in that round, with all of a
+// thread's reads of a round in flight together; the sums then come in a fixed order.
 template <bool AVG, int K>
-__global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
+__global__ __launch_bounds__(AVG ? 512 : 256, AVG ? 2 : 3) void unpool_band_kernel(
     const float* __restrict__ gout, const int64_t* __restrict__ idx, const float* __restrict__ map,
     float* __restrict__ gin, const int* __restrict__ table, int* __restrict__ gate, int planes,
     int H, int W, int OW, int M, int RB, int nbands, int chunks, int map_elems, int aligned) {
   if (table[0] == 0) return;
   constexpr int PG = 2;
+  // average unpooling: twice the threads with half the pooled pixels each (its sample-by-sample
+  // rounds hold a pixel's sums in registers beside its taps)
+  constexpr int BLK = AVG ? 512 : 256, IPT = kUbWindowPixels / BLK;
+  // average unpooling keeps the even columns of a band row in the row's first half and the odd
+  // ones in the second: the samples of a strided or dilated map land two columns apart, and
+  // a wave's adds would otherwise use half of the LDS banks
+  constexpr bool PERM = AVG;
   __shared__ __attribute__((aligned(16))) float acc[kUbLdsFloats];
   constexpr int KH = (K + 1) / 2;
   const int t = threadIdx.x;
@@ -401,13 +423,15 @@ __global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
   const int lo = hi1 > 0 ? kUbBig - table[9 + 2 * band] : 0;
   const int npw = hi1 > 0 ? (hi1 - lo) * OW : 0;   // pooled pixels that may reach the band
   const int pw0 = lo * OW;
+  const bool ordered = AVG && table[3] != 0 && table[8 + 2 * nbands + band] == 0;
 
-  unsigned offp[kUbIpt][KH];
+  const float2* map2 = reinterpret_cast<const float2*>(map);
+  unsigned offp[IPT][KH];
 #pragma unroll
-  for (int j = 0; j < kUbIpt; ++j) {
-    const int i = t + kBandBlock * j;
+  for (int j = 0; j < IPT; ++j) {
+    const int i = t + BLK * j;
     const int pix = pw0 + min(i, max(npw - 1, 0));
-    const float2* coords = reinterpret_cast<const float2*>(map) + (size_t)pix * K;
+    const float2* coords = map2 + (size_t)pix * K;
 #pragma unroll
     for (int h = 0; h < KH; ++h) {
       unsigned half[2];
@@ -420,26 +444,36 @@ __global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
           PointTaps<float, 0> tp;
           tp.set(c.x, c.y, H, W);
           const int ry = tp.ty[0] - y0;
+          const int col = PERM ? (tp.tx[0] >> 1) + (tp.tx[0] & 1) * (W >> 1) : tp.tx[0];
           if (i < npw && tp.off[0] >= 0 && (unsigned)ry < (unsigned)band_rows)
-            half[e] = (unsigned)(ry * W + tp.tx[0]);
+            half[e] = (unsigned)(ry * W + col);
         }
       }
       offp[j][h] = half[0] | (half[1] << 16);
     }
   }
   vec4* acc4 = reinterpret_cast<vec4*>(acc);
-  for (int v = t; v < PG * n_vec; v += kBandBlock) acc4[v] = vec4{0.f, 0.f, 0.f, 0.f};
+  for (int v = t; v < PG * n_vec; v += BLK) acc4[v] = vec4{0.f, 0.f, 0.f, 0.f};
   __syncthreads();
   // Stores the band sums of the planes q, q + 1 (the second only below p_end) and clears them.
   auto store_pass = [&](int q) {
-    for (int v = t; v < n_vec; v += kBandBlock) {
+    for (int v = t; v < n_vec; v += BLK) {
       vec4 a, b;
       if constexpr (AVG) {
-        const vec4 lo4 = acc4[2 * v], hi4 = acc4[2 * v + 1];   // (p0, p1) of four elements
-        acc4[2 * v] = vec4{0.f, 0.f, 0.f, 0.f};
-        acc4[2 * v + 1] = vec4{0.f, 0.f, 0.f, 0.f};
-        a = vec4{lo4[0], lo4[2], hi4[0], hi4[2]} / float(K);
-        b = vec4{lo4[1], lo4[3], hi4[1], hi4[3]} / float(K);
+        // (p0, p1) of two columns each: c, c + 1 and c + 2, c + 3, or with PERM c, c + 2 and
+        // c + 1, c + 3
+        const int ia = PERM ? (v / (W >> 2)) * (W >> 1) + v % (W >> 2) : 2 * v;
+        const int ib = PERM ? ia + (W >> 2) : 2 * v + 1;
+        const vec4 lo4 = acc4[ia], hi4 = acc4[ib];
+        acc4[ia] = vec4{0.f, 0.f, 0.f, 0.f};
+        acc4[ib] = vec4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (PERM) {
+          a = vec4{lo4[0], hi4[0], lo4[2], hi4[2]} / float(K);
+          b = vec4{lo4[1], hi4[1], lo4[3], hi4[3]} / float(K);
+        } else {
+          a = vec4{lo4[0], lo4[2], hi4[0], hi4[2]} / float(K);
+          b = vec4{lo4[1], lo4[3], hi4[1], hi4[3]} / float(K);
+        }
       } else {
         a = acc4[v];
         b = acc4[n_vec + v];
@@ -455,11 +489,11 @@ __global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
   for (int p = p_begin; p < p_end; p += PG) {
     // this pass's indices and gradients are requested first; the previous pass is stored
     // while they are on their way
-    int64_t sv[kUbIpt][PG];
-    float gv[kUbIpt][PG];
+    int64_t sv[IPT][PG];
+    float gv[IPT][PG];
 #pragma unroll
-    for (int j = 0; j < kUbIpt; ++j) {
-      const int i = t + kBandBlock * j;
+    for (int j = 0; j < IPT; ++j) {
+      const int i = t + BLK * j;
       const size_t at = (size_t)pw0 + min(i, max(npw - 1, 0));
 #pragma unroll
       for (int g = 0; g < PG; ++g) {
@@ -473,36 +507,56 @@ __global__ __launch_bounds__(kBandBlock, AVG ? 4 : 3) void unpool_band_kernel(
       __syncthreads();
     }
     const bool two = p + 1 < p_end;
+    if (AVG && ordered) {
+      float2* acc2 = reinterpret_cast<float2*>(acc);
 #pragma unroll
-    for (int j = 0; j < kUbIpt; ++j) {
-      const int i = t + kBandBlock * j;
-      if (i >= npw) continue;
-      if constexpr (AVG) {
-        float2* acc2 = reinterpret_cast<float2*>(acc);
-        const float gb = two ? gv[j][1] : 0.0f;
+      for (int k = 0; k < K; ++k) {
+        unsigned o[IPT];
+        float2 cur[IPT];
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-          const unsigned o16 = (offp[j][k >> 1] >> ((k & 1) * 16)) & 0xFFFFu;
-          if (o16 != kUbNone) lds_add_f32x2(acc2 + o16, gv[j][0], gb);
+        for (int j = 0; j < IPT; ++j) {
+          o[j] = (offp[j][k >> 1] >> ((k & 1) * 16)) & 0xFFFFu;   // kUbNone for i >= npw too
+          cur[j] = float2{0.0f, 0.0f};
+          if (o[j] != kUbNone) cur[j] = acc2[o[j]];
         }
-      } else {
-        const int first = (pw0 + i) * K * 2;   // map element of the pixel's first sample
 #pragma unroll
-        for (int g = 0; g < PG; ++g) {
-          if (g == 1 && !two) continue;
-          const int64_t s64 = sv[j][g];
-          const bool live = s64 >= 0 && s64 + 2 <= (int64_t)map_elems;   // others add nothing
-          const int d = (int)s64 - first;
-          const bool mine = d >= 0 && d < 2 * K && (d & 1) == 0;
-          stray |= live && !mine;
-          if (live && mine) {
-            const unsigned o16 = packed_tap<K>(offp[j], d >> 1);
-            if (o16 != kUbNone) lds_add_f32(acc + g * band_elems + o16, gv[j][g]);
+        for (int j = 0; j < IPT; ++j)
+          if (o[j] != kUbNone)
+            acc2[o[j]] = float2{cur[j].x + gv[j][0], cur[j].y + (two ? gv[j][1] : 0.0f)};
+        __syncthreads();
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) {
+        const int i = t + BLK * j;
+        if (i >= npw) continue;
+        if constexpr (AVG) {
+          float2* acc2 = reinterpret_cast<float2*>(acc);
+          const float gb = two ? gv[j][1] : 0.0f;
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            const unsigned o16 = (offp[j][k >> 1] >> ((k & 1) * 16)) & 0xFFFFu;
+            if (o16 != kUbNone) lds_add_f32x2(acc2 + o16, gv[j][0], gb);
+          }
+        } else {
+          const int first = (pw0 + i) * K * 2;   // map element of the pixel's first sample
+#pragma unroll
+          for (int g = 0; g < PG; ++g) {
+            if (g == 1 && !two) continue;
+            const int64_t s64 = sv[j][g];
+            const bool live = s64 >= 0 && s64 + 2 <= (int64_t)map_elems;   // others add nothing
+            const int d = (int)s64 - first;
+            const bool mine = d >= 0 && d < 2 * K && (d & 1) == 0;
+            stray |= live && !mine;
+            if (live && mine) {
+              const unsigned o16 = packed_tap<K>(offp[j], d >> 1);
+              if (o16 != kUbNone) lds_add_f32(acc + g * band_elems + o16, gv[j][g]);
+            }
           }
         }
       }
+      __syncthreads();
     }
-    __syncthreads();
   }
   store_pass(p_begin + (p_end - p_begin - 1) / PG * PG);   // the last pass
   if (stray) atomicAdd(gate, 1);
@@ -552,15 +606,15 @@ bool unpool_band_shape(int H, int W, int OH, int OW, int K) {
 size_t unpool_band_table_bytes(int H, int W) {
   const int rb = unpool_band_rows_per_band(W);
   const int64_t nbands = rb > 0 ? ceil_div(H, rb) : 0;
-  return (size_t)(8 + 2 * nbands) * sizeof(int);   // the verdict word is there for every plane
+  return (size_t)(8 + 3 * nbands) * sizeof(int);   // the verdict word is there for every plane
 }
 
 void unpool_band_build(const float* map, int* table, int H, int W, int OH, int OW, int K,
-                       hipStream_t stream) {
+                       hipStream_t stream, unsigned* seen) {
   const int rb = unpool_band_rows_per_band(W);
   const int M = OH * OW;
   launch(unpool_band_rows_kernel, dim3((unsigned)ceil_div(M, kBandBlock)), dim3(kBandBlock), stream,
-         map, M, OW, K, H, W, rb, table);
+         map, M, OW, K, H, W, rb, (int)ceil_div(H, rb), table, seen);
   launch(unpool_band_verdict_kernel, dim3(1), dim3(kBandBlock), stream, table,
          (int)ceil_div(H, rb), OW);
 }
@@ -570,17 +624,17 @@ void unpool_band_launch(bool avg, const float* gout, const int64_t* idx, const f
                         int OH, int OW, int K, hipStream_t stream) {
   const int rb = unpool_band_rows_per_band(W);
   const int nbands = (int)ceil_div(H, rb);
-  // one round of resident workgroups (three per CU for max unpooling, whose registers allow
-  // no more, four for average unpooling; measured: 102 against 112 us and 107 against 115 us
-  // on an 8 x 64 x 256 x 512 image), chunks in eighths (one per XCD), at least two planes each
-  int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(planes / 2, (avg ? 1024 : 768) / nbands));
+  // one round of resident workgroups (three of 256 threads per CU for max unpooling, two of
+  // 512 for average unpooling: as many as their registers allow), chunks in eighths (one per
+  // XCD), at least two planes each
+  int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(planes / 2, (avg ? 512 : 768) / nbands));
   chunks = std::max(8, chunks / 8 * 8);
   chunks = (int)std::min<int64_t>(chunks, planes);
   const unsigned grid = 8u * (unsigned)nbands * (unsigned)ceil_div(chunks, 8);
   const int M = OH * OW;
-#define UB(AVGv, Kv)                                                                          \
-  launch(unpool_band_kernel<AVGv, Kv>, dim3(grid), dim3(kBandBlock), stream, gout, idx, map, \
-         gin, table, gate, (int)planes, H, W, OW, M, rb, nbands, chunks, M * K * 2,               \
+#define UB(AVGv, Kv)                                                                        \
+  launch(unpool_band_kernel<AVGv, Kv>, dim3(grid), dim3(AVGv ? 512 : 256), stream, gout, idx, \
+         map, gin, table, gate, (int)planes, H, W, OW, M, rb, nbands, chunks, M * K * 2,      \
          ((uintptr_t)gin & 15) == 0 ? 1 : 0)
   if (K == 9) {
     if (avg) UB(true, 9); else UB(false, 9);

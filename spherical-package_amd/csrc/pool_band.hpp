@@ -20,8 +20,11 @@ bool pool_band_launch(bool avg, const float* in, const float* map, float* out, i
 // caller's other route has to run (it stays 0 when unpool_band_build is never called).
 bool unpool_band_shape(int H, int W, int OH, int OW, int K);
 size_t unpool_band_table_bytes(int H, int W);
+// seen: nullptr, or scratch of one zeroed 32-bit word per image pixel (not needed afterwards):
+// the build then also finds out whether average unpooling may add sample by sample without
+// atomics (no two pooled pixels with the same sample at one image pixel).
 void unpool_band_build(const float* map, int* table, int H, int W, int OH, int OW, int K,
-                       hipStream_t stream);
+                       hipStream_t stream, unsigned* seen = nullptr);
 // avg: every sample of a pooled pixel receives grad_output / K (idx unused); else the sample the
 // index names receives grad_output.  gate: raised when an index names a sample of another
 // pooled pixel than its own (the caller then redoes the call with its atomic route).
