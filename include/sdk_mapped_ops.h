@@ -319,7 +319,10 @@ int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
  * Negative or out-of-range indices contribute nothing.
  *
  * `workspace` is optional device scratch of sdk_mapped_max_unpool_workspace_bytes()
- * bytes (it depends on the input plane and the element size only).  With it the
+ * bytes (it depends on the input plane only: 32 bytes per 2048 input pixels,
+ * 12 bytes per band of 32 KB of image rows and, while that stays below 32 MiB,
+ * 40 KB per band for the band's pooled pixels with their taps resolved;
+ * 1.3 MB for a 256 x 512 plane).  With it the
  * call works by pieces of the input plane, whole rows (float32, single nearest
  * taps, kernel_size 4 or 9, width a multiple of 4) or tiles: the pooled pixels
  * that can reach a piece are found from the map, their contributions are summed

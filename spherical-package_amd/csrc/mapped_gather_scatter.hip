@@ -1320,6 +1320,8 @@ static size_t inverse_layout(int64_t HW, size_t esz, size_t (&off)[4]) {
 static UnpoolTiling unpool_tiling(int H, int W);
 static size_t unpool_layout(const UnpoolTiling& ut);
 static size_t unpool_layout_with_bands(const UnpoolTiling& ut);
+static size_t unpool_layout_with_taps(const UnpoolTiling& ut);
+static unsigned* unpool_taps_at(void* region, size_t region_bytes, const UnpoolTiling& ut);
 template <typename T>
 static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, int interp);
 template <typename T>
@@ -1438,6 +1440,8 @@ static int launch_resample_to_map(const T* in, const T* map, const T* wts, T* ou
     if (bands != nullptr && planes > 0) {
       if constexpr (sizeof(T) == 4) {
         unpool_band_launch(true, (const float*)in, nullptr, (const float*)map, (float*)out, bands,
+                           unpool_taps_at(ws + lists_bytes, workspace_bytes - lists_bytes,
+                                          unpool_tiling(H, W)),
                            nullptr, planes, H, W, MP / group / OW, OW, group, stream);
         SDK_LAUNCH_CHECK("mapped_avg_unpool(bands)");
       }
@@ -1637,6 +1641,21 @@ static size_t unpool_layout_with_bands(const UnpoolTiling& ut) {
   return unpool_layout(ut) + unpool_band_table_bytes(ut.H, ut.W);
 }
 
+// ... and, where they fit (unpool_band_taps_bytes), by the bands' packed taps, 256-byte aligned.
+static size_t unpool_layout_with_taps(const UnpoolTiling& ut) {
+  const size_t t = unpool_band_taps_bytes(ut.H, ut.W);
+  const size_t base = unpool_layout_with_bands(ut);
+  return t != 0 ? ((base + 255) & ~(size_t)255) + t : base;
+}
+
+// The packed taps inside a region laid out as above, nullptr where it has no room for them.
+static unsigned* unpool_taps_at(void* region, size_t region_bytes, const UnpoolTiling& ut) {
+  if (unpool_band_taps_bytes(ut.H, ut.W) == 0 || region_bytes < unpool_layout_with_taps(ut))
+    return nullptr;
+  return reinterpret_cast<unsigned*>(static_cast<char*>(region) +
+                                     ((unpool_layout_with_bands(ut) + 255) & ~(size_t)255));
+}
+
 // Whether the row-band kernels take this element type, interpolation and shape at all.
 template <typename T>
 static bool unpool_bands_possible(int H, int W, int OH, int OW, int K, int P, int interp) {
@@ -1662,7 +1681,9 @@ static int build_unpool_windows(const T* map, void* workspace, size_t workspace_
   const int* skip = nullptr;
   if (with_table && unpool_bands_possible<T>(H, W, OH, OW, K, P, interp)) {
     int* table = reinterpret_cast<int*>(ws + unpool_layout(ut));
-    unpool_band_build((const float*)map, table, H, W, OH, OW, K, stream, seen);
+    // (average unpooling is the caller that lends `seen`; its taps are laid out for it)
+    unpool_band_build((const float*)map, table, H, W, OH, OW, K, stream, seen,
+                      unpool_taps_at(workspace, workspace_bytes, ut), seen != nullptr);
     SDK_LAUNCH_CHECK("mapped_max_unpool(band table)");
     skip = table;
   }
@@ -1719,7 +1740,8 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
         if (bands == nullptr)
           return fail(SDK_ERR_INVALID_ARGUMENT, "mapped_max_unpool_planned_bands: no band table for this shape");
         unpool_band_launch(false, (const float*)gout, indices, (const float*)map, (float*)gin,
-                           bands, g, planes, H, W, OH, OW, K, stream);
+                           bands, unpool_taps_at(workspace, workspace_bytes, ut), g, planes, H,
+                           W, OH, OW, K, stream);
         SDK_LAUNCH_CHECK("mapped_max_unpool(bands)");
         const int64_t blocks = std::min<int64_t>(ceil_div((int64_t)total, kBlock), 4096);
         SDK_DISPATCH_INTERP(interp, P,
@@ -1743,7 +1765,8 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
     if (bands != nullptr) {
       if constexpr (sizeof(T) == 4) {
         unpool_band_launch(false, (const float*)gout, indices, (const float*)map, (float*)gin,
-                           bands, g, planes, H, W, OH, OW, K, stream);
+                           bands, unpool_taps_at(workspace, workspace_bytes, ut), g, planes, H,
+                           W, OH, OW, K, stream);
         SDK_LAUNCH_CHECK("mapped_max_unpool(bands)");
       }
     }
@@ -1882,7 +1905,7 @@ size_t sdk_resample_to_map_workspace_bytes(int64_t height, int64_t width, int32_
   size_t off[4];
   // the inverse lists, then the tile windows of the tiled average unpooling
   return inverse_layout(height * width, dtype == SDK_F64 ? 8 : 4, off) +
-         unpool_layout_with_bands(unpool_tiling((int)height, (int)width));
+         unpool_layout_with_taps(unpool_tiling((int)height, (int)width));
 }
 
 static int resample_to_map_entry(const void* input, const void* sample_map,
@@ -2154,7 +2177,7 @@ int sdk_mapped_avg_unpool(const void* grad_output, const void* sample_map,
 size_t sdk_mapped_max_unpool_workspace_bytes(int64_t height, int64_t width, int32_t dtype) {
   if (height < 1 || width < 1 || height * width >= ((int64_t)1 << 31)) return 0;
   (void)dtype;
-  return unpool_layout_with_bands(unpool_tiling((int)height, (int)width));
+  return unpool_layout_with_taps(unpool_tiling((int)height, (int)width));
 }
 
 int sdk_mapped_max_unpool(const void* grad_output, const int64_t* indices, const void* sample_map,

@@ -278,7 +278,7 @@ bool dispatch_ipt(int ipt, const float* in, const float* map, float* out, int64_
 //
 // table: [0] 1 when every band's range fits (kUbIpt * 256 pooled pixels), else 0 (the caller
 // then takes its other route); [3] 1 when the build looked for pooled pixels that have the
-// same sample k at the same image pixel; [8 + 2b] last pooled row of band b + 1 (0: nothing
+// same sample k at the same image pixel; [4] 1 when the packed taps behind the table are there; [8 + 2b] last pooled row of band b + 1 (0: nothing
 // reaches it); [9 + 2b] kUbBig - first pooled row; [8 + 2 nbands + b] raised when two such
 // pooled pixels meet in band b (where [3] is set and this is 0, average unpooling adds
 // band b sample by sample without atomics).  All grow by atomicMax from a zero fill.
@@ -339,6 +339,56 @@ __global__ __launch_bounds__(kBandBlock) void unpool_band_verdict_kernel(int* __
   if (threadIdx.x == 0) table[0] = bad ? 0 : 1;
 }
 
+constexpr int kUbTapWords = 5;   // packed taps of a pooled pixel, K <= 9 (two to a word)
+
+// Word h of a pooled pixel's packed taps: the positions inside the band (rows y0 .. y0 +
+// band_rows - 1) of its samples 2h and 2h + 1, kUbNone for a sample outside the band or the
+// image and where !on.  perm: the even columns of a band row in the row's first half, the odd
+// ones in the second (average unpooling: the samples of a strided or dilated map land two
+// columns apart, and a wave's adds would otherwise use half of the LDS banks).
+__device__ __forceinline__ unsigned packed_tap_word(const float2* coords, int h, int K, int H,
+                                                    int W, int y0, int band_rows, bool on,
+                                                    bool perm) {
+  unsigned half[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int k = 2 * h + e;
+    half[e] = kUbNone;
+    if (k < K) {
+      const float2 c = coords[k];
+      PointTaps<float, 0> tp;
+      tp.set(c.x, c.y, H, W);
+      const int ry = tp.ty[0] - y0;
+      const int col = perm ? (tp.tx[0] >> 1) + (tp.tx[0] & 1) * (W >> 1) : tp.tx[0];
+      if (on && tp.off[0] >= 0 && (unsigned)ry < (unsigned)band_rows)
+        half[e] = (unsigned)(ry * W + col);
+    }
+  }
+  return half[0] | (half[1] << 16);
+}
+
+// The packed taps of every band's pooled pixels, worked out once per map: taps[(band *
+// kUbTapWords + h) * kUbWindowPixels + i] for pooled pixel i of the band's range.  grid =
+// (kUbWindowPixels / 256, nbands).  Sets table[4] (read by the band kernel) when it has run.
+__global__ __launch_bounds__(kBandBlock) void unpool_band_taps_kernel(
+    const float* __restrict__ map, int* __restrict__ table, unsigned* __restrict__ taps, int K,
+    int H, int W, int OW, int RB, int perm) {
+  if (table[0] == 0) return;
+  const int band = blockIdx.y;
+  const int i = blockIdx.x * kBandBlock + threadIdx.x;
+  if (band == 0 && i == 0) table[4] = 1;
+  const int y0 = band * RB;
+  const int band_rows = min(RB, H - y0);
+  const int hi1 = table[8 + 2 * band];
+  const int lo = hi1 > 0 ? kUbBig - table[9 + 2 * band] : 0;
+  const int npw = hi1 > 0 ? (hi1 - lo) * OW : 0;
+  const int pix = lo * OW + min(i, max(npw - 1, 0));
+  const float2* coords = reinterpret_cast<const float2*>(map) + (size_t)pix * K;
+  for (int h = 0; h < (K + 1) / 2; ++h)
+    taps[((size_t)band * kUbTapWords + h) * kUbWindowPixels + i] =
+        packed_tap_word(coords, h, K, H, W, y0, band_rows, i < npw, perm != 0);
+}
+
 // One 64-bit compare-and-swap loop that adds (a, b) to an aligned pair of floats in LDS.
 __device__ __forceinline__ void lds_add_f32x2(float2* addr, float a, float b) {
   unsigned long long* ip = reinterpret_cast<unsigned long long*>(addr);
@@ -394,17 +444,15 @@ __device__ __forceinline__ unsigned packed_tap(const unsigned (&offp)[(K + 1) / 
 template <bool AVG, int K>
 __global__ __launch_bounds__(AVG ? 512 : 256, AVG ? 2 : 3) void unpool_band_kernel(
     const float* __restrict__ gout, const int64_t* __restrict__ idx, const float* __restrict__ map,
-    float* __restrict__ gin, const int* __restrict__ table, int* __restrict__ gate, int planes,
-    int H, int W, int OW, int M, int RB, int nbands, int chunks, int map_elems, int aligned) {
+    float* __restrict__ gin, const int* __restrict__ table, const unsigned* __restrict__ taps,
+    int* __restrict__ gate, int planes, int H, int W, int OW, int M, int RB, int nbands,
+    int chunks, int map_elems, int aligned) {
   if (table[0] == 0) return;
   constexpr int PG = 2;
   // average unpooling: twice the threads with half the pooled pixels each (its sample-by-sample
   // rounds hold a pixel's sums in registers beside its taps)
   constexpr int BLK = AVG ? 512 : 256, IPT = kUbWindowPixels / BLK;
-  // average unpooling keeps the even columns of a band row in the row's first half and the odd
-  // ones in the second: the samples of a strided or dilated map land two columns apart, and
-  // a wave's adds would otherwise use half of the LDS banks
-  constexpr bool PERM = AVG;
+  constexpr bool PERM = AVG;   // packed_tap_word
   __shared__ __attribute__((aligned(16))) float acc[kUbLdsFloats];
   constexpr int KH = (K + 1) / 2;
   const int t = threadIdx.x;
@@ -425,31 +473,25 @@ __global__ __launch_bounds__(AVG ? 512 : 256, AVG ? 2 : 3) void unpool_band_kern
   const int pw0 = lo * OW;
   const bool ordered = AVG && table[3] != 0 && table[8 + 2 * nbands + band] == 0;
 
-  const float2* map2 = reinterpret_cast<const float2*>(map);
+  // the packed taps of the thread's pooled pixels: from the plan where it holds them (one
+  // read of neighbouring words per word), else worked out here from the map
   unsigned offp[IPT][KH];
+  if (taps != nullptr && table[4] != 0) {
+    const unsigned* mine = taps + (size_t)band * kUbTapWords * kUbWindowPixels;
 #pragma unroll
-  for (int j = 0; j < IPT; ++j) {
-    const int i = t + BLK * j;
-    const int pix = pw0 + min(i, max(npw - 1, 0));
-    const float2* coords = map2 + (size_t)pix * K;
+    for (int j = 0; j < IPT; ++j)
 #pragma unroll
-    for (int h = 0; h < KH; ++h) {
-      unsigned half[2];
+      for (int h = 0; h < KH; ++h) offp[j][h] = mine[h * kUbWindowPixels + t + BLK * j];
+  } else {
+    const float2* map2 = reinterpret_cast<const float2*>(map);
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int k = 2 * h + e;
-        half[e] = kUbNone;
-        if (k < K) {
-          const float2 c = coords[k];
-          PointTaps<float, 0> tp;
-          tp.set(c.x, c.y, H, W);
-          const int ry = tp.ty[0] - y0;
-          const int col = PERM ? (tp.tx[0] >> 1) + (tp.tx[0] & 1) * (W >> 1) : tp.tx[0];
-          if (i < npw && tp.off[0] >= 0 && (unsigned)ry < (unsigned)band_rows)
-            half[e] = (unsigned)(ry * W + col);
-        }
-      }
-      offp[j][h] = half[0] | (half[1] << 16);
+    for (int j = 0; j < IPT; ++j) {
+      const int i = t + BLK * j;
+      const int pix = pw0 + min(i, max(npw - 1, 0));
+#pragma unroll
+      for (int h = 0; h < KH; ++h)
+        offp[j][h] = packed_tap_word(map2 + (size_t)pix * K, h, K, H, W, y0, band_rows, i < npw,
+                                     PERM);
     }
   }
   vec4* acc4 = reinterpret_cast<vec4*>(acc);
@@ -603,6 +645,13 @@ bool unpool_band_shape(int H, int W, int OH, int OW, int K) {
          (int64_t)OH * OW * K * 2 < ((int64_t)1 << 31);
 }
 
+size_t unpool_band_taps_bytes(int H, int W) {
+  const int rb = unpool_band_rows_per_band(W);
+  const int64_t nbands = rb > 0 ? ceil_div(H, rb) : 0;
+  const int64_t bytes = nbands * kUbTapWords * kUbWindowPixels * (int64_t)sizeof(unsigned);
+  return bytes <= ((int64_t)32 << 20) ? (size_t)bytes : 0;
+}
+
 size_t unpool_band_table_bytes(int H, int W) {
   const int rb = unpool_band_rows_per_band(W);
   const int64_t nbands = rb > 0 ? ceil_div(H, rb) : 0;
@@ -610,18 +659,21 @@ size_t unpool_band_table_bytes(int H, int W) {
 }
 
 void unpool_band_build(const float* map, int* table, int H, int W, int OH, int OW, int K,
-                       hipStream_t stream, unsigned* seen) {
+                       hipStream_t stream, unsigned* seen, unsigned* taps, bool perm) {
   const int rb = unpool_band_rows_per_band(W);
   const int M = OH * OW;
   launch(unpool_band_rows_kernel, dim3((unsigned)ceil_div(M, kBandBlock)), dim3(kBandBlock), stream,
          map, M, OW, K, H, W, rb, (int)ceil_div(H, rb), table, seen);
   launch(unpool_band_verdict_kernel, dim3(1), dim3(kBandBlock), stream, table,
          (int)ceil_div(H, rb), OW);
+  if (taps != nullptr)
+    launch(unpool_band_taps_kernel, dim3(kUbWindowPixels / kBandBlock, (unsigned)ceil_div(H, rb)),
+           dim3(kBandBlock), stream, map, table, taps, K, H, W, OW, rb, perm ? 1 : 0);
 }
 
 void unpool_band_launch(bool avg, const float* gout, const int64_t* idx, const float* map,
-                        float* gin, const int* table, int* gate, int64_t planes, int H, int W,
-                        int OH, int OW, int K, hipStream_t stream) {
+                        float* gin, const int* table, const unsigned* taps, int* gate,
+                        int64_t planes, int H, int W, int OH, int OW, int K, hipStream_t stream) {
   const int rb = unpool_band_rows_per_band(W);
   const int nbands = (int)ceil_div(H, rb);
   // one round of resident workgroups (three of 256 threads per CU for max unpooling, two of
@@ -634,7 +686,7 @@ void unpool_band_launch(bool avg, const float* gout, const int64_t* idx, const f
   const int M = OH * OW;
 #define UB(AVGv, Kv)                                                                        \
   launch(unpool_band_kernel<AVGv, Kv>, dim3(grid), dim3(AVGv ? 512 : 256), stream, gout, idx, \
-         map, gin, table, gate, (int)planes, H, W, OW, M, rb, nbands, chunks, M * K * 2,      \
+         map, gin, table, taps, gate, (int)planes, H, W, OW, M, rb, nbands, chunks, M * K * 2, \
          ((uintptr_t)gin & 15) == 0 ? 1 : 0)
   if (K == 9) {
     if (avg) UB(true, 9); else UB(false, 9);
