@@ -7,6 +7,7 @@
 #include <mutex>
 
 #include "conv_fused.hpp"
+#include "conv_small.hpp"
 #include "conv_internal.hpp"
 #include "sdk_host.hpp"
 
@@ -356,13 +357,27 @@ static int impl_mapped_conv_backward(const void* grad_output, const void* sample
              (int)kernel_size, num_interp_pts, interp, (int)out_width};
   rc = check_plan(what, g, dtype, compute, plan);
   if (rc) return rc;
-  hipEvent_t joined = nullptr;
-  rc = fork_side((hipStream_t)stream, &joined, side_worth(batch, out_channels, M, dtype),
-                 [&](hipStream_t s) {
-    return bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, s,
-                     s != (hipStream_t)stream);
-  });
   SharedPlan shared;   // the tap plan of the map is built once for both contractions
+  // A layer with at most four image channels runs three small kernels, each adding into a
+  // target that has to start from zero: the three targets are cleared by one launch.
+  if (dtype == SDK_F32 && compute != SDK_COMPUTE_UNFUSED && batch > 0 && fused_supported(g) &&
+      small_conv_supported(g) && small_wgrad_supported(g) &&
+      !side_worth(batch, out_channels, M, dtype)) {
+    rc = zero_fill3(grad_bias, sizeof(float) * (size_t)out_channels, grad_input,
+                    sizeof(float) * (size_t)batch * in_channels * height * width, grad_weight,
+                    sizeof(float) * (size_t)out_channels * in_channels * kernel_size,
+                    (hipStream_t)stream);
+    if (rc) return rc;
+    shared.cleared = true;
+    shared.bias_sum = static_cast<float*>(grad_bias);   // summed by the weight-gradient kernel
+  }
+  hipEvent_t joined = nullptr;
+  if (!shared.cleared)
+    rc = fork_side((hipStream_t)stream, &joined, side_worth(batch, out_channels, M, dtype),
+                   [&](hipStream_t s) {
+      return bias_grad(grad_output, grad_bias, batch, out_channels, M, dtype, s,
+                       s != (hipStream_t)stream);
+    });
   if (rc == SDK_OK)
     rc = run(what, GEMM_SCATTER, g, dtype, compute, grad_output, sample_map, interp_weights,
              weight, nullptr, grad_input, workspace, workspace_bytes, (hipStream_t)stream, &shared,

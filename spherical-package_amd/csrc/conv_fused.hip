@@ -1143,7 +1143,8 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
   int rc = SDK_OK;
   if (small_conv_supported(g)) {
     // images of a few channels: fill, then the packed scatter kernel
-    rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
+    if (!(shared != nullptr && shared->cleared && bias == nullptr))
+      rc = plane_fill<float>(img, bias, g.B * g.Cg, g.Cg, (size_t)g.H * g.W, stream);
     if (rc) return rc;
     if (shared != nullptr) shared->valid = false;
     return small_scatter(g, pix, map, wts, Wm, img, stream);
@@ -1280,10 +1281,12 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
                        const float* wts, const float* img, float* gW, float* workspace,
                        hipStream_t stream, const SharedPlan* shared, const CachedPlan* cached) {
   const bool bf16 = compute == SDK_COMPUTE_BF16;
-  int rc = zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
+  const bool cleared = shared != nullptr && shared->cleared && small_wgrad_supported(g);
+  int rc = cleared ? SDK_OK : zero_fill(gW, sizeof(float) * (size_t)g.Cp * g.Cg * g.K, stream);
   if (rc) return rc;
   if (g.B == 0) return SDK_OK;
-  if (small_wgrad_supported(g)) return small_wgrad(g, pix, map, wts, img, gW, stream);
+  if (small_wgrad_supported(g))
+    return small_wgrad(g, pix, map, wts, img, gW, stream, cleared ? shared->bias_sum : nullptr);
   if (planned_wgrad_supported(g)) {
     if (cached != nullptr)
       return wgrad_from_plan(g, matrix_mode(compute), cached->plan, pix, img, gW, workspace,

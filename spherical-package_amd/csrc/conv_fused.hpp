@@ -12,6 +12,12 @@ namespace sdk {
 struct SharedPlan {
   bool valid = false;
   Plan plan;
+  // The caller has cleared the scatter's image and the weight gradient already (the combined
+  // backward of a layer with at most four image channels, whose seven launches are its time).
+  bool cleared = false;
+  // ... and wants the bias gradient (the sum of the weight gradient's pixel-side operand over
+  // batch and pixels) from the weight-gradient kernel, into this cleared buffer.
+  float* bias_sum = nullptr;
 };
 
 // Everything the fused kernels derive from the sample map alone, built once into a

@@ -16,6 +16,9 @@ inline int matrix_mode(int compute) {
 }
 
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream);
+// Three buffers (sizes multiples of 4 bytes) cleared by one launch.
+int zero_fill3(void* a, size_t a_bytes, void* b, size_t b_bytes, void* c, size_t c_bytes,
+               hipStream_t stream);
 // grad_bias[c] = sum over batch and pixels (sdk_bias_grad).  beside_contractions: the variant
 // that uses no LDS, for a launch that runs concurrently with the contraction kernels.
 int bias_grad(const void* grad_output, void* grad_bias, int64_t batch, int64_t channels,

@@ -272,16 +272,18 @@ __global__ __launch_bounds__(kSmThreads) void small_scatter_kernel(
 // and image reads are in flight together) into an LDS tile, the pixel-side values are copied
 // beside it, and wave w multiplies pixels 16 w .. 16 w + 15.  The waves' accumulators (NB * CB
 // of 16 registers) are summed in LDS at the end and leave the workgroup as one float atomic per
-// element of gW.
+// element of gW.  gbias (optional): the bias gradient, the sum of the pixel-side rows the
+// kernel has in LDS anyway, one atomic per channel and workgroup (gbias must start from zero).
 constexpr int kSmTile = 64;       // pixels per tile
 constexpr int kSmLd = kSmTile + 1;   // row stride of the LDS tiles (floats): rows on distinct banks
 
 template <int INTERP, bool WEIGHTED, int NB, int CB>
 __global__ __launch_bounds__(kSmThreads) void small_wgrad_kernel(
     const float* __restrict__ pix, const float* __restrict__ img, const float* __restrict__ map,
-    const float* __restrict__ wts, float* __restrict__ gW, int Cg, int H, int W, int Cp, int M,
-    int K, int P) {
+    const float* __restrict__ wts, float* __restrict__ gW, float* __restrict__ gbias, int Cg,
+    int H, int W, int Cp, int M, int K, int P) {
   constexpr int COLS = 32 * CB, ROWS = 32 * NB;
+  float row_sum = 0.0f;   // thread n < ROWS: pixel-side row n over this workgroup's tiles
   constexpr int TILE_FLOATS = (COLS + ROWS) * kSmLd, SUM_FLOATS = ROWS * COLS;
   __shared__ float lds[TILE_FLOATS > SUM_FLOATS ? TILE_FLOATS : SUM_FLOATS];
   float* colT = lds;                  // [COLS][kSmLd]
@@ -332,6 +334,12 @@ __global__ __launch_bounds__(kSmThreads) void small_wgrad_kernel(
       }
     }
     __syncthreads();
+    if (gbias != nullptr && tid < ROWS) {
+      float s = 0.0f;
+#pragma unroll 8
+      for (int p = 0; p < kSmTile; ++p) s += pixT[tid * kSmLd + p];
+      row_sum += s;
+    }
     // ---- wave w: pixels 16 w + 2 s + h, s = 0..7
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -369,6 +377,7 @@ __global__ __launch_bounds__(kSmThreads) void small_wgrad_kernel(
     const int n = e / COLS, col = e - n * COLS;
     if (n < Cp && col < CK) atomic_add_noret(gW + (size_t)n * CK + col, sum[e]);
   }
+  if (gbias != nullptr && tid < Cp) atomic_add_noret(gbias + tid, row_sum);
 }
 
 }  // namespace
@@ -430,7 +439,7 @@ int small_scatter(const ConvGeom& g, const float* pix, const float* map, const f
 }
 
 int small_wgrad(const ConvGeom& g, const float* pix, const float* map, const float* wts,
-                const float* img, float* gW, hipStream_t stream) {
+                const float* img, float* gW, hipStream_t stream, float* gbias) {
   const int NB = (int)ceil_div(g.Cp, 32), CB = (int)ceil_div(g.Cg * g.K, 32);
   const int64_t tiles = ceil_div(g.M, kSmTile);
   // at most about two workgroups per CU over the whole grid: each ends with one atomic per
@@ -440,8 +449,8 @@ int small_wgrad(const ConvGeom& g, const float* pix, const float* map, const flo
 #define SW(NBv, CBv)                                                                            \
   SDK_DISPATCH_INTERP(g.interp, g.P,                                                            \
                       (launch((small_wgrad_kernel<INTERP, WEIGHTED, NBv, CBv>), grid,           \
-                              dim3(kSmThreads), stream, pix, img, map, wts, gW, g.Cg, g.H, g.W, \
-                              g.Cp, g.M, g.K, g.P)))
+                              dim3(kSmThreads), stream, pix, img, map, wts, gW, gbias, g.Cg,    \
+                              g.H, g.W, g.Cp, g.M, g.K, g.P)))
 #define SWN(CBv)                                                               \
   do {                                                                         \
     if (NB <= 1) SW(1, CBv); else if (NB == 2) SW(2, CBv); else SW(4, CBv);    \

@@ -18,7 +18,8 @@ int small_forward(const ConvGeom& g, const float* img, const float* map, const f
 int small_scatter(const ConvGeom& g, const float* pix, const float* map, const float* wts,
                   const float* Wm, float* img, hipStream_t stream);
 // gW += sum_b pix[b] x im2col(img[b])^T; gW must hold the values to add to (zeros).
+// gbias (optional, [Cp], zeros): receives the sum of pix over batch and pixels as well.
 int small_wgrad(const ConvGeom& g, const float* pix, const float* map, const float* wts,
-                const float* img, float* gW, hipStream_t stream);
+                const float* img, float* gW, hipStream_t stream, float* gbias = nullptr);
 
 }  // namespace sdk

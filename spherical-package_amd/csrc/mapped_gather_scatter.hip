@@ -58,6 +58,36 @@ __global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p, s
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) p[i] = z;
 }
 
+// Three buffers in one launch (the targets of a small layer's combined backward, where a launch
+// costs as much as the kernel it starts): 16-byte stores for the bulk of each, words for the rest.
+struct ZeroSeg {
+  unsigned* p;
+  size_t words;
+};
+__global__ __launch_bounds__(kBlock) void zero3_kernel(ZeroSeg s0, ZeroSeg s1, ZeroSeg s2) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const size_t first = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  const ZeroSeg segs[3] = {s0, s1, s2};
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const size_t n16 = (reinterpret_cast<uintptr_t>(segs[k].p) % 16 == 0) ? segs[k].words / 4 : 0;
+    uint4* p16 = reinterpret_cast<uint4*>(segs[k].p);
+    for (size_t i = first; i < n16; i += stride) p16[i] = make_uint4(0, 0, 0, 0);
+    for (size_t i = n16 * 4 + first; i < segs[k].words; i += stride) segs[k].p[i] = 0u;
+  }
+}
+
+int zero_fill3(void* a, size_t a_bytes, void* b, size_t b_bytes, void* c, size_t c_bytes,
+               hipStream_t stream) {
+  const size_t most = std::max(a_bytes, std::max(b_bytes, c_bytes));
+  if (most == 0) return SDK_OK;
+  const int blocks = (int)std::min<size_t>(ceil_div((int64_t)(most / 16 + 1), kBlock), 256 * 16);
+  launch(zero3_kernel, dim3(blocks), dim3(kBlock), stream, ZeroSeg{(unsigned*)a, a_bytes / 4},
+         ZeroSeg{(unsigned*)b, b_bytes / 4}, ZeroSeg{(unsigned*)c, c_bytes / 4});
+  SDK_LAUNCH_CHECK("zero_fill3");
+  return SDK_OK;
+}
+
 int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate);
 int zero_fill(void* ptr, size_t bytes, hipStream_t stream) {
   return zero_fill_gated(ptr, bytes, stream, nullptr);
