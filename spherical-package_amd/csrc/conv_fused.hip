@@ -27,6 +27,7 @@
 //   D, 16 registers v: D[i = 8*(v/4) + 4*(l/32) + v%4][j = l % 32]
 #include "conv_fused.hpp"
 #include "conv_small.hpp"
+#include "conv_product.hpp"
 #include "conv_plan.hpp"
 
 #include <hip/hip_runtime.h>
@@ -733,6 +734,7 @@ size_t fused_workspace_bytes(const ConvGeom& g) {
   if (gather_from_window(g)) need = std::max(need, gather_layout(g).total);
   if (plan_supported(g)) need = ((need + 255) & ~(size_t)255) + plan_bytes(g);
   if (scatter_tries_inverse(g)) need = std::max(need, inverse_ws_offset(g) + inverse_bytes(g));
+  need = std::max(need, product_workspace_bytes(g));
   // last: the weight gradient's tile lists and partial sums (the plan and, in a combined
   // backward call, everything before it are still in use when they are written)
   return ((need + 255) & ~(size_t)255) + wgrad_tail(g).total;
@@ -1149,6 +1151,13 @@ int fused_gemm_scatter(const ConvGeom& g, int compute, const float* pix, const f
     if (shared != nullptr) shared->valid = false;
     return small_scatter(g, pix, map, wts, Wm, img, stream);
   }
+  if (product_route(g)) {
+    // the image is finer than the pixel grid: products at the grid's resolution, then their
+    // splat as a gather (conv_product.hip)
+    if (shared != nullptr) shared->valid = false;
+    return product_gemm_scatter(g, pix, map, wts, Wm, bias, img, workspace, stream,
+                                cached != nullptr ? cached->col2im_lists : nullptr);
+  }
   const bool planned_fb = planned_scatter_supported(g);
   const int* generic_gate = nullptr;   // gate of the atomic scatter kernel at the end
   bool filled = false;
@@ -1331,8 +1340,8 @@ int fused_gather_wgrad(const ConvGeom& g, int compute, const float* pix, const f
 // ---------------------------------------------------------------------------
 namespace {
 struct CachedLayout {
-  size_t plan, lists, lists4, inverse, inverse_lists, total;
-  bool has_inverse;
+  size_t plan, lists, lists4, inverse, inverse_lists, col2im, total;
+  bool has_inverse, has_col2im;
 };
 CachedLayout cached_layout(const ConvGeom& g) {
   auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
@@ -1346,7 +1355,10 @@ CachedLayout cached_layout(const ConvGeom& g) {
                   plan_supported(inverse_geom(g)) &&
                   (int64_t)g.H * g.W * g.K < ((int64_t)1 << 31);
   l.inverse_lists = l.inverse + (l.has_inverse ? up(inverse_plan_bytes(g)) : 0);
-  l.total = l.inverse_lists + (l.has_inverse ? up(tile_lists_bytes(inverse_geom(g))) : 0);
+  l.col2im = l.inverse_lists + (l.has_inverse ? up(tile_lists_bytes(inverse_geom(g))) : 0);
+  // the inverted map of the product route (conv_product.hpp), where the map may take it
+  l.has_col2im = product_route_map(g);
+  l.total = l.col2im + (l.has_col2im ? up(col2im_lists_bytes(g.H, g.W, g.M, g.K, g.P, g.interp)) : 0);
   return l;
 }
 }  // namespace
@@ -1367,6 +1379,7 @@ void load_cached_plan(const ConvGeom& g, void* buffer, CachedPlan* out) {
     load_inverse_plan(g, b + l.inverse, &out->inverse);
     load_tile_lists(out->inverse.plan, b + l.inverse_lists, &out->inverse_lists);
   }
+  out->col2im_lists = l.has_col2im ? b + l.col2im : nullptr;
 }
 
 int build_cached_plan(const ConvGeom& g, const float* map, const float* wts, void* buffer,
@@ -1385,6 +1398,10 @@ int build_cached_plan(const ConvGeom& g, const float* map, const float* wts, voi
     if (rc) return rc;
     rc = build_tile_lists(cp.inverse.plan, b + l.inverse_lists, stream, &cp.inverse_lists, 0,
                           kProductCap);
+    if (rc) return rc;
+  }
+  if (l.has_col2im) {
+    rc = col2im_lists_build(map, wts, b + l.col2im, g.H, g.W, g.M, g.K, g.P, g.interp, stream);
     if (rc) return rc;
   }
   return SDK_OK;

@@ -29,6 +29,7 @@ struct CachedPlan {
   bool has_inverse = false;
   InversePlan inverse;
   TileLists inverse_lists;
+  const void* col2im_lists = nullptr;   // the inverted map of the product route, where kept
 };
 // g: only H, W, M, OW, K, P and interp matter.  0 bytes: no plan for this geometry.
 size_t cached_plan_bytes(const ConvGeom& g);

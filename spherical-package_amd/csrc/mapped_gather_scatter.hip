@@ -15,6 +15,7 @@
 #include <cfloat>
 #include <climits>
 
+#include "conv_product.hpp"
 #include "pool_band.hpp"
 #include "sdk_host.hpp"
 #include "sdk_taps.hpp"
@@ -1819,6 +1820,306 @@ static int launch_unpool(const T* gout, const int64_t* indices, const T* map, co
                               dim3(kBlock), stream, gout, indices, map, wts, gin, total, H, W,
                               (int)M, P, map_elems, gate)));
   SDK_LAUNCH_CHECK("mapped_max_unpool");
+  return SDK_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The splat of a convolution's column matrix (common/mapped_im2col.h:89-158) as a gather over
+// the inverted map, for conv_product.hip (declared in conv_product.hpp).  The map is inverted
+// into lists of exact length: per image element u the entries offset[u] .. offset[u + 1] - 1 of
+// (sample, coefficient), sample = m * K + k, sorted by sample, so
+// every element is written once, with its bias, as a sum in a fixed order; no list can
+// overflow.  count -> scan -> fill -> sort build them; they depend on the map alone.
+// ---------------------------------------------------------------------------
+namespace {
+
+// FILL = false: counts the taps of every image element; true: writes them at the slots the
+// scanned counts reserve.  Taps outside the image and taps with a zero coefficient are left
+// out (by both passes alike).
+template <int INTERP, bool WEIGHTED, bool FILL>
+__global__ __launch_bounds__(kBlock) void col2im_invert_kernel(
+    const float* __restrict__ map, const float* __restrict__ wts, int H, int W, int M, int K,
+    int P, int* __restrict__ counter, int* __restrict__ src, float* __restrict__ co) {
+  const int pix = blockIdx.x * kBlock + threadIdx.x;   // sample m * K + k
+  if (pix >= M * K) return;
+  const int q = WEIGHTED ? P : 1;
+  PointTaps<float, INTERP> t;
+  for (int p = 0; p < q; ++p) {
+    const size_t s = (size_t)pix * q + p;
+    t.set(map[s * 2], map[s * 2 + 1], H, W);
+    const float wt = WEIGHTED ? wts[s] : 1.0f;
+#pragma unroll
+    for (int i = 0; i < PointTaps<float, INTERP>::N; ++i) {
+      const float c = INTERP == 0 ? wt : t.w[i] * wt;
+      if (t.off[i] >= 0 && c != 0.0f) {
+        const int slot = atomicAdd(&counter[t.off[i]], 1);
+        if constexpr (FILL) {
+          src[slot] = pix;
+          co[slot] = c;
+        }
+      }
+    }
+  }
+}
+
+// Exclusive scan of n counters in three launches: per tile of 4096 counters (16 consecutive
+// ones per thread) the tile's sum; the sums scanned by one workgroup; every tile again, now
+// from its first slot.  offset[i] = cursor[i] = first slot of element i, offset[n] = all slots.
+constexpr int kScanPer = 16;
+constexpr int kScanTile = kBlock * kScanPer;
+
+// The block's exclusive scan of one value per thread; *total: the block's sum (every thread).
+__device__ __forceinline__ int block_exclusive_scan(int mine, int* total) {
+  __shared__ int wave_sum[kBlock / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = mine;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int below = __shfl_up(incl, d);
+    if (lane >= d) incl += below;
+  }
+  __syncthreads();   // (wave_sum may still be read from the previous call)
+  if (lane == 63) wave_sum[wave] = incl;
+  __syncthreads();
+  int before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < kBlock / 64; ++w) {
+    before += w < wave ? wave_sum[w] : 0;
+    all += wave_sum[w];
+  }
+  *total = all;
+  return before + incl - mine;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(const int* __restrict__ count,
+                                                                int n, int* __restrict__ sums) {
+  const int first = blockIdx.x * kScanTile + threadIdx.x * kScanPer;
+  int mine = 0;
+#pragma unroll
+  for (int i = 0; i < kScanPer; ++i) mine += first + i < n ? count[first + i] : 0;
+  int total;
+  block_exclusive_scan(mine, &total);
+  if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+// One workgroup: sums[0 .. tiles) -> their exclusive scan, in place.
+__global__ __launch_bounds__(kBlock) void scan_sums_kernel(int* __restrict__ sums, int tiles) {
+  int run = 0;
+  for (int base = 0; base < tiles; base += kBlock) {
+    const int i = base + threadIdx.x;
+    const int mine = i < tiles ? sums[i] : 0;
+    int total;
+    const int before = block_exclusive_scan(mine, &total);
+    if (i < tiles) sums[i] = run + before;
+    run += total;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(const int* __restrict__ count, int n,
+                                                            const int* __restrict__ sums,
+                                                            int* __restrict__ offset,
+                                                            int* __restrict__ cursor) {
+  const int first = blockIdx.x * kScanTile + threadIdx.x * kScanPer;
+  int c[kScanPer];
+  int mine = 0;
+#pragma unroll
+  for (int i = 0; i < kScanPer; ++i) {
+    c[i] = first + i < n ? count[first + i] : 0;
+    mine += c[i];
+  }
+  int total;
+  int run = sums[blockIdx.x] + block_exclusive_scan(mine, &total);
+#pragma unroll
+  for (int i = 0; i < kScanPer; ++i) {
+    if (first + i < n) {
+      offset[first + i] = run;
+      cursor[first + i] = run;
+    }
+    run += c[i];
+    if (first + i == n - 1) offset[n] = run;
+  }
+}
+
+// Every element's entries sorted by source, then coefficient (the fill appends in the order
+// its atomics are served); selection sort in place, the lists are short.
+__global__ __launch_bounds__(kBlock) void col2im_sort_kernel(const int* __restrict__ offset,
+                                                             int* __restrict__ src,
+                                                             float* __restrict__ co, int HW) {
+  const int u = blockIdx.x * kBlock + threadIdx.x;
+  if (u >= HW) return;
+  const int beg = offset[u], end = offset[u + 1];
+  for (int i = beg; i + 1 < end; ++i) {
+    int best = i, bs = src[i];
+    float bc = co[i];
+    const int first_s = bs;
+    const float first_c = bc;
+    for (int j = i + 1; j < end; ++j) {
+      const int sj = src[j];
+      const float cj = co[j];
+      if (sj < bs || (sj == bs && cj < bc)) {
+        best = j;
+        bs = sj;
+        bc = cj;
+      }
+    }
+    if (best != i) {
+      src[best] = first_s;
+      co[best] = first_c;
+      src[i] = bs;
+      co[i] = bc;
+    }
+  }
+}
+
+// col holds the products channels-last, col[b][sample][c]: a wave reads the Cg values of an
+// entry's sample as one run (lane = channel) and owns 16 consecutive image elements, whose
+// entries are one run of the lists: the lanes fetch that run together (lane l entry l), every
+// lane works out which of the 16 elements its entry belongs to, and the wave then walks the
+// entries in order, eight value reads in flight at a time, handing a finished element's sums
+// to an LDS tile from which the workgroup's 64 elements x 64 channels leave transposed, as
+// runs along the image.  grid (blocks of 64 image elements, batch).
+constexpr int kC2iTargets = 64;
+
+__global__ __launch_bounds__(kBlock) void col2im_gather_kernel(
+    const float* __restrict__ col, const int* __restrict__ offset, const int* __restrict__ src,
+    const float* __restrict__ co, const float* __restrict__ bias, float* __restrict__ img, int Cg,
+    int HW, size_t samples) {
+  __shared__ float tile[kC2iTargets * (kC2iTargets + 1)];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int u0 = blockIdx.x * kC2iTargets;
+  const float* col_b = col + (size_t)blockIdx.y * samples * Cg;
+  float* img_b = img + (size_t)blockIdx.y * Cg * HW;
+  // the 17 list boundaries of the wave's 16 elements (elements past the image: empty lists)
+  const int w_first = u0 + 16 * wave;
+  const int my_off = offset[min(w_first + min(lane, 16), HW)];
+  const int beg_w = __builtin_amdgcn_readlane(my_off, 0);
+  const int end_w = __builtin_amdgcn_readlane(my_off, 16);
+  for (int c0 = 0; c0 < Cg; c0 += 64) {
+    const int cc = min(c0 + lane, Cg - 1);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) tile[(16 * wave + t) * (kC2iTargets + 1) + lane] = 0.0f;
+    float acc = 0.0f;
+    int cur = -1;   // element (0..15) the sums belong to
+    for (int base = beg_w; base < end_w; base += 64) {
+      const int e = base + lane;
+      const bool on = e < end_w;
+      const int s_l = on ? src[e] : 0;
+      const float w_l = on ? co[e] : 0.0f;
+      int t_l = 0;   // boundaries 1..16 at or below e: the element of entry e
+#pragma unroll
+      for (int q = 1; q <= 16; ++q) t_l += __builtin_amdgcn_readlane(my_off, q) <= e ? 1 : 0;
+      const int n_here = min(64, end_w - base);   // (uniform)
+      for (int i0 = 0; i0 < n_here; i0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int s_i = __builtin_amdgcn_readlane(s_l, min(i0 + i, n_here - 1));
+          v[i] = col_b[(size_t)s_i * Cg + cc];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (i0 + i < n_here) {
+            const int t_i = __builtin_amdgcn_readlane(t_l, i0 + i);
+            const float w_i = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_l), i0 + i));
+            if (t_i != cur) {
+              if (cur >= 0) tile[(16 * wave + cur) * (kC2iTargets + 1) + lane] = acc;
+              acc = 0.0f;
+              cur = t_i;
+            }
+            acc += w_i * v[i];
+          }
+        }
+      }
+    }
+    if (cur >= 0) tile[(16 * wave + cur) * (kC2iTargets + 1) + lane] = acc;
+    __syncthreads();
+    // thread (wave, lane): element u0 + lane, channels c0 + wave + 4 i
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int c = c0 + wave + 4 * i;
+      if (c < Cg && u0 + lane < HW)
+        img_b[(size_t)c * HW + u0 + lane] =
+            tile[lane * (kC2iTargets + 1) + wave + 4 * i] + (bias != nullptr ? bias[c] : 0.0f);
+    }
+    __syncthreads();
+  }
+}
+
+struct Col2imLists {
+  int *count, *offset, *cursor, *sums, *src;
+  float* co;
+  size_t bytes;
+};
+Col2imLists col2im_lists_at(void* base, int H, int W, int M, int K, int P, int interp) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  const size_t HW = (size_t)H * W;
+  const size_t nnz = (size_t)M * K * (P > 0 ? P : 1) * (interp == 0 ? 1 : 4);
+  char* b = static_cast<char*>(base);
+  Col2imLists l;
+  size_t at = 0;
+  l.count = reinterpret_cast<int*>(b + at);
+  at += up(HW * 4);
+  l.offset = reinterpret_cast<int*>(b + at);
+  at += up((HW + 1) * 4);
+  l.cursor = reinterpret_cast<int*>(b + at);
+  at += up(HW * 4);
+  l.sums = reinterpret_cast<int*>(b + at);   // one per 4096 elements (the scan's tile sums)
+  at += up((HW / 4096 + 1) * 4);
+  l.src = reinterpret_cast<int*>(b + at);
+  at += up(nnz * 4);
+  l.co = reinterpret_cast<float*>(b + at);
+  at += up(nnz * 4);
+  l.bytes = at;
+  return l;
+}
+
+}  // namespace
+
+size_t col2im_lists_bytes(int H, int W, int M, int K, int P, int interp) {
+  const int64_t nnz = (int64_t)M * K * (P > 0 ? P : 1) * (interp == 0 ? 1 : 4);
+  if ((int64_t)H * W >= ((int64_t)1 << 31) - 1 || nnz >= ((int64_t)1 << 31)) return 0;
+  return col2im_lists_at(nullptr, H, W, M, K, P, interp).bytes;
+}
+
+int col2im_lists_build(const float* map, const float* wts, void* lists, int H, int W, int M,
+                       int K, int P, int interp, hipStream_t stream) {
+  const Col2imLists l = col2im_lists_at(lists, H, W, M, K, P, interp);
+  const int HW = H * W;
+  int rc = zero_fill(l.count, sizeof(int) * (size_t)HW, stream);
+  if (rc) return rc;
+  const dim3 grid((unsigned)ceil_div((int64_t)M * K, kBlock));
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((col2im_invert_kernel<INTERP, WEIGHTED, false>), grid, dim3(kBlock),
+                              stream, map, wts, H, W, M, K, P, l.count, (int*)nullptr,
+                              (float*)nullptr)));
+  const int tiles = (int)ceil_div(HW, kScanTile);
+  launch(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kBlock), stream, (const int*)l.count,
+         HW, l.sums);
+  launch(scan_sums_kernel, dim3(1), dim3(kBlock), stream, l.sums, tiles);
+  launch(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), stream, (const int*)l.count, HW,
+         (const int*)l.sums, l.offset, l.cursor);
+  SDK_DISPATCH_INTERP(interp, P,
+                      (launch((col2im_invert_kernel<INTERP, WEIGHTED, true>), grid, dim3(kBlock),
+                              stream, map, wts, H, W, M, K, P, l.cursor, l.src, l.co)));
+  launch(col2im_sort_kernel, dim3((unsigned)ceil_div(HW, kBlock)), dim3(kBlock), stream,
+         (const int*)l.offset, l.src, l.co, HW);
+  SDK_LAUNCH_CHECK("mapped_conv(inverted map)");
+  return SDK_OK;
+}
+
+int col2im_from_lists(const float* col, const float* bias, float* img, const void* lists,
+                      int64_t planes, int channels, int H, int W, int M, int K, int P, int interp,
+                      hipStream_t stream) {
+  const Col2imLists l = col2im_lists_at(const_cast<void*>(lists), H, W, M, K, P, interp);
+  const int HW = H * W;
+  const int64_t batch = planes / channels;
+  if (batch > 65535)
+    return fail(SDK_ERR_UNSUPPORTED, "mapped_conv: batch %lld too large", (long long)batch);
+  launch(col2im_gather_kernel, dim3((unsigned)ceil_div(HW, kC2iTargets), (unsigned)batch),
+         dim3(kBlock), stream, col, (const int*)l.offset, (const int*)l.src, (const float*)l.co,
+         bias, img, channels, HW, (size_t)M * K);
+  SDK_LAUNCH_CHECK("mapped_conv(col2im)");
   return SDK_OK;
 }
 
