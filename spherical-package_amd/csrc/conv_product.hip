@@ -118,28 +118,53 @@ __global__ __launch_bounds__(kPgThreads, 2) void product_gemm_kernel(
       for (int b = 0; b < 2; ++b)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
-#pragma unroll 8
-    for (int s = 0; s < NC * kPgChunk / 2; ++s) {
-      const float* ar = At + (2 * s + h) * kPgLd + wr + j;
-      const float* br = Bt + (2 * s + h) * kPgLd + wc + j;
-      const float a0 = ar[0], a1 = ar[32], b0 = br[0], b1 = br[32];
+    // (the operands of step s + 1 are read from LDS before the MFMAs of step s are issued)
+    constexpr int STEPS = NC * kPgChunk / 2;
+    const float* ar = At + h * kPgLd + wr + j;
+    const float* br = Bt + h * kPgLd + wc + j;
+    float a0 = ar[0], a1 = ar[32], b0 = br[0], b1 = br[32];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int sn1 = s + 1 < STEPS ? s + 1 : s;
+      const float na0 = ar[2 * sn1 * kPgLd], na1 = ar[2 * sn1 * kPgLd + 32];
+      const float nb0 = br[2 * sn1 * kPgLd], nb1 = br[2 * sn1 * kPgLd + 32];
+      __builtin_amdgcn_sched_barrier(0);
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
       acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
       acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
       acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      a0 = na0;
+      a1 = na1;
+      b0 = nb0;
+      b1 = nb1;
     }
     // D[pixel][column]: register v of lane l holds pixel 8 (v / 4) + 4 (l / 32) + v % 4 of
     // its 32, column l % 32
+    // (tiles inside the matrix store without tests, walking one pointer down the rows)
+    const bool whole = m0 + kPgTile <= M && j0 + kPgTile <= R;
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         const int jj = j0 + wc + 32 * b + j;
         float* out = col_b + (size_t)(m0 + wr + 32 * a + 4 * h) * R + jj;
+        if (whole) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int dm = 8 * (v >> 2) + (v & 3);
-          if (m0 + wr + 32 * a + 4 * h + dm < M && jj < R) out[(size_t)dm * R] = acc[a][b][v];
+          for (int g4 = 0; g4 < 4; ++g4) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              *out = acc[a][b][4 * g4 + e];
+              out += R;
+            }
+            out += 4 * (size_t)R;
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int dm = 8 * (v >> 2) + (v & 3);
+            if (m0 + wr + 32 * a + 4 * h + dm < M && jj < R) out[(size_t)dm * R] = acc[a][b][v];
+          }
         }
       }
   }
