@@ -205,10 +205,10 @@ int product_gemm_scatter(const ConvGeom& g, const float* pix, const float* map, 
   float* col = static_cast<float*>(workspace);
   void* own_lists = static_cast<char*>(workspace) + ((col_bytes(g) + 255) & ~(size_t)255);
   const int R = g.Cg * g.K;
-  // strips: about three rounds of two workgroups per CU over the whole grid
+  // strips: one round of two workgroups per CU over the whole grid
   const int m_tiles = (int)ceil_div(g.M, kPgTile);
   const int64_t others = ceil_div(R, kPgTile) * g.B;
-  const int strips = (int)std::max<int64_t>(1, std::min<int64_t>(m_tiles, ceil_div(1536, others)));
+  const int strips = (int)std::max<int64_t>(1, std::min<int64_t>(m_tiles, ceil_div(512, others)));
   const dim3 grid((unsigned)strips, (unsigned)ceil_div(R, kPgTile), (unsigned)g.B);
   const int nc = (int)ceil_div(g.Cp, kPgChunk);
 #define PG(NCv)                                                                             \
