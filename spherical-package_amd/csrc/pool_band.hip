@@ -271,17 +271,20 @@ bool dispatch_ipt(int ipt, const float* in, const float* map, float* out, int64_
 // range of planes, sums what reaches those rows in LDS and stores every element once, 16 bytes
 // at a time: no zero fill, no atomics in memory.  What can reach a band is fixed by the map:
 // a table (built once per map by unpool_band_rows_kernel, kept in the caller's workspace or
-// plan) holds per band the range of pooled rows with a tap in it.  A thread owns up to kUbIpt
-// pooled pixels of that range; the positions of their K taps inside the band are worked out
-// once, packed two to a register, and serve every plane, so per plane a pooled pixel costs
-// one index read, one gradient read, a select by the winning sample and one LDS add.
+// plan) holds per band the range of pooled rows with a tap in it.  A thread owns up to eight
+// pooled pixels of that range (four in average unpooling); the positions of their K taps
+// inside the band are worked out once, packed two to a register (in every workgroup, or once
+// per map into the plan: unpool_band_taps_kernel), and serve every plane, so per plane a
+// pooled pixel costs one index read, one gradient read, a select by the winning sample and
+// one LDS add.
 //
-// table: [0] 1 when every band's range fits (kUbIpt * 256 pooled pixels), else 0 (the caller
-// then takes its other route); [3] 1 when the build looked for pooled pixels that have the
-// same sample k at the same image pixel; [4] 1 when the packed taps behind the table are there; [8 + 2b] last pooled row of band b + 1 (0: nothing
-// reaches it); [9 + 2b] kUbBig - first pooled row; [8 + 2 nbands + b] raised when two such
-// pooled pixels meet in band b (where [3] is set and this is 0, average unpooling adds
-// band b sample by sample without atomics).  All grow by atomicMax from a zero fill.
+// table: [0] 1 when every band's range fits (kUbWindowPixels pooled pixels), else 0 (the
+// caller then takes its other route); [3] 1 when the build looked for pooled pixels that have
+// the same sample k at the same image pixel; [4] 1 when the packed taps behind the table are
+// there; [8 + 2b] last pooled row of band b + 1 (0: nothing reaches it); [9 + 2b] kUbBig -
+// first pooled row; [8 + 2 nbands + b] raised when two such pooled pixels meet in band b
+// (where [3] is set and this is 0, average unpooling adds band b sample by sample without
+// atomics).  All grow by atomicMax from a zero fill.
 // ---------------------------------------------------------------------------
 constexpr int kUbWindowPixels = 2048;   // pooled pixels a band's range may hold
 constexpr int kUbLdsBytes = 32 * 1024;
@@ -434,9 +437,9 @@ __device__ __forceinline__ unsigned packed_tap(const unsigned (&offp)[(K + 1) / 
 // Two planes per pass.  The LDS adds are compare-and-swap loops (the native float add to LDS
 // runs at a fraction of their rate on this GPU: 788 against 198 us for the average unpooling
 // of an 8 x 64 x 128 x 256 gradient), one after the other (issued as a batch, with the taps
-// outside the band masked or sent to a spare word, they were slower).  Max unpooling keeps the two planes apart (their
-// winners differ); average unpooling interleaves them, (plane 0, plane 1) per band element,
-// and adds both with one 64-bit swap per tap.  In a band where the table says that sample k of
+// outside the band masked or sent to a spare word, they were slower).  Max unpooling keeps
+// the two planes apart (their winners differ); average unpooling interleaves them, (plane 0,
+// plane 1) per band element, and adds both with one 64-bit swap per tap.  In a band where the table says that sample k of
 // different pooled pixels never shares an image pixel, average unpooling needs no atomics at
 // all: the samples are added one k at a time, a barrier between them, every lane reading,
 // adding to and writing back elements no other lane touches in that round, with all of a
