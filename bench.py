@@ -317,7 +317,7 @@ def bench_resample2(torch, ops, timer, steps, warmup, reps=8):
                                                        traffic=_measured_traffic("resample_to_map")))}
 
 
-def bench_pool3(torch, ops, timer, steps, warmup, reps=8):
+def bench_pool3(torch, ops, timer, steps, warmup, reps=8, with_cold=True):
     import workloads
     cfg = workloads.config3()
     dev = "cuda:0"
@@ -344,7 +344,7 @@ def bench_pool3(torch, ops, timer, steps, warmup, reps=8):
     # inputs used in turn, the last six outputs kept alive so that every call writes fresh
     # memory too (2 to 3 GB per row).  `ms` above is the steady state of a loop over one set
     # of tensors, part of which the cache holds from call to call; `cold_ms` is what HBM gives.
-    N = 6
+    N = 6 if with_cold else 1
     xs = [x] + [x.clone() for _ in range(N - 1)]
     gs = [g] + [g.clone() for _ in range(N - 1)]
     idxs = [idx] + [idx.clone() for _ in range(N - 1)]
@@ -358,22 +358,24 @@ def bench_pool3(torch, ops, timer, steps, warmup, reps=8):
             ring[k] = call(k)
         return fn
     cold = {}
-    cold["pool_forward"], _ = timer.run(rotating(lambda k: ops.mapped_max_pool(xs[k], m, None, K, 0)),
-                                        steps, warmup, reps=8)
-    cold["pool_backward"], _ = timer.run(rotating(
-        lambda k: ops.mapped_max_unpool(gs[k], idxs[k], m, None, H, W, K, 0)), steps, warmup, reps=8)
-    cold["avg_pool_forward"], _ = timer.run(rotating(lambda k: ops.mapped_avg_pool(xs[k], m, None, K, 0)),
+    if with_cold:
+        cold["pool_forward"], _ = timer.run(rotating(lambda k: ops.mapped_max_pool(xs[k], m, None, K, 0)),
                                             steps, warmup, reps=8)
-    cold["avg_pool_backward"], _ = timer.run(rotating(
-        lambda k: ops.mapped_avg_unpool(gs[k], m, None, H, W, K, 0)), steps, warmup, reps=8)
-    ys = [torch.empty_like(x) for _ in range(N)]
-    cold["copy_reference"], _ = timer.run(rotating(lambda k: ys[k].copy_(xs[k])), steps, warmup, reps=8)
-    del ys, xs, gs, idxs
+        cold["pool_backward"], _ = timer.run(rotating(
+            lambda k: ops.mapped_max_unpool(gs[k], idxs[k], m, None, H, W, K, 0)), steps, warmup, reps=8)
+        cold["avg_pool_forward"], _ = timer.run(rotating(lambda k: ops.mapped_avg_pool(xs[k], m, None, K, 0)),
+                                                steps, warmup, reps=8)
+        cold["avg_pool_backward"], _ = timer.run(rotating(
+            lambda k: ops.mapped_avg_unpool(gs[k], m, None, H, W, K, 0)), steps, warmup, reps=8)
+        ys = [torch.empty_like(x) for _ in range(N)]
+        cold["copy_reference"], _ = timer.run(rotating(lambda k: ys[k].copy_(xs[k])), steps, warmup, reps=8)
+        del ys, xs, gs, idxs
 
     def row(name, ms_, nbytes, entry):
         d = dict(ms=ms_, **_roof("hbm", nbytes, ms_, traffic=_measured_traffic(entry) if entry else None))
-        d["cold_ms"] = cold[name]
-        d["cold_frac"] = round(nbytes / (cold[name] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        if with_cold:
+            d["cold_ms"] = cold[name]
+            d["cold_frac"] = round(nbytes / (cold[name] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         return d
     return {"copy_reference": row("copy_reference", ms_c, 2 * _nbytes(x), None),
             "pool_forward": row("pool_forward", ms_f, fwd_bytes, "mapped_max_pool"),
@@ -490,6 +492,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of: conv4,conv4_bf16,conv4_split,conv1,resample2,pool3,ico5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cold", action="store_true",
+                    help="skip the second series of the pooling rows (tensors the cache does not hold)")
     ap.add_argument("--no-verify", action="store_true",
                     help="skip the oracle check of the timed configuration after the timed loop")
     args = ap.parse_args()
@@ -535,7 +539,8 @@ def main():
     if want("resample2"):
         kernels.update(bench_resample2(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
     if want("pool3"):
-        kernels.update(bench_pool3(torch, ops, timer, max(args.steps, 20), args.warmup + 3))
+        kernels.update(bench_pool3(torch, ops, timer, max(args.steps, 20), args.warmup + 3,
+                                   with_cold=not args.no_cold))
         torch.cuda.empty_cache()
     if want("ico5"):
         kernels.update(bench_ico5(torch, ops, timer, args.steps, args.warmup))
