@@ -12,6 +12,7 @@
 #include <algorithm>
 
 #include "sdk_host.hpp"
+#include "sdk_lane_runs.hpp"
 
 namespace sdk {
 
@@ -26,22 +27,30 @@ __global__ __launch_bounds__(kVoteBlock) void vote_clear_kernel(uint4* __restric
 // One thread per input pixel, grid.y over (batch element of this pass, channel): the plane
 // arithmetic is per workgroup, and the pixel's target (16 bytes of the map) and its label are
 // requested together.  A label outside [0, candidates) casts no vote (the reference would
-// write outside its histogram).
+// write outside its histogram).  Neighbouring lanes often vote for the same cell (pixels of a
+// label image that share a target): a run of them casts its votes with one atomic, from its
+// last lane.
 __global__ __launch_bounds__(kVoteBlock) void vote_kernel(
     const int64_t* __restrict__ labels, const int64_t* __restrict__ map,
     unsigned* __restrict__ votes, int in_pixels, int channels, int OH, int OW, int candidates,
     size_t element_stride) {
   const int pix = blockIdx.x * kVoteBlock + threadIdx.x;
-  if (pix >= in_pixels) return;
   const unsigned plane = blockIdx.y;
   const unsigned e = plane / (unsigned)channels, c = plane - e * (unsigned)channels;
-  const long long x = map[(size_t)pix * 2], y = map[(size_t)pix * 2 + 1];
-  const long long label = labels[(size_t)plane * in_pixels + pix];
-  if (x < 0 || x > OW - 1 || y < 0 || y > OH - 1 || label < 0 || label >= candidates) return;
+  const int at = min(pix, in_pixels - 1);
+  const long long x = map[(size_t)at * 2], y = map[(size_t)at * 2 + 1];
+  const long long label = labels[(size_t)plane * in_pixels + at];
+  const bool ok = pix < in_pixels && x >= 0 && x <= OW - 1 && y >= 0 && y <= OH - 1 &&
+                  label >= 0 && label < candidates;
   // channel offset in histogram elements as the reference has it (common/resample.h:127-129):
   // c * OH * OW, not c whole histograms, so the histograms of several channels overlap
-  atomicAdd(&votes[e * element_stride + (size_t)c * OH * OW +
-                   ((size_t)y * OW + (size_t)x) * candidates + (size_t)label], 1u);
+  const long long cell = ok ? (long long)(e * element_stride + (size_t)c * OH * OW +
+                                          ((size_t)y * OW + (size_t)x) * candidates +
+                                          (size_t)label)
+                            : -1;
+  const long long below = __shfl_up(cell, 1);
+  const LaneRuns runs(below == cell);
+  if (ok && runs.tail) atomicAdd(&votes[cell], (unsigned)(runs.dist + 1));
 }
 
 // One thread per output pixel, grid.y over (batch element of this pass, channel): index of
