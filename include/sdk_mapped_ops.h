@@ -184,6 +184,21 @@ int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const vo
                             int64_t batch, int64_t channels, int64_t num_textures,
                             int64_t tex_height, int64_t tex_width, int64_t height, int64_t width,
                             int32_t interp, int32_t dtype, sdk_stream_t stream);
+/* The buckets depend on quad_idx alone and can be kept between calls (the reference has no
+ * counterpart: uv_resample_layer.h:48-74 is stateless).  _plan_build fills a caller-owned
+ * buffer of sdk_resample_to_uv_maps_workspace_bytes() bytes (not 0); _planned is
+ * sdk_resample_to_uv_maps with that buffer, which it only reads, in place of the workspace:
+ * it launches the texture sums alone. */
+int sdk_resample_to_uv_maps_plan_build(const int64_t* quad_idx, void* plan, size_t plan_bytes,
+                                       int64_t num_textures, int64_t tex_height,
+                                       int64_t tex_width, int64_t height, int64_t width,
+                                       int32_t dtype, sdk_stream_t stream);
+int sdk_resample_to_uv_maps_planned(const void* input, const int64_t* quad_idx, const void* tex_uv,
+                                    void* textures, const void* plan, size_t plan_bytes,
+                                    int64_t batch, int64_t channels, int64_t num_textures,
+                                    int64_t tex_height, int64_t tex_width, int64_t height,
+                                    int64_t width, int32_t interp, int32_t dtype,
+                                    sdk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Voting resample (integer labels).  input [B,C,IH,IW] int64 labels in [0, num_candidates);

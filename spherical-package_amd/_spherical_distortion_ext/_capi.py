@@ -24,6 +24,8 @@ SIGNATURES = {
     "sdk_normalize_by_weight_sum": [_vp, _vp, ctypes.c_double, _i64, _i64, _i32, _vp],
     "sdk_resample_from_uv_maps": [_vp] * 4 + [_i64] * 7 + [_i32] * 2 + [_vp],
     "sdk_resample_to_uv_maps": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 2 + [_vp],
+    "sdk_resample_to_uv_maps_plan_build": [_vp, _vp, _sz] + [_i64] * 5 + [_i32, _vp],
+    "sdk_resample_to_uv_maps_planned": [_vp] * 5 + [_sz] + [_i64] * 7 + [_i32] * 2 + [_vp],
     "sdk_equirect_kernel_map": [_vp] + [_i64] * 6 + [_i32] * 2 + [_vp],
     "sdk_gnomonic_kernel_at": [_vp, _vp] + [_i64] * 3 + [ctypes.c_double] * 2 + [_i64] * 2
                               + [_i32, _vp],

@@ -695,6 +695,30 @@ def resample_from_uv_maps(textures, quad_idx, tex_uv, interp):
     return out
 
 
+def _uv_plan(ref, quad_idx, NT, TH, TW, H, W, nbytes):
+    """The image pixels bucketed by texture (sdk_resample_to_uv_maps_plan_build), kept per
+    quad_idx tensor like the other plans; None when the cache is off or cannot key the tensor
+    (the call then builds the buckets in its workspace)."""
+    if not _plan_cache_enabled:
+        return None
+    kq = _tensor_key(quad_idx)
+    if _uncacheable(kq):
+        return None
+    dt = _DTYPES[ref.dtype]
+    key = ("uv_scatter", ref.device, dt, kq, NT, TH, TW, H, W)
+    cur = torch.cuda.current_stream(ref.device)
+    ent = _cache_lookup(key, cur)
+    if ent is not None:
+        return ent.plan
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    plan = torch.empty(nbytes, dtype=torch.uint8, device=ref.device)
+    _capi.call("sdk_resample_to_uv_maps_plan_build", _ptr(quad_idx), _ptr(plan), nbytes, NT, TH,
+               TW, H, W, dt, _stream(ref))
+    _cache_insert(key, _PlanEntry(plan, nbytes, (quad_idx.untyped_storage(),), cur))
+    return plan
+
+
 def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp):
     _check(x, x=x, quad_idx=quad_idx, tex_uv=tex_uv)
     H, W = _uv_dims(quad_idx, tex_uv)
@@ -706,6 +730,12 @@ def resample_to_uv_maps(x, quad_idx, tex_uv, num_textures, tex_h, tex_w, interp)
     with torch.cuda.device(x.device):
         nws = _capi.load().sdk_resample_to_uv_maps_workspace_bytes(NT, TH, TW, H, W,
                                                                    _DTYPES[x.dtype])
+        plan = _uv_plan(x, quad_idx, NT, TH, TW, H, W, nws) if nws else None
+        if plan is not None:
+            _capi.call("sdk_resample_to_uv_maps_planned", _ptr(x), _ptr(quad_idx), _ptr(tex_uv),
+                       _ptr(out), _ptr(plan), nws, B, C, NT, TH, TW, H, W, int(interp),
+                       _DTYPES[x.dtype], _stream(x))
+            return out
         ws = torch.empty(nws, dtype=torch.uint8, device=x.device) if nws else None
         _capi.call("sdk_resample_to_uv_maps", _ptr(x), _ptr(quad_idx), _ptr(tex_uv), _ptr(out),
                    _ptr(ws), nws, B, C, NT, TH, TW, H, W, int(interp), _DTYPES[x.dtype],

@@ -1565,30 +1565,46 @@ static bool uv_by_texture_fits(int64_t NT, int64_t THW, size_t esz) {
   return NT <= kUvMaxTextures && THW * (int64_t)esz <= kUvLdsBytes;
 }
 
+// The image pixels bucketed by texture (a function of quad_idx alone) into `workspace`
+// (uv_layout bytes): offset[t] .. offset[t + 1] - 1 of `list` are texture t's pixels.
+static int build_uv_buckets(const int64_t* quad, void* workspace, int NT, int MP,
+                            hipStream_t stream) {
+  size_t off[4];
+  uv_layout(NT, MP, off);
+  char* ws = static_cast<char*>(workspace);
+  int* count = reinterpret_cast<int*>(ws + off[0]);
+  int* offset = reinterpret_cast<int*>(ws + off[1]);
+  int* cursor = reinterpret_cast<int*>(ws + off[2]);
+  int* list = reinterpret_cast<int*>(ws + off[3]);
+  int rc = zero_fill(count, off[1], stream);
+  if (rc != SDK_OK) return rc;
+  const dim3 pixel_grid((unsigned)ceil_div(MP, kBlock));
+  const int copies = uv_counter_copies(NT);
+  launch(uv_count_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, count);
+  launch(uv_scan_kernel, dim3(1), dim3(kBlock), stream, (const int*)count, NT, copies, offset,
+         cursor);
+  launch(uv_fill_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, cursor, list);
+  SDK_LAUNCH_CHECK("resample_to_uv_maps(bucket)");
+  return SDK_OK;
+}
+
 // The adjoint: with a workspace (and textures that fit in LDS) by texture, see
 // uv_texture_scatter_kernel; otherwise a zero fill and atomic adds in memory.
+// prebuilt: `workspace` already holds the buckets of this quad_idx (build_uv_buckets).
 template <typename T>
 static int launch_uv_scatter(const T* in, const int64_t* quad, const T* uv, T* textures,
                              void* workspace, size_t workspace_bytes, int64_t planes, int NT,
-                             int TH, int TW, int MP, int interp, hipStream_t stream) {
+                             int TH, int TW, int MP, int interp, hipStream_t stream,
+                             bool prebuilt = false) {
   const int THW = TH * TW;
   size_t off[4];
   if (workspace != nullptr && uv_by_texture_fits(NT, THW, sizeof(T)) &&
       workspace_bytes >= uv_layout(NT, MP, off)) {
     char* ws = static_cast<char*>(workspace);
-    int* count = reinterpret_cast<int*>(ws + off[0]);
     int* offset = reinterpret_cast<int*>(ws + off[1]);
-    int* cursor = reinterpret_cast<int*>(ws + off[2]);
     int* list = reinterpret_cast<int*>(ws + off[3]);
-    int rc = zero_fill(count, off[1], stream);
+    int rc = prebuilt ? SDK_OK : build_uv_buckets(quad, workspace, NT, MP, stream);
     if (rc != SDK_OK) return rc;
-    const dim3 pixel_grid((unsigned)ceil_div(MP, kBlock));
-    const int copies = uv_counter_copies(NT);
-    launch(uv_count_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, count);
-    launch(uv_scan_kernel, dim3(1), dim3(kBlock), stream, (const int*)count, NT, copies, offset,
-           cursor);
-    launch(uv_fill_kernel, pixel_grid, dim3(kBlock), stream, quad, NT, MP, copies, cursor, list);
-    SDK_LAUNCH_CHECK("resample_to_uv_maps(bucket)");
     // planes per workgroup: as many as LDS holds while the grid still fills the GPU; few
     // textures: several workgroups share one and add their parts to a zero-filled output
     int pl = 1;
@@ -2326,6 +2342,45 @@ int sdk_resample_to_uv_maps(const void* input, const int64_t* quad_idx, const vo
                                 workspace, workspace_bytes, planes, (int)num_textures,
                                 (int)tex_height, (int)tex_width, (int)(height * width), interp,
                                 (hipStream_t)stream));
+  return SDK_OK;
+}
+
+int sdk_resample_to_uv_maps_plan_build(const int64_t* quad_idx, void* plan, size_t plan_bytes,
+                                       int64_t num_textures, int64_t tex_height,
+                                       int64_t tex_width, int64_t height, int64_t width,
+                                       int32_t dtype, sdk_stream_t stream) {
+  SDK_REQUIRE(quad_idx && plan, "resample_to_uv_maps_plan_build: NULL pointer");
+  const size_t need = sdk_resample_to_uv_maps_workspace_bytes(num_textures, tex_height, tex_width,
+                                                              height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "resample_to_uv_maps_plan_build: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  return build_uv_buckets(quad_idx, plan, (int)num_textures, (int)(height * width),
+                          (hipStream_t)stream);
+}
+
+int sdk_resample_to_uv_maps_planned(const void* input, const int64_t* quad_idx, const void* tex_uv,
+                                    void* textures, const void* plan, size_t plan_bytes,
+                                    int64_t batch, int64_t channels, int64_t num_textures,
+                                    int64_t tex_height, int64_t tex_width, int64_t height,
+                                    int64_t width, int32_t interp, int32_t dtype,
+                                    sdk_stream_t stream) {
+  int rc = check_uv(input, quad_idx, tex_uv, textures, batch, channels, num_textures, tex_height,
+                    tex_width, height, width, "resample_to_uv_maps_planned");
+  if (rc) return rc;
+  SDK_REQUIRE(plan, "resample_to_uv_maps_planned: NULL pointer");
+  const size_t need = sdk_resample_to_uv_maps_workspace_bytes(num_textures, tex_height, tex_width,
+                                                              height, width, dtype);
+  if (need == 0 || plan_bytes < need)
+    return fail(SDK_ERR_WORKSPACE, "resample_to_uv_maps_planned: plan of %zu bytes, need %zu",
+                plan_bytes, need);
+  const int64_t planes = batch * channels;
+  if (planes == 0) return SDK_OK;
+  SDK_DISPATCH_DTYPE(dtype, return launch_uv_scatter<T>(
+                                (const T*)input, quad_idx, (const T*)tex_uv, (T*)textures,
+                                const_cast<void*>(plan), plan_bytes, planes, (int)num_textures,
+                                (int)tex_height, (int)tex_width, (int)(height * width), interp,
+                                (hipStream_t)stream, true));
   return SDK_OK;
 }
 

@@ -123,6 +123,42 @@ def test_uv_resample_both_directions(ops, oracle, case):
             assert (nws == 0) == (TH * TW * np.dtype(dt).itemsize > 65536)
 
 
+def test_uv_scatter_plan_matches_the_plain_call(ops, oracle):
+    """sdk_resample_to_uv_maps_plan_build / _planned: the buckets kept between calls (two calls
+    on one plan, different inputs), through the C ABI and through the operator's cache (on and
+    off); too small a plan is refused."""
+    from _spherical_distortion_ext import _capi
+    B, C, NT, TH, TW, H, W = 2, 5, 9, 12, 10, 40, 66
+    rng = np.random.default_rng(77)
+    _, quad, uv, y = _uv_case(rng, np.float32, B, C, NT, TH, TW, H, W, crowd=0.1)
+    tq, tu = _t(quad), _t(uv)
+    n = _capi.load().sdk_resample_to_uv_maps_workspace_bytes(NT, TH, TW, H, W, 0)
+    assert n > 0
+    plan = torch.empty(n, dtype=torch.uint8, device=DEV)
+    _capi.call("sdk_resample_to_uv_maps_plan_build", ops._ptr(tq), ops._ptr(plan), n, NT, TH, TW,
+               H, W, 0, ops._stream(tq))
+    for scale in (1.0, -0.5):
+        ty = _t(y * np.float32(scale))
+        out = torch.full((B, C, NT, TH, TW), 7.0, device=DEV)
+        _capi.call("sdk_resample_to_uv_maps_planned", ops._ptr(ty), ops._ptr(tq), ops._ptr(tu),
+                   ops._ptr(out), ops._ptr(plan), n, B, C, NT, TH, TW, H, W, 1, 0, ops._stream(ty))
+        want = oracle.resample_to_uv_maps(y * np.float32(scale), quad, uv, NT, TH, TW, 1)
+        assert relerr(_n(out), want) <= 1e-4
+        plain, _ = _to_uv_capi(ops, y * np.float32(scale), quad, uv, NT, TH, TW, 1, True)
+        assert relerr(_n(out), plain) <= 1e-5
+    with pytest.raises(RuntimeError, match="plan of"):
+        _capi.call("sdk_resample_to_uv_maps_plan_build", ops._ptr(tq), ops._ptr(plan), n - 1, NT,
+                   TH, TW, H, W, 0, ops._stream(tq))
+    want = oracle.resample_to_uv_maps(y, quad, uv, NT, TH, TW, 1)
+    for cached in (True, True, False):
+        ops.set_conv_plan_cache(cached)
+        try:
+            got = _n(ops.resample_to_uv_maps(_t(y), tq, tu, NT, TH, TW, 1))
+        finally:
+            ops.set_conv_plan_cache(True)
+        assert relerr(got, want) <= 1e-4
+
+
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("coherent", [True, False])
 def test_uv_scatter_with_crowded_texels(ops, oracle, interp, coherent):
