@@ -282,6 +282,12 @@ def bench_resample2(torch, ops, timer, steps, warmup, reps=8):
     ms_g, _ = timer.run(lambda: ops.resample_from_map(x, m, None, 1), steps, warmup, reps=8)
     ms_s, _ = timer.run(lambda: ops.resample_to_map_normalized(patches, m, None, H, W, 1, 1e-12),
                         steps, warmup, reps=8)
+    # what the tensor library's copy reaches on tensors of this size (x to a second buffer,
+    # 50 MB moved): the rate a 20 us memory-bound call can be held against
+    xc = torch.empty_like(x)
+    ms_c, _ = timer.run(lambda: xc.copy_(x), steps, warmup, reps=8)
+    copy_small = dict(ms=ms_c, **_roof("hbm", 2 * _nbytes(x), ms_c))
+    del xc
     gather_bytes = _nbytes(x, m, patches)
     scatter_bytes = _nbytes(patches, m, x) + H * W * 4.0
     # the UV way back: every image pixel reads its face's patch at (u, v); and its adjoint
@@ -305,7 +311,8 @@ def bench_resample2(torch, ops, timer, steps, warmup, reps=8):
     ms_v, _ = timer.run(lambda: ops.voting_resample_to_map(labels, vmap, H // 2, W // 2, 13),
                         steps, warmup, reps=8)
     vote_bytes = _nbytes(labels, vmap) + B * (H // 2) * (W // 2) * 8.0
-    return {"voting_resample": dict(ms=ms_v, **_roof("hbm", vote_bytes, ms_v)),
+    return {"copy_reference_50MB": copy_small,
+            "voting_resample": dict(ms=ms_v, **_roof("hbm", vote_bytes, ms_v)),
             "map_generation": dict(ms=ms_map, **_roof("hbm", map_bytes, ms_map)),
             "uv_gather": dict(ms=ms_uf, **_roof("hbm", uv_bytes, ms_uf,
                                                 traffic=_measured_traffic("resample_from_uv_maps"))),
