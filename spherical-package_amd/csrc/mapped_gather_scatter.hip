@@ -119,9 +119,15 @@ int zero_fill_gated(void* ptr, size_t bytes, hipStream_t stream, const int* gate
 // :85-107.  planes = B*C; image plane stride HW; out plane stride MP.
 // ---------------------------------------------------------------------------
 // PC planes per thread: 8 when there are many planes, fewer for small batches so that the grid
-// still fills the GPU and no lane idles on planes that do not exist (12 planes: 25 us with 4,
-// 32 us with 8 at configuration 2).
+// still fills the GPU and no lane idles on planes that do not exist.
 inline int planes_per_thread(int64_t planes) { return planes >= 32 ? 8 : (planes > 8 ? 4 : 2); }
+// ... of the gather: 2 below 16 planes (12 planes at configuration 2: 17.7 us with 2, 19.7 with
+// 4, 21.8 with 8; a wave's reads of a polar patch touch 30 to 40 lines per plane and row, and
+// with fewer planes in flight the rows of neighbouring waves still find each other's lines in
+// the vector cache)
+inline int gather_planes_per_thread(int64_t planes) {
+  return planes >= 32 ? 8 : (planes >= 16 ? 4 : 2);
+}
 
 template <typename T, int INTERP, bool WEIGHTED, int PC>
 __global__ __launch_bounds__(kBlock) void resample_from_map_kernel(
@@ -1303,7 +1309,7 @@ template <typename T>
 static int launch_resample_from_map(const T* image, const T* map, const T* wts, T* out,
                                     int64_t planes, int H, int W, int MP, int P, int interp,
                                     hipStream_t stream) {
-  const int pc = planes_per_thread(planes);
+  const int pc = gather_planes_per_thread(planes);
 #define RFM(PCv)                                                                              \
   SDK_DISPATCH_INTERP(interp, P,                                                              \
                       (launch((resample_from_map_kernel<T, INTERP, WEIGHTED, PCv>),           \
