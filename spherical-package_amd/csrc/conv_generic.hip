@@ -269,9 +269,9 @@ int launch_bias_grad(const T* gout, T* gbias, int64_t B, int64_t C, int64_t M,
   int rc = zero_fill(gbias, sizeof(T) * (size_t)C, stream);
   if (rc) return rc;
   if (B * M == 0 || C == 0) return SDK_OK;
-  // about 8192 blocks overall, at least 4096 elements each; slices of a multiple of 4 elements
+  // about 8192 blocks overall, at least 16384 elements each; slices of a multiple of 4 elements
   int64_t slices = std::min<int64_t>(std::max<int64_t>(1, ceil_div(8192, C * B)),
-                                     std::max<int64_t>(1, M / 4096));
+                                     std::max<int64_t>(1, M / 16384));
   int64_t per_block = ceil_div(ceil_div(M, slices), 4) * 4;
   slices = ceil_div(M, per_block);
   if (B * slices > 65535)
